@@ -1,0 +1,145 @@
+/*
+ * thundersvm_amd -- C ABI of the MI355X (gfx950) back end for ThunderSVM's SMO-training and
+ * kernel-evaluation path.
+ *
+ * Every entry point replaces one function of the reference's `svm_kernel::` namespace
+ * (include/thundersvm/kernel/kernelmatrix_kernel.h:12-68, include/thundersvm/kernel/smo_kernel.h:24-45),
+ * taking raw device pointers where the reference takes SyncArray<T>&.  All pointers are DEVICE
+ * pointers unless a parameter is named host_*; the caller owns every buffer, the library keeps
+ * none of them after the call returns.  Work is enqueued on `stream` (a hipStream_t, NULL = the
+ * default stream) and is asynchronous unless stated otherwise.
+ *
+ * Return value: 0 on success, a positive hipError_t value for a runtime failure, a negative
+ * TSVM_E* value for a rejected argument.  tsvm_last_error() describes the last failure of the
+ * calling thread.  (The reference throws std::bad_alloc on out-of-memory and aborts otherwise,
+ * include/thundersvm/util/common.h:33-42; the C++ wrappers above this ABI map
+ * hipErrorOutOfMemory (2) to std::bad_alloc.)
+ *
+ * float_type and kernel_type are double (the reference built with -DUSE_DOUBLE=ON).
+ */
+#ifndef THUNDERSVM_AMD_H
+#define THUNDERSVM_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TSVM_EINVAL (-1)   /* bad argument */
+#define TSVM_ENOSPC (-2)   /* caller workspace too small */
+
+/* SvmParam::KERNEL_TYPE (include/thundersvm/svmparam.h:36-38) */
+enum tsvm_kernel_type { TSVM_K_LINEAR = 0, TSVM_K_POLY = 1, TSVM_K_RBF = 2, TSVM_K_SIGMOID = 3, TSVM_K_PRECOMPUTED = 4 };
+
+typedef void *tsvm_stream;
+
+const char *tsvm_last_error(void);
+int tsvm_version(void);
+
+/* ---------------------------------------------------------------------------------------------
+ * KernelMatrix::get_rows / diag  (src/thundersvm/kernelmatrix.cpp:183-316)
+ * ------------------------------------------------------------------------------------------- */
+
+/* Row self dot products of a CSR matrix: self_dot[i] = sum_j val^2 in stored order
+ * (KernelMatrix constructor, kernelmatrix.cpp:195-205). */
+int tsvm_csr_self_dot(const double *val, const int64_t *row_ptr, int64_t n, double *self_dot, tsvm_stream stream);
+
+/* Row self dot products of a dense row-major matrix [n][ld], over columns 0..d-1 in ascending order. */
+int tsvm_dense_self_dot(const double *x, int64_t ld, int64_t n, int d, double *self_dot, tsvm_stream stream);
+
+/* diag[i] = kappa(x_i, x_i) from the self dot products (kernelmatrix.cpp:225-247; poly_kernel /
+ * sigmoid_kernel of kernelmatrix_kernel.cpp:94-108 applied to self_dot). */
+int tsvm_kernel_diag(const double *self_dot, int64_t n, int kernel_type, double gamma, double coef0, int degree,
+                     double *diag, tsvm_stream stream);
+
+/* Scatter CSR rows into a zero-filled dense row-major matrix [n][ld] (column c = feature id c):
+ * get_working_set_ins, kernelmatrix_kernel.cpp:9-25, applied to all rows once.  Entries with
+ * col >= ld are dropped (the test-row rule of kernelmatrix.cpp:392). */
+int tsvm_csr_to_dense(const double *val, const int *col, const int64_t *row_ptr, int64_t n, double *x, int64_t ld,
+                      tsvm_stream stream);
+
+/* Dense get_rows: out[i*ldo + j] = kappa(a_i, x_j), i < m, j < n, where a_i is row a_idx[i] of `a`
+ * (a_idx == NULL: row i).  Replaces get_working_set_ins + dns_csr_mul + RBF_kernel/poly_kernel/
+ * sigmoid_kernel (kernelmatrix.cpp:251-312; kernelmatrix_kernel.cpp:9-25,61-108,149-160) in one
+ * launch.  x is [n][ldx], a is [*][lda], both row-major fp64 with zero padding up to a multiple of
+ * 8 columns (ldx % 8 == 0, lda % 8 == 0, d <= min(ldx, lda)).  The dot product is accumulated over
+ * ascending column index with fused multiply-adds.  sd_x[j] / sd_a[a_idx[i]] are the self dot
+ * products (used by RBF only). */
+int tsvm_get_rows_dense(const double *x, int64_t ldx, int64_t n, int d, const double *sd_x, const double *a,
+                        int64_t lda, const int *a_idx, int m, const double *sd_a, int kernel_type, double gamma,
+                        double coef0, int degree, double *out, int64_t ldo, tsvm_stream stream);
+
+/* Transposed dense staging of selected CSR rows: w[c*m + i] = value of feature c in row idx[i]
+ * (idx == NULL: row i of the given CSR), w is [n_features][m] and is zero-filled first.
+ * The sparse-path counterpart of get_working_set_ins (kernelmatrix_kernel.cpp:9-25). */
+int tsvm_csr_stage_rows(const double *val, const int *col, const int64_t *row_ptr, const int *idx, int m,
+                        int n_features, double *w, tsvm_stream stream);
+
+/* CSR get_rows: out[i*ldo + j] = kappa(w_i, x_j) with x in CSR (n rows) and the m working rows
+ * staged by tsvm_csr_stage_rows.  Accumulates over the stored order of row j's non-zeros
+ * (dns_csr_mul, kernelmatrix_kernel.cpp:149-160) and applies the epilogue.  sd_w[i] are the
+ * working rows' self dot products (already gathered, length m). */
+int tsvm_get_rows_csr(const double *val, const int *col, const int64_t *row_ptr, int64_t n, const double *sd_x,
+                      const double *w, int m, const double *sd_w, int kernel_type, double gamma, double coef0,
+                      int degree, double *out, int64_t ldo, tsvm_stream stream);
+
+/* out[i] = in[idx[i]] for doubles (gathers working-set self dots). */
+int tsvm_gather_f64(const double *in, const int *idx, int m, double *out, tsvm_stream stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * smo_kernel.cpp
+ * ------------------------------------------------------------------------------------------- */
+
+/* update_f (smo_kernel.cpp:300-319): f[j] -= sum_{t<ws, alpha_diff[t]!=0} alpha_diff[t]*K_t[j], the
+ * sum taken in ascending t with fused multiply-adds.  Kernel row t starts at
+ * k_rows + slots[t]*ld (slots == NULL: slot t), so rows kept from the previous working set are
+ * addressed in place instead of being copied (csmosolver.cpp:75). */
+int tsvm_update_f(double *f, const double *alpha_diff, int ws_size, const double *k_rows, const int *slots,
+                  int64_t ld, int64_t n, tsvm_stream stream);
+
+/* Bytes of device workspace tsvm_c_smo_solve / tsvm_nu_smo_solve need for a working set of ws_size. */
+size_t tsvm_smo_solve_workspace(int ws_size);
+
+/* c_smo_solve (smo_kernel.cpp:12-125).  One workgroup solves the working-set sub-problem.
+ * diff[0] = initial low-up gap, diff[1] = number of inner iterations.  k_rows/slots/ld as in
+ * tsvm_update_f; workspace from tsvm_smo_solve_workspace. */
+int tsvm_c_smo_solve(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
+                     int ws_size, double Cp, double Cn, const double *k_rows, const int *slots, int64_t ld,
+                     const double *k_diag, double eps, double *diff, int max_iter, void *workspace,
+                     tsvm_stream stream);
+
+/* nu_smo_solve (smo_kernel.cpp:127-298), same conventions; diff[1] is left untouched as in the
+ * reference's CPU code. */
+int tsvm_nu_smo_solve(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
+                      int ws_size, double C, const double *k_rows, const int *slots, int64_t ld,
+                      const double *k_diag, double eps, double *diff, int max_iter, void *workspace,
+                      tsvm_stream stream);
+
+/* Bytes of device workspace tsvm_select_working_set needs for n instances. */
+size_t tsvm_select_workspace(int64_t n);
+
+/* sort_f + select_working_set fused (smo_kernel.cpp:321-332; csmosolver.cpp:123-165;
+ * nusmosolver.cpp:48-118): writes into out[0..n_select) the ids the reference's alternating scan
+ * over the (f, index)-sorted order would pick, skipping the ids in marked[0..n_marked).
+ * nu != 0 selects the four-pointer NuSMOSolver rule. */
+int tsvm_select_working_set(const double *f, const int *y, const double *alpha, int64_t n, double Cp, double Cn,
+                            const int *marked, int n_marked, int *out, int n_select, int nu, void *workspace,
+                            tsvm_stream stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * predict (kernelmatrix_kernel.cpp:110-147)
+ * ------------------------------------------------------------------------------------------- */
+
+/* sum_kernel_values: dec[r*P + p] = sum_{l in SV_i} coef[(j-1)*T + l]*K[r][l]
+ *                                  + sum_{l in SV_j} coef[i*T + l]*K[r][l] - rho[p]
+ * for every class pair p = (i<j), P = k(k-1)/2, T = total_sv, K is [n_instances][ldk]. */
+int tsvm_sum_kernel_values(const double *coef, int total_sv, const int *sv_start, const int *sv_count,
+                           const double *rho, const double *k_mat, int64_t ldk, double *dec_values, int n_classes,
+                           int64_t n_instances, tsvm_stream stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,168 @@
+"""GPU parity: KernelMatrix::get_rows / diag and sum_kernel_values through the C ABI vs the CPU oracle.
+
+Mirrors src/test/test_kernelmatrix.cpp (same fixture, same row sets, all four kernels) and adds
+ragged shapes.  Bars: linear and RBF bit-exact (the oracle runs its restated expf, expf_mode=1);
+poly / sigmoid within 1 float32 ulp and >= 99.9% identical (double pow/tanh rounded to float on both sides,
+but from two different math libraries); decision values 1e-9.
+"""
+import numpy as np
+import pytest
+import torch
+
+import gpu_util as G
+import oracle_lib as O
+from thundersvm_amd import capi
+from thundersvm_amd.data import load_libsvm, from_dense, CsrData
+
+pytestmark = pytest.mark.gpu
+FIXTURE = __import__("os").path.join(__import__("os").path.dirname(__file__), "golden", "test_dataset.txt")
+
+KERNELS = [
+    ("rbf", O.RBF, dict(gamma=0.5)),
+    ("poly", O.POLY, dict(gamma=0.5, degree=3, coef0=0.1)),
+    ("linear", O.LINEAR, dict()),
+    ("sigmoid", O.SIGMOID, dict(gamma=0.5, coef0=0.1)),
+]
+
+
+def _check(name, got, want):
+    if name in ("rbf", "linear"):
+        bad = np.flatnonzero(got.ravel() != want.ravel())
+        assert bad.size == 0, "%s: %d mismatching entries, first %s got %r want %r" % (
+            name, bad.size, bad[:1], got.ravel()[bad[:1]], want.ravel()[bad[:1]])
+    else:
+        assert G.float_ulp_diff(got, want).max() <= 1
+        assert (got != want).mean() < 1e-3
+
+
+def _device_km(data, kt, prm):
+    xh, nf, ld = G.dense_padded(data)
+    x_d = G.dev(xh)
+    sd = torch.empty(data.n, dtype=torch.float64, device="cuda")
+    capi.call("tsvm_dense_self_dot", G.ptr(x_d), ld, data.n, nf, G.ptr(sd), G.stream())
+    diag = torch.empty(data.n, dtype=torch.float64, device="cuda")
+    capi.call("tsvm_kernel_diag", G.ptr(sd), data.n, kt, prm.get("gamma", 0.0), prm.get("coef0", 0.0),
+              prm.get("degree", 3), G.ptr(diag), G.stream())
+    return x_d, nf, ld, sd, diag
+
+
+@pytest.mark.parametrize("name,kt,prm", KERNELS)
+def test_fixture_rows_and_diag(name, kt, prm):
+    data = load_libsvm(FIXTURE)
+    p = O.make_param(kernel_type=kt, expf_mode=1, **prm)
+    okm = O.KernelMatrix(data.ptr, data.col, data.val, p)
+    x_d, nf, ld, sd, diag = _device_km(data, kt, prm)
+    assert nf == okm.n_features
+    assert np.array_equal(G.host(sd), okm.self_dot())
+    _check(name, G.host(diag), okm.diag())
+    rows = np.arange(10, dtype=np.int32) * 3 + 4          # test_kernelmatrix.cpp:83-86
+    rows_d = G.dev(rows)
+    got = G.get_rows_dense(x_d, ld, data.n, nf, sd, x_d, ld, rows_d, len(rows), sd, kt, **prm)
+    _check(name, G.host(got), okm.get_rows(rows))
+    # get_rows(instances): first 10 rows as an external batch (test_kernelmatrix.cpp:108-118)
+    batch = data.rows(np.arange(10))
+    bh = batch.to_dense(ld)
+    b_d = G.dev(bh)
+    sdb = torch.empty(10, dtype=torch.float64, device="cuda")
+    capi.call("tsvm_dense_self_dot", G.ptr(b_d), ld, 10, ld, G.ptr(sdb), G.stream())
+    got = G.get_rows_dense(x_d, ld, data.n, nf, sd, b_d, ld, None, 10, sdb, kt, **prm)
+    _check(name, G.host(got), okm.get_rows_instances(batch.ptr, batch.col, batch.val))
+
+
+@pytest.mark.parametrize("n,d,m,density", [(1, 1, 1, 1.0), (130, 9, 1, 1.0), (257, 33, 129, 1.0), (1000, 54, 512, 0.3),
+                                           (515, 100, 64, 0.2), (2049, 784, 16, 0.2)])
+@pytest.mark.parametrize("name,kt,prm", KERNELS[:1] + KERNELS[2:3])
+def test_random_dense(name, kt, prm, n, d, m, density):
+    rng = np.random.default_rng(n * 1000 + d)
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    x[rng.random((n, d)) > density] = 0
+    data = from_dense(x)
+    if data.nnz == 0:
+        data = from_dense(np.ones((n, d), dtype=np.float32))
+    p = O.make_param(kernel_type=kt, expf_mode=1, **prm)
+    okm = O.KernelMatrix(data.ptr, data.col, data.val, p)
+    x_d, nf, ld, sd, diag = _device_km(data, kt, prm)
+    idx = rng.integers(0, n, size=m).astype(np.int32)
+    idx_d = G.dev(idx)
+    got = G.get_rows_dense(x_d, ld, n, nf, sd, x_d, ld, idx_d, m, sd, kt, **prm)
+    _check(name, G.host(got), okm.get_rows(idx))
+
+
+@pytest.mark.parametrize("name,kt,prm", KERNELS)
+def test_csr_path(name, kt, prm):
+    rng = np.random.default_rng(7)
+    n, d, m = 700, 3000, 70
+    ptr = [0]
+    col, val = [], []
+    for i in range(n):
+        k = rng.integers(0, 40)          # includes empty rows
+        c = np.sort(rng.choice(d, size=k, replace=False)) + 1
+        col.extend(c)
+        val.extend(rng.standard_normal(k).astype(np.float32))
+        ptr.append(len(col))
+    data = CsrData(ptr, col, np.asarray(val, dtype=np.float64))
+    p = O.make_param(kernel_type=kt, expf_mode=1, **prm)
+    okm = O.KernelMatrix(data.ptr, data.col, data.val, p)
+    nf = okm.n_features
+    val_d, col_d, ptr_d = G.dev(data.val), G.dev(data.col), G.dev(data.ptr)
+    sd = torch.empty(n, dtype=torch.float64, device="cuda")
+    capi.call("tsvm_csr_self_dot", G.ptr(val_d), G.ptr(ptr_d), n, G.ptr(sd), G.stream())
+    assert np.array_equal(G.host(sd), okm.self_dot())
+    idx = rng.integers(0, n, size=m).astype(np.int32)
+    idx_d = G.dev(idx)
+    w = torch.empty((nf, m), dtype=torch.float64, device="cuda")
+    capi.call("tsvm_csr_stage_rows", G.ptr(val_d), G.ptr(col_d), G.ptr(ptr_d), G.ptr(idx_d), m, nf, G.ptr(w), G.stream())
+    sdw = torch.empty(m, dtype=torch.float64, device="cuda")
+    capi.call("tsvm_gather_f64", G.ptr(sd), G.ptr(idx_d), m, G.ptr(sdw), G.stream())
+    out = torch.empty((m, n), dtype=torch.float64, device="cuda")
+    capi.call("tsvm_get_rows_csr", G.ptr(val_d), G.ptr(col_d), G.ptr(ptr_d), n, G.ptr(sd), G.ptr(w), m, G.ptr(sdw), kt,
+              prm.get("gamma", 0.0), prm.get("coef0", 0.0), prm.get("degree", 3), G.ptr(out), n, G.stream())
+    _check(name, G.host(out), okm.get_rows(idx))
+    # the dense path on the same data gives the same bits (both sum in ascending feature order)
+    xh, nf2, ld = G.dense_padded(data)
+    x_d = G.dev(xh)
+    got = G.get_rows_dense(x_d, ld, n, nf2, sd, x_d, ld, idx_d, m, sd, kt, **prm)
+    _check(name, G.host(got), okm.get_rows(idx))
+
+
+def test_out_of_range_test_features():
+    """Test rows with feature ids beyond the SV set's: dropped from the dot, kept in the self dot (kernelmatrix.cpp:290-295,392)."""
+    rng = np.random.default_rng(3)
+    sv = from_dense(rng.standard_normal((50, 6)).astype(np.float32))
+    tst = from_dense(rng.standard_normal((20, 9)).astype(np.float32))
+    p = O.make_param(kernel_type=O.RBF, gamma=0.3, expf_mode=1)
+    okm = O.KernelMatrix(sv.ptr, sv.col, sv.val, p)
+    want = okm.get_rows_instances(tst.ptr, tst.col, tst.val)
+    xh, nf, ld = G.dense_padded(sv)
+    x_d = G.dev(xh)
+    sd = torch.empty(sv.n, dtype=torch.float64, device="cuda")
+    capi.call("tsvm_dense_self_dot", G.ptr(x_d), ld, sv.n, nf, G.ptr(sd), G.stream())
+    # batch: CSR -> dense (columns >= ld dropped), self dot over the full CSR row
+    val_d, col_d, ptr_d = G.dev(tst.val), G.dev(tst.col), G.dev(tst.ptr)
+    b_d = torch.empty((tst.n, ld), dtype=torch.float64, device="cuda")
+    capi.call("tsvm_csr_to_dense", G.ptr(val_d), G.ptr(col_d), G.ptr(ptr_d), tst.n, G.ptr(b_d), ld, G.stream())
+    b_d[:, nf:] = 0
+    sdb = torch.empty(tst.n, dtype=torch.float64, device="cuda")
+    capi.call("tsvm_csr_self_dot", G.ptr(val_d), G.ptr(ptr_d), tst.n, G.ptr(sdb), G.stream())
+    got = G.get_rows_dense(x_d, ld, sv.n, nf, sd, b_d, ld, None, tst.n, sdb, O.RBF, gamma=0.3)
+    assert np.array_equal(G.host(got), want)
+
+
+@pytest.mark.parametrize("n_classes,rows", [(2, 5), (3, 150), (7, 333)])
+def test_sum_kernel_values(n_classes, rows):
+    rng = np.random.default_rng(n_classes)
+    cnt = rng.integers(1, 300, size=n_classes).astype(np.int32)
+    if n_classes == 7:
+        cnt[3] = 0
+    start = np.concatenate([[0], np.cumsum(cnt)[:-1]]).astype(np.int32)
+    T = int(cnt.sum())
+    coef = rng.standard_normal((n_classes - 1, T))
+    nb = n_classes * (n_classes - 1) // 2
+    rho = rng.standard_normal(nb)
+    k = rng.random((rows, T))
+    want = O.sum_kernel_values(coef, T, start, cnt, rho, k, n_classes, rows)
+    dec = torch.empty((rows, nb), dtype=torch.float64, device="cuda")
+    coef_d, start_d, cnt_d, rho_d, k_d = G.dev(coef), G.dev(start), G.dev(cnt), G.dev(rho), G.dev(k)
+    capi.call("tsvm_sum_kernel_values", G.ptr(coef_d), T, G.ptr(start_d), G.ptr(cnt_d), G.ptr(rho_d), G.ptr(k_d), T,
+              G.ptr(dec), n_classes, rows, G.stream())
+    assert np.abs(G.host(dec) - want).max() < 1e-9

@@ -1,0 +1,128 @@
+"""GPU parity: update_f, c_smo_solve, nu_smo_solve and the fused sort_f + select_working_set
+through the C ABI vs the CPU oracle.  All bit-exact / index-exact."""
+import numpy as np
+import pytest
+import torch
+
+import gpu_util as G
+import oracle_lib as O
+from thundersvm_amd import capi
+from thundersvm_amd.data import from_dense
+
+pytestmark = pytest.mark.gpu
+
+
+def _problem(n, d, seed, gamma=0.5):
+    rng = np.random.default_rng(seed)
+    y = np.where(rng.random(n) < 0.5, 1, -1).astype(np.int32)
+    x = (rng.standard_normal((n, d)) + 0.4 * y[:, None]).astype(np.float32)
+    data = from_dense(x)
+    p = O.make_param(kernel_type=O.RBF, gamma=gamma, expf_mode=1)
+    km = O.KernelMatrix(data.ptr, data.col, data.val, p)
+    return rng, y, km
+
+
+@pytest.mark.parametrize("n,ws,zero_frac", [(1, 1, 0.0), (1000, 1024, 0.5), (1537, 512, 0.0), (4099, 37, 0.9), (513, 2050, 0.3)])
+def test_update_f(n, ws, zero_frac):
+    rng = np.random.default_rng(n + ws)
+    ld = n + 3
+    k = rng.random((ws + 5, ld))
+    ad = rng.standard_normal(ws)
+    ad[rng.random(ws) < zero_frac] = 0
+    f = rng.standard_normal(n)
+    slots = rng.permutation(ws + 5)[:ws].astype(np.int32)
+    want = O.update_f(f, ad, np.ascontiguousarray(k[slots][:, :n]), n)
+    f_d, ad_d, k_d, s_d = G.dev(f), G.dev(ad), G.dev(k), G.dev(slots)
+    capi.call("tsvm_update_f", G.ptr(f_d), G.ptr(ad_d), ws, G.ptr(k_d), G.ptr(s_d), ld, n, G.stream())
+    assert np.array_equal(G.host(f_d), want)
+    # slots == NULL: identity
+    want = O.update_f(f, ad, np.ascontiguousarray(k[:ws, :n]), n)
+    f_d = G.dev(f)
+    capi.call("tsvm_update_f", G.ptr(f_d), G.ptr(ad_d), ws, G.ptr(k_d), None, ld, n, G.stream())
+    assert np.array_equal(G.host(f_d), want)
+
+
+def _solver_inputs(n, d, ws, seed, C, nu=False):
+    rng, y, km = _problem(n, d, seed)
+    alpha = np.zeros(n)
+    # a mid-training state: some alphas at bounds, some free
+    r = rng.random(n)
+    alpha[r < 0.2] = C
+    alpha[(r >= 0.2) & (r < 0.5)] = rng.random(int(((r >= 0.2) & (r < 0.5)).sum())) * C
+    f = rng.standard_normal(n)
+    ws_ids = rng.permutation(n)[:ws].astype(np.int32)
+    k_rows = km.get_rows(ws_ids)
+    diag = km.diag()
+    return y, alpha, f, ws_ids, k_rows, diag
+
+
+@pytest.mark.parametrize("n,ws,max_iter", [(300, 16, 100000), (2000, 1024, 100000), (1500, 512, 7), (700, 100, 100000), (64, 64, 0)])
+def test_c_smo_solve(n, ws, max_iter):
+    Cp, Cn, eps = 10.0, 4.0, 1e-3
+    y, alpha, f, ws_ids, k_rows, diag = _solver_inputs(n, 12, ws, n + ws, Cn)
+    a_want, ad_want, diff_want = O.c_smo_solve(y, f, alpha, ws_ids, Cp, Cn, k_rows, diag, n, eps, max_iter)
+    slots = np.random.default_rng(1).permutation(ws).astype(np.int32)
+    k_phys = np.empty_like(k_rows)
+    k_phys[slots] = k_rows
+    y_d, f_d, a_d, ws_d, k_d, s_d, dg_d = G.dev(y), G.dev(f), G.dev(alpha), G.dev(ws_ids), G.dev(k_phys), G.dev(slots), G.dev(diag)
+    ad_d = torch.zeros(ws, dtype=torch.float64, device="cuda")
+    diff_d = torch.zeros(2, dtype=torch.float64, device="cuda")
+    wsp = torch.empty(capi.kernel_lib().tsvm_smo_solve_workspace(ws), dtype=torch.uint8, device="cuda")
+    capi.call("tsvm_c_smo_solve", G.ptr(y_d), G.ptr(f_d), G.ptr(a_d), G.ptr(ad_d), G.ptr(ws_d), ws, Cp, Cn, G.ptr(k_d),
+              G.ptr(s_d), n, G.ptr(dg_d), eps, G.ptr(diff_d), max_iter, G.ptr(wsp), G.stream())
+    assert np.array_equal(G.host(diff_d), diff_want)
+    assert np.array_equal(G.host(a_d), a_want)
+    assert np.array_equal(G.host(ad_d), ad_want)
+    assert diff_want[1] > 0 or max_iter == 0 or diff_want[0] < eps
+
+
+@pytest.mark.parametrize("n,ws", [(300, 16), (2000, 1024), (900, 200)])
+def test_nu_smo_solve(n, ws):
+    Cc, eps = 1.0, 1e-3
+    y, alpha, f, ws_ids, k_rows, diag = _solver_inputs(n, 10, ws, 5 * n + ws, Cc)
+    a_want, ad_want, diff_want = O.nu_smo_solve(y, f, alpha, ws_ids, Cc, k_rows, diag, n, eps, 100000)
+    y_d, f_d, a_d, ws_d, k_d, dg_d = G.dev(y), G.dev(f), G.dev(alpha), G.dev(ws_ids), G.dev(k_rows), G.dev(diag)
+    ad_d = torch.zeros(ws, dtype=torch.float64, device="cuda")
+    diff_d = torch.zeros(2, dtype=torch.float64, device="cuda")
+    wsp = torch.empty(capi.kernel_lib().tsvm_smo_solve_workspace(ws), dtype=torch.uint8, device="cuda")
+    capi.call("tsvm_nu_smo_solve", G.ptr(y_d), G.ptr(f_d), G.ptr(a_d), G.ptr(ad_d), G.ptr(ws_d), ws, Cc, G.ptr(k_d), None,
+              n, G.ptr(dg_d), eps, G.ptr(diff_d), 100000, G.ptr(wsp), G.stream())
+    assert G.host(diff_d)[0] == diff_want[0]
+    assert np.array_equal(G.host(a_d), a_want)
+    assert np.array_equal(G.host(ad_d), ad_want)
+
+
+def _select_case(n, n_select, n_marked, seed, tie_mode, nu):
+    rng = np.random.default_rng(seed)
+    y = np.where(rng.random(n) < 0.5, 1, -1).astype(np.int32)
+    C = 2.0
+    alpha = np.zeros(n)
+    r = rng.random(n)
+    alpha[r < 0.25] = C
+    free = (r >= 0.25) & (r < 0.5)
+    alpha[free] = rng.random(int(free.sum())) * C
+    if tie_mode == 0:
+        f = rng.standard_normal(n)
+    elif tie_mode == 1:
+        f = -y.astype(np.float64)               # the initial state of C-SVC: massive ties
+    else:
+        f = np.round(rng.standard_normal(n), 1)  # few distinct values, signed zeros
+        f[rng.random(n) < 0.1] = -0.0
+    marked = rng.permutation(n)[:n_marked].astype(np.int32)
+    return f, y, alpha, C, marked
+
+
+@pytest.mark.parametrize("nu", [0, 1])
+@pytest.mark.parametrize("tie_mode", [0, 1, 2])
+@pytest.mark.parametrize("n,n_select,n_marked", [(2, 2, 0), (150, 128, 0), (150, 64, 64), (3200, 1024, 0), (3200, 512, 512),
+                                                 (100000, 512, 512), (70001, 1024, 0), (1100, 1024, 0), (1030, 512, 512)])
+def test_select_working_set(n, n_select, n_marked, tie_mode, nu):
+    f, y, alpha, C, marked = _select_case(n, n_select, n_marked, n + n_select + tie_mode, tie_mode, nu)
+    want = O.select_working_set(f, y, alpha, C, C, marked, n_select, nu=bool(nu))
+    f_d, y_d, a_d, m_d = G.dev(f), G.dev(y), G.dev(alpha), G.dev(marked)
+    out_d = torch.full((n_select,), -7, dtype=torch.int32, device="cuda")
+    wsp = torch.empty(capi.kernel_lib().tsvm_select_workspace(n), dtype=torch.uint8, device="cuda")
+    capi.call("tsvm_select_working_set", G.ptr(f_d), G.ptr(y_d), G.ptr(a_d), n, C, C, G.ptr(m_d) if n_marked else None,
+              n_marked, G.ptr(out_d), n_select, nu, G.ptr(wsp), G.stream())
+    got = G.host(out_d)
+    assert np.array_equal(got, want), "first mismatch at %s" % np.flatnonzero(got != want)[:5]

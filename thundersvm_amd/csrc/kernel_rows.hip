@@ -1,0 +1,444 @@
+// KernelMatrix::get_rows / diag and the predict reduction as gfx950 kernels.
+//
+// Reference behaviour restated here: src/thundersvm/kernelmatrix.cpp:183-316 and
+// src/thundersvm/kernel/kernelmatrix_kernel.cpp:9-160 (the USE_CUDA=OFF, USE_DOUBLE=ON build).
+#include "../../include/thundersvm_amd.h"
+#include "tsvm_device.h"
+#include "tsvm_internal.h"
+
+typedef double v4d __attribute__((ext_vector_type(4)));
+
+// ------------------------------------------------------------------------------------------------
+// Dense get_rows: fp64 MFMA tiled GEMM  out = epilogue(A_ws . X^T)
+//
+// v_mfma_f64_16x16x4f64 accumulates its four k-slots as a chain of fused multiply-adds in
+// ascending slot order, so feeding k-slots in ascending column order reproduces, bit for bit, the
+// serial  acc = fma(a[k], x[k], acc), k = 0..d-1  dot product.
+//
+// Operand layout of the instruction (64 lanes): A lane l holds A[row l%16][k l/16], B lane l
+// holds B[k l/16][col l%16], D register v of lane l holds D[row 4v + l/16][col l%16].
+// Working-set rows are the A operand (D rows), all-rows X is the B operand (D columns), so the 16
+// lanes l%16 of one store cover 16 consecutive j: a 128-byte run of an output row.
+//
+// Workgroup = 256 threads = 4 wavefronts in a 2x2 grid; each wavefront owns a 64x64 block of the
+// 128x128 output tile as 4x4 MFMA tiles (64 accumulator doubles per lane).  K is walked in tiles
+// of 8 columns staged through LDS in k-major order [8][130]: the stride of 130 doubles keeps both
+// the staging writes and the operand reads free of bank conflicts.
+// ------------------------------------------------------------------------------------------------
+#define GR_BM 128
+#define GR_BN 128
+#define GR_KT 8
+#define GR_LS 130
+
+__global__ __launch_bounds__(256) void get_rows_dense_kernel(
+    const double *__restrict__ x, int64_t ldx, int64_t n, int d, const double *__restrict__ sd_x,
+    const double *__restrict__ a, int64_t lda, const int *__restrict__ a_idx, int m, const double *__restrict__ sd_a,
+    KernelParam kp, double *__restrict__ out, int64_t ldo, unsigned m_blocks) {
+    __shared__ double As[GR_KT * GR_LS];
+    __shared__ double Bs[GR_KT * GR_LS];
+    __shared__ uint64_t exp_tab[32];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wi = wave >> 1, wj = wave & 1;
+    if (tid < 32) exp_tab[tid] = TSVM_EXP2F_TAB[tid];
+    __syncthreads();
+
+    const unsigned logical = xcd_remap(blockIdx.x, gridDim.x);
+    const int64_t j0 = (int64_t) (logical / m_blocks) * GR_BN;
+    const int i0 = (int) (logical % m_blocks) * GR_BM;
+
+    // staging assignment: thread -> (row = tid/2, 4 consecutive k at 4*(tid&1))
+    const int srow = tid >> 1;
+    const int skh = (tid & 1) * 4;
+    const double *a_ptr = nullptr;
+    const double *x_ptr = nullptr;
+    {
+        int ai = i0 + srow;
+        if (ai < m) {
+            int64_t r = a_idx ? (int64_t) a_idx[ai] : (int64_t) ai;
+            a_ptr = a + r * lda + skh;
+        }
+        int64_t xj = j0 + srow;
+        if (xj < n) x_ptr = x + xj * ldx + skh;
+    }
+
+    v4d acc[4][4];
+#pragma unroll
+    for (int ti = 0; ti < 4; ++ti)
+#pragma unroll
+        for (int tj = 0; tj < 4; ++tj) acc[ti][tj] = (v4d){0.0, 0.0, 0.0, 0.0};
+
+    const int n_kt = (d + GR_KT - 1) / GR_KT;
+    v4d ra = (v4d){0.0, 0.0, 0.0, 0.0}, rb = (v4d){0.0, 0.0, 0.0, 0.0};
+    if (a_ptr) ra = *(const v4d *) a_ptr;
+    if (x_ptr) rb = *(const v4d *) x_ptr;
+
+    const int lrow = lane & 15;
+    const int lk = lane >> 4;
+
+    for (int kt = 0; kt < n_kt; ++kt) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            As[(skh + e) * GR_LS + srow] = ra[e];
+            Bs[(skh + e) * GR_LS + srow] = rb[e];
+        }
+        __syncthreads();
+        if (kt + 1 < n_kt) {
+            if (a_ptr) ra = *(const v4d *) (a_ptr + (kt + 1) * GR_KT);
+            if (x_ptr) rb = *(const v4d *) (x_ptr + (kt + 1) * GR_KT);
+        }
+#pragma unroll
+        for (int ks = 0; ks < GR_KT / 4; ++ks) {
+            double af[4], bf[4];
+            const int kk = (ks * 4 + lk) * GR_LS;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                af[t] = As[kk + wi * 64 + t * 16 + lrow];
+                bf[t] = Bs[kk + wj * 64 + t * 16 + lrow];
+            }
+#pragma unroll
+            for (int ti = 0; ti < 4; ++ti)
+#pragma unroll
+                for (int tj = 0; tj < 4; ++tj)
+                    acc[ti][tj] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[ti], bf[tj], acc[ti][tj], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+
+    // epilogue + store
+    double sdj[4];
+    int64_t jj[4];
+#pragma unroll
+    for (int tj = 0; tj < 4; ++tj) {
+        jj[tj] = j0 + wj * 64 + tj * 16 + lrow;
+        sdj[tj] = (jj[tj] < n && sd_x) ? sd_x[jj[tj]] : 0.0;
+    }
+#pragma unroll
+    for (int ti = 0; ti < 4; ++ti) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int i = i0 + wi * 64 + ti * 16 + 4 * v + lk;
+            if (i >= m) continue;
+            double sdi = 0.0;
+            if (sd_a) sdi = sd_a[a_idx ? a_idx[i] : i];
+            double *orow = out + (int64_t) i * ldo;
+#pragma unroll
+            for (int tj = 0; tj < 4; ++tj) {
+                if (jj[tj] < n) orow[jj[tj]] = tsvm_epilogue(acc[ti][tj][v], sdi, sdj[tj], kp, exp_tab);
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// CSR get_rows: out[i][j] = epilogue( sum over row j's non-zeros, in stored order, of v * w[col][i] )
+// One workgroup = 256 working rows i (one per thread) x 16 consecutive rows j; the 16 dot products
+// live in registers and each thread stores its 16 results as one 128-byte run of output row i.
+// ------------------------------------------------------------------------------------------------
+#define CS_JB 16
+
+__global__ __launch_bounds__(256) void get_rows_csr_kernel(
+    const double *__restrict__ val, const int *__restrict__ col, const int64_t *__restrict__ row_ptr, int64_t n,
+    const double *__restrict__ sd_x, const double *__restrict__ w, int m, const double *__restrict__ sd_w,
+    KernelParam kp, double *__restrict__ out, int64_t ldo, unsigned i_blocks) {
+    __shared__ uint64_t exp_tab[32];
+    const int tid = threadIdx.x;
+    if (tid < 32) exp_tab[tid] = TSVM_EXP2F_TAB[tid];
+    __syncthreads();
+    const unsigned logical = xcd_remap(blockIdx.x, gridDim.x);
+    const int64_t j0 = (int64_t) (logical / i_blocks) * CS_JB;
+    const int i = (int) (logical % i_blocks) * 256 + tid;
+    const bool active = i < m;
+    const int ic = active ? i : 0;
+    double acc[CS_JB];
+#pragma unroll
+    for (int jj = 0; jj < CS_JB; ++jj) {
+        acc[jj] = 0.0;
+        const int64_t j = j0 + jj;
+        if (j < n) {
+            const int64_t e0 = row_ptr[j], e1 = row_ptr[j + 1];
+            double s = 0.0;
+            for (int64_t e = e0; e < e1; ++e) {
+                const double v = val[e];
+                const int c = col[e];
+                s = __builtin_fma(v, w[(int64_t) c * m + ic], s);
+            }
+            acc[jj] = s;
+        }
+    }
+    if (!active) return;
+    const double sdi = sd_w ? sd_w[i] : 0.0;
+    double *orow = out + (int64_t) i * ldo;
+#pragma unroll
+    for (int jj = 0; jj < CS_JB; ++jj) {
+        const int64_t j = j0 + jj;
+        if (j < n) orow[j] = tsvm_epilogue(acc[jj], sdi, sd_x ? sd_x[j] : 0.0, kp, exp_tab);
+    }
+}
+
+__global__ void fill_f64_kernel(double *p, int64_t count, double v) {
+    for (int64_t e = (int64_t) blockIdx.x * blockDim.x + threadIdx.x; e < count; e += (int64_t) gridDim.x * blockDim.x)
+        p[e] = v;
+}
+
+// w[c*m + i] = value of feature c in CSR row idx[i]; one wavefront per staged row.
+__global__ void csr_stage_rows_kernel(const double *__restrict__ val, const int *__restrict__ col,
+                                      const int64_t *__restrict__ row_ptr, const int *__restrict__ idx, int m,
+                                      int n_features, double *__restrict__ w) {
+    const int i = (int) ((blockIdx.x * (int64_t) blockDim.x + threadIdx.x) >> 6);
+    const int lane = threadIdx.x & 63;
+    if (i >= m) return;
+    const int64_t r = idx ? (int64_t) idx[i] : (int64_t) i;
+    for (int64_t e = row_ptr[r] + lane; e < row_ptr[r + 1]; e += 64) {
+        const int c = col[e];
+        if (c < n_features) w[(int64_t) c * m + i] = val[e];
+    }
+}
+
+// x[r*ld + c] = value of feature c in row r; one wavefront per row.
+__global__ void csr_to_dense_kernel(const double *__restrict__ val, const int *__restrict__ col,
+                                    const int64_t *__restrict__ row_ptr, int64_t n, double *__restrict__ x, int64_t ld) {
+    const int64_t r = (blockIdx.x * (int64_t) blockDim.x + threadIdx.x) >> 6;
+    const int lane = threadIdx.x & 63;
+    if (r >= n) return;
+    for (int64_t e = row_ptr[r] + lane; e < row_ptr[r + 1]; e += 64) {
+        const int c = col[e];
+        if (c < ld) x[r * ld + c] = val[e];
+    }
+}
+
+// self_dot[i] = serial fma chain over the row's values (kernelmatrix.cpp:195-205).
+__global__ void csr_self_dot_kernel(const double *__restrict__ val, const int64_t *__restrict__ row_ptr, int64_t n,
+                                    double *__restrict__ self_dot) {
+    const int64_t i = blockIdx.x * (int64_t) blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    double s = 0.0;
+    for (int64_t e = row_ptr[i]; e < row_ptr[i + 1]; ++e) s = __builtin_fma(val[e], val[e], s);
+    self_dot[i] = s;
+}
+
+__global__ void dense_self_dot_kernel(const double *__restrict__ x, int64_t ld, int64_t n, int d,
+                                      double *__restrict__ self_dot) {
+    const int64_t i = blockIdx.x * (int64_t) blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    double s = 0.0;
+    const double *r = x + i * ld;
+    for (int k = 0; k < d; ++k) s = __builtin_fma(r[k], r[k], s);
+    self_dot[i] = s;
+}
+
+__global__ void kernel_diag_kernel(const double *__restrict__ self_dot, int64_t n, KernelParam kp,
+                                   double *__restrict__ diag) {
+    const int64_t i = blockIdx.x * (int64_t) blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    double v;
+    switch (kp.kernel_type) {
+        case TSVM_RBF:
+        case TSVM_PRECOMPUTED: v = 1.0; break;
+        case TSVM_LINEAR: v = self_dot[i]; break;
+        default: v = tsvm_epilogue(self_dot[i], 0.0, 0.0, kp, TSVM_EXP2F_TAB); break;
+    }
+    diag[i] = v;
+}
+
+__global__ void gather_f64_kernel(const double *__restrict__ in, const int *__restrict__ idx, int m,
+                                  double *__restrict__ out) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < m) out[i] = in[idx[i]];
+}
+
+// ------------------------------------------------------------------------------------------------
+// sum_kernel_values (kernelmatrix_kernel.cpp:110-147).
+// One workgroup handles SK_R test rows.  For coefficient row c (0..k-2) and SV class s the segment
+// sum S[c][s] = sum_{l in SV_s} coef[c*T + l] * K[r][l] is accumulated by 256 threads striding over
+// the segment and tree-reduced through LDS; dec(i,j) = S[j-1][i] + S[i][j] - rho.  The summation
+// order differs from the reference's serial loop (results agree to ~1e-13 relative, inside the
+// 1e-6 absolute tolerance on decision values).
+// ------------------------------------------------------------------------------------------------
+#define SK_R 4
+#define SK_T 256
+
+__global__ __launch_bounds__(SK_T) void sum_kernel_values_kernel(
+    const double *__restrict__ coef, int total_sv, const int *__restrict__ sv_start, const int *__restrict__ sv_count,
+    const double *__restrict__ rho, const double *__restrict__ k_mat, int64_t ldk, double *__restrict__ dec,
+    int n_classes, int64_t n_instances) {
+    extern __shared__ double sm[];  // [SK_R][(k-1)*k] segment sums, then reduction scratch [SK_T/64][SK_R]
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int64_t r0 = (int64_t) blockIdx.x * SK_R;
+    const int km1 = n_classes - 1;
+    double *S = sm;
+    double *red = sm + SK_R * km1 * n_classes;
+    const int P = n_classes * km1 / 2;
+    for (int s = 0; s < n_classes; ++s) {
+        const int st = sv_start[s], cnt = sv_count[s];
+        for (int c = 0; c < km1; ++c) {
+            // every (c, s) is used by exactly one pair: (i=s, j=c+1) when c >= s, (i=c, j=s) when c < s
+            const double *cf = coef + (int64_t) c * total_sv + st;
+            double part[SK_R];
+#pragma unroll
+            for (int rr = 0; rr < SK_R; ++rr) part[rr] = 0.0;
+            for (int l = tid; l < cnt; l += SK_T) {
+                const double cv = cf[l];
+#pragma unroll
+                for (int rr = 0; rr < SK_R; ++rr) {
+                    const int64_t r = r0 + rr;
+                    if (r < n_instances) part[rr] = __builtin_fma(cv, k_mat[r * ldk + st + l], part[rr]);
+                }
+            }
+#pragma unroll
+            for (int rr = 0; rr < SK_R; ++rr) {
+                double v = part[rr];
+#pragma unroll
+                for (int msk = 32; msk >= 1; msk >>= 1) v += shfl_xor_f64(v, msk);
+                if (lane == 0) red[wave * SK_R + rr] = v;
+            }
+            __syncthreads();
+            if (tid < SK_R) {
+                double t = 0.0;
+                for (int wv = 0; wv < SK_T / 64; ++wv) t += red[wv * SK_R + tid];
+                S[(tid * km1 + c) * n_classes + s] = t;
+            }
+            __syncthreads();
+        }
+    }
+    __syncthreads();
+    for (int e = tid; e < SK_R * P; e += SK_T) {
+        const int rr = e / P, p = e % P;
+        const int64_t r = r0 + rr;
+        if (r >= n_instances) continue;
+        // decode pair index p -> (i, j)
+        int i = 0, rem = p;
+        while (rem >= n_classes - 1 - i) { rem -= n_classes - 1 - i; ++i; }
+        const int j = i + 1 + rem;
+        const double sum = S[(rr * km1 + (j - 1)) * n_classes + i] + S[(rr * km1 + i) * n_classes + j];
+        dec[r * P + p] = sum - rho[p];
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// C ABI
+// ------------------------------------------------------------------------------------------------
+static inline unsigned grid_for(int64_t n, int block) { return (unsigned) ((n + block - 1) / block); }
+
+extern "C" {
+
+int tsvm_csr_self_dot(const double *val, const int64_t *row_ptr, int64_t n, double *self_dot, tsvm_stream stream) {
+    TSVM_REQUIRE(n >= 0 && row_ptr && self_dot, "tsvm_csr_self_dot: bad argument");
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(csr_self_dot_kernel, dim3(grid_for(n, 256)), dim3(256), 0, tsvm_s(stream), val, row_ptr, n, self_dot);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+int tsvm_dense_self_dot(const double *x, int64_t ld, int64_t n, int d, double *self_dot, tsvm_stream stream) {
+    TSVM_REQUIRE(n >= 0 && x && self_dot && d >= 0 && d <= ld, "tsvm_dense_self_dot: bad argument");
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(dense_self_dot_kernel, dim3(grid_for(n, 256)), dim3(256), 0, tsvm_s(stream), x, ld, n, d, self_dot);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+int tsvm_kernel_diag(const double *self_dot, int64_t n, int kernel_type, double gamma, double coef0, int degree,
+                     double *diag, tsvm_stream stream) {
+    TSVM_REQUIRE(n >= 0 && self_dot && diag, "tsvm_kernel_diag: bad argument");
+    TSVM_REQUIRE(kernel_type >= 0 && kernel_type <= 4, "tsvm_kernel_diag: unknown kernel type %d", kernel_type);
+    if (n == 0) return 0;
+    KernelParam kp{kernel_type, degree, gamma, coef0};
+    hipLaunchKernelGGL(kernel_diag_kernel, dim3(grid_for(n, 256)), dim3(256), 0, tsvm_s(stream), self_dot, n, kp, diag);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+int tsvm_csr_to_dense(const double *val, const int *col, const int64_t *row_ptr, int64_t n, double *x, int64_t ld,
+                      tsvm_stream stream) {
+    TSVM_REQUIRE(n >= 0 && row_ptr && x && ld > 0, "tsvm_csr_to_dense: bad argument");
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(fill_f64_kernel, dim3(2048), dim3(256), 0, tsvm_s(stream), x, n * ld, 0.0);
+    TSVM_LAUNCH_CHECK();
+    hipLaunchKernelGGL(csr_to_dense_kernel, dim3(grid_for(n * 64, 256)), dim3(256), 0, tsvm_s(stream), val, col, row_ptr,
+                       n, x, ld);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+int tsvm_get_rows_dense(const double *x, int64_t ldx, int64_t n, int d, const double *sd_x, const double *a,
+                        int64_t lda, const int *a_idx, int m, const double *sd_a, int kernel_type, double gamma,
+                        double coef0, int degree, double *out, int64_t ldo, tsvm_stream stream) {
+    TSVM_REQUIRE(x && a && out, "tsvm_get_rows_dense: null pointer");
+    TSVM_REQUIRE(n >= 0 && m >= 0 && d >= 0, "tsvm_get_rows_dense: negative size");
+    TSVM_REQUIRE(ldx % 8 == 0 && lda % 8 == 0, "tsvm_get_rows_dense: ldx (%lld) and lda (%lld) must be multiples of 8",
+                 (long long) ldx, (long long) lda);
+    TSVM_REQUIRE(d <= ldx && d <= lda, "tsvm_get_rows_dense: d (%d) exceeds a leading dimension", d);
+    TSVM_REQUIRE(ldo >= n, "tsvm_get_rows_dense: ldo (%lld) < n (%lld)", (long long) ldo, (long long) n);
+    TSVM_REQUIRE(((uintptr_t) x % 32 == 0) && ((uintptr_t) a % 32 == 0), "tsvm_get_rows_dense: x and a must be 32-byte aligned");
+    TSVM_REQUIRE(kernel_type >= 0 && kernel_type <= 4, "tsvm_get_rows_dense: unknown kernel type %d", kernel_type);
+    TSVM_REQUIRE((kernel_type != TSVM_RBF && kernel_type != TSVM_PRECOMPUTED) || (sd_x && sd_a),
+                 "tsvm_get_rows_dense: RBF needs self dot products");
+    if (n == 0 || m == 0) return 0;
+    KernelParam kp{kernel_type, degree, gamma, coef0};
+    const unsigned m_blocks = (unsigned) ((m + GR_BM - 1) / GR_BM);
+    const int64_t n_blocks = (n + GR_BN - 1) / GR_BN;
+    TSVM_REQUIRE(n_blocks * m_blocks < (int64_t) 0x7fffffff, "tsvm_get_rows_dense: grid too large");
+    hipLaunchKernelGGL(get_rows_dense_kernel, dim3((unsigned) (n_blocks * m_blocks)), dim3(256), 0, tsvm_s(stream), x, ldx,
+                       n, d, sd_x, a, lda, a_idx, m, sd_a, kp, out, ldo, m_blocks);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+int tsvm_csr_stage_rows(const double *val, const int *col, const int64_t *row_ptr, const int *idx, int m,
+                        int n_features, double *w, tsvm_stream stream) {
+    TSVM_REQUIRE(row_ptr && w && m >= 0 && n_features >= 0, "tsvm_csr_stage_rows: bad argument");
+    if (m == 0 || n_features == 0) return 0;
+    hipLaunchKernelGGL(fill_f64_kernel, dim3(2048), dim3(256), 0, tsvm_s(stream), w, (int64_t) m * n_features, 0.0);
+    TSVM_LAUNCH_CHECK();
+    hipLaunchKernelGGL(csr_stage_rows_kernel, dim3(grid_for((int64_t) m * 64, 256)), dim3(256), 0, tsvm_s(stream), val, col,
+                       row_ptr, idx, m, n_features, w);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+int tsvm_get_rows_csr(const double *val, const int *col, const int64_t *row_ptr, int64_t n, const double *sd_x,
+                      const double *w, int m, const double *sd_w, int kernel_type, double gamma, double coef0,
+                      int degree, double *out, int64_t ldo, tsvm_stream stream) {
+    TSVM_REQUIRE(row_ptr && w && out, "tsvm_get_rows_csr: null pointer");
+    TSVM_REQUIRE(n >= 0 && m >= 0 && ldo >= n, "tsvm_get_rows_csr: bad size");
+    TSVM_REQUIRE(kernel_type >= 0 && kernel_type <= 4, "tsvm_get_rows_csr: unknown kernel type %d", kernel_type);
+    TSVM_REQUIRE((kernel_type != TSVM_RBF && kernel_type != TSVM_PRECOMPUTED) || (sd_x && sd_w),
+                 "tsvm_get_rows_csr: RBF needs self dot products");
+    if (n == 0 || m == 0) return 0;
+    KernelParam kp{kernel_type, degree, gamma, coef0};
+    const unsigned i_blocks = (unsigned) ((m + 255) / 256);
+    const int64_t j_blocks = (n + CS_JB - 1) / CS_JB;
+    TSVM_REQUIRE(j_blocks * i_blocks < (int64_t) 0x7fffffff, "tsvm_get_rows_csr: grid too large");
+    hipLaunchKernelGGL(get_rows_csr_kernel, dim3((unsigned) (j_blocks * i_blocks)), dim3(256), 0, tsvm_s(stream), val, col,
+                       row_ptr, n, sd_x, w, m, sd_w, kp, out, ldo, i_blocks);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+int tsvm_gather_f64(const double *in, const int *idx, int m, double *out, tsvm_stream stream) {
+    TSVM_REQUIRE(in && idx && out && m >= 0, "tsvm_gather_f64: bad argument");
+    if (m == 0) return 0;
+    hipLaunchKernelGGL(gather_f64_kernel, dim3(grid_for(m, 256)), dim3(256), 0, tsvm_s(stream), in, idx, m, out);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+int tsvm_sum_kernel_values(const double *coef, int total_sv, const int *sv_start, const int *sv_count,
+                           const double *rho, const double *k_mat, int64_t ldk, double *dec_values, int n_classes,
+                           int64_t n_instances, tsvm_stream stream) {
+    TSVM_REQUIRE(sv_start && sv_count && rho && dec_values, "tsvm_sum_kernel_values: null pointer");
+    TSVM_REQUIRE(n_classes >= 2 && n_classes <= 32, "tsvm_sum_kernel_values: n_classes %d outside [2, 32]", n_classes);
+    TSVM_REQUIRE(total_sv >= 0 && ldk >= total_sv && n_instances >= 0, "tsvm_sum_kernel_values: bad size");
+    if (n_instances == 0) return 0;
+    const size_t shm = sizeof(double) * ((size_t) SK_R * (n_classes - 1) * n_classes + (SK_T / 64) * SK_R);
+    hipLaunchKernelGGL(sum_kernel_values_kernel, dim3(grid_for(n_instances, SK_R)), dim3(SK_T), shm, tsvm_s(stream), coef,
+                       total_sv, sv_start, sv_count, rho, k_mat, ldk, dec_values, n_classes, n_instances);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,869 @@
+// SMO device kernels for gfx950: update_f, the single-workgroup local solvers and the fused
+// sort_f + select_working_set.
+//
+// Reference behaviour restated here: src/thundersvm/kernel/smo_kernel.cpp:12-332,
+// src/thundersvm/solver/csmosolver.cpp:123-165, src/thundersvm/solver/nusmosolver.cpp:48-118
+// (the USE_CUDA=OFF, USE_DOUBLE=ON build: first-index tie breaks, serial summation order).
+#include "../../include/thundersvm_amd.h"
+#include "tsvm_device.h"
+#include "tsvm_internal.h"
+
+#define TSVM_INF __builtin_inf()
+#define MAX_WS 1024
+
+// ------------------------------------------------------------------------------------------------
+// update_f: f[j] -= sum_t alpha_diff[t] * K_t[j]  (smo_kernel.cpp:300-319)
+// Bandwidth-bound stream over the ws x n kernel rows.  The non-zero alpha_diff entries are
+// compacted (in order) into LDS once per workgroup; rows with alpha_diff == 0 are never read.
+// Each thread owns two columns j and keeps eight row loads in flight per column.
+// ------------------------------------------------------------------------------------------------
+#define UF_T 256
+#define UF_CHUNK 1024
+#define UF_UNROLL 8
+
+__global__ __launch_bounds__(UF_T) void update_f_kernel(double *__restrict__ f, const double *__restrict__ alpha_diff,
+                                                        int ws, const double *__restrict__ k_rows,
+                                                        const int *__restrict__ slots, int64_t ld, int64_t n) {
+    __shared__ double s_ad[UF_CHUNK];
+    __shared__ int64_t s_off[UF_CHUNK];
+    __shared__ int s_wave_cnt[UF_T / 64];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int64_t j0 = (int64_t) blockIdx.x * (UF_T * 2) + tid;
+    const int64_t j1 = j0 + UF_T;
+    const bool a0 = j0 < n, a1 = j1 < n;
+    double sum0 = 0.0, sum1 = 0.0;
+    for (int base = 0; base < ws; base += UF_CHUNK) {
+        // ordered compaction of this chunk's non-zero entries: thread t owns entries 4t..4t+3
+        double v[4];
+        int cnt = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int t = base + tid * 4 + e;
+            v[e] = t < ws ? alpha_diff[t] : 0.0;
+            cnt += (v[e] != 0.0);
+        }
+        int incl = cnt;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            int o = __shfl_up(incl, d, 64);
+            if (lane >= d) incl += o;
+        }
+        if (lane == 63) s_wave_cnt[wave] = incl;
+        __syncthreads();
+        int wave_base = 0, total = 0;
+#pragma unroll
+        for (int w = 0; w < UF_T / 64; ++w) {
+            if (w < wave) wave_base += s_wave_cnt[w];
+            total += s_wave_cnt[w];
+        }
+        int pos = wave_base + incl - cnt;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (v[e] != 0.0) {
+                const int t = base + tid * 4 + e;
+                s_ad[pos] = v[e];
+                s_off[pos] = (int64_t) (slots ? slots[t] : t) * ld;
+                ++pos;
+            }
+        }
+        __syncthreads();
+        int u = 0;
+        for (; u + UF_UNROLL <= total; u += UF_UNROLL) {
+            double k0[UF_UNROLL], k1[UF_UNROLL];
+#pragma unroll
+            for (int e = 0; e < UF_UNROLL; ++e) {
+                const double *row = k_rows + s_off[u + e];
+                k0[e] = a0 ? row[j0] : 0.0;
+                k1[e] = a1 ? row[j1] : 0.0;
+            }
+#pragma unroll
+            for (int e = 0; e < UF_UNROLL; ++e) {
+                sum0 = __builtin_fma(s_ad[u + e], k0[e], sum0);
+                sum1 = __builtin_fma(s_ad[u + e], k1[e], sum1);
+            }
+        }
+        for (; u < total; ++u) {
+            const double *row = k_rows + s_off[u];
+            if (a0) sum0 = __builtin_fma(s_ad[u], row[j0], sum0);
+            if (a1) sum1 = __builtin_fma(s_ad[u], row[j1], sum1);
+        }
+        __syncthreads();
+    }
+    if (a0) f[j0] -= sum0;
+    if (a1) f[j1] -= sum1;
+}
+
+// ------------------------------------------------------------------------------------------------
+// Working-set block gather: kws[r*ws + t] = K_r[working_set[t]].  Turns the local solver's two
+// scattered row gathers per inner iteration (smo_kernel.cpp:50-52,107-110) into coalesced reads.
+// ------------------------------------------------------------------------------------------------
+__global__ void gather_ws_block_kernel(const double *__restrict__ k_rows, const int *__restrict__ slots, int64_t ld,
+                                       const int *__restrict__ working_set, int ws, double *__restrict__ kws) {
+    const int r = blockIdx.x;
+    const double *row = k_rows + (int64_t) (slots ? slots[r] : r) * ld;
+    for (int t = threadIdx.x; t < ws; t += blockDim.x) kws[(int64_t) r * ws + t] = row[working_set[t]];
+}
+
+// ------------------------------------------------------------------------------------------------
+// c_smo_solve (smo_kernel.cpp:12-114): one workgroup, one thread per working-set element.
+// f, alpha, y live in registers; per inner iteration: one reduction round for (i, up, low), one
+// for j2, two coalesced row reads of the gathered ws x ws block.  Reductions are lexicographic
+// (value, index) minima so ties resolve to the lowest index exactly as the serial loops do.
+// ------------------------------------------------------------------------------------------------
+template <int NW>
+__device__ __forceinline__ void block_argmin(const double *s_v, const int *s_i, double &v, int &i) {
+    v = s_v[0];
+    i = s_i[0];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) {
+        const double ov = s_v[w];
+        const int oi = s_i[w];
+        if (ov < v || (ov == v && oi < i)) { v = ov; i = oi; }
+    }
+}
+
+template <int NW>
+__global__ __launch_bounds__(NW * 64) void c_smo_solve_kernel(
+    const int *__restrict__ label, const double *__restrict__ f_val, double *__restrict__ alpha,
+    double *__restrict__ alpha_diff, const int *__restrict__ working_set, int ws, double Cp, double Cn,
+    const double *__restrict__ kws, const double *__restrict__ k_diag, double eps, double *__restrict__ diff,
+    int max_iter) {
+    __shared__ double s_kd[NW * 64];
+    __shared__ float s_y[NW * 64];
+    __shared__ double s_a[2][NW * 64];
+    __shared__ double s_f[2][NW * 64];
+    __shared__ double s_kI[NW * 64];
+    __shared__ double sA_v[NW], sA_l[NW], sB_v[NW];
+    __shared__ int sA_i[NW], sB_i[NW];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const bool active = tid < ws;
+    const int wsi = active ? working_set[tid] : 0;
+    double f = active ? f_val[wsi] : 0.0;
+    double a = active ? alpha[wsi] : 0.0;
+    const double a_old = a;
+    const double y = active ? (double) label[wsi] : 0.0;
+    const double kd = active ? k_diag[wsi] : 0.0;
+    s_kd[tid] = kd;
+    s_y[tid] = (float) y;
+    double local_eps = 0.0;
+    int numOfIter = 0;
+    while (true) {
+        const int par = numOfIter & 1;
+        s_a[par][tid] = a;
+        s_f[par][tid] = f;
+        // i = first argmin of f over I_up; low = max of f over I_low
+        double v = (active && is_I_up(a, y, Cp, Cn) && f < TSVM_INF) ? f : TSVM_INF;
+        int vi = tid;
+        double lw = (active && is_I_low(a, y, Cp, Cn) && f > -TSVM_INF) ? f : -TSVM_INF;
+        wave_argmin(v, vi);
+        lw = wave_max(lw);
+        if (lane == 0) { sA_v[wave] = v; sA_i[wave] = vi; sA_l[wave] = lw; }
+        __syncthreads();
+        double up_value;
+        int i;
+        block_argmin<NW>(sA_v, sA_i, up_value, i);
+        double low_value = sA_l[0];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) low_value = sA_l[w] > low_value ? sA_l[w] : low_value;
+        if (!(up_value < TSVM_INF)) i = 0;
+        const double local_diff = low_value - up_value;
+        if (numOfIter == 0) {
+            const double t = 0.1f * local_diff;
+            local_eps = eps > t ? eps : t;
+            if (tid == 0) diff[0] = local_diff;
+        }
+        if (numOfIter > max_iter || local_diff < local_eps) break;
+        const double kI = active ? kws[(int64_t) i * ws + tid] : 0.0;
+        s_kI[tid] = kI;
+        const double kd_i = s_kd[i];
+        // j2 = first argmin of -b^2/a over I_low with f > up
+        double ft = TSVM_INF;
+        if (active && -up_value > -f && is_I_low(a, y, Cp, Cn)) {
+            const double aIJ = kd_i + kd - 2 * kI;
+            const double bIJ = -up_value + f;
+            const double t = -bIJ * bIJ / aIJ;
+            if (t < TSVM_INF) ft = t;
+        }
+        int fi = tid;
+        wave_argmin(ft, fi);
+        if (lane == 0) { sB_v[wave] = ft; sB_i[wave] = fi; }
+        __syncthreads();
+        double min_t;
+        int j2;
+        block_argmin<NW>(sB_v, sB_i, min_t, j2);
+        if (!(min_t < TSVM_INF)) j2 = 0;
+        const double a_i = s_a[par][i], y_i = (double) s_y[i];
+        const double a_j = s_a[par][j2], y_j = (double) s_y[j2];
+        const double alpha_i_diff = y_i > 0 ? Cp - a_i : a_i;
+        const double q1 = y_j > 0 ? a_j : Cn - a_j;
+        const double q2 = (-up_value + s_f[par][j2]) / (kd_i + s_kd[j2] - 2 * s_kI[j2]);
+        const double alpha_j_diff = q1 < q2 ? q1 : q2;
+        const double l = alpha_i_diff < alpha_j_diff ? alpha_i_diff : alpha_j_diff;
+        if (tid == i) a += l * y;
+        if (tid == j2) a -= l * y;
+        const double kJ = active ? kws[(int64_t) j2 * ws + tid] : 0.0;
+        f = __builtin_fma(-l, kJ - kI, f);
+        ++numOfIter;
+    }
+    if (active) {
+        alpha_diff[tid] = -(a - a_old) * y;
+        alpha[wsi] = a;
+    }
+    if (tid == 0) diff[1] = (double) numOfIter;
+}
+
+// ------------------------------------------------------------------------------------------------
+// nu_smo_solve (smo_kernel.cpp:127-287).  Same structure with four extrema.  Keeps the CPU code's
+// j2n score, which uses kd[ip] and K[ip, .] (smo_kernel.cpp:239), and does not write diff[1].
+// ------------------------------------------------------------------------------------------------
+template <int NW>
+__global__ __launch_bounds__(NW * 64) void nu_smo_solve_kernel(
+    const int *__restrict__ label, const double *__restrict__ f_val, double *__restrict__ alpha,
+    double *__restrict__ alpha_diff, const int *__restrict__ working_set, int ws, double C,
+    const double *__restrict__ kws, const double *__restrict__ k_diag, double eps, double *__restrict__ diff,
+    int max_iter) {
+    __shared__ double s_kd[NW * 64];
+    __shared__ float s_y[NW * 64];
+    __shared__ double s_a[2][NW * 64];
+    __shared__ double s_f[2][NW * 64];
+    __shared__ double s_kIp[NW * 64], s_kIn[NW * 64];
+    __shared__ double sA_vp[NW], sA_vn[NW], sA_lp[NW], sA_ln[NW], sB_vp[NW], sB_vn[NW];
+    __shared__ int sA_ip[NW], sA_in[NW], sB_ip[NW], sB_in[NW];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const bool active = tid < ws;
+    const int wsi = active ? working_set[tid] : 0;
+    double f = active ? f_val[wsi] : 0.0;
+    double a = active ? alpha[wsi] : 0.0;
+    const double a_old = a;
+    const int yi_ = active ? label[wsi] : 0;
+    const double y = (double) yi_;
+    const double kd = active ? k_diag[wsi] : 0.0;
+    s_kd[tid] = kd;
+    s_y[tid] = (float) y;
+    double local_eps = 0.0;
+    int numOfIter = 0;
+    while (true) {
+        const int par = numOfIter & 1;
+        s_a[par][tid] = a;
+        s_f[par][tid] = f;
+        double vp = (active && yi_ > 0 && a < C && f < TSVM_INF) ? f : TSVM_INF;
+        double vn = (active && yi_ < 0 && a > 0 && f < TSVM_INF) ? f : TSVM_INF;
+        double lp = (active && yi_ > 0 && a > 0 && f > -TSVM_INF) ? f : -TSVM_INF;
+        double ln = (active && yi_ < 0 && a < C && f > -TSVM_INF) ? f : -TSVM_INF;
+        int ipi = tid, ini = tid;
+        wave_argmin(vp, ipi);
+        wave_argmin(vn, ini);
+        lp = wave_max(lp);
+        ln = wave_max(ln);
+        if (lane == 0) {
+            sA_vp[wave] = vp; sA_ip[wave] = ipi; sA_vn[wave] = vn; sA_in[wave] = ini;
+            sA_lp[wave] = lp; sA_ln[wave] = ln;
+        }
+        __syncthreads();
+        double up_value_p, up_value_n;
+        int ip, in;
+        block_argmin<NW>(sA_vp, sA_ip, up_value_p, ip);
+        block_argmin<NW>(sA_vn, sA_in, up_value_n, in);
+        if (!(up_value_p < TSVM_INF)) ip = 0;
+        if (!(up_value_n < TSVM_INF)) in = 0;
+        double low_value_p = sA_lp[0], low_value_n = sA_ln[0];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) {
+            low_value_p = sA_lp[w] > low_value_p ? sA_lp[w] : low_value_p;
+            low_value_n = sA_ln[w] > low_value_n ? sA_ln[w] : low_value_n;
+        }
+        const double dp = low_value_p - up_value_p, dn = low_value_n - up_value_n;
+        const double local_diff = dp > dn ? dp : dn;  // max(x, y) = x > y ? x : y
+        if (numOfIter == 0) {
+            const double t = 0.1 * local_diff;
+            local_eps = eps > t ? eps : t;
+            if (tid == 0) diff[0] = local_diff;
+        }
+        if (numOfIter > max_iter || local_diff < local_eps) break;
+        const double kIp = active ? kws[(int64_t) ip * ws + tid] : 0.0;
+        const double kIn = active ? kws[(int64_t) in * ws + tid] : 0.0;
+        s_kIp[tid] = kIp;
+        s_kIn[tid] = kIn;
+        const double kd_ip = s_kd[ip];
+        double ftp = TSVM_INF, ftn = TSVM_INF;
+        if (active && -up_value_p > -f && yi_ > 0 && a > 0) {
+            const double aIJ = kd_ip + kd - 2 * kIp;
+            const double bIJ = -up_value_p + f;
+            const double t = -bIJ * bIJ / aIJ;
+            if (t < TSVM_INF) ftp = t;
+        }
+        if (active && -up_value_n > -f && yi_ < 0 && a < C) {
+            const double aIJ = kd_ip + kd - 2 * kIp;
+            const double bIJ = -up_value_n + f;
+            const double t = -bIJ * bIJ / aIJ;
+            if (t < TSVM_INF) ftn = t;
+        }
+        int jpi = tid, jni = tid;
+        wave_argmin(ftp, jpi);
+        wave_argmin(ftn, jni);
+        if (lane == 0) { sB_vp[wave] = ftp; sB_ip[wave] = jpi; sB_vn[wave] = ftn; sB_in[wave] = jni; }
+        __syncthreads();
+        double f_val_j2p, f_val_j2n;
+        int j2p, j2n;
+        block_argmin<NW>(sB_vp, sB_ip, f_val_j2p, j2p);
+        block_argmin<NW>(sB_vn, sB_in, f_val_j2n, j2n);
+        if (!(f_val_j2p < TSVM_INF)) j2p = 0;
+        if (!(f_val_j2n < TSVM_INF)) j2n = 0;
+        int i, j2;
+        double up_value, kIj2, kI;
+        if (f_val_j2p < f_val_j2n) {
+            i = ip; j2 = j2p; up_value = up_value_p; kIj2 = s_kIp[j2p]; kI = kIp;
+        } else {
+            i = in; j2 = j2n; up_value = up_value_n; kIj2 = s_kIn[j2n]; kI = kIn;
+        }
+        const double a_i = s_a[par][i], y_i = (double) s_y[i];
+        const double a_j = s_a[par][j2], y_j = (double) s_y[j2];
+        const double alpha_i_diff = y_i > 0 ? C - a_i : a_i;
+        const double q1 = y_j > 0 ? a_j : C - a_j;
+        const double q2 = (-up_value + s_f[par][j2]) / (s_kd[i] + s_kd[j2] - 2 * kIj2);
+        const double alpha_j_diff = q1 < q2 ? q1 : q2;
+        const double l = alpha_i_diff < alpha_j_diff ? alpha_i_diff : alpha_j_diff;
+        if (tid == i) a += l * y;
+        if (tid == j2) a -= l * y;
+        const double kJ = active ? kws[(int64_t) j2 * ws + tid] : 0.0;
+        f = __builtin_fma(-l, kJ - kI, f);
+        ++numOfIter;
+    }
+    if (active) {
+        alpha_diff[tid] = -(a - a_old) * y;
+        alpha[wsi] = a;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Fused sort_f + select_working_set.
+//
+// The reference sorts (f, index) pairs ascending (smo_kernel.cpp:321-332) and then walks the
+// sorted order from both ends, alternately taking the next unmarked I_up element from the low end
+// and the next unmarked I_low element from the high end (csmosolver.cpp:123-165).  Only the first
+// n_select candidates from each end can ever be taken, so instead of sorting n pairs this selects,
+// per side, the n_select smallest composite keys (f-bits, index) among that side's candidates with
+// an MSB-first radix select (11-bit digits, one pass over the keys per digit, early exit once the
+// boundary bucket is exactly consumed), sorts those <= 1024 entries in LDS with a bitonic network
+// and replays the alternating scan on them.  The high end is handled by complementing key and
+// index, so every side is an ascending selection.  Composite keys are unique, which makes the
+// result independent of any thread ordering.
+//
+// Sides: C-SMO 0 = I_up (ascending), 1 = I_low (descending);
+//        nu-SMO 0 = I_up&y>0, 1 = I_up&y<0 (ascending), 2 = I_low&y>0, 3 = I_low&y<0 (descending).
+// ------------------------------------------------------------------------------------------------
+#define SEL_BINS 2048
+#define SEL_DIGIT 11
+#define SEL_MAX_PASS 9
+#define SEL_MAX_SIDES 4
+#define SEL_T 256
+
+struct SelState {
+    uint64_t pk;      // resolved high bits of the key part
+    uint32_t pi;      // resolved high bits of the index part
+    uint32_t k_rem;   // entries still to take from inside the boundary bucket
+    uint32_t done;    // 1: selection decided; entries matching the prefix are all taken
+    uint32_t pad;     // number of digits held by the prefix
+};
+
+struct SelWorkspace {   // device-side layout, carved from the caller's workspace
+    uint64_t *keys;     // [n] order-preserving transform of f
+    uint8_t *flags;     // [n] side membership bits
+    uint8_t *ind;       // [n] ws_indicator
+    uint32_t *hist;     // [SEL_MAX_PASS][SEL_MAX_SIDES][SEL_BINS]
+    SelState *state;    // [SEL_MAX_PASS + 1][SEL_MAX_SIDES]
+    uint32_t *count;    // [SEL_MAX_SIDES]
+    uint64_t *list_key; // [SEL_MAX_SIDES][MAX_WS]
+    uint32_t *list_idx; // [SEL_MAX_SIDES][MAX_WS]
+};
+
+static size_t sel_align(size_t v) { return (v + 255) & ~(size_t) 255; }
+
+static size_t sel_carve(void *base, int64_t n, SelWorkspace *w) {
+    size_t off = 0;
+    char *b = (char *) base;
+    auto take = [&](size_t bytes) { size_t o = off; off += sel_align(bytes); return b ? b + o : nullptr; };
+    void *keys = take(sizeof(uint64_t) * (size_t) n);
+    void *flags = take((size_t) n);
+    void *ind = take((size_t) n);
+    void *hist = take(sizeof(uint32_t) * SEL_MAX_PASS * SEL_MAX_SIDES * SEL_BINS);
+    void *state = take(sizeof(SelState) * (SEL_MAX_PASS + 1) * SEL_MAX_SIDES);
+    void *count = take(sizeof(uint32_t) * SEL_MAX_SIDES);
+    void *lk = take(sizeof(uint64_t) * SEL_MAX_SIDES * MAX_WS);
+    void *li = take(sizeof(uint32_t) * SEL_MAX_SIDES * MAX_WS);
+    if (w) {
+        w->keys = (uint64_t *) keys; w->flags = (uint8_t *) flags; w->ind = (uint8_t *) ind;
+        w->hist = (uint32_t *) hist; w->state = (SelState *) state; w->count = (uint32_t *) count;
+        w->list_key = (uint64_t *) lk; w->list_idx = (uint32_t *) li;
+    }
+    return off;
+}
+
+struct SelGeom {
+    int n_sides;
+    int n_pass;
+    int idx_bits;
+    uint32_t idx_mask;
+    uint32_t k;   // n_select
+};
+
+// digit p of the composite (key: 6 digits of 11,11,11,11,11,9 bits; then the index digits)
+__device__ __forceinline__ void sel_digit_geom(int p, int idx_bits, bool &is_key, int &shift, int &width) {
+    if (p < 6) {
+        is_key = true;
+        width = p < 5 ? SEL_DIGIT : 9;
+        shift = p < 5 ? 64 - SEL_DIGIT * (p + 1) : 0;
+    } else {
+        is_key = false;
+        const int rb = idx_bits - SEL_DIGIT * (p - 6);
+        width = rb < SEL_DIGIT ? rb : SEL_DIGIT;
+        shift = rb - width;
+    }
+}
+__device__ __forceinline__ int sel_resolved_key_bits(int p) { return p >= 6 ? 64 : SEL_DIGIT * p; }
+__device__ __forceinline__ int sel_resolved_idx_bits(int p, int idx_bits) {
+    if (p <= 6) return 0;
+    const int r = SEL_DIGIT * (p - 6);
+    return r < idx_bits ? r : idx_bits;
+}
+
+// -1 / 0 / +1: composite (k, i) versus the prefix on the bits resolved before pass p
+__device__ __forceinline__ int sel_cmp_prefix(uint64_t k, uint32_t i, const SelState &st, int p, int idx_bits) {
+    const int rk = sel_resolved_key_bits(p);
+    if (rk > 0) {
+        const uint64_t a = rk == 64 ? k : (k >> (64 - rk));
+        const uint64_t b = rk == 64 ? st.pk : (st.pk >> (64 - rk));
+        if (a < b) return -1;
+        if (a > b) return 1;
+    }
+    const int ri = sel_resolved_idx_bits(p, idx_bits);
+    if (ri > 0) {
+        const uint32_t a = i >> (idx_bits - ri);
+        const uint32_t b = st.pi >> (idx_bits - ri);
+        if (a < b) return -1;
+        if (a > b) return 1;
+    }
+    return 0;
+}
+
+__device__ __forceinline__ uint64_t f_to_key(double f) {
+    if (f == 0.0) f = 0.0;  // -0.0 and +0.0 compare equal in the reference's sort
+    uint64_t u = (uint64_t) __double_as_longlong(f);
+    return (u >> 63) ? ~u : (u | 0x8000000000000000ull);
+}
+
+__device__ __forceinline__ bool sel_side_descending(int side, int n_sides) { return n_sides == 2 ? side == 1 : side >= 2; }
+
+__global__ void sel_init_kernel(SelWorkspace w, int64_t n, SelGeom g) {
+    const int64_t gid = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t) gridDim.x * blockDim.x;
+    for (int64_t j = gid; j < n; j += stride) w.ind[j] = 0;
+    for (int64_t e = gid; e < (int64_t) SEL_MAX_PASS * SEL_MAX_SIDES * SEL_BINS; e += stride) w.hist[e] = 0;
+    if (gid < SEL_MAX_SIDES) {
+        w.count[gid] = 0;
+        SelState st;
+        st.pk = 0; st.pi = 0; st.k_rem = g.k; st.done = 0; st.pad = 0;
+        w.state[gid] = st;  // state before pass 0
+    }
+}
+
+__global__ void sel_mark_kernel(uint8_t *ind, const int *__restrict__ marked, int n_marked) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n_marked) ind[marked[i]] = 1;
+}
+
+// Computes, in LDS, the state after pass p-1's histogram has been consumed (st_out), from the
+// state before it (global state[p-1]) and hist[p-1].  Every workgroup does this redundantly.
+__device__ void sel_advance_state(const SelWorkspace &w, const SelGeom &g, int p, SelState *st_out /* LDS [sides] */,
+                                  uint32_t *scratch /* LDS [SEL_T + 8] */) {
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    for (int s = 0; s < g.n_sides; ++s) {
+        SelState st = w.state[(p - 1) * SEL_MAX_SIDES + s];
+        if (!st.done) {
+            const uint32_t *h = w.hist + ((size_t) (p - 1) * SEL_MAX_SIDES + s) * SEL_BINS;
+            uint32_t c[SEL_BINS / SEL_T];
+            uint32_t sum = 0;
+#pragma unroll
+            for (int e = 0; e < SEL_BINS / SEL_T; ++e) { c[e] = h[tid * (SEL_BINS / SEL_T) + e]; sum += c[e]; }
+            uint32_t incl = sum;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                uint32_t o = __shfl_up(incl, d, 64);
+                if (lane >= d) incl += o;
+            }
+            if (lane == 63) scratch[wave] = incl;
+            __syncthreads();
+            uint32_t wave_base = 0, total = 0;
+            for (int wv = 0; wv < SEL_T / 64; ++wv) {
+                if (wv < wave) wave_base += scratch[wv];
+                total += scratch[wv];
+            }
+            const uint32_t excl = wave_base + incl - sum;
+            if (total < st.k_rem) {
+                // fewer candidates than requested (only possible on the first digit): take them all
+                if (tid == 0) { st.done = 1; st.k_rem = total; st_out[s] = st; }
+            } else if (excl < st.k_rem && st.k_rem <= excl + sum) {
+                uint32_t below = excl;
+                int b = 0;
+                for (int e = 0; e < SEL_BINS / SEL_T; ++e) {
+                    if (below + c[e] >= st.k_rem) { b = tid * (SEL_BINS / SEL_T) + e; break; }
+                    below += c[e];
+                }
+                const uint32_t cb = h[b];
+                bool is_key; int shift, width;
+                sel_digit_geom(p - 1, g.idx_bits, is_key, shift, width);
+                if (is_key) st.pk |= (uint64_t) b << shift; else st.pi |= (uint32_t) b << shift;
+                st.k_rem -= below;
+                st.pad = (uint32_t) p;
+                if (cb == st.k_rem || p == g.n_pass) st.done = 1;
+                st_out[s] = st;
+            }
+            __syncthreads();
+        } else {
+            if (tid == 0) st_out[s] = st;
+            __syncthreads();
+        }
+    }
+    __syncthreads();
+}
+
+// Pass p: (p == 0: also builds keys/flags) histogram digit p of the not-yet-decided candidates.
+__global__ __launch_bounds__(SEL_T) void sel_pass_kernel(SelWorkspace w, const double *__restrict__ f,
+                                                         const int *__restrict__ y, const double *__restrict__ alpha,
+                                                         int64_t n, double Cp, double Cn, SelGeom g, int p) {
+    __shared__ uint32_t lhist[SEL_MAX_SIDES][SEL_BINS];
+    __shared__ SelState st[SEL_MAX_SIDES];
+    __shared__ uint32_t scratch[SEL_T + 16];
+    const int tid = threadIdx.x;
+    if (p == 0) {
+        if (tid < g.n_sides) st[tid] = w.state[tid];
+        __syncthreads();
+    } else {
+        sel_advance_state(w, g, p, st, scratch);
+        if (blockIdx.x == 0 && tid < g.n_sides) w.state[p * SEL_MAX_SIDES + tid] = st[tid];
+    }
+    bool any = false;
+    for (int s = 0; s < g.n_sides; ++s) any |= !st[s].done;
+    if (!any) return;
+    for (int e = tid; e < SEL_MAX_SIDES * SEL_BINS; e += SEL_T) (&lhist[0][0])[e] = 0;
+    __syncthreads();
+    bool is_key; int shift, width;
+    sel_digit_geom(p, g.idx_bits, is_key, shift, width);
+    const uint32_t dmask = (1u << width) - 1;
+    const int64_t stride = (int64_t) gridDim.x * SEL_T;
+    for (int64_t j = (int64_t) blockIdx.x * SEL_T + tid; j < n; j += stride) {
+        uint64_t key;
+        uint32_t fl;
+        if (p == 0) {
+            const double a = alpha[j];
+            const double yy = (double) y[j];
+            key = f_to_key(f[j]);
+            fl = 0;
+            if (!w.ind[j]) {
+                const bool up = is_I_up(a, yy, Cp, Cn), low = is_I_low(a, yy, Cp, Cn);
+                if (g.n_sides == 2) {
+                    fl = (up ? 1u : 0u) | (low ? 2u : 0u);
+                } else {
+                    fl = ((up && yy > 0) ? 1u : 0u) | ((up && yy < 0) ? 2u : 0u) | ((low && yy > 0) ? 4u : 0u) |
+                         ((low && yy < 0) ? 8u : 0u);
+                }
+            }
+            w.keys[j] = key;
+            w.flags[j] = (uint8_t) fl;
+        } else {
+            fl = w.flags[j];
+            if (!fl) continue;
+            key = w.keys[j];
+        }
+        for (int s = 0; s < g.n_sides; ++s) {
+            if (!(fl & (1u << s)) || st[s].done) continue;
+            const bool desc = sel_side_descending(s, g.n_sides);
+            const uint64_t k2 = desc ? ~key : key;
+            const uint32_t i2 = desc ? g.idx_mask - (uint32_t) j : (uint32_t) j;
+            if (sel_cmp_prefix(k2, i2, st[s], p, g.idx_bits) != 0) continue;
+            const uint32_t dg = is_key ? (uint32_t) (k2 >> shift) & dmask : (i2 >> shift) & dmask;
+            atomicAdd(&lhist[s][dg], 1u);
+        }
+    }
+    __syncthreads();
+    uint32_t *gh = w.hist + (size_t) p * SEL_MAX_SIDES * SEL_BINS;
+    for (int e = tid; e < g.n_sides * SEL_BINS; e += SEL_T) {
+        const uint32_t c = (&lhist[0][0])[e];
+        if (c) atomicAdd(&gh[e], c);
+    }
+}
+
+// After the last pass: finalise the state and append every selected candidate to its side's list.
+__global__ __launch_bounds__(SEL_T) void sel_compact_kernel(SelWorkspace w, int64_t n, SelGeom g) {
+    __shared__ SelState st[SEL_MAX_SIDES];
+    __shared__ uint32_t scratch[SEL_T + 16];
+    const int tid = threadIdx.x;
+    sel_advance_state(w, g, g.n_pass, st, scratch);
+    const int64_t stride = (int64_t) gridDim.x * SEL_T;
+    for (int64_t j = (int64_t) blockIdx.x * SEL_T + tid; j < n; j += stride) {
+        const uint32_t fl = w.flags[j];
+        if (!fl) continue;
+        const uint64_t key = w.keys[j];
+        for (int s = 0; s < g.n_sides; ++s) {
+            if (!(fl & (1u << s))) continue;
+            const bool desc = sel_side_descending(s, g.n_sides);
+            const uint64_t k2 = desc ? ~key : key;
+            const uint32_t i2 = desc ? g.idx_mask - (uint32_t) j : (uint32_t) j;
+            // all digits count as resolved once the side is done: compare on the digits it consumed
+            int cmp;
+            if (st[s].k_rem == 0 && st[s].done) {
+                cmp = 1;  // nothing to take on this side
+            } else {
+                // number of passes whose digit is part of the prefix = passes consumed by this side
+                cmp = sel_cmp_prefix(k2, i2, st[s], (int) st[s].pad, g.idx_bits);
+            }
+            if (cmp <= 0) {
+                const uint32_t pos = atomicAdd(&w.count[s], 1u);
+                if (pos < MAX_WS) {
+                    w.list_key[s * MAX_WS + pos] = k2;
+                    w.list_idx[s * MAX_WS + pos] = i2;
+                }
+            }
+        }
+    }
+}
+
+// Final step: sort each side's list, replay the alternating scan, write the selection.
+__device__ __forceinline__ bool comp_less(uint64_t ka, uint32_t ia, uint64_t kb, uint32_t ib) {
+    return ka < kb || (ka == kb && ia < ib);
+}
+
+__global__ __launch_bounds__(MAX_WS) void sel_final_kernel(SelWorkspace w, SelGeom g, int *__restrict__ out) {
+    __shared__ uint64_t sk[SEL_MAX_SIDES][MAX_WS];
+    __shared__ uint32_t si[SEL_MAX_SIDES][MAX_WS];
+    __shared__ int pos_other[SEL_MAX_SIDES][MAX_WS];  // position of the same instance in the paired side's list, or -1
+    __shared__ int cnt[SEL_MAX_SIDES];
+    __shared__ int conflict;
+    const int tid = threadIdx.x;
+    if (tid < SEL_MAX_SIDES) {
+        int c = tid < g.n_sides ? (int) w.count[tid] : 0;
+        cnt[tid] = c > MAX_WS ? MAX_WS : c;
+    }
+    if (tid == 0) conflict = 0;
+    __syncthreads();
+    for (int s = 0; s < g.n_sides; ++s) {
+        if (tid < cnt[s]) {
+            sk[s][tid] = w.list_key[s * MAX_WS + tid];
+            si[s][tid] = w.list_idx[s * MAX_WS + tid];
+        } else {
+            sk[s][tid] = ~0ull;
+            si[s][tid] = ~0u;
+        }
+    }
+    __syncthreads();
+    // bitonic sort, ascending composite, all sides at once
+    for (int size = 2; size <= MAX_WS; size <<= 1) {
+        for (int strd = size >> 1; strd > 0; strd >>= 1) {
+            const int partner = tid ^ strd;
+            if (partner > tid) {
+                const bool asc = (tid & size) == 0;
+                for (int s = 0; s < g.n_sides; ++s) {
+                    const uint64_t ka = sk[s][tid], kb = sk[s][partner];
+                    const uint32_t ia = si[s][tid], ib = si[s][partner];
+                    const bool sw = asc ? comp_less(kb, ib, ka, ia) : comp_less(ka, ia, kb, ib);
+                    if (sw) { sk[s][tid] = kb; sk[s][partner] = ka; si[s][tid] = ib; si[s][partner] = ia; }
+                }
+            }
+            __syncthreads();
+        }
+    }
+    // real instance ids; descending sides stored idx_mask - id
+    for (int s = 0; s < g.n_sides; ++s)
+        if (tid < cnt[s] && sel_side_descending(s, g.n_sides)) si[s][tid] = g.idx_mask - si[s][tid];
+    __syncthreads();
+    // position of each entry in the paired side's list (binary search on the paired side's order)
+    const int half = g.n_sides / 2;
+    for (int s = 0; s < g.n_sides; ++s) {
+        const int o = s < half ? s + half : s - half;
+        int res = -1;
+        if (tid < cnt[s]) {
+            // key of this instance as the paired side stores it: complement of ours (or of the complement)
+            const uint64_t k_here = sk[s][tid];
+            const uint64_t k_o = ~k_here;
+            const uint32_t id = si[s][tid];
+            const uint32_t i_o = sel_side_descending(o, g.n_sides) ? g.idx_mask - id : id;
+            int lo = 0, hi = cnt[o];
+            while (lo < hi) {
+                const int mid = (lo + hi) >> 1;
+                const uint32_t im = sel_side_descending(o, g.n_sides) ? g.idx_mask - si[o][mid] : si[o][mid];
+                if (comp_less(sk[o][mid], im, k_o, i_o)) lo = mid + 1; else hi = mid;
+            }
+            if (lo < cnt[o] && sk[o][lo] == k_o && si[o][lo] == id) res = lo;
+        }
+        pos_other[s][tid] = res;
+    }
+    __syncthreads();
+    const int k = (int) g.k;
+    // fast path: round r takes entry r of every side, provided no entry is already consumed by its pair
+    const int per = k / g.n_sides;
+    bool ok = (k % g.n_sides) == 0;
+    for (int s = 0; s < g.n_sides; ++s) ok = ok && cnt[s] >= per;
+    if (ok && tid < per) {
+        for (int s = 0; s < g.n_sides; ++s) {
+            const int po = pos_other[s][tid];
+            if (po < 0) continue;
+            // the paired side has consumed `tid` entries before this pick if it runs later in the round,
+            // `tid + 1` if it runs earlier
+            const int o = s < half ? s + half : s - half;
+            const int consumed = o < s ? tid + 1 : tid;
+            if (po < consumed) atomicOr(&conflict, 1);
+        }
+    }
+    __syncthreads();
+    if (ok && !conflict) {
+        if (tid < per)
+            for (int s = 0; s < g.n_sides; ++s) out[tid * g.n_sides + s] = (int) si[s][tid];
+        return;
+    }
+    // general path: replay the scan serially (small problems, or sides that run dry)
+    if (tid == 0) {
+        int ptr[SEL_MAX_SIDES] = {0, 0, 0, 0};
+        int n_sel = 0;
+        while (n_sel < k) {
+            bool progressed = false;
+            for (int s = 0; s < g.n_sides; ++s) {
+                const int o = s < half ? s + half : s - half;
+                while (ptr[s] < cnt[s] && pos_other[s][ptr[s]] >= 0 && pos_other[s][ptr[s]] < ptr[o]) ++ptr[s];
+                if (ptr[s] < cnt[s] && n_sel < k) {
+                    out[n_sel++] = (int) si[s][ptr[s]];
+                    ++ptr[s];
+                    progressed = true;
+                }
+            }
+            if (!progressed) break;
+        }
+        for (; n_sel < k; ++n_sel) out[n_sel] = -1;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// C ABI
+// ------------------------------------------------------------------------------------------------
+extern "C" {
+
+int tsvm_update_f(double *f, const double *alpha_diff, int ws_size, const double *k_rows, const int *slots,
+                  int64_t ld, int64_t n, tsvm_stream stream) {
+    TSVM_REQUIRE(f && alpha_diff && k_rows, "tsvm_update_f: null pointer");
+    TSVM_REQUIRE(ws_size >= 0 && n >= 0 && ld >= n, "tsvm_update_f: bad size (ws=%d n=%lld ld=%lld)", ws_size,
+                 (long long) n, (long long) ld);
+    if (n == 0 || ws_size == 0) return 0;
+    const unsigned grid = (unsigned) ((n + UF_T * 2 - 1) / (UF_T * 2));
+    hipLaunchKernelGGL(update_f_kernel, dim3(grid), dim3(UF_T), 0, tsvm_s(stream), f, alpha_diff, ws_size, k_rows, slots,
+                       ld, n);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+size_t tsvm_smo_solve_workspace(int ws_size) {
+    if (ws_size < 0) return 0;
+    return sizeof(double) * (size_t) ws_size * (size_t) ws_size + 256;
+}
+
+static int launch_gather(const double *k_rows, const int *slots, int64_t ld, const int *working_set, int ws,
+                         void *workspace, hipStream_t s) {
+    hipLaunchKernelGGL(gather_ws_block_kernel, dim3(ws), dim3(ws < 256 ? 64 : 256), 0, s, k_rows, slots, ld, working_set,
+                       ws, (double *) workspace);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+#define TSVM_DISPATCH_NW(KERNEL, ...)                                                                          \
+    do {                                                                                                       \
+        const int nw_ = (ws_size + 63) / 64;                                                                   \
+        if (nw_ <= 1) hipLaunchKernelGGL(KERNEL<1>, dim3(1), dim3(64), 0, s, __VA_ARGS__);                      \
+        else if (nw_ <= 2) hipLaunchKernelGGL(KERNEL<2>, dim3(1), dim3(128), 0, s, __VA_ARGS__);                \
+        else if (nw_ <= 4) hipLaunchKernelGGL(KERNEL<4>, dim3(1), dim3(256), 0, s, __VA_ARGS__);                \
+        else if (nw_ <= 8) hipLaunchKernelGGL(KERNEL<8>, dim3(1), dim3(512), 0, s, __VA_ARGS__);                \
+        else hipLaunchKernelGGL(KERNEL<16>, dim3(1), dim3(1024), 0, s, __VA_ARGS__);                            \
+    } while (0)
+
+int tsvm_c_smo_solve(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
+                     int ws_size, double Cp, double Cn, const double *k_rows, const int *slots, int64_t ld,
+                     const double *k_diag, double eps, double *diff, int max_iter, void *workspace,
+                     tsvm_stream stream) {
+    TSVM_REQUIRE(y && f_val && alpha && alpha_diff && working_set && k_rows && k_diag && diff && workspace,
+                 "tsvm_c_smo_solve: null pointer");
+    TSVM_REQUIRE(ws_size >= 1 && ws_size <= MAX_WS, "tsvm_c_smo_solve: ws_size %d outside [1, %d]", ws_size, MAX_WS);
+    hipStream_t s = tsvm_s(stream);
+    int rc = launch_gather(k_rows, slots, ld, working_set, ws_size, workspace, s);
+    if (rc) return rc;
+    const double *kws = (const double *) workspace;
+    TSVM_DISPATCH_NW(c_smo_solve_kernel, y, f_val, alpha, alpha_diff, working_set, ws_size, Cp, Cn, kws, k_diag, eps, diff,
+                     max_iter);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+int tsvm_nu_smo_solve(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
+                      int ws_size, double C, const double *k_rows, const int *slots, int64_t ld,
+                      const double *k_diag, double eps, double *diff, int max_iter, void *workspace,
+                      tsvm_stream stream) {
+    TSVM_REQUIRE(y && f_val && alpha && alpha_diff && working_set && k_rows && k_diag && diff && workspace,
+                 "tsvm_nu_smo_solve: null pointer");
+    TSVM_REQUIRE(ws_size >= 1 && ws_size <= MAX_WS, "tsvm_nu_smo_solve: ws_size %d outside [1, %d]", ws_size, MAX_WS);
+    hipStream_t s = tsvm_s(stream);
+    int rc = launch_gather(k_rows, slots, ld, working_set, ws_size, workspace, s);
+    if (rc) return rc;
+    const double *kws = (const double *) workspace;
+    TSVM_DISPATCH_NW(nu_smo_solve_kernel, y, f_val, alpha, alpha_diff, working_set, ws_size, C, kws, k_diag, eps, diff,
+                     max_iter);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+size_t tsvm_select_workspace(int64_t n) {
+    if (n < 0) return 0;
+    return sel_carve(nullptr, n, nullptr) + 256;
+}
+
+int tsvm_select_working_set(const double *f, const int *y, const double *alpha, int64_t n, double Cp, double Cn,
+                            const int *marked, int n_marked, int *out, int n_select, int nu, void *workspace,
+                            tsvm_stream stream) {
+    TSVM_REQUIRE(f && y && alpha && out && workspace, "tsvm_select_working_set: null pointer");
+    TSVM_REQUIRE(n >= 1 && n <= 0x7fffffffLL, "tsvm_select_working_set: n %lld outside [1, 2^31)", (long long) n);
+    TSVM_REQUIRE(n_select >= 0 && n_select <= MAX_WS, "tsvm_select_working_set: n_select %d outside [0, %d]", n_select,
+                 MAX_WS);
+    TSVM_REQUIRE(n_marked >= 0 && (n_marked == 0 || marked), "tsvm_select_working_set: bad marked list");
+    if (n_select == 0) return 0;
+    hipStream_t s = tsvm_s(stream);
+    SelWorkspace w;
+    void *base = (void *) (((uintptr_t) workspace + 255) & ~(uintptr_t) 255);
+    sel_carve(base, n, &w);
+    SelGeom g;
+    g.n_sides = nu ? 4 : 2;
+    int bits = 1;
+    while (((int64_t) 1 << bits) < n) ++bits;
+    g.idx_bits = bits;
+    g.idx_mask = (uint32_t) (((uint64_t) 1 << bits) - 1);
+    g.n_pass = 6 + (bits + SEL_DIGIT - 1) / SEL_DIGIT;
+    g.k = (uint32_t) n_select;
+    const unsigned grid = (unsigned) std::min<int64_t>((n + SEL_T - 1) / SEL_T, 1024);
+    hipLaunchKernelGGL(sel_init_kernel, dim3(grid), dim3(SEL_T), 0, s, w, n, g);
+    TSVM_LAUNCH_CHECK();
+    if (n_marked > 0) {
+        hipLaunchKernelGGL(sel_mark_kernel, dim3((n_marked + 255) / 256), dim3(256), 0, s, w.ind, marked, n_marked);
+        TSVM_LAUNCH_CHECK();
+    }
+    for (int p = 0; p < g.n_pass; ++p) {
+        hipLaunchKernelGGL(sel_pass_kernel, dim3(grid), dim3(SEL_T), 0, s, w, f, y, alpha, n, Cp, Cn, g, p);
+        TSVM_LAUNCH_CHECK();
+    }
+    hipLaunchKernelGGL(sel_compact_kernel, dim3(grid), dim3(SEL_T), 0, s, w, n, g);
+    TSVM_LAUNCH_CHECK();
+    hipLaunchKernelGGL(sel_final_kernel, dim3(1), dim3(MAX_WS), 0, s, w, g, out);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,127 @@
+// Device-side helpers shared by the gfx950 kernels: the float-rounded kernel epilogues, the
+// index-set predicates and wavefront reductions.  Everything here is plain IEEE arithmetic with
+// explicit fma(); the library is built with -ffp-contract=off so nothing else fuses.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define TSVM_WAVE 64
+
+enum { TSVM_LINEAR = 0, TSVM_POLY = 1, TSVM_RBF = 2, TSVM_SIGMOID = 3, TSVM_PRECOMPUTED = 4 };
+
+struct KernelParam {
+    int kernel_type;
+    int degree;
+    double gamma;
+    double coef0;
+};
+
+// 2^(i/32) table with i << 47 subtracted (so the integer part of k can be added into the exponent field).
+__constant__ const uint64_t TSVM_EXP2F_TAB[32] = {
+    0x3ff0000000000000ull, 0x3fefd9b0d3158574ull, 0x3fefb5586cf9890full, 0x3fef9301d0125b51ull,
+    0x3fef72b83c7d517bull, 0x3fef54873168b9aaull, 0x3fef387a6e756238ull, 0x3fef1e9df51fdee1ull,
+    0x3fef06fe0a31b715ull, 0x3feef1a7373aa9cbull, 0x3feedea64c123422ull, 0x3feece086061892dull,
+    0x3feebfdad5362a27ull, 0x3feeb42b569d4f82ull, 0x3feeab07dd485429ull, 0x3feea47eb03a5585ull,
+    0x3feea09e667f3bcdull, 0x3fee9f75e8ec5f74ull, 0x3feea11473eb0187ull, 0x3feea589994cce13ull,
+    0x3feeace5422aa0dbull, 0x3feeb737b0cdc5e5ull, 0x3feec49182a3f090ull, 0x3feed503b23e255dull,
+    0x3feee89f995ad3adull, 0x3feeff76f2fb5e47ull, 0x3fef199bdd85529cull, 0x3fef3720dcef9069ull,
+    0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full, 0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull};
+
+// expf of a float argument, evaluated in double and rounded once to float: the table-driven
+// algorithm glibc (>= 2.27) uses for expf.  `tab` points at the 32-entry table (LDS or constant).
+// The reference's kernels call libm expf on the host (kernelmatrix_kernel.cpp:71-72,87-89).
+__device__ __forceinline__ float tsvm_expf(float x, const uint64_t *tab) {
+    if (x != x) return x;
+    if (x > 0x1.62e42ep6f) return __builtin_inff();
+    if (x < -0x1.9fe368p6f) return 0.0f;
+    const double InvLn2N = 0x1.71547652b82fep+0 * 32;
+    const double SHIFT = 0x1.8p+52;
+    const double C0 = 0x1.c6af84b912394p-5 / 32 / 32 / 32;
+    const double C1 = 0x1.ebfce50fac4f3p-3 / 32 / 32;
+    const double C2 = 0x1.62e42ff0c52d6p-1 / 32;
+    double xd = (double) x;
+    double z = InvLn2N * xd;
+    double kd = z + SHIFT;
+    uint64_t ki = (uint64_t) __double_as_longlong(kd);
+    kd -= SHIFT;
+    double r = z - kd;
+    uint64_t t = tab[ki & 31];
+    t += ki << 47;
+    double s = __longlong_as_double((long long) t);
+    double zz = __builtin_fma(C0, r, C1);
+    double r2 = r * r;
+    double y = __builtin_fma(C2, r, 1.0);
+    y = __builtin_fma(zz, r2, y);
+    y = y * s;
+    return (float) y;
+}
+
+// Kernel epilogues (kernelmatrix_kernel.cpp:61-108).  sd0/sd1 are the two rows' self dot products.
+__device__ __forceinline__ double tsvm_epilogue(double dot, double sd0, double sd1, const KernelParam &p,
+                                                const uint64_t *tab) {
+    switch (p.kernel_type) {
+        case TSVM_RBF:
+        case TSVM_PRECOMPUTED: {
+            double arg = -(sd0 + sd1 - dot * 2) * p.gamma;
+            return (double) tsvm_expf((float) arg, tab);
+        }
+        case TSVM_POLY: {
+            // powf / tanhf of a float-rounded argument: evaluated in double and rounded once to float
+            const float arg = (float) __builtin_fma(p.gamma, dot, p.coef0);
+            return (double) (float) pow((double) arg, (double) p.degree);
+        }
+        case TSVM_SIGMOID: {
+            const float arg = (float) __builtin_fma(p.gamma, dot, p.coef0);
+            return (double) (float) tanh((double) arg);
+        }
+        default:
+            return dot;
+    }
+}
+
+// include/thundersvm/kernel/smo_kernel.h:13-23
+__device__ __forceinline__ bool is_I_up(double a, double y, double Cp, double Cn) {
+    return (y > 0 && a < Cp) || (y < 0 && a > 0);
+}
+__device__ __forceinline__ bool is_I_low(double a, double y, double Cp, double Cn) {
+    return (y > 0 && a > 0) || (y < 0 && a < Cn);
+}
+
+__device__ __forceinline__ double shfl_xor_f64(double v, int mask) {
+    int lo = __double2loint(v), hi = __double2hiint(v);
+    lo = __shfl_xor(lo, mask, TSVM_WAVE);
+    hi = __shfl_xor(hi, mask, TSVM_WAVE);
+    return __hiloint2double(hi, lo);
+}
+
+// Lexicographic (value, index) minimum across the wavefront: the smallest value wins and, among
+// equal values, the smallest index -- the serial loops' "first strict improvement" rule
+// (smo_kernel.cpp:43-49,80-89).
+__device__ __forceinline__ void wave_argmin(double &v, int &i) {
+#pragma unroll
+    for (int m = 1; m < TSVM_WAVE; m <<= 1) {
+        double ov = shfl_xor_f64(v, m);
+        int oi = __shfl_xor(i, m, TSVM_WAVE);
+        if (ov < v || (ov == v && oi < i)) { v = ov; i = oi; }
+    }
+}
+
+__device__ __forceinline__ double wave_max(double v) {
+#pragma unroll
+    for (int m = 1; m < TSVM_WAVE; m <<= 1) {
+        double ov = shfl_xor_f64(v, m);
+        if (ov > v) v = ov;
+    }
+    return v;
+}
+
+// Maps the launch's linear workgroup id to a logical one so that logical neighbours run on the
+// same XCD (the hardware deals consecutive workgroup ids round-robin over the 8 XCDs, each with
+// its own L2).
+__device__ __forceinline__ unsigned xcd_remap(unsigned pid, unsigned nwg) {
+    const unsigned NX = 8;
+    unsigned per = nwg / NX, rem = nwg % NX;
+    unsigned xcd = pid % NX, local = pid / NX;
+    unsigned base = xcd < rem ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per;
+    return base + local;
+}
