@@ -1,0 +1,85 @@
+/*
+ * thundersvm_amd -- model-level C ABI (libthundersvm.so).
+ *
+ * The role the reference's extern "C" scikit layer plays for its Python binding
+ * (src/thundersvm/thundersvm-scikit.cpp:15-400: model_new / *_model_scikit / get_sv / get_coef /
+ * get_rho / *_decision / save / load), with float64 arrays and CSR input so that coefficients, rho
+ * and decision values cross the boundary unrounded.  All pointers are HOST pointers.  A model handle
+ * is an opaque SvmModel* owned by the caller (tsvm_model_new / tsvm_model_free).
+ *
+ * Return value: 0 on success, 2 when the device ran out of memory (the reference's std::bad_alloc),
+ * -1 otherwise; tsvm_model_last_error() describes the failure.
+ */
+#ifndef THUNDERSVM_AMD_MODEL_H
+#define THUNDERSVM_AMD_MODEL_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* SvmParam (include/thundersvm/svmparam.h:14-66) */
+typedef struct tsvm_param {
+    int svm_type;      /* 0 C_SVC, 1 NU_SVC, 2 ONE_CLASS, 3 EPSILON_SVR, 4 NU_SVR */
+    int kernel_type;   /* 0 LINEAR, 1 POLY, 2 RBF, 3 SIGMOID, 4 PRECOMPUTED */
+    int degree;
+    int max_iter;      /* outer-iteration cap, -1 = none (SvmModel::set_max_iter) */
+    double gamma;
+    double coef0;
+    double C;
+    double nu;
+    double p;
+    double epsilon;
+    int64_t max_mem_size;   /* bytes, reference default 8192 MiB */
+    int nr_weight;
+    int verbose;
+    const int *weight_label;
+    const double *weight;
+} tsvm_param;
+
+const char *tsvm_model_last_error(void);
+
+void *tsvm_model_new(int svm_type);
+void tsvm_model_free(void *model);
+
+/* SvmModel::train on rows given as CSR (feature ids as in the LibSVM file, values float32-exact).
+ * ws_override > 0 forces the working-set size; keep_binary keeps each binary sub-problem's alpha*y
+ * and f for tsvm_model_binary; trace_cap > 0 records that many outer iterations of the first
+ * sub-problem; profile != 0 times the solver phases with device events. */
+int tsvm_model_train_csr(void *model, int64_t n, const int64_t *row_ptr, const int *col, const double *val,
+                         const double *y, const tsvm_param *param, int ws_override, int keep_binary, int trace_cap,
+                         int profile);
+
+/* SvmModel::train on a LibSVM text file (DataSet::load_from_file). */
+int tsvm_model_train_file(void *model, const char *path, const tsvm_param *param);
+
+int tsvm_model_info(void *model, int *n_classes, int *n_binary_models, int *total_sv, int64_t *sv_nnz);
+
+/* get_n_sv / get_rho / get_coef / get_sv_ind / svs (svmmodel.cpp:385-411); any pointer may be NULL.
+ * coef is [(n_classes-1)][total_sv] for classifiers and [total_sv] otherwise. */
+int tsvm_model_get(void *model, int *label, int *n_sv, double *rho, double *coef, int *sv_indices, int64_t *sv_ptr,
+                   int *sv_col, double *sv_val);
+
+/* Solver diagnostics of binary sub-problem k: outer iterations, inner iterations, objective and
+ * device milliseconds per phase (select, get_rows, local solve, update_f; zeros unless profiled). */
+int tsvm_model_stats(void *model, int k, int64_t *n_iter, int64_t *local_iter, double *obj, double *phase_ms);
+
+int64_t tsvm_model_binary_size(void *model, int k);
+int tsvm_model_binary(void *model, int k, double *alpha_signed, double *f);
+
+/* Recorded trajectory of the first sub-problem: returns the number of iterations recorded. */
+int tsvm_model_trace(void *model, int *ws_size, const double **diff, const int **ws);
+
+/* SvmModel::predict (svmmodel.cpp:157-171; SVC::predict svc.cpp:179-185): dec_values is
+ * [nrows][n_binary_models], labels [nrows] (class label, regression value or +-1). */
+int tsvm_model_predict_csr(void *model, int64_t nrows, const int64_t *row_ptr, const int *col, const double *val,
+                           int batch_size, double *dec_values, double *labels);
+
+int tsvm_model_save(void *model, const char *path);
+int tsvm_model_load(void *model, const char *path);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

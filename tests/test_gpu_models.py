@@ -1,0 +1,129 @@
+"""GPU parity of whole training / prediction runs (host C++ layer + kernels) against the CPU oracle.
+
+Modelled on the reference's model tests (src/test/test_svc.cpp, test_svr.cpp, test_nusvc.cpp,
+test_nusvr.cpp, test_oneclass_svc.cpp: same fixture, same parameters, same golden values), then the
+five benchmark workloads at reduced row counts.  Tolerances as stated for the path: coefficients
+and rho 1e-6 relative, decision values 1e-6 absolute, labels identical; in practice the
+trajectories are identical and the values agree to the last bit.
+"""
+import os
+
+import numpy as np
+import pytest
+
+import oracle_lib as O
+from thundersvm_amd import data as D
+from thundersvm_amd.model import Model, make_param
+
+pytestmark = pytest.mark.gpu
+FIXTURE = os.path.join(os.path.dirname(__file__), "golden", "test_dataset.txt")
+
+
+def _oparam(prm):
+    return O.make_param(svm_type=prm.svm_type, kernel_type=prm.kernel_type, degree=prm.degree, gamma=prm.gamma,
+                        coef0=prm.coef0, C_=prm.C, nu=prm.nu, p=prm.p, epsilon=prm.epsilon, max_iter=prm.max_iter,
+                        expf_mode=1)
+
+
+def _compare(train, test, prm, ws=0, trace=8):
+    gm = Model(prm.svm_type).train(train, prm, ws_override=ws, keep_binary=True, trace_cap=trace)
+    om = O.Model(train.ptr, train.col, train.val, train.y, _oparam(prm), ws_override=ws, want_trace=True)
+    gd, gw = gm.trace()
+    od, ow = om.trace()
+    k = min(len(gd), len(od), trace)
+    assert np.array_equal(gw[:k], ow[:k]), "working sets diverge at outer iteration %d" % np.flatnonzero(
+        (gw[:k] != ow[:k]).any(axis=1))[0]
+    assert np.array_equal(gd[:k], od[:k])
+    for b in range(gm.n_binary):
+        st = gm.stats(b)
+        assert st["n_iter"] == om.n_iter[b] and st["local_iter"] == om.local_iter[b]
+        ga, gf = gm.binary(b)
+        oa, of = om.binary(b)
+        np.testing.assert_allclose(ga, oa, rtol=1e-6, atol=1e-12)
+        np.testing.assert_allclose(gf, of, rtol=1e-6, atol=1e-9)
+    assert gm.total_sv == om.total_sv
+    assert np.array_equal(gm.n_sv, om.n_sv) and np.array_equal(gm.sv_indices, om.sv_indices)
+    np.testing.assert_allclose(gm.rho, om.rho, rtol=1e-6, atol=1e-12)
+    np.testing.assert_allclose(gm.coef, om.coef, rtol=1e-6, atol=1e-12)
+    tst = test if test is not None else train
+    glab, gdec = gm.predict(tst, 100)
+    olab, odec = om.predict(tst.ptr, tst.col, tst.val, 100)
+    assert np.abs(gdec - odec).max() < 1e-6
+    assert np.array_equal(glab, olab) or prm.svm_type in (3, 4)
+    if prm.svm_type in (3, 4):
+        assert np.abs(glab - olab).max() < 1e-6
+    return gm, om, glab, tst
+
+
+def test_fixture_csvc():            # test_svc.cpp:33-37
+    d = D.load_libsvm(FIXTURE)
+    gm, om, lab, tst = _compare(d, d, make_param(svm_type=0, kernel_type=2, gamma=0.5, C=100))
+    assert abs((lab == d.y).mean() - 0.98) < 1e-5
+
+
+def test_fixture_svr():             # test_svr.cpp:35-39
+    d = D.load_libsvm(FIXTURE)
+    gm, om, lab, tst = _compare(d, d, make_param(svm_type=3, kernel_type=2, gamma=0.5, C=100))
+    assert abs(((lab - d.y) ** 2).mean() - 0.020752) < 1e-3
+
+
+def test_fixture_nusvc():           # test_nusvc.cpp:40-44
+    d = D.load_libsvm(FIXTURE)
+    gm, om, lab, tst = _compare(d, d, make_param(svm_type=1, kernel_type=2, gamma=0.5, nu=0.1, C=100))
+    assert abs((lab == d.y).mean() - 0.98) < 1e-3
+
+
+def test_fixture_nusvr():           # test_nusvr.cpp:38-42
+    d = D.load_libsvm(FIXTURE)
+    gm, om, lab, tst = _compare(d, d, make_param(svm_type=4, kernel_type=2, gamma=0.5, nu=0.1, C=100))
+    assert abs(((lab - d.y) ** 2).mean() - 0.028369) < 1.2e-5
+
+
+def test_fixture_oneclass(tmp_path):   # test_oneclass_svc.cpp:7-30: train, save, load, predict
+    d = D.load_libsvm(FIXTURE)
+    gm, om, lab, tst = _compare(d, d, make_param(svm_type=2, kernel_type=2, gamma=0.5, nu=0.1))
+    path = str(tmp_path / "one_class.model")
+    gm.save(path)
+    m2 = Model(2).load(path)
+    lab2, _ = m2.predict(d, 100)
+    assert int((lab2 > 0).sum()) == 135
+
+
+@pytest.mark.parametrize("kt,prm", [(0, {}), (1, dict(gamma=0.5, degree=3, coef0=0.1)), (3, dict(gamma=0.5, coef0=0.1))])
+def test_fixture_other_kernels(kt, prm):
+    d = D.load_libsvm(FIXTURE)
+    _compare(d, d, make_param(svm_type=0, kernel_type=kt, C=10, **prm))
+
+
+def test_workload_c1():
+    w = D.workload_c1()
+    _compare(w["train"], w["test"], make_param(**w["params"]), trace=64)
+
+
+def test_workload_c2_small():
+    w = D.workload_c2(scale=0.03)
+    _compare(w["train"], w["test"], make_param(**w["params"]), trace=64)
+
+
+@pytest.mark.parametrize("kernel", ["linear", "rbf"])
+def test_workload_c3_small(kernel):
+    w = D.workload_c3(scale=0.04, kernel=kernel)
+    _compare(w["train"], None, make_param(**w["params"]), trace=64)
+
+
+def test_workload_c4_small():
+    w = D.workload_c4(scale=0.01, n_test=500)
+    _compare(w["train"], w["test"], make_param(**w["params"]), trace=64)
+
+
+def test_workload_c5_small():
+    w = D.workload_c5(scale=0.01)
+    _compare(w["train"], w["test"], make_param(**w["params"]), trace=64)
+
+
+def test_max_iter_cap():
+    w = D.workload_c1(scale=0.5)
+    prm = make_param(**w["params"])
+    prm.max_iter = 3
+    gm, om, _, _ = _compare(w["train"], w["test"], prm)
+    assert gm.stats(0)["n_iter"] == 4

@@ -31,15 +31,15 @@ def build_host(extra=()):
     srcs = sorted(os.path.join(HOST, f) for f in os.listdir(HOST) if f.endswith(".cpp") and not f.startswith("main_"))
     if not srcs:
         return None
-    _run(["hipcc", "-O2", "-fPIC", "-std=c++17", "-ffp-contract=off", "-fopenmp", "-x", "c++", *extra, *srcs, "-x", "none",
-          "-shared", "-o", HOST_LIB, "-I", os.path.join(HERE, "..", "include"),
-          "-L", HERE, "-ltsvm_hip", "-Wl,-rpath,$ORIGIN", "-L/opt/rocm/lib", "-lamdhip64"])
+    _run(["g++", "-O2", "-fPIC", "-std=c++17", "-ffp-contract=off", "-fopenmp", "-D__HIP_PLATFORM_AMD__",
+          "-I/opt/rocm/include", *extra, *srcs, "-shared", "-o", HOST_LIB,
+          "-L", HERE, "-ltsvm_hip", "-Wl,-rpath,$ORIGIN", "-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,/opt/rocm/lib"])
     for main in sorted(f for f in os.listdir(HOST) if f.startswith("main_") and f.endswith(".cpp")):
         exe = os.path.join(HERE, "bin", main[len("main_"):-len(".cpp")].replace("_", "-"))
         os.makedirs(os.path.dirname(exe), exist_ok=True)
-        _run(["hipcc", "-O2", "-std=c++17", "-fopenmp", "-x", "c++", os.path.join(HOST, main), "-x", "none", "-o", exe,
-              "-I", os.path.join(HERE, "..", "include"), "-L", HERE, "-lthundersvm", "-ltsvm_hip",
-              "-Wl,-rpath,$ORIGIN/..", "-L/opt/rocm/lib", "-lamdhip64"])
+        _run(["g++", "-O2", "-std=c++17", "-fopenmp", "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include",
+              os.path.join(HOST, main), "-o", exe, "-L", HERE, "-lthundersvm", "-ltsvm_hip",
+              "-Wl,-rpath,$ORIGIN/..", "-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,/opt/rocm/lib"])
     return HOST_LIB
 
 

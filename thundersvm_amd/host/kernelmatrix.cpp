@@ -1,0 +1,135 @@
+#include "kernelmatrix.h"
+
+#include <algorithm>
+
+using tsvm::abi_check;
+
+namespace tsvm {
+size_t &device_bytes_in_use() {
+    static size_t bytes = 0;
+    return bytes;
+}
+}  // namespace tsvm
+
+// Dense rows cost d_pad MFMA k-steps per output, CSR rows cost one L2 gather per stored non-zero;
+// the matrix cores run roughly 30 k-steps in the time of one gather, so dense wins unless rows
+// are very sparse.  Dense storage is also capped at 64 GiB.
+bool KernelMatrix::choose_dense(size_t n, size_t n_features, size_t nnz) {
+    if (n == 0) return true;
+    const size_t ld = (n_features + 7) / 8 * 8;
+    const double avg = (double) nnz / (double) n;
+    if ((double) ld * (double) n * 8.0 > 64.0 * 1024 * 1024 * 1024) return false;
+    return (double) ld <= 32.0 * std::max(avg, 1.0);
+}
+
+KernelMatrix::KernelMatrix(const DataSet::node2d &instances, SvmParam param) : param(param) {
+    build(instances, nullptr, instances.size(), 1);
+}
+
+KernelMatrix::KernelMatrix(const DataSet::node2d &all, const int *rows, size_t n_rows, SvmParam param, int repeat)
+    : param(param) {
+    build(all, rows, n_rows, repeat);
+}
+
+// CSR assembly on the host (kernelmatrix.cpp:183-207): n_features_ = largest feature id + 1, ids kept
+// as given.  `repeat` stacks the same rows several times (the 2n-row problem of SVR, svr.cpp:14-15).
+void KernelMatrix::build(const DataSet::node2d &all, const int *rows, size_t n_rows, int repeat) {
+    n_instances_ = n_rows * repeat;
+    std::vector<int64_t> ptr(n_instances_ + 1, 0);
+    size_t total = 0;
+    int max_index = 0;
+    for (size_t r = 0; r < n_rows; ++r) {
+        const auto &row = all[rows ? rows[r] : r];
+        total += row.size();
+        for (const auto &nd : row) max_index = std::max(max_index, nd.index);
+    }
+    nnz_ = total * repeat;
+    n_features_ = (size_t) max_index + 1;
+    std::vector<kernel_type> val(nnz_);
+    std::vector<int> col(nnz_);
+    size_t e = 0;
+    for (int rep = 0; rep < repeat; ++rep) {
+        for (size_t r = 0; r < n_rows; ++r) {
+            const auto &row = all[rows ? rows[r] : r];
+            for (const auto &nd : row) { val[e] = nd.value; col[e] = nd.index; ++e; }
+            ptr[rep * n_rows + r + 1] = (int64_t) e;
+        }
+    }
+    val_.upload(val);
+    col_ind_.upload(col);
+    row_ptr_.upload(ptr);
+    self_dot_.resize(n_instances_);
+    diag_.resize(n_instances_);
+    abi_check(tsvm_csr_self_dot(val_.data(), row_ptr_.data(), (int64_t) n_instances_, self_dot_.data(), nullptr));
+    abi_check(tsvm_kernel_diag(self_dot_.data(), (int64_t) n_instances_, (int) param.kernel_type, param.gamma, param.coef0,
+                               param.degree, diag_.data(), nullptr));
+    dense_ = choose_dense(n_instances_, n_features_, nnz_);
+    if (dense_) {
+        ld_ = (int64_t) ((n_features_ + 7) / 8 * 8);
+        x_.resize(n_instances_ * (size_t) ld_);
+        abi_check(tsvm_csr_to_dense(val_.data(), col_ind_.data(), row_ptr_.data(), (int64_t) n_instances_, x_.data(), ld_,
+                                    nullptr));
+        TSVM_HIP_CHECK(hipDeviceSynchronize());
+        val_.release();
+        col_ind_.release();
+        row_ptr_.release();
+    }
+}
+
+void KernelMatrix::get_rows(const int *d_idx, int m, kernel_type *d_out, int64_t ld) const {
+    const int n = (int) n_instances_;
+    if (dense_) {
+        abi_check(tsvm_get_rows_dense(x_.data(), ld_, n, (int) n_features_, self_dot_.data(), x_.data(), ld_, d_idx, m,
+                                      self_dot_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
+                                      d_out, ld, nullptr));
+        return;
+    }
+    if (stage_.size() < (size_t) m * n_features_) stage_.resize((size_t) m * n_features_);
+    if (stage_sd_.size() < (size_t) m) stage_sd_.resize(m);
+    abi_check(tsvm_csr_stage_rows(val_.data(), col_ind_.data(), row_ptr_.data(), d_idx, m, (int) n_features_,
+                                  stage_.data(), nullptr));
+    abi_check(tsvm_gather_f64(self_dot_.data(), d_idx, m, stage_sd_.data(), nullptr));
+    abi_check(tsvm_get_rows_csr(val_.data(), col_ind_.data(), row_ptr_.data(), n, self_dot_.data(), stage_.data(), m,
+                                stage_sd_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree, d_out,
+                                ld, nullptr));
+}
+
+// External batch (kernelmatrix.cpp:281-312, 385-406): features with id >= n_features_ are left out of
+// the dot product but stay in the batch row's self dot.
+void KernelMatrix::get_rows(const DataSet::node2d &instances, kernel_type *d_out, int64_t ld) const {
+    const int m = (int) instances.size();
+    if (m == 0) return;
+    std::vector<int64_t> ptr(m + 1, 0);
+    size_t total = 0;
+    for (const auto &row : instances) total += row.size();
+    std::vector<kernel_type> val(total);
+    std::vector<int> col(total);
+    size_t e = 0;
+    for (int r = 0; r < m; ++r) {
+        for (const auto &nd : instances[r]) { val[e] = nd.value; col[e] = nd.index; ++e; }
+        ptr[r + 1] = (int64_t) e;
+    }
+    if (b_val_.size() < total) { b_val_.resize(total); b_col_.resize(total); }
+    if (b_ptr_.size() < (size_t) m + 1) b_ptr_.resize(m + 1);
+    b_val_.upload(val.data(), total);
+    b_col_.upload(col.data(), total);
+    b_ptr_.upload(ptr.data(), m + 1);
+    if (stage_sd_.size() < (size_t) m) stage_sd_.resize(m);
+    abi_check(tsvm_csr_self_dot(b_val_.data(), b_ptr_.data(), m, stage_sd_.data(), nullptr));
+    const int n = (int) n_instances_;
+    if (dense_) {
+        if (stage_.size() < (size_t) m * ld_) stage_.resize((size_t) m * ld_);
+        // columns >= n_features_ are dropped: the staging matrix is only n_features_ wide
+        abi_check(tsvm_csr_to_dense(b_val_.data(), b_col_.data(), b_ptr_.data(), m, stage_.data(), ld_, nullptr));
+        abi_check(tsvm_get_rows_dense(x_.data(), ld_, n, (int) n_features_, self_dot_.data(), stage_.data(), ld_, nullptr, m,
+                                      stage_sd_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
+                                      d_out, ld, nullptr));
+    } else {
+        if (stage_.size() < (size_t) m * n_features_) stage_.resize((size_t) m * n_features_);
+        abi_check(tsvm_csr_stage_rows(b_val_.data(), b_col_.data(), b_ptr_.data(), nullptr, m, (int) n_features_,
+                                      stage_.data(), nullptr));
+        abi_check(tsvm_get_rows_csr(val_.data(), col_ind_.data(), row_ptr_.data(), n, self_dot_.data(), stage_.data(), m,
+                                    stage_sd_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
+                                    d_out, ld, nullptr));
+    }
+}

@@ -1,0 +1,53 @@
+// KernelMatrix: the training (or support-vector) rows resident in HBM, serving kernel rows by id or
+// for an external batch.  Public surface of include/thundersvm/kernelmatrix.h:39-72 with device
+// pointers in place of SyncArray.
+//
+// Layout in HBM: either dense row-major fp64 [n][ld] (ld = n_features rounded up to 8, column c =
+// feature id c) for the MFMA path, or CSR (fp64 values, int32 columns, int64 row offsets) for the
+// sparse path.  The layout is chosen from the average row fill (see choose_dense()).
+#pragma once
+#include "dataset.h"
+#include "device.h"
+#include "svmparam.h"
+
+class KernelMatrix {
+public:
+    KernelMatrix(const DataSet::node2d &instances, SvmParam param);
+    // Rows `rows[0..n_rows)` of `all`, without materialising a node2d copy.
+    KernelMatrix(const DataSet::node2d &all, const int *rows, size_t n_rows, SvmParam param, int repeat = 1);
+
+    // kernel rows of stored instances d_idx[0..m) (device ids) -> d_out[i*ld + j]
+    void get_rows(const int *d_idx, int m, kernel_type *d_out, int64_t ld) const;
+    // kernel rows of an external batch -> d_out[i*ld + j]
+    void get_rows(const DataSet::node2d &instances, kernel_type *d_out, int64_t ld) const;
+
+    const kernel_type *diag() const { return diag_.data(); }          // device
+    const kernel_type *self_dot() const { return self_dot_.data(); }  // device
+    size_t n_instances() const { return n_instances_; }
+    size_t n_features() const { return n_features_; }
+    size_t nnz() const { return nnz_; }
+    bool dense_layout() const { return dense_; }
+    const SvmParam &get_param() const { return param; }
+
+    static bool choose_dense(size_t n, size_t n_features, size_t nnz);
+
+private:
+    void build(const DataSet::node2d &all, const int *rows, size_t n_rows, int repeat);
+
+    SvmParam param;
+    size_t n_instances_ = 0, n_features_ = 0, nnz_ = 0;
+    bool dense_ = false;
+    int64_t ld_ = 0;
+    tsvm::DeviceBuffer<kernel_type> x_;          // dense layout
+    tsvm::DeviceBuffer<kernel_type> val_;        // CSR layout
+    tsvm::DeviceBuffer<int> col_ind_;
+    tsvm::DeviceBuffer<int64_t> row_ptr_;
+    tsvm::DeviceBuffer<kernel_type> self_dot_;
+    tsvm::DeviceBuffer<kernel_type> diag_;
+    // reusable staging for the sparse path and for external batches
+    mutable tsvm::DeviceBuffer<kernel_type> stage_;
+    mutable tsvm::DeviceBuffer<kernel_type> stage_sd_;
+    mutable tsvm::DeviceBuffer<kernel_type> b_val_;
+    mutable tsvm::DeviceBuffer<int> b_col_;
+    mutable tsvm::DeviceBuffer<int64_t> b_ptr_;
+};

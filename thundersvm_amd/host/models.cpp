@@ -1,0 +1,540 @@
+#include "models.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <fstream>
+#include <iomanip>
+#include <stdexcept>
+
+using tsvm::abi_check;
+using tsvm::DeviceBuffer;
+
+const char *SvmParam::kernel_type_name[6] = {"linear", "polynomial", "rbf", "sigmoid", "precomputed", "NULL"};
+const char *SvmParam::svm_type_name[6] = {"c_svc", "nu_svc", "one_class", "epsilon_svr", "nu_svr", "NULL"};
+
+std::unique_ptr<SvmModel> make_model(SvmParam::SVM_TYPE type) {
+    switch (type) {
+        case SvmParam::C_SVC: return std::unique_ptr<SvmModel>(new SVC());
+        case SvmParam::NU_SVC: return std::unique_ptr<SvmModel>(new NuSVC());
+        case SvmParam::ONE_CLASS: return std::unique_ptr<SvmModel>(new OneClassSVC());
+        case SvmParam::EPSILON_SVR: return std::unique_ptr<SvmModel>(new SVR());
+        case SvmParam::NU_SVR: return std::unique_ptr<SvmModel>(new NuSVR());
+    }
+    throw std::runtime_error("unknown svm type");
+}
+
+// ------------------------------------------------------------------------------------------------
+// SvmModel
+// ------------------------------------------------------------------------------------------------
+void SvmModel::model_setup(const DataSet &, SvmParam &p) {   // svmmodel.cpp:22-29
+    n_binary_models = n_classes * (n_classes - 1) / 2;
+    rho.assign(n_binary_models, 0);
+    n_sv.assign(n_classes, 0);
+    sv.clear();
+    sv_indices.clear();
+    coef.clear();
+    linear_coef.clear();
+    solver_stats.clear();
+    binary_alpha.clear();
+    binary_f.clear();
+    param = p;
+}
+
+static int max2power(double n) { return (int) pow(2, floor(log2f(float(n)))); }   // util/common.h:20-23
+
+// svmmodel.cpp:437-451.  The reference subtracts the bytes its SyncMem counter holds; the device
+// allocations of this build play that role.
+int SvmModel::get_working_set_size(int n_instances, int n_features) {
+    if (ws_override > 0) return ws_override;
+    const size_t used = tsvm::device_bytes_in_use();
+    if (param.max_mem_size < used) throw std::bad_alloc();
+    const size_t free_mem = param.max_mem_size - used;
+    const size_t by_mem = (size_t) max2power((double) (free_mem / sizeof(kernel_type) / ((size_t) n_instances + n_features)));
+    const int ws = std::min(max2power(n_instances), (int) std::min(by_mem, (size_t) 1024));
+    TSVM_LOG << "working set size = " << ws;
+    return ws;
+}
+
+void SvmModel::run_solver(CSMOSolver &solver, const KernelMatrix &k_mat, const std::vector<int> &y,
+                          std::vector<float_type> &alpha, float_type &rho_out, std::vector<float_type> &f_val,
+                          float_type Cp, float_type Cn) {
+    const int ws = get_working_set_size((int) k_mat.n_instances(), (int) k_mat.n_features());
+    solver.profile = profile;
+    solver.trace = solver_stats.empty() ? trace_first : nullptr;
+    solver.solve(k_mat, y, alpha, rho_out, f_val, param.epsilon, Cp, Cn, ws, max_iter);
+    solver_stats.push_back(solver.stats);
+    if (keep_binary) binary_f.push_back(f_val);
+}
+
+// Decision values for a batch of rows (svmmodel.cpp:74-117): kernel values against all support
+// vectors, then the per-class-pair reduction, batch by batch, all on the device.
+void SvmModel::predict_dec_values(const DataSet::node2d &instances, std::vector<float_type> &dec, int batch_size) const {
+    dec.assign(instances.size() * (size_t) n_binary_models, 0);
+    if (instances.empty()) return;
+    std::vector<int> sv_start(n_classes, 0);
+    for (int c = 1; c < n_classes; ++c) sv_start[c] = sv_start[c - 1] + n_sv[c - 1];
+    const size_t T = sv.size();
+    if (T == 0) {
+        for (size_t r = 0; r < instances.size(); ++r)
+            for (int p = 0; p < n_binary_models; ++p) dec[r * n_binary_models + p] = -rho[p];
+        return;
+    }
+    KernelMatrix k_mat(sv, param);
+    if (batch_size == -1) {
+        const size_t used = tsvm::device_bytes_in_use();
+        const size_t free_mem = param.max_mem_size > used ? param.max_mem_size - used : 0;
+        batch_size = (int) std::min(free_mem / sizeof(float_type) / (T + k_mat.n_features()), size_t(10000));
+        if (batch_size < 1) batch_size = 1;
+    }
+    DeviceBuffer<int> d_start, d_count;
+    DeviceBuffer<float_type> d_coef, d_rho;
+    d_start.upload(sv_start);
+    d_count.upload(n_sv);
+    d_coef.upload(coef);
+    d_rho.upload(rho);
+    const size_t bmax = std::min((size_t) batch_size, instances.size());
+    DeviceBuffer<kernel_type> d_k(bmax * T);
+    DeviceBuffer<float_type> d_dec(bmax * n_binary_models);
+    for (size_t b0 = 0; b0 < instances.size(); b0 += batch_size) {
+        const size_t bm = std::min((size_t) batch_size, instances.size() - b0);
+        DataSet::node2d batch(instances.begin() + b0, instances.begin() + b0 + bm);
+        k_mat.get_rows(batch, d_k.data(), (int64_t) T);
+        abi_check(tsvm_sum_kernel_values(d_coef.data(), (int) T, d_start.data(), d_count.data(), d_rho.data(), d_k.data(),
+                                         (int64_t) T, d_dec.data(), n_classes, (int64_t) bm, nullptr));
+        d_dec.download(dec.data() + b0 * n_binary_models, bm * n_binary_models);
+    }
+}
+
+std::vector<float_type> SvmModel::predict(const DataSet::node2d &instances, int batch_size) {   // svmmodel.cpp:157-171
+    predict_dec_values(instances, dec_values, batch_size);
+    return dec_values;
+}
+
+// Stratified folds in class order (svmmodel.cpp:31-71).
+std::vector<float_type> SvmModel::cross_validation(DataSet dataset, SvmParam p, int n_fold) {
+    dataset.group_classes(this->param.svm_type == SvmParam::C_SVC);
+    std::vector<float_type> y_predict_all(dataset.n_instances());
+    for (int k = 0; k < n_fold; ++k) {
+        DataSet::node2d x_train, x_test;
+        std::vector<float_type> y_train;
+        std::vector<int> test_idx;
+        for (size_t c = 0; c < dataset.n_classes(); ++c) {
+            const int fold = dataset.count()[c] / n_fold;
+            const std::vector<int> ids = dataset.original_index((int) c);
+            const size_t lo = (size_t) fold * k;
+            const size_t hi = (k == n_fold - 1) ? ids.size() : std::min(ids.size(), lo + fold);
+            for (size_t t = 0; t < ids.size(); ++t) {
+                if (t >= lo && t < hi) {
+                    x_test.push_back(dataset.instances()[ids[t]]);
+                    test_idx.push_back(ids[t]);
+                } else {
+                    x_train.push_back(dataset.instances()[ids[t]]);
+                    y_train.push_back(dataset.y()[ids[t]]);
+                }
+            }
+        }
+        DataSet train_set(x_train, (int) dataset.n_features(), y_train);
+        this->train(train_set, p);
+        std::vector<float_type> y_predict = this->predict(x_test, 1000);
+        for (size_t i = 0; i < y_predict.size(); ++i) y_predict_all[test_idx[i]] = y_predict[i];
+    }
+    return y_predict_all;
+}
+
+void SvmModel::compute_linear_coef_single_model(size_t n_feature, bool zero_based) {
+    linear_coef.assign(zero_based ? n_feature + 1 : n_feature, 0);
+    for (size_t i = 0; i < sv.size(); ++i)
+        for (const auto &nd : sv[i]) linear_coef[zero_based ? nd.index : nd.index - 1] += coef[i] * nd.value;
+}
+
+// LibSVM text model (svmmodel.cpp:193-264): rho/gamma at stream default precision, coefficients with
+// 16 significant digits, SV values with 8.
+std::string SvmModel::save_to_string() {
+    std::ostringstream s;
+    s << "svm_type " << SvmParam::svm_type_name[param.svm_type] << std::endl;
+    s << "kernel_type " << SvmParam::kernel_type_name[param.kernel_type] << std::endl;
+    if (param.kernel_type == SvmParam::POLY) s << "degree " << param.degree << std::endl;
+    if (param.kernel_type == SvmParam::POLY || param.kernel_type == SvmParam::RBF || param.kernel_type == SvmParam::SIGMOID)
+        s << "gamma " << param.gamma << std::endl;
+    if (param.kernel_type == SvmParam::POLY || param.kernel_type == SvmParam::SIGMOID)
+        s << "coef0 " << param.coef0 << std::endl;
+    s << "nr_class " << n_classes << std::endl;
+    s << "total_sv " << sv.size() << std::endl;
+    s << "rho ";
+    for (int i = 0; i < n_binary_models; ++i) s << rho[i] << " ";
+    s << std::endl;
+    if (param.svm_type == SvmParam::NU_SVC || param.svm_type == SvmParam::C_SVC) {
+        s << "label ";
+        for (int i = 0; i < n_classes; ++i) s << label[i] << " ";
+        s << std::endl << "nr_sv ";
+        for (int i = 0; i < n_classes; ++i) s << n_sv[i] << " ";
+        s << std::endl;
+    }
+    if (param.probability == 1) {
+        s << "probA ";
+        for (int i = 0; i < n_binary_models; ++i) s << probA[i] << " ";
+        s << std::endl << "probB ";
+        for (int i = 0; i < n_binary_models; ++i) s << probB[i] << " ";
+        s << std::endl;
+    }
+    if (param.kernel_type == SvmParam::LINEAR) {
+        s << "coef " << std::endl;
+        for (size_t i = 0; i < linear_coef.size(); ++i) s << std::setprecision(16) << linear_coef[i] << " ";
+        s << std::endl;
+    }
+    s << "SV " << std::endl;
+    const int rows = (param.svm_type == SvmParam::NU_SVC || param.svm_type == SvmParam::C_SVC) ? n_classes - 1 : 1;
+    for (size_t i = 0; i < sv.size(); ++i) {
+        for (int j = 0; j < rows; ++j) s << std::setprecision(16) << coef[j * sv.size() + i] << " ";
+        for (const auto &nd : sv[i]) s << nd.index << ":" << std::setprecision(8) << nd.value << " ";
+        s << std::endl;
+    }
+    return s.str();
+}
+
+void SvmModel::save_to_file(std::string path) {
+    std::ofstream out(path.c_str(), std::ios_base::out | std::ios_base::trunc);
+    if (!out.is_open()) throw std::runtime_error("create file " + path + " failed");
+    out << save_to_string();
+}
+
+void SvmModel::load_from_file(std::string path) {
+    std::ifstream in(path.c_str());
+    if (!in.is_open()) throw std::runtime_error("file " + path + " not found");
+    std::stringstream ss;
+    ss << in.rdbuf();
+    load_from_string(ss.str());
+}
+
+// svmmodel.cpp:280-383
+void SvmModel::load_from_string(std::string data) {
+    std::stringstream iss(data);
+    std::string key;
+    while (iss >> key) {
+        if (key == "svm_type") {
+            std::string v;
+            iss >> v;
+            for (int i = 0; i < 5; ++i) if (v == SvmParam::svm_type_name[i]) param.svm_type = (SvmParam::SVM_TYPE) i;
+        } else if (key == "kernel_type") {
+            std::string v;
+            iss >> v;
+            for (int i = 0; i < 5; ++i) if (v == SvmParam::kernel_type_name[i]) param.kernel_type = (SvmParam::KERNEL_TYPE) i;
+        } else if (key == "degree") {
+            iss >> param.degree;
+        } else if (key == "gamma") {
+            iss >> param.gamma;
+        } else if (key == "coef0") {
+            iss >> param.coef0;
+        } else if (key == "nr_class") {
+            iss >> n_classes;
+            n_binary_models = n_classes * (n_classes - 1) / 2;
+            rho.assign(n_binary_models, 0);
+            n_sv.assign(n_classes, 0);
+        } else if (key == "total_sv") {
+            iss >> n_total_sv;
+        } else if (key == "rho") {
+            for (int i = 0; i < n_binary_models; ++i) iss >> rho[i];
+        } else if (key == "label") {
+            label.assign(n_classes, 0);
+            for (int i = 0; i < n_classes; ++i) iss >> label[i];
+        } else if (key == "nr_sv") {
+            for (int i = 0; i < n_classes; ++i) iss >> n_sv[i];
+        } else if (key == "probA") {
+            param.probability = 1;
+            probA.assign(n_binary_models, 0);
+            for (int i = 0; i < n_binary_models; ++i) iss >> probA[i];
+        } else if (key == "probB") {
+            probB.assign(n_binary_models, 0);
+            for (int i = 0; i < n_binary_models; ++i) iss >> probB[i];
+        } else if (key == "coef") {
+            std::string line;
+            std::getline(iss, line);
+            std::getline(iss, line);
+            std::stringstream ls(line);
+            linear_coef.clear();
+            float_type v;
+            while (ls >> v) linear_coef.push_back(v);
+        } else if (key == "SV") {
+            const bool cls = param.svm_type == SvmParam::C_SVC || param.svm_type == SvmParam::NU_SVC;
+            const int rows = cls ? n_classes - 1 : 1;
+            sv.clear();
+            coef.assign((size_t) rows * n_total_sv, 0);
+            std::string line;
+            std::getline(iss, line);
+            for (int i = 0; i < n_total_sv; ++i) {
+                std::getline(iss, line);
+                std::stringstream ls(line);
+                for (int j = 0; j < rows; ++j) ls >> coef[(size_t) j * n_total_sv + i];
+                sv.emplace_back();
+                std::string tuple;
+                while (ls >> tuple) {
+                    int idx;
+                    double v;
+                    if (sscanf(tuple.c_str(), "%d:%lf", &idx, &v) != 2) throw std::runtime_error("error when loading model file");
+                    sv.back().emplace_back(idx, v);
+                    sv_max_index = std::max(sv_max_index, idx);
+                }
+            }
+        }
+    }
+    if (param.svm_type != SvmParam::C_SVC && param.svm_type != SvmParam::NU_SVC) {
+        n_sv.assign(2, 0);
+        n_sv[0] = n_total_sv;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// SVC (svc.cpp)
+// ------------------------------------------------------------------------------------------------
+void SVC::model_setup(const DataSet &dataset, SvmParam &p) {   // svc.cpp:16-39
+    n_classes = (int) dataset.n_classes();
+    label = dataset.label();
+    SvmModel::model_setup(dataset, p);
+    param.svm_type = SvmParam::C_SVC;
+    c_weight.assign(n_classes, 1);
+    for (int w = 0; w < p.nr_weight; ++w) {
+        bool found = false;
+        for (int c = 0; c < n_classes && !found; ++c)
+            if (p.weight_label[w] == label[c]) { c_weight[c] *= p.weight[w]; found = true; }
+        if (!found) TSVM_LOG << "weighted label " << p.weight_label[w] << " not found";
+    }
+}
+
+void SVC::train(const DataSet &dataset, SvmParam p) {   // svc.cpp:41-145
+    DataSet grouped = dataset;
+    grouped.group_classes();
+    model_setup(grouped, p);
+    const int n = (int) grouped.n_instances();
+    std::vector<std::vector<float_type>> alpha(n_binary_models);
+    std::vector<char> is_sv(n, 0);
+    int k = 0;
+    for (int i = 0; i < n_classes; ++i)
+        for (int j = i + 1; j < n_classes; ++j, ++k) {
+            train_binary(grouped, i, j, alpha[k], rho[k]);
+            const std::vector<int> ids = grouped.original_index(i, j);
+            for (size_t l = 0; l < ids.size(); ++l)
+                if (alpha[k][l] != 0) is_sv[ids[l]] = 1;
+            if (keep_binary) binary_alpha.push_back(alpha[k]);
+        }
+    // support vectors class by class, in grouped order
+    for (int c = 0; c < n_classes; ++c)
+        for (int id : grouped.original_index(c))
+            if (is_sv[id]) {
+                n_sv[c]++;
+                sv.push_back(grouped.instances()[id]);
+                sv_indices.push_back(id);
+            }
+    n_total_sv = (int) sv.size();
+    TSVM_LOG << "#total unique sv = " << n_total_sv;
+    // LibSVM coefficient layout: pair (i<j) stores class i's SVs in row j-1 and class j's SVs in row i
+    coef.assign((size_t) (n_classes - 1) * n_total_sv, 0);
+    std::vector<int> sv_start(n_classes, 0);
+    for (int c = 1; c < n_classes; ++c) sv_start[c] = sv_start[c - 1] + n_sv[c - 1];
+    k = 0;
+    for (int i = 0; i < n_classes; ++i)
+        for (int j = i + 1; j < n_classes; ++j, ++k) {
+            const std::vector<int> ids = grouped.original_index(i, j);
+            const int ci = grouped.count()[i];
+            int at = sv_start[i];
+            for (int l = 0; l < ci; ++l)
+                if (is_sv[ids[l]]) coef[(size_t) (j - 1) * n_total_sv + at++] = alpha[k][l];
+            at = sv_start[j];
+            for (size_t l = ci; l < ids.size(); ++l)
+                if (is_sv[ids[l]]) coef[(size_t) i * n_total_sv + at++] = alpha[k][l];
+        }
+    if (param.kernel_type == SvmParam::LINEAR) {   // explicit w per pair (svc.cpp:111-135)
+        const size_t nf = grouped.n_features();
+        linear_coef.assign((size_t) n_binary_models * (grouped.is_zero_based() ? nf + 1 : nf), 0);
+        k = 0;
+        for (int i = 0; i < n_classes; ++i)
+            for (int j = i + 1; j < n_classes; ++j, ++k) {
+                const std::vector<int> ids = grouped.original_index(i, j);
+                for (size_t l = 0; l < ids.size(); ++l) {
+                    if (alpha[k][l] == 0) continue;
+                    for (const auto &nd : grouped.instances()[ids[l]])
+                        linear_coef[k * nf + (grouped.is_zero_based() ? nd.index : nd.index - 1)] += alpha[k][l] * nd.value;
+                }
+            }
+    }
+    if (param.probability == 1) throw std::runtime_error("probability estimates are not part of this build");
+}
+
+void SVC::train_binary(const DataSet &dataset, int i, int j, std::vector<float_type> &alpha, float_type &rho_out) {   // svc.cpp:147-177
+    const std::vector<int> ids = dataset.original_index(i, j);
+    const int ci = dataset.count()[i], n = (int) ids.size();
+    std::vector<int> y(n);
+    std::vector<float_type> f_val(n);
+    alpha.assign(n, 0);
+    for (int l = 0; l < n; ++l) {
+        y[l] = l < ci ? +1 : -1;
+        f_val[l] = l < ci ? -1 : +1;
+    }
+    KernelMatrix k_mat(dataset.instances(), ids.data(), ids.size(), param);
+    CSMOSolver solver;
+    run_solver(solver, k_mat, y, alpha, rho_out, f_val, param.C * c_weight[i], param.C * c_weight[j]);
+    int count = 0;
+    for (int l = 0; l < n; ++l) {
+        alpha[l] *= y[l];
+        if (alpha[l] != 0) count++;
+    }
+    TSVM_LOG << "rho = " << rho_out << ", #sv = " << count;
+}
+
+std::vector<float_type> SVC::predict(const DataSet::node2d &instances, int batch_size) {   // svc.cpp:179-185
+    predict_dec_values(instances, dec_values, batch_size);
+    return predict_label(dec_values, (int) instances.size());
+}
+
+// One-vs-one vote, ties to the lowest class index (svc.cpp:265-288).
+std::vector<float_type> SVC::predict_label(const std::vector<float_type> &dec, int n_instances) const {
+    std::vector<float_type> out(n_instances);
+    std::vector<int> votes(n_classes);
+    for (int r = 0; r < n_instances; ++r) {
+        std::fill(votes.begin(), votes.end(), 0);
+        int k = 0;
+        for (int i = 0; i < n_classes; ++i)
+            for (int j = i + 1; j < n_classes; ++j, ++k) votes[dec[(size_t) r * n_binary_models + k] > 0 ? i : j]++;
+        int best = 0;
+        for (int c = 1; c < n_classes; ++c) if (votes[c] > votes[best]) best = c;
+        out[r] = (float) label[best];
+    }
+    return out;
+}
+
+// ------------------------------------------------------------------------------------------------
+// NuSVC (nusvc.cpp)
+// ------------------------------------------------------------------------------------------------
+void NuSVC::model_setup(const DataSet &dataset, SvmParam &p) {
+    SVC::model_setup(dataset, p);
+    param.svm_type = SvmParam::NU_SVC;
+}
+
+void NuSVC::train_binary(const DataSet &dataset, int i, int j, std::vector<float_type> &alpha, float_type &rho_out) {
+    const std::vector<int> ids = dataset.original_index(i, j);
+    const int n_pos = dataset.count()[i], n = (int) ids.size();
+    std::vector<int> y(n);
+    std::vector<float_type> f_val(n, 0);
+    alpha.assign(n, 0);
+    float_type sum_pos = param.nu * n / 2;
+    float_type sum_neg = sum_pos;
+    for (int l = 0; l < n; ++l) {
+        float_type &budget = l < n_pos ? sum_pos : sum_neg;
+        y[l] = l < n_pos ? +1 : -1;
+        alpha[l] = std::min(1., budget);
+        budget -= alpha[l];
+    }
+    KernelMatrix k_mat(dataset.instances(), ids.data(), ids.size(), param);
+    NuSMOSolver solver(false);
+    run_solver(solver, k_mat, y, alpha, rho_out, f_val, 1, 1);
+    for (int l = 0; l < n; ++l) alpha[l] *= y[l];
+}
+
+// ------------------------------------------------------------------------------------------------
+// SVR / NuSVR (svr.cpp, nusvr.cpp): the 2n-variable problem, instances stacked twice
+// ------------------------------------------------------------------------------------------------
+void SVR::model_setup(const DataSet &dataset, SvmParam &p) {
+    n_classes = 2;
+    SvmModel::model_setup(dataset, p);
+    param.svm_type = SvmParam::EPSILON_SVR;
+}
+
+void SVR::train(const DataSet &dataset, SvmParam p) {
+    model_setup(dataset, p);
+    const int n = (int) dataset.n_instances();
+    KernelMatrix k_mat(dataset.instances(), nullptr, n, param, 2);
+    std::vector<float_type> f_val(2 * (size_t) n), alpha_2(2 * (size_t) n, 0);
+    std::vector<int> y(2 * (size_t) n);
+    for (int i = 0; i < n; ++i) {
+        f_val[i] = param.p - dataset.y()[i];
+        y[i] = +1;
+        f_val[i + n] = -param.p - dataset.y()[i];
+        y[i + n] = -1;
+    }
+    CSMOSolver solver;
+    run_solver(solver, k_mat, y, alpha_2, rho[0], f_val, param.C, param.C);
+    if (keep_binary) binary_alpha.push_back(alpha_2);
+    save_svr_coef(alpha_2, dataset.instances());
+    if (param.kernel_type == SvmParam::LINEAR) compute_linear_coef_single_model(dataset.n_features(), dataset.is_zero_based());
+}
+
+void SVR::save_svr_coef(const std::vector<float_type> &alpha_2, const DataSet::node2d &instances) {   // svr.cpp:43-62
+    const size_t n = alpha_2.size() / 2;
+    for (size_t i = 0; i < n; ++i) {
+        const float_type a = alpha_2[i] - alpha_2[i + n];
+        if (a != 0) {
+            sv.push_back(instances[i]);
+            sv_indices.push_back((int) i);
+            coef.push_back(a);
+        }
+    }
+    n_sv[0] = (int) sv.size();
+    n_sv[1] = 0;
+    n_total_sv = (int) sv.size();
+    TSVM_LOG << "rho = " << rho[0] << ", #sv = " << sv.size();
+}
+
+void NuSVR::model_setup(const DataSet &dataset, SvmParam &p) {
+    SVR::model_setup(dataset, p);
+    param.svm_type = SvmParam::NU_SVR;
+}
+
+void NuSVR::train(const DataSet &dataset, SvmParam p) {   // nusvr.cpp:7-41
+    model_setup(dataset, p);
+    const int n = (int) dataset.n_instances();
+    KernelMatrix k_mat(dataset.instances(), nullptr, n, param, 2);
+    std::vector<float_type> f_val(2 * (size_t) n), alpha_2(2 * (size_t) n);
+    std::vector<int> y(2 * (size_t) n);
+    float_type sum = param.C * param.nu * n / 2;
+    for (int i = 0; i < n; ++i) {
+        alpha_2[i] = alpha_2[i + n] = std::min(sum, param.C);
+        sum -= alpha_2[i];
+        f_val[i] = f_val[i + n] = -dataset.y()[i];
+        y[i] = +1;
+        y[i + n] = -1;
+    }
+    NuSMOSolver solver(true);
+    run_solver(solver, k_mat, y, alpha_2, rho[0], f_val, param.C, param.C);
+    if (keep_binary) binary_alpha.push_back(alpha_2);
+    save_svr_coef(alpha_2, dataset.instances());
+    if (param.kernel_type == SvmParam::LINEAR) compute_linear_coef_single_model(dataset.n_features(), dataset.is_zero_based());
+}
+
+// ------------------------------------------------------------------------------------------------
+// OneClassSVC (oneclass_svc.cpp)
+// ------------------------------------------------------------------------------------------------
+void OneClassSVC::model_setup(const DataSet &dataset, SvmParam &p) {
+    n_classes = 2;
+    SvmModel::model_setup(dataset, p);
+    param.svm_type = SvmParam::ONE_CLASS;
+}
+
+void OneClassSVC::train(const DataSet &dataset, SvmParam p) {
+    model_setup(dataset, p);
+    const int n = (int) dataset.n_instances();
+    KernelMatrix k_mat(dataset.instances(), param);
+    std::vector<float_type> alpha(n, 0), f_val(n, 0);
+    std::vector<int> y(n, 1);
+    const int full = static_cast<int>(param.nu * n);
+    for (int i = 0; i < full; ++i) alpha[i] = 1;
+    if (full < n) alpha[full] = param.nu * n - full;
+    CSMOSolver solver;
+    run_solver(solver, k_mat, y, alpha, rho[0], f_val, 1, 1);
+    if (keep_binary) binary_alpha.push_back(alpha);
+    for (int i = 0; i < n; ++i)
+        if (alpha[i] != 0) {
+            sv.push_back(dataset.instances()[i]);
+            sv_indices.push_back(i);
+            coef.push_back(alpha[i]);
+        }
+    n_sv[0] = (int) sv.size();
+    n_sv[1] = 0;
+    n_total_sv = (int) sv.size();
+    if (param.kernel_type == SvmParam::LINEAR) compute_linear_coef_single_model(dataset.n_features(), dataset.is_zero_based());
+}
+
+std::vector<float_type> OneClassSVC::predict(const DataSet::node2d &instances, int batch_size) {   // oneclass_svc.cpp:59-66
+    std::vector<float_type> dec = SvmModel::predict(instances, batch_size);
+    for (auto &v : dec) v = v > 0 ? 1 : -1;
+    return dec;
+}

@@ -1,0 +1,238 @@
+#include "solver.h"
+
+#include <climits>
+#include <cmath>
+#include <algorithm>
+
+using tsvm::abi_check;
+using tsvm::DeviceBuffer;
+
+namespace {
+
+inline bool up_set(float_type a, float_type y, float_type Cp, float_type Cn) { return (y > 0 && a < Cp) || (y < 0 && a > 0); }
+inline bool low_set(float_type a, float_type y, float_type Cp, float_type Cn) { return (y > 0 && a > 0) || (y < 0 && a < Cn); }
+inline bool free_sv(float_type a, float_type y, float_type Cp, float_type Cn) { return a > 0 && (y > 0 ? a < Cp : a < Cn); }
+
+struct PhaseTimer {
+    bool on;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    explicit PhaseTimer(bool on) : on(on) {
+        if (on) { TSVM_HIP_CHECK(hipEventCreate(&e0)); TSVM_HIP_CHECK(hipEventCreate(&e1)); }
+    }
+    ~PhaseTimer() { if (on) { (void) hipEventDestroy(e0); (void) hipEventDestroy(e1); } }
+    void begin() { if (on) TSVM_HIP_CHECK(hipEventRecord(e0, nullptr)); }
+    void end(double &acc) {
+        if (!on) return;
+        TSVM_HIP_CHECK(hipEventRecord(e1, nullptr));
+        TSVM_HIP_CHECK(hipEventSynchronize(e1));
+        float ms = 0;
+        TSVM_HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
+        acc += ms;
+    }
+};
+
+}  // namespace
+
+void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std::vector<float_type> &alpha,
+                       float_type &rho, std::vector<float_type> &f_val, float_type eps, float_type Cp, float_type Cn,
+                       int ws_size, int out_max_iter) const {
+    const int n = (int) k_mat.n_instances();
+    const int q = ws_size / 2;
+    const int64_t ld = ((int64_t) n + 1) / 2 * 2;   // even row stride keeps every kernel row 16-byte aligned
+    const bool nu = is_nu();
+    stats = SolverStats();
+
+    DeviceBuffer<int> d_y(n), d_ws(ws_size), d_slots_even(ws_size), d_slots_odd(ws_size);
+    DeviceBuffer<float_type> d_alpha(n), d_f(n), d_alpha_diff(ws_size), d_diff(2);
+    DeviceBuffer<kernel_type> d_k_rows((size_t) ws_size * ld);
+    DeviceBuffer<unsigned char> d_sel_ws(tsvm_select_workspace(n));
+    DeviceBuffer<unsigned char> d_smo_ws(tsvm_smo_solve_workspace(ws_size));
+    d_y.upload(y.data(), n);
+    d_alpha.upload(alpha.data(), n);
+    d_f.upload(f_val.data(), n);
+    d_diff.zero();
+    d_alpha_diff.zero();
+    {
+        // Rows kept from the previous working set are re-addressed, not copied (csmosolver.cpp:69,75):
+        // logical row t of the working set lives in physical row slot[t]; the two halves swap every iteration.
+        std::vector<int> even(ws_size), odd(ws_size);
+        for (int t = 0; t < ws_size; ++t) { even[t] = t; odd[t] = (t + q) % ws_size; }
+        d_slots_even.upload(even.data(), ws_size);
+        d_slots_odd.upload(odd.data(), ws_size);
+    }
+    double *h_diff = nullptr;
+    TSVM_HIP_CHECK(hipHostMalloc((void **) &h_diff, 2 * sizeof(double)));
+    h_diff[0] = h_diff[1] = 0;
+
+    init_f(alpha, y, k_mat, d_f.data());
+
+    const int max_iter = std::max(100000, ws_size > INT_MAX / 100 ? INT_MAX : 100 * ws_size);
+    long long local_iter = 0;
+    int same_local_diff_cnt = 0, swap_local_diff_cnt = 0;
+    float_type previous_local_diff = INFINITY, last_local_diff = INFINITY, second_last_local_diff = INFINITY;
+    PhaseTimer timer(profile);
+    if (trace) {
+        trace->ws_size = ws_size;
+        trace->diff.clear();
+        trace->ws.clear();
+    }
+
+    for (int iter = 0;; ++iter) {
+        const int *slots = (iter % 2 == 0) ? d_slots_even.data() : d_slots_odd.data();
+        timer.begin();
+        if (iter == 0) {
+            abi_check(tsvm_select_working_set(d_f.data(), d_y.data(), d_alpha.data(), n, Cp, Cn, nullptr, 0, d_ws.data(),
+                                              ws_size, nu, d_sel_ws.data(), nullptr));
+        } else {
+            TSVM_HIP_CHECK(hipMemcpyAsync(d_ws.data(), d_ws.data() + q, sizeof(int) * q, hipMemcpyDeviceToDevice, nullptr));
+            abi_check(tsvm_select_working_set(d_f.data(), d_y.data(), d_alpha.data(), n, Cp, Cn, d_ws.data(), q,
+                                              d_ws.data() + q, q, nu, d_sel_ws.data(), nullptr));
+        }
+        timer.end(stats.ms_select);
+        timer.begin();
+        if (iter == 0) {
+            k_mat.get_rows(d_ws.data(), ws_size, d_k_rows.data(), ld);
+        } else {
+            // new rows go to the physical half that the dropped rows occupied
+            const int phys0 = (iter % 2 == 0) ? q : 0;
+            k_mat.get_rows(d_ws.data() + q, q, d_k_rows.data() + (size_t) phys0 * ld, ld);
+        }
+        timer.end(stats.ms_get_rows);
+        timer.begin();
+        if (nu) {
+            abi_check(tsvm_nu_smo_solve(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), d_ws.data(), ws_size, Cp,
+                                        d_k_rows.data(), slots, ld, k_mat.diag(), eps, d_diff.data(), max_iter,
+                                        d_smo_ws.data(), nullptr));
+        } else {
+            abi_check(tsvm_c_smo_solve(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), d_ws.data(), ws_size, Cp,
+                                       Cn, d_k_rows.data(), slots, ld, k_mat.diag(), eps, d_diff.data(), max_iter,
+                                       d_smo_ws.data(), nullptr));
+        }
+        timer.end(stats.ms_local);
+        timer.begin();
+        abi_check(tsvm_update_f(d_f.data(), d_alpha_diff.data(), ws_size, d_k_rows.data(), slots, ld, n, nullptr));
+        timer.end(stats.ms_update_f);
+        TSVM_HIP_CHECK(hipMemcpyAsync(h_diff, d_diff.data(), 2 * sizeof(double), hipMemcpyDeviceToHost, nullptr));
+        TSVM_HIP_CHECK(hipStreamSynchronize(nullptr));
+        const double diff0 = h_diff[0], diff1 = h_diff[1];
+        local_iter += (long long) diff1;
+        if (trace && iter < trace->cap_iters) {
+            trace->diff.push_back(diff0);
+            trace->diff.push_back(diff1);
+            std::vector<int> w = d_ws.to_host();
+            trace->ws.insert(trace->ws.end(), w.begin(), w.end());
+        }
+
+        // stall guards and stopping rule (csmosolver.cpp:86-111)
+        if (fabs(diff0 - previous_local_diff) < eps * 0.001) {
+            same_local_diff_cnt++;
+        } else {
+            same_local_diff_cnt = 0;
+            previous_local_diff = diff0;
+        }
+        if (fabs(diff0 - second_last_local_diff) < eps * 0.001) swap_local_diff_cnt++;
+        else swap_local_diff_cnt = 0;
+        second_last_local_diff = last_local_diff;
+        last_local_diff = diff0;
+        if (iter % 100 == 0)
+            TSVM_LOG << "global iter = " << iter << ", total local iter = " << local_iter << ", diff = " << diff0;
+        const bool stalled = (same_local_diff_cnt >= 10 || swap_local_diff_cnt >= 10) && fabs(diff0 - 2.0) > eps;
+        if (stalled || diff0 < eps || (out_max_iter != -1 && iter == out_max_iter)) {
+            d_alpha.download(alpha.data(), n);
+            d_f.download(f_val.data(), n);
+            rho = calculate_rho(f_val, y, alpha, Cp, Cn);
+            stats.n_iter = iter + 1;
+            stats.local_iter = local_iter;
+            stats.obj = calculate_obj(f_val, alpha, y);
+            TSVM_LOG << "global iter = " << iter << ", total local iter = " << local_iter << ", diff = " << diff0
+                     << ", obj = " << stats.obj;
+            break;
+        }
+    }
+    (void) hipHostFree(h_diff);
+}
+
+// csmosolver.cpp:189-214: f starts from a non-zero alpha in batches of 101 rows.
+void CSMOSolver::init_f(const std::vector<float_type> &alpha, const std::vector<int> &y, const KernelMatrix &k_mat,
+                        float_type *d_f) const {
+    const size_t batch_size = 100;
+    const int n = (int) k_mat.n_instances();
+    const int64_t ld = ((int64_t) n + 1) / 2 * 2;
+    std::vector<int> idx_vec;
+    std::vector<float_type> alpha_diff_vec;
+    DeviceBuffer<int> d_idx;
+    DeviceBuffer<float_type> d_ad;
+    DeviceBuffer<kernel_type> d_rows;
+    for (size_t i = 0; i < alpha.size(); ++i) {
+        if (alpha[i] != 0) {
+            idx_vec.push_back((int) i);
+            alpha_diff_vec.push_back(-alpha[i] * y[i]);
+        }
+        if (idx_vec.size() > batch_size || (i == alpha.size() - 1 && !idx_vec.empty())) {
+            const int m = (int) idx_vec.size();
+            if (d_rows.size() == 0) {
+                d_idx.resize(batch_size + 1);
+                d_ad.resize(batch_size + 1);
+                d_rows.resize((batch_size + 1) * (size_t) ld);
+            }
+            d_idx.upload(idx_vec.data(), m);
+            d_ad.upload(alpha_diff_vec.data(), m);
+            k_mat.get_rows(d_idx.data(), m, d_rows.data(), ld);
+            abi_check(tsvm_update_f(d_f, d_ad.data(), m, d_rows.data(), nullptr, ld, n, nullptr));
+            TSVM_HIP_CHECK(hipStreamSynchronize(nullptr));
+            idx_vec.clear();
+            alpha_diff_vec.clear();
+        }
+    }
+}
+
+// csmosolver.cpp:167-187
+float_type CSMOSolver::calculate_rho(const std::vector<float_type> &f_val, const std::vector<int> &y,
+                                     std::vector<float_type> &alpha, float_type Cp, float_type Cn) const {
+    int n_free = 0;
+    double sum_free = 0;
+    float_type up_value = INFINITY, low_value = -INFINITY;
+    for (size_t i = 0; i < alpha.size(); ++i) {
+        if (free_sv(alpha[i], y[i], Cp, Cn)) { n_free++; sum_free += f_val[i]; }
+        if (up_set(alpha[i], y[i], Cp, Cn)) up_value = std::min(up_value, f_val[i]);
+        if (low_set(alpha[i], y[i], Cp, Cn)) low_value = std::max(low_value, f_val[i]);
+    }
+    return n_free != 0 ? sum_free / n_free : -(up_value + low_value) / 2;
+}
+
+// csmosolver.cpp:227-239
+float_type CSMOSolver::calculate_obj(const std::vector<float_type> &f_val, const std::vector<float_type> &alpha,
+                                     const std::vector<int> &y) const {
+    float_type obj = 0;
+    for (size_t i = 0; i < f_val.size(); ++i) obj += alpha[i] - (f_val[i] + y[i]) * alpha[i] * y[i] / 2;
+    return -obj;
+}
+
+// nusmosolver.cpp:9-46,120-126
+float_type NuSMOSolver::calculate_rho(const std::vector<float_type> &f_val, const std::vector<int> &y,
+                                      std::vector<float_type> &alpha, float_type Cp, float_type Cn) const {
+    int n_free_p = 0, n_free_n = 0;
+    float_type sum_free_p = 0, sum_free_n = 0;
+    float_type up_p = INFINITY, up_n = INFINITY, low_p = -INFINITY, low_n = -INFINITY;
+    for (size_t i = 0; i < alpha.size(); ++i) {
+        const float_type a = alpha[i], nf = -f_val[i];
+        if (y[i] > 0) {
+            if (a > 0 && a < Cp) { n_free_p++; sum_free_p += f_val[i]; }
+            if (up_set(a, y[i], Cp, Cn)) up_p = std::min(up_p, nf);
+            if (low_set(a, y[i], Cp, Cn)) low_p = std::max(low_p, nf);
+        } else {
+            if (a > 0 && a < Cn) { n_free_n++; sum_free_n += nf; }
+            if (up_set(a, y[i], Cp, Cn)) up_n = std::min(up_n, nf);
+            if (low_set(a, y[i], Cp, Cn)) low_n = std::max(low_n, nf);
+        }
+    }
+    const float_type r1 = n_free_p != 0 ? sum_free_p / n_free_p : -(up_p + low_p) / 2;
+    const float_type r2 = n_free_n != 0 ? sum_free_n / n_free_n : -(up_n + low_n) / 2;
+    float_type rho = (r1 - r2) / 2;
+    if (!for_svr) {   // scale_alpha_rho: nu-SVC rescales, nu-SVR does not
+        const float_type r = (r1 + r2) / 2;
+        for (auto &a : alpha) a /= r;
+        rho /= r;
+    }
+    return rho;
+}
