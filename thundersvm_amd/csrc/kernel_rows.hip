@@ -20,23 +20,30 @@ typedef double v4d __attribute__((ext_vector_type(4)));
 // Working-set rows are the A operand (D rows), all-rows X is the B operand (D columns), so the 16
 // lanes l%16 of one store cover 16 consecutive j: a 128-byte run of an output row.
 //
-// Workgroup = 256 threads = 4 wavefronts in a 2x2 grid; each wavefront owns a 64x64 block of the
-// 128x128 output tile as 4x4 MFMA tiles (64 accumulator doubles per lane).  K is walked in tiles
+// Workgroup = 256 threads = 4 wavefronts in a 2x2 grid; each wavefront owns a (16*TI)x64 block of the
+// (32*TI)x128 output tile as TIx4 MFMA tiles (16*TI accumulator doubles per lane).  K is walked in tiles
 // of 8 columns staged through LDS in k-major order [8][130]: the stride of 130 doubles keeps both
 // the staging writes and the operand reads free of bank conflicts.
 // ------------------------------------------------------------------------------------------------
-#define GR_BM 128
 #define GR_BN 128
 #define GR_KT 8
 #define GR_LS 130
 
-__global__ __launch_bounds__(256) void get_rows_dense_kernel(
+// KT: kernel type (compile-time so that only one epilogue is instantiated); TI: 16-row MFMA tiles
+// per wavefront in the working-row direction (4 -> 128-row workgroup tile, 2 -> 64-row tile with
+// half the accumulators and twice the resident wavefronts, used when d is small and the epilogue
+// and stores dominate).
+template <int KT, int TI>
+__global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
     const double *__restrict__ x, int64_t ldx, int64_t n, int d, const double *__restrict__ sd_x,
     const double *__restrict__ a, int64_t lda, const int *__restrict__ a_idx, int m, const double *__restrict__ sd_a,
-    KernelParam kp, double *__restrict__ out, int64_t ldo, unsigned m_blocks) {
+    KernelParam kp_in, double *__restrict__ out, int64_t ldo, unsigned m_blocks) {
+    constexpr int BM = 32 * TI;
     __shared__ double As[GR_KT * GR_LS];
     __shared__ double Bs[GR_KT * GR_LS];
     __shared__ uint64_t exp_tab[32];
+    KernelParam kp = kp_in;
+    kp.kernel_type = KT;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -47,16 +54,16 @@ __global__ __launch_bounds__(256) void get_rows_dense_kernel(
 
     const unsigned logical = xcd_remap(blockIdx.x, gridDim.x);
     const int64_t j0 = (int64_t) (logical / m_blocks) * GR_BN;
-    const int i0 = (int) (logical % m_blocks) * GR_BM;
+    const int i0 = (int) (logical % m_blocks) * BM;
 
-    // staging assignment: thread -> (row = tid/2, 4 consecutive k at 4*(tid&1))
+    // staging assignment: thread -> (row = tid/2, 4 consecutive k at 4*(tid&1)); the A tile has BM rows
     const int srow = tid >> 1;
     const int skh = (tid & 1) * 4;
     const double *a_ptr = nullptr;
     const double *x_ptr = nullptr;
     {
         int ai = i0 + srow;
-        if (ai < m) {
+        if (srow < BM && ai < m) {
             int64_t r = a_idx ? (int64_t) a_idx[ai] : (int64_t) ai;
             a_ptr = a + r * lda + skh;
         }
@@ -64,9 +71,9 @@ __global__ __launch_bounds__(256) void get_rows_dense_kernel(
         if (xj < n) x_ptr = x + xj * ldx + skh;
     }
 
-    v4d acc[4][4];
+    v4d acc[TI][4];
 #pragma unroll
-    for (int ti = 0; ti < 4; ++ti)
+    for (int ti = 0; ti < TI; ++ti)
 #pragma unroll
         for (int tj = 0; tj < 4; ++tj) acc[ti][tj] = (v4d){0.0, 0.0, 0.0, 0.0};
 
@@ -81,7 +88,7 @@ __global__ __launch_bounds__(256) void get_rows_dense_kernel(
     for (int kt = 0; kt < n_kt; ++kt) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            As[(skh + e) * GR_LS + srow] = ra[e];
+            if (srow < BM) As[(skh + e) * GR_LS + srow] = ra[e];
             Bs[(skh + e) * GR_LS + srow] = rb[e];
         }
         __syncthreads();
@@ -91,15 +98,14 @@ __global__ __launch_bounds__(256) void get_rows_dense_kernel(
         }
 #pragma unroll
         for (int ks = 0; ks < GR_KT / 4; ++ks) {
-            double af[4], bf[4];
+            double af[TI], bf[4];
             const int kk = (ks * 4 + lk) * GR_LS;
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                af[t] = As[kk + wi * 64 + t * 16 + lrow];
-                bf[t] = Bs[kk + wj * 64 + t * 16 + lrow];
-            }
+            for (int t = 0; t < TI; ++t) af[t] = As[kk + wi * (16 * TI) + t * 16 + lrow];
 #pragma unroll
-            for (int ti = 0; ti < 4; ++ti)
+            for (int t = 0; t < 4; ++t) bf[t] = Bs[kk + wj * 64 + t * 16 + lrow];
+#pragma unroll
+            for (int ti = 0; ti < TI; ++ti)
 #pragma unroll
                 for (int tj = 0; tj < 4; ++tj)
                     acc[ti][tj] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[ti], bf[tj], acc[ti][tj], 0, 0, 0);
@@ -116,10 +122,10 @@ __global__ __launch_bounds__(256) void get_rows_dense_kernel(
         sdj[tj] = (jj[tj] < n && sd_x) ? sd_x[jj[tj]] : 0.0;
     }
 #pragma unroll
-    for (int ti = 0; ti < 4; ++ti) {
+    for (int ti = 0; ti < TI; ++ti) {
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
-            const int i = i0 + wi * 64 + ti * 16 + 4 * v + lk;
+            const int i = i0 + wi * (16 * TI) + ti * 16 + 4 * v + lk;
             if (i >= m) continue;
             double sdi = 0.0;
             if (sd_a) sdi = sd_a[a_idx ? a_idx[i] : i];
@@ -379,11 +385,28 @@ int tsvm_get_rows_dense(const double *x, int64_t ldx, int64_t n, int d, const do
                  "tsvm_get_rows_dense: RBF needs self dot products");
     if (n == 0 || m == 0) return 0;
     KernelParam kp{kernel_type, degree, gamma, coef0};
-    const unsigned m_blocks = (unsigned) ((m + GR_BM - 1) / GR_BM);
+    // small feature counts: the epilogue and the stores dominate, run the 64-row tile at higher occupancy
+    const int ti = d <= 256 ? 2 : 4;
+    const unsigned m_blocks = (unsigned) ((m + 32 * ti - 1) / (32 * ti));
     const int64_t n_blocks = (n + GR_BN - 1) / GR_BN;
     TSVM_REQUIRE(n_blocks * m_blocks < (int64_t) 0x7fffffff, "tsvm_get_rows_dense: grid too large");
-    hipLaunchKernelGGL(get_rows_dense_kernel, dim3((unsigned) (n_blocks * m_blocks)), dim3(256), 0, tsvm_s(stream), x, ldx,
-                       n, d, sd_x, a, lda, a_idx, m, sd_a, kp, out, ldo, m_blocks);
+    const dim3 grid((unsigned) (n_blocks * m_blocks)), block(256);
+#define GR_LAUNCH(KTYPE)                                                                                              \
+    do {                                                                                                              \
+        if (ti == 2)                                                                                                  \
+            hipLaunchKernelGGL((get_rows_dense_kernel<KTYPE, 2>), grid, block, 0, tsvm_s(stream), x, ldx, n, d, sd_x, a, \
+                               lda, a_idx, m, sd_a, kp, out, ldo, m_blocks);                                          \
+        else                                                                                                          \
+            hipLaunchKernelGGL((get_rows_dense_kernel<KTYPE, 4>), grid, block, 0, tsvm_s(stream), x, ldx, n, d, sd_x, a, \
+                               lda, a_idx, m, sd_a, kp, out, ldo, m_blocks);                                          \
+    } while (0)
+    switch (kernel_type) {
+        case TSVM_LINEAR: GR_LAUNCH(TSVM_LINEAR); break;
+        case TSVM_POLY: GR_LAUNCH(TSVM_POLY); break;
+        case TSVM_SIGMOID: GR_LAUNCH(TSVM_SIGMOID); break;
+        default: GR_LAUNCH(TSVM_RBF); break;
+    }
+#undef GR_LAUNCH
     TSVM_LAUNCH_CHECK();
     return 0;
 }

@@ -95,252 +95,6 @@ __global__ __launch_bounds__(UF_T) void update_f_kernel(double *__restrict__ f, 
 }
 
 // ------------------------------------------------------------------------------------------------
-// Working-set block gather: kws[r*ws + t] = K_r[working_set[t]].  Turns the local solver's two
-// scattered row gathers per inner iteration (smo_kernel.cpp:50-52,107-110) into coalesced reads.
-// ------------------------------------------------------------------------------------------------
-__global__ void gather_ws_block_kernel(const double *__restrict__ k_rows, const int *__restrict__ slots, int64_t ld,
-                                       const int *__restrict__ working_set, int ws, double *__restrict__ kws) {
-    const int r = blockIdx.x;
-    const double *row = k_rows + (int64_t) (slots ? slots[r] : r) * ld;
-    for (int t = threadIdx.x; t < ws; t += blockDim.x) kws[(int64_t) r * ws + t] = row[working_set[t]];
-}
-
-// ------------------------------------------------------------------------------------------------
-// c_smo_solve (smo_kernel.cpp:12-114): one workgroup, one thread per working-set element.
-// f, alpha, y live in registers; per inner iteration: one reduction round for (i, up, low), one
-// for j2, two coalesced row reads of the gathered ws x ws block.  Reductions are lexicographic
-// (value, index) minima so ties resolve to the lowest index exactly as the serial loops do.
-// ------------------------------------------------------------------------------------------------
-template <int NW>
-__device__ __forceinline__ void block_argmin(const double *s_v, const int *s_i, double &v, int &i) {
-    v = s_v[0];
-    i = s_i[0];
-#pragma unroll
-    for (int w = 1; w < NW; ++w) {
-        const double ov = s_v[w];
-        const int oi = s_i[w];
-        if (ov < v || (ov == v && oi < i)) { v = ov; i = oi; }
-    }
-}
-
-template <int NW>
-__global__ __launch_bounds__(NW * 64) void c_smo_solve_kernel(
-    const int *__restrict__ label, const double *__restrict__ f_val, double *__restrict__ alpha,
-    double *__restrict__ alpha_diff, const int *__restrict__ working_set, int ws, double Cp, double Cn,
-    const double *__restrict__ kws, const double *__restrict__ k_diag, double eps, double *__restrict__ diff,
-    int max_iter) {
-    __shared__ double s_kd[NW * 64];
-    __shared__ float s_y[NW * 64];
-    __shared__ double s_a[2][NW * 64];
-    __shared__ double s_f[2][NW * 64];
-    __shared__ double s_kI[NW * 64];
-    __shared__ double sA_v[NW], sA_l[NW], sB_v[NW];
-    __shared__ int sA_i[NW], sB_i[NW];
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
-    const bool active = tid < ws;
-    const int wsi = active ? working_set[tid] : 0;
-    double f = active ? f_val[wsi] : 0.0;
-    double a = active ? alpha[wsi] : 0.0;
-    const double a_old = a;
-    const double y = active ? (double) label[wsi] : 0.0;
-    const double kd = active ? k_diag[wsi] : 0.0;
-    s_kd[tid] = kd;
-    s_y[tid] = (float) y;
-    double local_eps = 0.0;
-    int numOfIter = 0;
-    while (true) {
-        const int par = numOfIter & 1;
-        s_a[par][tid] = a;
-        s_f[par][tid] = f;
-        // i = first argmin of f over I_up; low = max of f over I_low
-        double v = (active && is_I_up(a, y, Cp, Cn) && f < TSVM_INF) ? f : TSVM_INF;
-        int vi = tid;
-        double lw = (active && is_I_low(a, y, Cp, Cn) && f > -TSVM_INF) ? f : -TSVM_INF;
-        wave_argmin(v, vi);
-        lw = wave_max(lw);
-        if (lane == 0) { sA_v[wave] = v; sA_i[wave] = vi; sA_l[wave] = lw; }
-        __syncthreads();
-        double up_value;
-        int i;
-        block_argmin<NW>(sA_v, sA_i, up_value, i);
-        double low_value = sA_l[0];
-#pragma unroll
-        for (int w = 1; w < NW; ++w) low_value = sA_l[w] > low_value ? sA_l[w] : low_value;
-        if (!(up_value < TSVM_INF)) i = 0;
-        const double local_diff = low_value - up_value;
-        if (numOfIter == 0) {
-            const double t = 0.1f * local_diff;
-            local_eps = eps > t ? eps : t;
-            if (tid == 0) diff[0] = local_diff;
-        }
-        if (numOfIter > max_iter || local_diff < local_eps) break;
-        const double kI = active ? kws[(int64_t) i * ws + tid] : 0.0;
-        s_kI[tid] = kI;
-        const double kd_i = s_kd[i];
-        // j2 = first argmin of -b^2/a over I_low with f > up
-        double ft = TSVM_INF;
-        if (active && -up_value > -f && is_I_low(a, y, Cp, Cn)) {
-            const double aIJ = kd_i + kd - 2 * kI;
-            const double bIJ = -up_value + f;
-            const double t = -bIJ * bIJ / aIJ;
-            if (t < TSVM_INF) ft = t;
-        }
-        int fi = tid;
-        wave_argmin(ft, fi);
-        if (lane == 0) { sB_v[wave] = ft; sB_i[wave] = fi; }
-        __syncthreads();
-        double min_t;
-        int j2;
-        block_argmin<NW>(sB_v, sB_i, min_t, j2);
-        if (!(min_t < TSVM_INF)) j2 = 0;
-        const double a_i = s_a[par][i], y_i = (double) s_y[i];
-        const double a_j = s_a[par][j2], y_j = (double) s_y[j2];
-        const double alpha_i_diff = y_i > 0 ? Cp - a_i : a_i;
-        const double q1 = y_j > 0 ? a_j : Cn - a_j;
-        const double q2 = (-up_value + s_f[par][j2]) / (kd_i + s_kd[j2] - 2 * s_kI[j2]);
-        const double alpha_j_diff = q1 < q2 ? q1 : q2;
-        const double l = alpha_i_diff < alpha_j_diff ? alpha_i_diff : alpha_j_diff;
-        if (tid == i) a += l * y;
-        if (tid == j2) a -= l * y;
-        const double kJ = active ? kws[(int64_t) j2 * ws + tid] : 0.0;
-        f = __builtin_fma(-l, kJ - kI, f);
-        ++numOfIter;
-    }
-    if (active) {
-        alpha_diff[tid] = -(a - a_old) * y;
-        alpha[wsi] = a;
-    }
-    if (tid == 0) diff[1] = (double) numOfIter;
-}
-
-// ------------------------------------------------------------------------------------------------
-// nu_smo_solve (smo_kernel.cpp:127-287).  Same structure with four extrema.  Keeps the CPU code's
-// j2n score, which uses kd[ip] and K[ip, .] (smo_kernel.cpp:239), and does not write diff[1].
-// ------------------------------------------------------------------------------------------------
-template <int NW>
-__global__ __launch_bounds__(NW * 64) void nu_smo_solve_kernel(
-    const int *__restrict__ label, const double *__restrict__ f_val, double *__restrict__ alpha,
-    double *__restrict__ alpha_diff, const int *__restrict__ working_set, int ws, double C,
-    const double *__restrict__ kws, const double *__restrict__ k_diag, double eps, double *__restrict__ diff,
-    int max_iter) {
-    __shared__ double s_kd[NW * 64];
-    __shared__ float s_y[NW * 64];
-    __shared__ double s_a[2][NW * 64];
-    __shared__ double s_f[2][NW * 64];
-    __shared__ double s_kIp[NW * 64], s_kIn[NW * 64];
-    __shared__ double sA_vp[NW], sA_vn[NW], sA_lp[NW], sA_ln[NW], sB_vp[NW], sB_vn[NW];
-    __shared__ int sA_ip[NW], sA_in[NW], sB_ip[NW], sB_in[NW];
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
-    const bool active = tid < ws;
-    const int wsi = active ? working_set[tid] : 0;
-    double f = active ? f_val[wsi] : 0.0;
-    double a = active ? alpha[wsi] : 0.0;
-    const double a_old = a;
-    const int yi_ = active ? label[wsi] : 0;
-    const double y = (double) yi_;
-    const double kd = active ? k_diag[wsi] : 0.0;
-    s_kd[tid] = kd;
-    s_y[tid] = (float) y;
-    double local_eps = 0.0;
-    int numOfIter = 0;
-    while (true) {
-        const int par = numOfIter & 1;
-        s_a[par][tid] = a;
-        s_f[par][tid] = f;
-        double vp = (active && yi_ > 0 && a < C && f < TSVM_INF) ? f : TSVM_INF;
-        double vn = (active && yi_ < 0 && a > 0 && f < TSVM_INF) ? f : TSVM_INF;
-        double lp = (active && yi_ > 0 && a > 0 && f > -TSVM_INF) ? f : -TSVM_INF;
-        double ln = (active && yi_ < 0 && a < C && f > -TSVM_INF) ? f : -TSVM_INF;
-        int ipi = tid, ini = tid;
-        wave_argmin(vp, ipi);
-        wave_argmin(vn, ini);
-        lp = wave_max(lp);
-        ln = wave_max(ln);
-        if (lane == 0) {
-            sA_vp[wave] = vp; sA_ip[wave] = ipi; sA_vn[wave] = vn; sA_in[wave] = ini;
-            sA_lp[wave] = lp; sA_ln[wave] = ln;
-        }
-        __syncthreads();
-        double up_value_p, up_value_n;
-        int ip, in;
-        block_argmin<NW>(sA_vp, sA_ip, up_value_p, ip);
-        block_argmin<NW>(sA_vn, sA_in, up_value_n, in);
-        if (!(up_value_p < TSVM_INF)) ip = 0;
-        if (!(up_value_n < TSVM_INF)) in = 0;
-        double low_value_p = sA_lp[0], low_value_n = sA_ln[0];
-#pragma unroll
-        for (int w = 1; w < NW; ++w) {
-            low_value_p = sA_lp[w] > low_value_p ? sA_lp[w] : low_value_p;
-            low_value_n = sA_ln[w] > low_value_n ? sA_ln[w] : low_value_n;
-        }
-        const double dp = low_value_p - up_value_p, dn = low_value_n - up_value_n;
-        const double local_diff = dp > dn ? dp : dn;  // max(x, y) = x > y ? x : y
-        if (numOfIter == 0) {
-            const double t = 0.1 * local_diff;
-            local_eps = eps > t ? eps : t;
-            if (tid == 0) diff[0] = local_diff;
-        }
-        if (numOfIter > max_iter || local_diff < local_eps) break;
-        const double kIp = active ? kws[(int64_t) ip * ws + tid] : 0.0;
-        const double kIn = active ? kws[(int64_t) in * ws + tid] : 0.0;
-        s_kIp[tid] = kIp;
-        s_kIn[tid] = kIn;
-        const double kd_ip = s_kd[ip];
-        double ftp = TSVM_INF, ftn = TSVM_INF;
-        if (active && -up_value_p > -f && yi_ > 0 && a > 0) {
-            const double aIJ = kd_ip + kd - 2 * kIp;
-            const double bIJ = -up_value_p + f;
-            const double t = -bIJ * bIJ / aIJ;
-            if (t < TSVM_INF) ftp = t;
-        }
-        if (active && -up_value_n > -f && yi_ < 0 && a < C) {
-            const double aIJ = kd_ip + kd - 2 * kIp;
-            const double bIJ = -up_value_n + f;
-            const double t = -bIJ * bIJ / aIJ;
-            if (t < TSVM_INF) ftn = t;
-        }
-        int jpi = tid, jni = tid;
-        wave_argmin(ftp, jpi);
-        wave_argmin(ftn, jni);
-        if (lane == 0) { sB_vp[wave] = ftp; sB_ip[wave] = jpi; sB_vn[wave] = ftn; sB_in[wave] = jni; }
-        __syncthreads();
-        double f_val_j2p, f_val_j2n;
-        int j2p, j2n;
-        block_argmin<NW>(sB_vp, sB_ip, f_val_j2p, j2p);
-        block_argmin<NW>(sB_vn, sB_in, f_val_j2n, j2n);
-        if (!(f_val_j2p < TSVM_INF)) j2p = 0;
-        if (!(f_val_j2n < TSVM_INF)) j2n = 0;
-        int i, j2;
-        double up_value, kIj2, kI;
-        if (f_val_j2p < f_val_j2n) {
-            i = ip; j2 = j2p; up_value = up_value_p; kIj2 = s_kIp[j2p]; kI = kIp;
-        } else {
-            i = in; j2 = j2n; up_value = up_value_n; kIj2 = s_kIn[j2n]; kI = kIn;
-        }
-        const double a_i = s_a[par][i], y_i = (double) s_y[i];
-        const double a_j = s_a[par][j2], y_j = (double) s_y[j2];
-        const double alpha_i_diff = y_i > 0 ? C - a_i : a_i;
-        const double q1 = y_j > 0 ? a_j : C - a_j;
-        const double q2 = (-up_value + s_f[par][j2]) / (s_kd[i] + s_kd[j2] - 2 * kIj2);
-        const double alpha_j_diff = q1 < q2 ? q1 : q2;
-        const double l = alpha_i_diff < alpha_j_diff ? alpha_i_diff : alpha_j_diff;
-        if (tid == i) a += l * y;
-        if (tid == j2) a -= l * y;
-        const double kJ = active ? kws[(int64_t) j2 * ws + tid] : 0.0;
-        f = __builtin_fma(-l, kJ - kI, f);
-        ++numOfIter;
-    }
-    if (active) {
-        alpha_diff[tid] = -(a - a_old) * y;
-        alpha[wsi] = a;
-    }
-}
-
-// ------------------------------------------------------------------------------------------------
 // Fused sort_f + select_working_set.
 //
 // The reference sorts (f, index) pairs ascending (smo_kernel.cpp:321-332) and then walks the
@@ -761,63 +515,6 @@ int tsvm_update_f(double *f, const double *alpha_diff, int ws_size, const double
     const unsigned grid = (unsigned) ((n + UF_T * 2 - 1) / (UF_T * 2));
     hipLaunchKernelGGL(update_f_kernel, dim3(grid), dim3(UF_T), 0, tsvm_s(stream), f, alpha_diff, ws_size, k_rows, slots,
                        ld, n);
-    TSVM_LAUNCH_CHECK();
-    return 0;
-}
-
-size_t tsvm_smo_solve_workspace(int ws_size) {
-    if (ws_size < 0) return 0;
-    return sizeof(double) * (size_t) ws_size * (size_t) ws_size + 256;
-}
-
-static int launch_gather(const double *k_rows, const int *slots, int64_t ld, const int *working_set, int ws,
-                         void *workspace, hipStream_t s) {
-    hipLaunchKernelGGL(gather_ws_block_kernel, dim3(ws), dim3(ws < 256 ? 64 : 256), 0, s, k_rows, slots, ld, working_set,
-                       ws, (double *) workspace);
-    TSVM_LAUNCH_CHECK();
-    return 0;
-}
-
-#define TSVM_DISPATCH_NW(KERNEL, ...)                                                                          \
-    do {                                                                                                       \
-        const int nw_ = (ws_size + 63) / 64;                                                                   \
-        if (nw_ <= 1) hipLaunchKernelGGL(KERNEL<1>, dim3(1), dim3(64), 0, s, __VA_ARGS__);                      \
-        else if (nw_ <= 2) hipLaunchKernelGGL(KERNEL<2>, dim3(1), dim3(128), 0, s, __VA_ARGS__);                \
-        else if (nw_ <= 4) hipLaunchKernelGGL(KERNEL<4>, dim3(1), dim3(256), 0, s, __VA_ARGS__);                \
-        else if (nw_ <= 8) hipLaunchKernelGGL(KERNEL<8>, dim3(1), dim3(512), 0, s, __VA_ARGS__);                \
-        else hipLaunchKernelGGL(KERNEL<16>, dim3(1), dim3(1024), 0, s, __VA_ARGS__);                            \
-    } while (0)
-
-int tsvm_c_smo_solve(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
-                     int ws_size, double Cp, double Cn, const double *k_rows, const int *slots, int64_t ld,
-                     const double *k_diag, double eps, double *diff, int max_iter, void *workspace,
-                     tsvm_stream stream) {
-    TSVM_REQUIRE(y && f_val && alpha && alpha_diff && working_set && k_rows && k_diag && diff && workspace,
-                 "tsvm_c_smo_solve: null pointer");
-    TSVM_REQUIRE(ws_size >= 1 && ws_size <= MAX_WS, "tsvm_c_smo_solve: ws_size %d outside [1, %d]", ws_size, MAX_WS);
-    hipStream_t s = tsvm_s(stream);
-    int rc = launch_gather(k_rows, slots, ld, working_set, ws_size, workspace, s);
-    if (rc) return rc;
-    const double *kws = (const double *) workspace;
-    TSVM_DISPATCH_NW(c_smo_solve_kernel, y, f_val, alpha, alpha_diff, working_set, ws_size, Cp, Cn, kws, k_diag, eps, diff,
-                     max_iter);
-    TSVM_LAUNCH_CHECK();
-    return 0;
-}
-
-int tsvm_nu_smo_solve(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
-                      int ws_size, double C, const double *k_rows, const int *slots, int64_t ld,
-                      const double *k_diag, double eps, double *diff, int max_iter, void *workspace,
-                      tsvm_stream stream) {
-    TSVM_REQUIRE(y && f_val && alpha && alpha_diff && working_set && k_rows && k_diag && diff && workspace,
-                 "tsvm_nu_smo_solve: null pointer");
-    TSVM_REQUIRE(ws_size >= 1 && ws_size <= MAX_WS, "tsvm_nu_smo_solve: ws_size %d outside [1, %d]", ws_size, MAX_WS);
-    hipStream_t s = tsvm_s(stream);
-    int rc = launch_gather(k_rows, slots, ld, working_set, ws_size, workspace, s);
-    if (rc) return rc;
-    const double *kws = (const double *) workspace;
-    TSVM_DISPATCH_NW(nu_smo_solve_kernel, y, f_val, alpha, alpha_diff, working_set, ws_size, C, kws, k_diag, eps, diff,
-                     max_iter);
     TSVM_LAUNCH_CHECK();
     return 0;
 }

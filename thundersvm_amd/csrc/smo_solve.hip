@@ -1,0 +1,367 @@
+// The local SMO solvers: c_smo_solve / nu_smo_solve (src/thundersvm/kernel/smo_kernel.cpp:12-287,
+// USE_CUDA=OFF semantics) as one LDS-resident workgroup on gfx950.
+//
+// Shape of the kernel.  One workgroup of 256 threads (one wavefront per SIMD of the CU) holds the
+// whole working set: element t = e*256 + tid lives in register slot e of thread tid (E = ws/256
+// slots, up to 4), with its f, alpha, y and diagonal.  One inner iteration is
+//   1. (i, up) = first argmin of f over I_up and low = max of f over I_low: a per-thread scan of
+//      its E slots, a DPP reduction inside each wavefront, four partial results through LDS;
+//   2. row K[i, .] of the gathered ws x ws block (coalesced);
+//   3. j2 = first argmin of -b^2/a over I_low with f > up: same reduction shape;
+//   4. the two-variable step, row K[j2, .], f -= l * (K[j2, .] - K[i, .]).
+// Two workgroup barriers per iteration.  Reductions are lexicographic (value, element index)
+// minima, so ties go to the lowest index exactly as the reference's serial loops resolve them, and
+// all arithmetic is the reference's expression order in IEEE double (the library is compiled with
+// -ffp-contract=off; the one fused operation, f -= l*(kJ - kI), is an explicit fma as gcc -O3
+// contracts it on an FMA host).
+#include "../../include/thundersvm_amd.h"
+#include "tsvm_device.h"
+#include "tsvm_internal.h"
+
+#define TSVM_INF __builtin_inf()
+#define MAX_WS 1024
+#define SV_T 256           // threads of the solver workgroup
+#define SV_W (SV_T / 64)   // wavefronts
+
+// kws[r*ws + t] = K_r[working_set[t]]: the ws x ws block the solver reads, gathered once per call so
+// that the two row reads per inner iteration (smo_kernel.cpp:50-52,107-110) are contiguous.
+__global__ void gather_ws_block_kernel(const double *__restrict__ k_rows, const int *__restrict__ slots, int64_t ld,
+                                       const int *__restrict__ working_set, int ws, double *__restrict__ kws) {
+    const int r = blockIdx.x;
+    const double *row = k_rows + (int64_t) (slots ? slots[r] : r) * ld;
+    for (int t = threadIdx.x; t < ws; t += blockDim.x) kws[(int64_t) r * ws + t] = row[working_set[t]];
+}
+
+// Combines the per-wavefront partial results (one LDS entry per wavefront) in wavefront order.
+__device__ __forceinline__ void block_argmin(const double *s_v, const int *s_i, double &v, int &i) {
+    v = s_v[0];
+    i = s_i[0];
+#pragma unroll
+    for (int w = 1; w < SV_W; ++w) lexmin(v, i, s_v[w], s_i[w]);
+}
+__device__ __forceinline__ double block_max(const double *s_v) {
+    double v = s_v[0];
+#pragma unroll
+    for (int w = 1; w < SV_W; ++w) v = s_v[w] > v ? s_v[w] : v;
+    return v;
+}
+
+template <int E>
+__global__ __launch_bounds__(SV_T) void c_smo_solve_kernel(
+    const int *__restrict__ label, const double *__restrict__ f_val, double *__restrict__ alpha,
+    double *__restrict__ alpha_diff, const int *__restrict__ working_set, int ws, double Cp, double Cn,
+    const double *__restrict__ kws, const double *__restrict__ k_diag, double eps, double *__restrict__ diff,
+    int max_iter) {
+    __shared__ double s_kd[E * SV_T];
+    __shared__ float s_y[E * SV_T];
+    __shared__ double s_a[2][E * SV_T];
+    __shared__ double s_f[2][E * SV_T];
+    __shared__ double s_kI[E * SV_T];
+    __shared__ double sA_v[SV_W], sA_l[SV_W], sB_v[SV_W];
+    __shared__ int sA_i[SV_W], sB_i[SV_W];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    double f[E], a[E], a_old[E], y[E], kd[E], kI[E];
+    int wsi[E];
+    bool active[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        const int t = e * SV_T + tid;
+        active[e] = t < ws;
+        wsi[e] = active[e] ? working_set[t] : 0;
+        f[e] = active[e] ? f_val[wsi[e]] : 0.0;
+        a[e] = active[e] ? alpha[wsi[e]] : 0.0;
+        a_old[e] = a[e];
+        y[e] = active[e] ? (double) label[wsi[e]] : 0.0;
+        kd[e] = active[e] ? k_diag[wsi[e]] : 0.0;
+        s_kd[t] = kd[e];
+        s_y[t] = (float) y[e];
+    }
+    double local_eps = 0.0;
+    int numOfIter = 0;
+    while (true) {
+        const int par = numOfIter & 1;
+        // i = first argmin of f over I_up; low = max of f over I_low (smo_kernel.cpp:41-59)
+        double v = TSVM_INF, lw = -TSVM_INF;
+        int vi = MAX_WS;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            const int t = e * SV_T + tid;
+            s_a[par][t] = a[e];
+            s_f[par][t] = f[e];
+            if (active[e] && is_I_up(a[e], y[e], Cp, Cn) && f[e] < v) { v = f[e]; vi = t; }
+            if (active[e] && is_I_low(a[e], y[e], Cp, Cn) && f[e] > lw) lw = f[e];
+        }
+        wave_argmin(v, vi);
+        lw = wave_max(lw);
+        if (lane == 0) { sA_v[wave] = v; sA_i[wave] = vi; sA_l[wave] = lw; }
+        __syncthreads();
+        double up_value;
+        int i;
+        block_argmin(sA_v, sA_i, up_value, i);
+        const double low_value = block_max(sA_l);
+        if (!(up_value < TSVM_INF)) i = 0;
+        const double local_diff = low_value - up_value;
+        if (numOfIter == 0) {
+            const double t = 0.1f * local_diff;   // float literal, as in the reference (smo_kernel.cpp:64)
+            local_eps = eps > t ? eps : t;
+            if (tid == 0) diff[0] = local_diff;
+        }
+        if (numOfIter > max_iter || local_diff < local_eps) break;
+        const double *row_i = kws + (int64_t) i * ws;
+#pragma unroll
+        for (int e = 0; e < E; ++e) kI[e] = active[e] ? row_i[e * SV_T + tid] : 0.0;
+        const double kd_i = s_kd[i];
+        // j2 = first argmin of -b^2/a over I_low with f > up (smo_kernel.cpp:77-90)
+        double ft = TSVM_INF;
+        int fi = MAX_WS;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            const int t = e * SV_T + tid;
+            s_kI[t] = kI[e];
+            if (active[e] && -up_value > -f[e] && is_I_low(a[e], y[e], Cp, Cn)) {
+                const double aIJ = kd_i + kd[e] - 2 * kI[e];
+                const double bIJ = -up_value + f[e];
+                const double q = -bIJ * bIJ / aIJ;
+                if (q < ft) { ft = q; fi = t; }
+            }
+        }
+        wave_argmin(ft, fi);
+        if (lane == 0) { sB_v[wave] = ft; sB_i[wave] = fi; }
+        __syncthreads();
+        double min_t;
+        int j2;
+        block_argmin(sB_v, sB_i, min_t, j2);
+        if (!(min_t < TSVM_INF)) j2 = 0;
+        // two-variable step (smo_kernel.cpp:92-103)
+        const double a_i = s_a[par][i], y_i = (double) s_y[i];
+        const double a_j = s_a[par][j2], y_j = (double) s_y[j2];
+        const double alpha_i_diff = y_i > 0 ? Cp - a_i : a_i;
+        const double q1 = y_j > 0 ? a_j : Cn - a_j;
+        const double q2 = (-up_value + s_f[par][j2]) / (kd_i + s_kd[j2] - 2 * s_kI[j2]);
+        const double alpha_j_diff = q1 < q2 ? q1 : q2;
+        const double l = alpha_i_diff < alpha_j_diff ? alpha_i_diff : alpha_j_diff;
+        const double *row_j = kws + (int64_t) j2 * ws;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            const int t = e * SV_T + tid;
+            if (t == i) a[e] += l * y[e];
+            if (t == j2) a[e] -= l * y[e];
+            const double kJ = active[e] ? row_j[t] : 0.0;
+            f[e] = __builtin_fma(-l, kJ - kI[e], f[e]);
+        }
+        ++numOfIter;
+    }
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        if (active[e]) {
+            alpha_diff[e * SV_T + tid] = -(a[e] - a_old[e]) * y[e];
+            alpha[wsi[e]] = a[e];
+        }
+    }
+    if (tid == 0) diff[1] = (double) numOfIter;
+}
+
+// nu variant (smo_kernel.cpp:127-287): four extrema, two second-order candidates.  Keeps the CPU
+// code's j2n score, which uses kd[ip] and K[ip, .] (smo_kernel.cpp:239), and leaves diff[1] alone.
+template <int E>
+__global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
+    const int *__restrict__ label, const double *__restrict__ f_val, double *__restrict__ alpha,
+    double *__restrict__ alpha_diff, const int *__restrict__ working_set, int ws, double C,
+    const double *__restrict__ kws, const double *__restrict__ k_diag, double eps, double *__restrict__ diff,
+    int max_iter) {
+    __shared__ double s_kd[E * SV_T];
+    __shared__ float s_y[E * SV_T];
+    __shared__ double s_a[2][E * SV_T];
+    __shared__ double s_f[2][E * SV_T];
+    __shared__ double s_kIp[E * SV_T], s_kIn[E * SV_T];
+    __shared__ double sA_vp[SV_W], sA_vn[SV_W], sA_lp[SV_W], sA_ln[SV_W], sB_vp[SV_W], sB_vn[SV_W];
+    __shared__ int sA_ip[SV_W], sA_in[SV_W], sB_ip[SV_W], sB_in[SV_W];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    double f[E], a[E], a_old[E], y[E], kd[E], kIp[E], kIn[E];
+    int wsi[E];
+    bool active[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        const int t = e * SV_T + tid;
+        active[e] = t < ws;
+        wsi[e] = active[e] ? working_set[t] : 0;
+        f[e] = active[e] ? f_val[wsi[e]] : 0.0;
+        a[e] = active[e] ? alpha[wsi[e]] : 0.0;
+        a_old[e] = a[e];
+        y[e] = active[e] ? (double) label[wsi[e]] : 0.0;
+        kd[e] = active[e] ? k_diag[wsi[e]] : 0.0;
+        s_kd[t] = kd[e];
+        s_y[t] = (float) y[e];
+    }
+    double local_eps = 0.0;
+    int numOfIter = 0;
+    while (true) {
+        const int par = numOfIter & 1;
+        double vp = TSVM_INF, vn = TSVM_INF, lp = -TSVM_INF, ln = -TSVM_INF;
+        int ipi = MAX_WS, ini = MAX_WS;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            const int t = e * SV_T + tid;
+            s_a[par][t] = a[e];
+            s_f[par][t] = f[e];
+            if (!active[e]) continue;
+            if (y[e] > 0 && a[e] < C && f[e] < vp) { vp = f[e]; ipi = t; }
+            if (y[e] < 0 && a[e] > 0 && f[e] < vn) { vn = f[e]; ini = t; }
+            if (y[e] > 0 && a[e] > 0 && f[e] > lp) lp = f[e];
+            if (y[e] < 0 && a[e] < C && f[e] > ln) ln = f[e];
+        }
+        wave_argmin(vp, ipi);
+        wave_argmin(vn, ini);
+        lp = wave_max(lp);
+        ln = wave_max(ln);
+        if (lane == 0) {
+            sA_vp[wave] = vp; sA_ip[wave] = ipi; sA_vn[wave] = vn; sA_in[wave] = ini;
+            sA_lp[wave] = lp; sA_ln[wave] = ln;
+        }
+        __syncthreads();
+        double up_value_p, up_value_n;
+        int ip, in;
+        block_argmin(sA_vp, sA_ip, up_value_p, ip);
+        block_argmin(sA_vn, sA_in, up_value_n, in);
+        if (!(up_value_p < TSVM_INF)) ip = 0;
+        if (!(up_value_n < TSVM_INF)) in = 0;
+        const double low_value_p = block_max(sA_lp), low_value_n = block_max(sA_ln);
+        const double dp = low_value_p - up_value_p, dn = low_value_n - up_value_n;
+        const double local_diff = dp > dn ? dp : dn;
+        if (numOfIter == 0) {
+            const double t = 0.1 * local_diff;
+            local_eps = eps > t ? eps : t;
+            if (tid == 0) diff[0] = local_diff;
+        }
+        if (numOfIter > max_iter || local_diff < local_eps) break;
+        const double *row_p = kws + (int64_t) ip * ws;
+        const double *row_n = kws + (int64_t) in * ws;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            kIp[e] = active[e] ? row_p[e * SV_T + tid] : 0.0;
+            kIn[e] = active[e] ? row_n[e * SV_T + tid] : 0.0;
+        }
+        const double kd_ip = s_kd[ip];
+        double ftp = TSVM_INF, ftn = TSVM_INF;
+        int jpi = MAX_WS, jni = MAX_WS;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            const int t = e * SV_T + tid;
+            s_kIp[t] = kIp[e];
+            s_kIn[t] = kIn[e];
+            if (!active[e]) continue;
+            const double aIJ = kd_ip + kd[e] - 2 * kIp[e];
+            if (-up_value_p > -f[e] && y[e] > 0 && a[e] > 0) {
+                const double bIJ = -up_value_p + f[e];
+                const double q = -bIJ * bIJ / aIJ;
+                if (q < ftp) { ftp = q; jpi = t; }
+            }
+            if (-up_value_n > -f[e] && y[e] < 0 && a[e] < C) {
+                const double bIJ = -up_value_n + f[e];
+                const double q = -bIJ * bIJ / aIJ;
+                if (q < ftn) { ftn = q; jni = t; }
+            }
+        }
+        wave_argmin(ftp, jpi);
+        wave_argmin(ftn, jni);
+        if (lane == 0) { sB_vp[wave] = ftp; sB_ip[wave] = jpi; sB_vn[wave] = ftn; sB_in[wave] = jni; }
+        __syncthreads();
+        double f_val_j2p, f_val_j2n;
+        int j2p, j2n;
+        block_argmin(sB_vp, sB_ip, f_val_j2p, j2p);
+        block_argmin(sB_vn, sB_in, f_val_j2n, j2n);
+        if (!(f_val_j2p < TSVM_INF)) j2p = 0;
+        if (!(f_val_j2n < TSVM_INF)) j2n = 0;
+        const bool take_p = f_val_j2p < f_val_j2n;
+        const int i = take_p ? ip : in;
+        const int j2 = take_p ? j2p : j2n;
+        const double up_value = take_p ? up_value_p : up_value_n;
+        const double kIj2 = take_p ? s_kIp[j2] : s_kIn[j2];
+        const double a_i = s_a[par][i], y_i = (double) s_y[i];
+        const double a_j = s_a[par][j2], y_j = (double) s_y[j2];
+        const double alpha_i_diff = y_i > 0 ? C - a_i : a_i;
+        const double q1 = y_j > 0 ? a_j : C - a_j;
+        const double q2 = (-up_value + s_f[par][j2]) / (s_kd[i] + s_kd[j2] - 2 * kIj2);
+        const double alpha_j_diff = q1 < q2 ? q1 : q2;
+        const double l = alpha_i_diff < alpha_j_diff ? alpha_i_diff : alpha_j_diff;
+        const double *row_j = kws + (int64_t) j2 * ws;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            const int t = e * SV_T + tid;
+            if (t == i) a[e] += l * y[e];
+            if (t == j2) a[e] -= l * y[e];
+            const double kJ = active[e] ? row_j[t] : 0.0;
+            f[e] = __builtin_fma(-l, kJ - (take_p ? kIp[e] : kIn[e]), f[e]);
+        }
+        ++numOfIter;
+    }
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        if (active[e]) {
+            alpha_diff[e * SV_T + tid] = -(a[e] - a_old[e]) * y[e];
+            alpha[wsi[e]] = a[e];
+        }
+    }
+}
+
+extern "C" {
+
+size_t tsvm_smo_solve_workspace(int ws_size) {
+    if (ws_size < 0) return 0;
+    return sizeof(double) * (size_t) ws_size * (size_t) ws_size + 256;
+}
+
+static int launch_gather(const double *k_rows, const int *slots, int64_t ld, const int *working_set, int ws,
+                         void *workspace, hipStream_t s) {
+    hipLaunchKernelGGL(gather_ws_block_kernel, dim3(ws), dim3(ws < 256 ? 64 : 256), 0, s, k_rows, slots, ld, working_set,
+                       ws, (double *) workspace);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+#define TSVM_DISPATCH_E(KERNEL, ...)                                                            \
+    do {                                                                                        \
+        if (ws_size <= SV_T) hipLaunchKernelGGL(KERNEL<1>, dim3(1), dim3(SV_T), 0, s, __VA_ARGS__);      \
+        else if (ws_size <= 2 * SV_T) hipLaunchKernelGGL(KERNEL<2>, dim3(1), dim3(SV_T), 0, s, __VA_ARGS__); \
+        else hipLaunchKernelGGL(KERNEL<4>, dim3(1), dim3(SV_T), 0, s, __VA_ARGS__);                      \
+    } while (0)
+
+int tsvm_c_smo_solve(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
+                     int ws_size, double Cp, double Cn, const double *k_rows, const int *slots, int64_t ld,
+                     const double *k_diag, double eps, double *diff, int max_iter, void *workspace,
+                     tsvm_stream stream) {
+    TSVM_REQUIRE(y && f_val && alpha && alpha_diff && working_set && k_rows && k_diag && diff && workspace,
+                 "tsvm_c_smo_solve: null pointer");
+    TSVM_REQUIRE(ws_size >= 1 && ws_size <= MAX_WS, "tsvm_c_smo_solve: ws_size %d outside [1, %d]", ws_size, MAX_WS);
+    hipStream_t s = tsvm_s(stream);
+    int rc = launch_gather(k_rows, slots, ld, working_set, ws_size, workspace, s);
+    if (rc) return rc;
+    const double *kws = (const double *) workspace;
+    TSVM_DISPATCH_E(c_smo_solve_kernel, y, f_val, alpha, alpha_diff, working_set, ws_size, Cp, Cn, kws, k_diag, eps, diff,
+                    max_iter);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+int tsvm_nu_smo_solve(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
+                      int ws_size, double C, const double *k_rows, const int *slots, int64_t ld,
+                      const double *k_diag, double eps, double *diff, int max_iter, void *workspace,
+                      tsvm_stream stream) {
+    TSVM_REQUIRE(y && f_val && alpha && alpha_diff && working_set && k_rows && k_diag && diff && workspace,
+                 "tsvm_nu_smo_solve: null pointer");
+    TSVM_REQUIRE(ws_size >= 1 && ws_size <= MAX_WS, "tsvm_nu_smo_solve: ws_size %d outside [1, %d]", ws_size, MAX_WS);
+    hipStream_t s = tsvm_s(stream);
+    int rc = launch_gather(k_rows, slots, ld, working_set, ws_size, workspace, s);
+    if (rc) return rc;
+    const double *kws = (const double *) workspace;
+    TSVM_DISPATCH_E(nu_smo_solve_kernel, y, f_val, alpha, alpha_diff, working_set, ws_size, C, kws, k_diag, eps, diff,
+                    max_iter);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+}  // extern "C"

@@ -94,25 +94,70 @@ __device__ __forceinline__ double shfl_xor_f64(double v, int mask) {
     return __hiloint2double(hi, lo);
 }
 
-// Lexicographic (value, index) minimum across the wavefront: the smallest value wins and, among
-// equal values, the smallest index -- the serial loops' "first strict improvement" rule
-// (smo_kernel.cpp:43-49,80-89).
-__device__ __forceinline__ void wave_argmin(double &v, int &i) {
-#pragma unroll
-    for (int m = 1; m < TSVM_WAVE; m <<= 1) {
-        double ov = shfl_xor_f64(v, m);
-        int oi = __shfl_xor(i, m, TSVM_WAVE);
-        if (ov < v || (ov == v && oi < i)) { v = ov; i = oi; }
-    }
+// Cross-lane moves on the VALU (DPP) instead of the LDS crossbar: quad_perm xor-1 / xor-2,
+// row_half_mirror and row_mirror make every lane of a 16-lane row see the row's result in four
+// steps; the four row results are then read with v_readlane and combined uniformly.
+#define TSVM_DPP_XOR1 0xB1          /* quad_perm [1,0,3,2] */
+#define TSVM_DPP_XOR2 0x4E          /* quad_perm [2,3,0,1] */
+#define TSVM_DPP_HALF_MIRROR 0x141
+#define TSVM_DPP_MIRROR 0x140
+
+template <int CTRL>
+__device__ __forceinline__ int dpp_i32(int x) {
+    return __builtin_amdgcn_update_dpp(x, x, CTRL, 0xf, 0xf, false);
+}
+template <int CTRL>
+__device__ __forceinline__ double dpp_f64(double v) {
+    int lo = dpp_i32<CTRL>(__double2loint(v)), hi = dpp_i32<CTRL>(__double2hiint(v));
+    return __hiloint2double(hi, lo);
+}
+__device__ __forceinline__ double readlane_f64(double v, int lane) {
+    int lo = __builtin_amdgcn_readlane(__double2loint(v), lane), hi = __builtin_amdgcn_readlane(__double2hiint(v), lane);
+    return __hiloint2double(hi, lo);
 }
 
-__device__ __forceinline__ double wave_max(double v) {
+// Lexicographic (value, index) minimum across the wavefront: the smallest value wins and, among
+// equal values, the smallest index -- the serial loops' "first strict improvement" rule
+// (smo_kernel.cpp:43-49,80-89).  Every lane returns the wavefront's result.
+__device__ __forceinline__ void lexmin(double &v, int &i, double ov, int oi) {
+    if (ov < v || (ov == v && oi < i)) { v = ov; i = oi; }
+}
+template <int CTRL>
+__device__ __forceinline__ void argmin_step(double &v, int &i) {
+    const double ov = dpp_f64<CTRL>(v);
+    const int oi = dpp_i32<CTRL>(i);
+    lexmin(v, i, ov, oi);
+}
+__device__ __forceinline__ void wave_argmin(double &v, int &i) {
+    argmin_step<TSVM_DPP_XOR1>(v, i);
+    argmin_step<TSVM_DPP_XOR2>(v, i);
+    argmin_step<TSVM_DPP_HALF_MIRROR>(v, i);
+    argmin_step<TSVM_DPP_MIRROR>(v, i);
+    double rv = readlane_f64(v, 0);
+    int ri = __builtin_amdgcn_readlane(i, 0);
 #pragma unroll
-    for (int m = 1; m < TSVM_WAVE; m <<= 1) {
-        double ov = shfl_xor_f64(v, m);
-        if (ov > v) v = ov;
+    for (int r = 1; r < 4; ++r) lexmin(rv, ri, readlane_f64(v, 16 * r), __builtin_amdgcn_readlane(i, 16 * r));
+    v = rv;
+    i = ri;
+}
+
+template <int CTRL>
+__device__ __forceinline__ void max_step(double &v) {
+    const double ov = dpp_f64<CTRL>(v);
+    if (ov > v) v = ov;
+}
+__device__ __forceinline__ double wave_max(double v) {
+    max_step<TSVM_DPP_XOR1>(v);
+    max_step<TSVM_DPP_XOR2>(v);
+    max_step<TSVM_DPP_HALF_MIRROR>(v);
+    max_step<TSVM_DPP_MIRROR>(v);
+    double rv = readlane_f64(v, 0);
+#pragma unroll
+    for (int r = 1; r < 4; ++r) {
+        const double ov = readlane_f64(v, 16 * r);
+        if (ov > rv) rv = ov;
     }
-    return v;
+    return rv;
 }
 
 // Maps the launch's linear workgroup id to a logical one so that logical neighbours run on the
