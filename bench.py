@@ -37,6 +37,8 @@ def parse():
     ap.add_argument("--scale", type=float, default=1.0, help="row-count scale of the workload (1.0 = benchmark shape)")
     ap.add_argument("--cpu-iters", type=int, default=-1, help="outer iterations of the CPU baseline sample (-1 = auto, 0 = skip)")
     ap.add_argument("--extra-c4", type=int, default=1, help="also time one training pass of C4 (500k x 54, 7 classes)")
+    ap.add_argument("--kernels-only", action="store_true",
+                    help="only launch get_rows / update_f at the workload's shape plus a 1 GiB device copy (for rocprofv3 counter runs)")
     return ap.parse_args()
 
 
@@ -166,6 +168,15 @@ def main():
     w = gen[args.workload](args.scale)
     train, test, params = w["train"], w.get("test"), w["params"]
     prm = make_param(**params)
+
+    if args.kernels_only:
+        src = torch.empty(1 << 27, dtype=torch.float64, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)                      # plain copy of known size: 1 GiB read + 1 GiB written
+        torch.cuda.synchronize()
+        del src, dst
+        print(json.dumps(kernel_figures(train, params)))
+        return
 
     def one_train():
         m = Model(prm.svm_type)

@@ -1,0 +1,55 @@
+"""The C-ABI libraries load without a GPU and export every symbol the headers under include/ declare;
+compute calls fail loudly instead of falling back to a CPU path."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from thundersvm_amd import capi, model
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tsvm_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_kernel_library_exports():
+    lib = capi.kernel_lib()
+    names = _declared("thundersvm_amd.h")
+    assert len(names) >= 15
+    for n in names:
+        assert hasattr(lib, n), n
+    assert set(names) == set(capi.SIGNATURES), set(names) ^ set(capi.SIGNATURES)
+    assert lib.tsvm_version() >= 100
+
+
+def test_model_library_exports():
+    lib = model.host_lib()
+    names = _declared("thundersvm_amd_model.h")
+    assert len(names) >= 12
+    for n in names:
+        assert hasattr(lib, n), n
+
+
+def test_argument_checks_do_not_need_a_gpu():
+    lib = capi.kernel_lib()
+    rc = lib.tsvm_update_f(None, None, 4, None, None, 8, 8, None)
+    assert rc == -1 and b"null pointer" in lib.tsvm_last_error()
+    rc = lib.tsvm_get_rows_dense(8, 12, 4, 4, 8, 8, 12, None, 1, 8, 2, 0.5, 0.0, 3, 8, 4, None)
+    assert rc == -1 and b"multiples of 8" in lib.tsvm_last_error()
+    assert lib.tsvm_select_workspace(1000) > 1000 * 10
+    assert lib.tsvm_smo_solve_workspace(1024) >= 8 * 1024 * 1024
+
+
+def test_no_cpu_fallback():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("GPU present")
+    from thundersvm_amd import data as D
+    w = D.workload_c1(0.05)
+    with pytest.raises((capi.TsvmError, MemoryError)):
+        model.Model(0).train(w["train"], model.make_param(**w["params"]))
