@@ -15,24 +15,27 @@
 // update_f: f[j] -= sum_t alpha_diff[t] * K_t[j]  (smo_kernel.cpp:300-319)
 // Bandwidth-bound stream over the ws x n kernel rows.  The non-zero alpha_diff entries are
 // compacted (in order) into LDS once per workgroup; rows with alpha_diff == 0 are never read.
-// Each thread owns two columns j and keeps eight row loads in flight per column.
+// Each thread owns one or two adjacent columns and keeps 16 (or 8 two-column) row loads in flight.
 // ------------------------------------------------------------------------------------------------
 #define UF_T 256
 #define UF_CHUNK 1024
-#define UF_UNROLL 8
 
+// COLS columns per thread (consecutive, loaded as one 8*COLS-byte vector), UNROLL rows in flight.
+template <int COLS, int UNROLL>
 __global__ __launch_bounds__(UF_T) void update_f_kernel(double *__restrict__ f, const double *__restrict__ alpha_diff,
                                                         int ws, const double *__restrict__ k_rows,
                                                         const int *__restrict__ slots, int64_t ld, int64_t n) {
+    typedef double vec_t __attribute__((ext_vector_type(COLS)));
     __shared__ double s_ad[UF_CHUNK];
     __shared__ int64_t s_off[UF_CHUNK];
     __shared__ int s_wave_cnt[UF_T / 64];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    const int64_t j0 = (int64_t) blockIdx.x * (UF_T * 2) + tid;
-    const int64_t j1 = j0 + UF_T;
-    const bool a0 = j0 < n, a1 = j1 < n;
-    double sum0 = 0.0, sum1 = 0.0;
+    const int64_t j = ((int64_t) blockIdx.x * UF_T + tid) * COLS;
+    const bool act = j < n;   // n is a multiple of COLS whenever COLS > 1 (checked by the launcher)
+    double sum[COLS];
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) sum[c] = 0.0;
     for (int base = 0; base < ws; base += UF_CHUNK) {
         // ordered compaction of this chunk's non-zero entries: thread t owns entries 4t..4t+3
         double v[4];
@@ -68,30 +71,32 @@ __global__ __launch_bounds__(UF_T) void update_f_kernel(double *__restrict__ f, 
             }
         }
         __syncthreads();
-        int u = 0;
-        for (; u + UF_UNROLL <= total; u += UF_UNROLL) {
-            double k0[UF_UNROLL], k1[UF_UNROLL];
+        if (act) {
+            int u = 0;
+            for (; u + UNROLL <= total; u += UNROLL) {
+                vec_t k[UNROLL];
 #pragma unroll
-            for (int e = 0; e < UF_UNROLL; ++e) {
-                const double *row = k_rows + s_off[u + e];
-                k0[e] = a0 ? row[j0] : 0.0;
-                k1[e] = a1 ? row[j1] : 0.0;
-            }
+                for (int e = 0; e < UNROLL; ++e) k[e] = *(const vec_t *) (k_rows + s_off[u + e] + j);
 #pragma unroll
-            for (int e = 0; e < UF_UNROLL; ++e) {
-                sum0 = __builtin_fma(s_ad[u + e], k0[e], sum0);
-                sum1 = __builtin_fma(s_ad[u + e], k1[e], sum1);
+                for (int e = 0; e < UNROLL; ++e) {
+                    const double ad = s_ad[u + e];
+#pragma unroll
+                    for (int c = 0; c < COLS; ++c) sum[c] = __builtin_fma(ad, k[e][c], sum[c]);
+                }
             }
-        }
-        for (; u < total; ++u) {
-            const double *row = k_rows + s_off[u];
-            if (a0) sum0 = __builtin_fma(s_ad[u], row[j0], sum0);
-            if (a1) sum1 = __builtin_fma(s_ad[u], row[j1], sum1);
+            for (; u < total; ++u) {
+                const vec_t k = *(const vec_t *) (k_rows + s_off[u] + j);
+                const double ad = s_ad[u];
+#pragma unroll
+                for (int c = 0; c < COLS; ++c) sum[c] = __builtin_fma(ad, k[c], sum[c]);
+            }
         }
         __syncthreads();
     }
-    if (a0) f[j0] -= sum0;
-    if (a1) f[j1] -= sum1;
+    if (act) {
+#pragma unroll
+        for (int c = 0; c < COLS; ++c) f[j + c] -= sum[c];
+    }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -512,9 +517,18 @@ int tsvm_update_f(double *f, const double *alpha_diff, int ws_size, const double
     TSVM_REQUIRE(ws_size >= 0 && n >= 0 && ld >= n, "tsvm_update_f: bad size (ws=%d n=%lld ld=%lld)", ws_size,
                  (long long) n, (long long) ld);
     if (n == 0 || ws_size == 0) return 0;
-    const unsigned grid = (unsigned) ((n + UF_T * 2 - 1) / (UF_T * 2));
-    hipLaunchKernelGGL(update_f_kernel, dim3(grid), dim3(UF_T), 0, tsvm_s(stream), f, alpha_diff, ws_size, k_rows, slots,
-                       ld, n);
+    // 16-byte loads need every row start and f itself 16-byte aligned and an even column count
+    const bool vec2 = n % 2 == 0 && ld % 2 == 0 && ((uintptr_t) k_rows % 16 == 0) && ((uintptr_t) f % 16 == 0) &&
+                      n >= (int64_t) UF_T * 2 * 512;
+    if (vec2) {
+        const unsigned grid = (unsigned) ((n / 2 + UF_T - 1) / UF_T);
+        hipLaunchKernelGGL((update_f_kernel<2, 8>), dim3(grid), dim3(UF_T), 0, tsvm_s(stream), f, alpha_diff, ws_size,
+                           k_rows, slots, ld, n);
+    } else {
+        const unsigned grid = (unsigned) ((n + UF_T - 1) / UF_T);
+        hipLaunchKernelGGL((update_f_kernel<1, 16>), dim3(grid), dim3(UF_T), 0, tsvm_s(stream), f, alpha_diff, ws_size,
+                           k_rows, slots, ld, n);
+    }
     TSVM_LAUNCH_CHECK();
     return 0;
 }

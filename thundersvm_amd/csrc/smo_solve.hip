@@ -9,7 +9,9 @@
 //   2. row K[i, .] of the gathered ws x ws block (coalesced);
 //   3. j2 = first argmin of -b^2/a over I_low with f > up: same reduction shape;
 //   4. the two-variable step, row K[j2, .], f -= l * (K[j2, .] - K[i, .]).
-// Two workgroup barriers per iteration.  Reductions are lexicographic (value, element index)
+// Two workgroup barriers per iteration.  The loop body is written with selects instead of branches:
+// with one wavefront per SIMD nothing hides a taken branch (the same loop written with if-blocks
+// measured about 1.3x slower per inner iteration).  Reductions are lexicographic (value, element index)
 // minima, so ties go to the lowest index exactly as the reference's serial loops resolve them, and
 // all arithmetic is the reference's expression order in IEEE double (the library is compiled with
 // -ffp-contract=off; the one fused operation, f -= l*(kJ - kI), is an explicit fma as gcc -O3
@@ -23,60 +25,70 @@
 #define SV_T 256           // threads of the solver workgroup
 #define SV_W (SV_T / 64)   // wavefronts
 
-// kws[r*ws + t] = K_r[working_set[t]]: the ws x ws block the solver reads, gathered once per call so
-// that the two row reads per inner iteration (smo_kernel.cpp:50-52,107-110) are contiguous.
+// kws[r*ldk + t] = K_r[working_set[t]] for t < ws, 0 for ws <= t < ldk: the ws x ws block the solver
+// reads, gathered once per call so that the two row reads per inner iteration
+// (smo_kernel.cpp:50-52,107-110) are contiguous; rows are padded to the solver's thread x slot grid
+// so every thread can load without a bounds test.
 __global__ void gather_ws_block_kernel(const double *__restrict__ k_rows, const int *__restrict__ slots, int64_t ld,
-                                       const int *__restrict__ working_set, int ws, double *__restrict__ kws) {
+                                       const int *__restrict__ working_set, int ws, int ldk, double *__restrict__ kws) {
     const int r = blockIdx.x;
     const double *row = k_rows + (int64_t) (slots ? slots[r] : r) * ld;
-    for (int t = threadIdx.x; t < ws; t += blockDim.x) kws[(int64_t) r * ws + t] = row[working_set[t]];
+    for (int t = threadIdx.x; t < ldk; t += blockDim.x) kws[(int64_t) r * ldk + t] = t < ws ? row[working_set[t]] : 0.0;
 }
 
-// Combines the per-wavefront partial results (one LDS entry per wavefront) in wavefront order.
-__device__ __forceinline__ void block_argmin(const double *s_v, const int *s_i, double &v, int &i) {
-    v = s_v[0];
-    i = s_i[0];
+// Cross-wavefront combination of the per-wavefront (value, index) minima held in LDS.
+__device__ __forceinline__ void block_argmin(const double *s_v, const int *s_i, double &v, int &i, int none) {
+    double m = s_v[0];
 #pragma unroll
-    for (int w = 1; w < SV_W; ++w) lexmin(v, i, s_v[w], s_i[w]);
+    for (int w = 1; w < SV_W; ++w) m = fmin_sel(m, s_v[w]);
+    int r = none;
+#pragma unroll
+    for (int w = 0; w < SV_W; ++w) r = imin_sel(r, s_v[w] == m ? s_i[w] : none);
+    v = m;
+    i = r;
 }
 __device__ __forceinline__ double block_max(const double *s_v) {
     double v = s_v[0];
 #pragma unroll
-    for (int w = 1; w < SV_W; ++w) v = s_v[w] > v ? s_v[w] : v;
+    for (int w = 1; w < SV_W; ++w) v = fmax_sel(v, s_v[w]);
     return v;
 }
 
+// Elements beyond ws are given y = 0, which puts them in neither I_up nor I_low.
 template <int E>
 __global__ __launch_bounds__(SV_T) void c_smo_solve_kernel(
     const int *__restrict__ label, const double *__restrict__ f_val, double *__restrict__ alpha,
     double *__restrict__ alpha_diff, const int *__restrict__ working_set, int ws, double Cp, double Cn,
     const double *__restrict__ kws, const double *__restrict__ k_diag, double eps, double *__restrict__ diff,
     int max_iter) {
-    __shared__ double s_kd[E * SV_T];
-    __shared__ float s_y[E * SV_T];
-    __shared__ double s_a[2][E * SV_T];
-    __shared__ double s_f[2][E * SV_T];
-    __shared__ double s_kI[E * SV_T];
+    constexpr int LDK = E * SV_T;
+    __shared__ double s_kd[LDK];
+    __shared__ float s_y[LDK];
+    __shared__ double s_a[2][LDK];
+    __shared__ double s_f[2][LDK];
+    __shared__ double s_kI[LDK];
     __shared__ double sA_v[SV_W], sA_l[SV_W], sB_v[SV_W];
     __shared__ int sA_i[SV_W], sB_i[SV_W];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     double f[E], a[E], a_old[E], y[E], kd[E], kI[E];
+    bool upm[E], lowm[E];
     int wsi[E];
-    bool active[E];
 #pragma unroll
     for (int e = 0; e < E; ++e) {
         const int t = e * SV_T + tid;
-        active[e] = t < ws;
-        wsi[e] = active[e] ? working_set[t] : 0;
-        f[e] = active[e] ? f_val[wsi[e]] : 0.0;
-        a[e] = active[e] ? alpha[wsi[e]] : 0.0;
+        const bool active = t < ws;
+        wsi[e] = active ? working_set[t] : 0;
+        f[e] = active ? f_val[wsi[e]] : 0.0;
+        a[e] = active ? alpha[wsi[e]] : 0.0;
         a_old[e] = a[e];
-        y[e] = active[e] ? (double) label[wsi[e]] : 0.0;
-        kd[e] = active[e] ? k_diag[wsi[e]] : 0.0;
+        y[e] = active ? (double) label[wsi[e]] : 0.0;
+        kd[e] = active ? k_diag[wsi[e]] : 1.0;
         s_kd[t] = kd[e];
         s_y[t] = (float) y[e];
+        upm[e] = is_I_up(a[e], y[e], Cp, Cn);
+        lowm[e] = is_I_low(a[e], y[e], Cp, Cn);
     }
     double local_eps = 0.0;
     int numOfIter = 0;
@@ -90,18 +102,20 @@ __global__ __launch_bounds__(SV_T) void c_smo_solve_kernel(
             const int t = e * SV_T + tid;
             s_a[par][t] = a[e];
             s_f[par][t] = f[e];
-            if (active[e] && is_I_up(a[e], y[e], Cp, Cn) && f[e] < v) { v = f[e]; vi = t; }
-            if (active[e] && is_I_low(a[e], y[e], Cp, Cn) && f[e] > lw) lw = f[e];
+            const bool c = upm[e] & (f[e] < v);
+            v = c ? f[e] : v;
+            vi = c ? t : vi;
+            lw = (lowm[e] & (f[e] > lw)) ? f[e] : lw;
         }
-        wave_argmin(v, vi);
-        lw = wave_max(lw);
+        wave_argmin(v, vi, MAX_WS);
+        lw = wave_max_f64(lw);
         if (lane == 0) { sA_v[wave] = v; sA_i[wave] = vi; sA_l[wave] = lw; }
         __syncthreads();
         double up_value;
         int i;
-        block_argmin(sA_v, sA_i, up_value, i);
+        block_argmin(sA_v, sA_i, up_value, i, MAX_WS);
         const double low_value = block_max(sA_l);
-        if (!(up_value < TSVM_INF)) i = 0;
+        i = up_value < TSVM_INF ? i : 0;
         const double local_diff = low_value - up_value;
         if (numOfIter == 0) {
             const double t = 0.1f * local_diff;   // float literal, as in the reference (smo_kernel.cpp:64)
@@ -109,9 +123,9 @@ __global__ __launch_bounds__(SV_T) void c_smo_solve_kernel(
             if (tid == 0) diff[0] = local_diff;
         }
         if (numOfIter > max_iter || local_diff < local_eps) break;
-        const double *row_i = kws + (int64_t) i * ws;
+        const double *row_i = kws + (int64_t) i * LDK + tid;
 #pragma unroll
-        for (int e = 0; e < E; ++e) kI[e] = active[e] ? row_i[e * SV_T + tid] : 0.0;
+        for (int e = 0; e < E; ++e) kI[e] = row_i[e * SV_T];
         const double kd_i = s_kd[i];
         // j2 = first argmin of -b^2/a over I_low with f > up (smo_kernel.cpp:77-90)
         double ft = TSVM_INF;
@@ -120,20 +134,24 @@ __global__ __launch_bounds__(SV_T) void c_smo_solve_kernel(
         for (int e = 0; e < E; ++e) {
             const int t = e * SV_T + tid;
             s_kI[t] = kI[e];
-            if (active[e] && -up_value > -f[e] && is_I_low(a[e], y[e], Cp, Cn)) {
-                const double aIJ = kd_i + kd[e] - 2 * kI[e];
-                const double bIJ = -up_value + f[e];
-                const double q = -bIJ * bIJ / aIJ;
-                if (q < ft) { ft = q; fi = t; }
-            }
+            const double aIJ = kd_i + kd[e] - 2 * kI[e];
+            const double bIJ = -up_value + f[e];
+            const double q = -bIJ * bIJ / aIJ;
+            const bool c = lowm[e] & (-up_value > -f[e]) & (q < ft);
+            ft = c ? q : ft;
+            fi = c ? t : fi;
         }
-        wave_argmin(ft, fi);
+        wave_argmin(ft, fi, MAX_WS);
         if (lane == 0) { sB_v[wave] = ft; sB_i[wave] = fi; }
         __syncthreads();
         double min_t;
         int j2;
-        block_argmin(sB_v, sB_i, min_t, j2);
-        if (!(min_t < TSVM_INF)) j2 = 0;
+        block_argmin(sB_v, sB_i, min_t, j2, MAX_WS);
+        j2 = min_t < TSVM_INF ? j2 : 0;
+        const double *row_j = kws + (int64_t) j2 * LDK + tid;
+        double kJ[E];
+#pragma unroll
+        for (int e = 0; e < E; ++e) kJ[e] = row_j[e * SV_T];
         // two-variable step (smo_kernel.cpp:92-103)
         const double a_i = s_a[par][i], y_i = (double) s_y[i];
         const double a_j = s_a[par][j2], y_j = (double) s_y[j2];
@@ -142,21 +160,22 @@ __global__ __launch_bounds__(SV_T) void c_smo_solve_kernel(
         const double q2 = (-up_value + s_f[par][j2]) / (kd_i + s_kd[j2] - 2 * s_kI[j2]);
         const double alpha_j_diff = q1 < q2 ? q1 : q2;
         const double l = alpha_i_diff < alpha_j_diff ? alpha_i_diff : alpha_j_diff;
-        const double *row_j = kws + (int64_t) j2 * ws;
 #pragma unroll
         for (int e = 0; e < E; ++e) {
             const int t = e * SV_T + tid;
-            if (t == i) a[e] += l * y[e];
-            if (t == j2) a[e] -= l * y[e];
-            const double kJ = active[e] ? row_j[t] : 0.0;
-            f[e] = __builtin_fma(-l, kJ - kI[e], f[e]);
+            a[e] = t == i ? a[e] + l * y[e] : a[e];
+            a[e] = t == j2 ? a[e] - l * y[e] : a[e];
+            upm[e] = is_I_up(a[e], y[e], Cp, Cn);
+            lowm[e] = is_I_low(a[e], y[e], Cp, Cn);
+            f[e] = __builtin_fma(-l, kJ[e] - kI[e], f[e]);
         }
         ++numOfIter;
     }
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-        if (active[e]) {
-            alpha_diff[e * SV_T + tid] = -(a[e] - a_old[e]) * y[e];
+        const int t = e * SV_T + tid;
+        if (t < ws) {
+            alpha_diff[t] = -(a[e] - a_old[e]) * y[e];
             alpha[wsi[e]] = a[e];
         }
     }
@@ -171,11 +190,12 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
     double *__restrict__ alpha_diff, const int *__restrict__ working_set, int ws, double C,
     const double *__restrict__ kws, const double *__restrict__ k_diag, double eps, double *__restrict__ diff,
     int max_iter) {
-    __shared__ double s_kd[E * SV_T];
-    __shared__ float s_y[E * SV_T];
-    __shared__ double s_a[2][E * SV_T];
-    __shared__ double s_f[2][E * SV_T];
-    __shared__ double s_kIp[E * SV_T], s_kIn[E * SV_T];
+    constexpr int LDK = E * SV_T;
+    __shared__ double s_kd[LDK];
+    __shared__ float s_y[LDK];
+    __shared__ double s_a[2][LDK];
+    __shared__ double s_f[2][LDK];
+    __shared__ double s_kIp[LDK], s_kIn[LDK];
     __shared__ double sA_vp[SV_W], sA_vn[SV_W], sA_lp[SV_W], sA_ln[SV_W], sB_vp[SV_W], sB_vn[SV_W];
     __shared__ int sA_ip[SV_W], sA_in[SV_W], sB_ip[SV_W], sB_in[SV_W];
 
@@ -183,17 +203,16 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
     const int lane = tid & 63, wave = tid >> 6;
     double f[E], a[E], a_old[E], y[E], kd[E], kIp[E], kIn[E];
     int wsi[E];
-    bool active[E];
 #pragma unroll
     for (int e = 0; e < E; ++e) {
         const int t = e * SV_T + tid;
-        active[e] = t < ws;
-        wsi[e] = active[e] ? working_set[t] : 0;
-        f[e] = active[e] ? f_val[wsi[e]] : 0.0;
-        a[e] = active[e] ? alpha[wsi[e]] : 0.0;
+        const bool active = t < ws;
+        wsi[e] = active ? working_set[t] : 0;
+        f[e] = active ? f_val[wsi[e]] : 0.0;
+        a[e] = active ? alpha[wsi[e]] : 0.0;
         a_old[e] = a[e];
-        y[e] = active[e] ? (double) label[wsi[e]] : 0.0;
-        kd[e] = active[e] ? k_diag[wsi[e]] : 0.0;
+        y[e] = active ? (double) label[wsi[e]] : 0.0;
+        kd[e] = active ? k_diag[wsi[e]] : 1.0;
         s_kd[t] = kd[e];
         s_y[t] = (float) y[e];
     }
@@ -208,16 +227,20 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
             const int t = e * SV_T + tid;
             s_a[par][t] = a[e];
             s_f[par][t] = f[e];
-            if (!active[e]) continue;
-            if (y[e] > 0 && a[e] < C && f[e] < vp) { vp = f[e]; ipi = t; }
-            if (y[e] < 0 && a[e] > 0 && f[e] < vn) { vn = f[e]; ini = t; }
-            if (y[e] > 0 && a[e] > 0 && f[e] > lp) lp = f[e];
-            if (y[e] < 0 && a[e] < C && f[e] > ln) ln = f[e];
+            const bool pos = y[e] > 0, neg = y[e] < 0;
+            const bool cp = pos & (a[e] < C) & (f[e] < vp);
+            vp = cp ? f[e] : vp;
+            ipi = cp ? t : ipi;
+            const bool cn = neg & (a[e] > 0) & (f[e] < vn);
+            vn = cn ? f[e] : vn;
+            ini = cn ? t : ini;
+            lp = (pos & (a[e] > 0) & (f[e] > lp)) ? f[e] : lp;
+            ln = (neg & (a[e] < C) & (f[e] > ln)) ? f[e] : ln;
         }
-        wave_argmin(vp, ipi);
-        wave_argmin(vn, ini);
-        lp = wave_max(lp);
-        ln = wave_max(ln);
+        wave_argmin(vp, ipi, MAX_WS);
+        wave_argmin(vn, ini, MAX_WS);
+        lp = wave_max_f64(lp);
+        ln = wave_max_f64(ln);
         if (lane == 0) {
             sA_vp[wave] = vp; sA_ip[wave] = ipi; sA_vn[wave] = vn; sA_in[wave] = ini;
             sA_lp[wave] = lp; sA_ln[wave] = ln;
@@ -225,10 +248,10 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
         __syncthreads();
         double up_value_p, up_value_n;
         int ip, in;
-        block_argmin(sA_vp, sA_ip, up_value_p, ip);
-        block_argmin(sA_vn, sA_in, up_value_n, in);
-        if (!(up_value_p < TSVM_INF)) ip = 0;
-        if (!(up_value_n < TSVM_INF)) in = 0;
+        block_argmin(sA_vp, sA_ip, up_value_p, ip, MAX_WS);
+        block_argmin(sA_vn, sA_in, up_value_n, in, MAX_WS);
+        ip = up_value_p < TSVM_INF ? ip : 0;
+        in = up_value_n < TSVM_INF ? in : 0;
         const double low_value_p = block_max(sA_lp), low_value_n = block_max(sA_ln);
         const double dp = low_value_p - up_value_p, dn = low_value_n - up_value_n;
         const double local_diff = dp > dn ? dp : dn;
@@ -238,12 +261,12 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
             if (tid == 0) diff[0] = local_diff;
         }
         if (numOfIter > max_iter || local_diff < local_eps) break;
-        const double *row_p = kws + (int64_t) ip * ws;
-        const double *row_n = kws + (int64_t) in * ws;
+        const double *row_p = kws + (int64_t) ip * LDK + tid;
+        const double *row_n = kws + (int64_t) in * LDK + tid;
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            kIp[e] = active[e] ? row_p[e * SV_T + tid] : 0.0;
-            kIn[e] = active[e] ? row_n[e * SV_T + tid] : 0.0;
+            kIp[e] = row_p[e * SV_T];
+            kIn[e] = row_n[e * SV_T];
         }
         const double kd_ip = s_kd[ip];
         double ftp = TSVM_INF, ftn = TSVM_INF;
@@ -253,33 +276,34 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
             const int t = e * SV_T + tid;
             s_kIp[t] = kIp[e];
             s_kIn[t] = kIn[e];
-            if (!active[e]) continue;
             const double aIJ = kd_ip + kd[e] - 2 * kIp[e];
-            if (-up_value_p > -f[e] && y[e] > 0 && a[e] > 0) {
-                const double bIJ = -up_value_p + f[e];
-                const double q = -bIJ * bIJ / aIJ;
-                if (q < ftp) { ftp = q; jpi = t; }
-            }
-            if (-up_value_n > -f[e] && y[e] < 0 && a[e] < C) {
-                const double bIJ = -up_value_n + f[e];
-                const double q = -bIJ * bIJ / aIJ;
-                if (q < ftn) { ftn = q; jni = t; }
-            }
+            const double bp = -up_value_p + f[e], bn = -up_value_n + f[e];
+            const double qp = -bp * bp / aIJ, qn = -bn * bn / aIJ;
+            const bool cp = (-up_value_p > -f[e]) & (y[e] > 0) & (a[e] > 0) & (qp < ftp);
+            ftp = cp ? qp : ftp;
+            jpi = cp ? t : jpi;
+            const bool cn = (-up_value_n > -f[e]) & (y[e] < 0) & (a[e] < C) & (qn < ftn);
+            ftn = cn ? qn : ftn;
+            jni = cn ? t : jni;
         }
-        wave_argmin(ftp, jpi);
-        wave_argmin(ftn, jni);
+        wave_argmin(ftp, jpi, MAX_WS);
+        wave_argmin(ftn, jni, MAX_WS);
         if (lane == 0) { sB_vp[wave] = ftp; sB_ip[wave] = jpi; sB_vn[wave] = ftn; sB_in[wave] = jni; }
         __syncthreads();
         double f_val_j2p, f_val_j2n;
         int j2p, j2n;
-        block_argmin(sB_vp, sB_ip, f_val_j2p, j2p);
-        block_argmin(sB_vn, sB_in, f_val_j2n, j2n);
-        if (!(f_val_j2p < TSVM_INF)) j2p = 0;
-        if (!(f_val_j2n < TSVM_INF)) j2n = 0;
+        block_argmin(sB_vp, sB_ip, f_val_j2p, j2p, MAX_WS);
+        block_argmin(sB_vn, sB_in, f_val_j2n, j2n, MAX_WS);
+        j2p = f_val_j2p < TSVM_INF ? j2p : 0;
+        j2n = f_val_j2n < TSVM_INF ? j2n : 0;
         const bool take_p = f_val_j2p < f_val_j2n;
         const int i = take_p ? ip : in;
         const int j2 = take_p ? j2p : j2n;
         const double up_value = take_p ? up_value_p : up_value_n;
+        const double *row_j = kws + (int64_t) j2 * LDK + tid;
+        double kJ[E];
+#pragma unroll
+        for (int e = 0; e < E; ++e) kJ[e] = row_j[e * SV_T];
         const double kIj2 = take_p ? s_kIp[j2] : s_kIn[j2];
         const double a_i = s_a[par][i], y_i = (double) s_y[i];
         const double a_j = s_a[par][j2], y_j = (double) s_y[j2];
@@ -288,21 +312,20 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
         const double q2 = (-up_value + s_f[par][j2]) / (s_kd[i] + s_kd[j2] - 2 * kIj2);
         const double alpha_j_diff = q1 < q2 ? q1 : q2;
         const double l = alpha_i_diff < alpha_j_diff ? alpha_i_diff : alpha_j_diff;
-        const double *row_j = kws + (int64_t) j2 * ws;
 #pragma unroll
         for (int e = 0; e < E; ++e) {
             const int t = e * SV_T + tid;
-            if (t == i) a[e] += l * y[e];
-            if (t == j2) a[e] -= l * y[e];
-            const double kJ = active[e] ? row_j[t] : 0.0;
-            f[e] = __builtin_fma(-l, kJ - (take_p ? kIp[e] : kIn[e]), f[e]);
+            a[e] = t == i ? a[e] + l * y[e] : a[e];
+            a[e] = t == j2 ? a[e] - l * y[e] : a[e];
+            f[e] = __builtin_fma(-l, kJ[e] - (take_p ? kIp[e] : kIn[e]), f[e]);
         }
         ++numOfIter;
     }
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-        if (active[e]) {
-            alpha_diff[e * SV_T + tid] = -(a[e] - a_old[e]) * y[e];
+        const int t = e * SV_T + tid;
+        if (t < ws) {
+            alpha_diff[t] = -(a[e] - a_old[e]) * y[e];
             alpha[wsi[e]] = a[e];
         }
     }
@@ -310,15 +333,17 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
 
 extern "C" {
 
+static int solver_ldk(int ws_size) { return ws_size <= SV_T ? SV_T : (ws_size <= 2 * SV_T ? 2 * SV_T : 4 * SV_T); }
+
 size_t tsvm_smo_solve_workspace(int ws_size) {
     if (ws_size < 0) return 0;
-    return sizeof(double) * (size_t) ws_size * (size_t) ws_size + 256;
+    return sizeof(double) * (size_t) ws_size * (size_t) solver_ldk(ws_size) + 256;
 }
 
 static int launch_gather(const double *k_rows, const int *slots, int64_t ld, const int *working_set, int ws,
                          void *workspace, hipStream_t s) {
-    hipLaunchKernelGGL(gather_ws_block_kernel, dim3(ws), dim3(ws < 256 ? 64 : 256), 0, s, k_rows, slots, ld, working_set,
-                       ws, (double *) workspace);
+    hipLaunchKernelGGL(gather_ws_block_kernel, dim3(ws), dim3(256), 0, s, k_rows, slots, ld, working_set, ws,
+                       solver_ldk(ws), (double *) workspace);
     TSVM_LAUNCH_CHECK();
     return 0;
 }

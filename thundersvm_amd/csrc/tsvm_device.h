@@ -116,48 +116,45 @@ __device__ __forceinline__ double readlane_f64(double v, int lane) {
     return __hiloint2double(hi, lo);
 }
 
-// Lexicographic (value, index) minimum across the wavefront: the smallest value wins and, among
-// equal values, the smallest index -- the serial loops' "first strict improvement" rule
-// (smo_kernel.cpp:43-49,80-89).  Every lane returns the wavefront's result.
-__device__ __forceinline__ void lexmin(double &v, int &i, double ov, int oi) {
-    if (ov < v || (ov == v && oi < i)) { v = ov; i = oi; }
-}
-template <int CTRL>
-__device__ __forceinline__ void argmin_step(double &v, int &i) {
-    const double ov = dpp_f64<CTRL>(v);
-    const int oi = dpp_i32<CTRL>(i);
-    lexmin(v, i, ov, oi);
-}
-__device__ __forceinline__ void wave_argmin(double &v, int &i) {
-    argmin_step<TSVM_DPP_XOR1>(v, i);
-    argmin_step<TSVM_DPP_XOR2>(v, i);
-    argmin_step<TSVM_DPP_HALF_MIRROR>(v, i);
-    argmin_step<TSVM_DPP_MIRROR>(v, i);
-    double rv = readlane_f64(v, 0);
-    int ri = __builtin_amdgcn_readlane(i, 0);
-#pragma unroll
-    for (int r = 1; r < 4; ++r) lexmin(rv, ri, readlane_f64(v, 16 * r), __builtin_amdgcn_readlane(i, 16 * r));
-    v = rv;
-    i = ri;
-}
+// Wavefront reductions used by the local solvers.  A (value, index) lexicographic minimum -- the
+// smallest value wins and, among equal values, the smallest index: the serial loops' "first strict
+// improvement" rule (smo_kernel.cpp:43-49,80-89) -- is taken in two branch-free passes: the minimum
+// value (v_min_f64 over DPP moves), then the minimum index among the lanes that hold that value.
+// Every lane returns the wavefront's result.  Callers never pass NaN.
+__device__ __forceinline__ double fmin_sel(double a, double b) { return b < a ? b : a; }
+__device__ __forceinline__ double fmax_sel(double a, double b) { return b > a ? b : a; }
+__device__ __forceinline__ int imin_sel(int a, int b) { return b < a ? b : a; }
 
-template <int CTRL>
-__device__ __forceinline__ void max_step(double &v) {
-    const double ov = dpp_f64<CTRL>(v);
-    if (ov > v) v = ov;
+__device__ __forceinline__ double wave_min_f64(double v) {
+    v = fmin_sel(v, dpp_f64<TSVM_DPP_XOR1>(v));
+    v = fmin_sel(v, dpp_f64<TSVM_DPP_XOR2>(v));
+    v = fmin_sel(v, dpp_f64<TSVM_DPP_HALF_MIRROR>(v));
+    v = fmin_sel(v, dpp_f64<TSVM_DPP_MIRROR>(v));
+    const double r0 = readlane_f64(v, 0), r1 = readlane_f64(v, 16), r2 = readlane_f64(v, 32), r3 = readlane_f64(v, 48);
+    return fmin_sel(fmin_sel(r0, r1), fmin_sel(r2, r3));
 }
-__device__ __forceinline__ double wave_max(double v) {
-    max_step<TSVM_DPP_XOR1>(v);
-    max_step<TSVM_DPP_XOR2>(v);
-    max_step<TSVM_DPP_HALF_MIRROR>(v);
-    max_step<TSVM_DPP_MIRROR>(v);
-    double rv = readlane_f64(v, 0);
-#pragma unroll
-    for (int r = 1; r < 4; ++r) {
-        const double ov = readlane_f64(v, 16 * r);
-        if (ov > rv) rv = ov;
-    }
-    return rv;
+__device__ __forceinline__ double wave_max_f64(double v) {
+    v = fmax_sel(v, dpp_f64<TSVM_DPP_XOR1>(v));
+    v = fmax_sel(v, dpp_f64<TSVM_DPP_XOR2>(v));
+    v = fmax_sel(v, dpp_f64<TSVM_DPP_HALF_MIRROR>(v));
+    v = fmax_sel(v, dpp_f64<TSVM_DPP_MIRROR>(v));
+    const double r0 = readlane_f64(v, 0), r1 = readlane_f64(v, 16), r2 = readlane_f64(v, 32), r3 = readlane_f64(v, 48);
+    return fmax_sel(fmax_sel(r0, r1), fmax_sel(r2, r3));
+}
+__device__ __forceinline__ int wave_min_i32(int v) {
+    v = imin_sel(v, dpp_i32<TSVM_DPP_XOR1>(v));
+    v = imin_sel(v, dpp_i32<TSVM_DPP_XOR2>(v));
+    v = imin_sel(v, dpp_i32<TSVM_DPP_HALF_MIRROR>(v));
+    v = imin_sel(v, dpp_i32<TSVM_DPP_MIRROR>(v));
+    const int r0 = __builtin_amdgcn_readlane(v, 0), r1 = __builtin_amdgcn_readlane(v, 16);
+    const int r2 = __builtin_amdgcn_readlane(v, 32), r3 = __builtin_amdgcn_readlane(v, 48);
+    return imin_sel(imin_sel(r0, r1), imin_sel(r2, r3));
+}
+// v, i: this lane's candidate; on return the wavefront's lexicographic minimum.
+__device__ __forceinline__ void wave_argmin(double &v, int &i, int none) {
+    const double m = wave_min_f64(v);
+    i = wave_min_i32(v == m ? i : none);
+    v = m;
 }
 
 // Maps the launch's linear workgroup id to a logical one so that logical neighbours run on the
