@@ -77,7 +77,7 @@ def kernel_figures(train, params):
         x = torch.empty((n, ld), dtype=torch.float64, device="cuda")
         capi.call("tsvm_csr_to_dense", val_d.data_ptr(), col_d.data_ptr(), ptr_d.data_ptr(), n, x.data_ptr(), ld, None)
         ms = event_time(lambda: capi.call("tsvm_get_rows_dense", x.data_ptr(), ld, n, nf, sd.data_ptr(), x.data_ptr(), ld,
-                                          idx.data_ptr(), m, sd.data_ptr(), kt, gamma, 0.0, 3, k_out.data_ptr(), n, None), 20)
+                                          idx.data_ptr(), m, sd.data_ptr(), kt, gamma, 0.0, 3, k_out.data_ptr(), None, n, None), 20)
         flops = 2.0 * m * n * d
         out["get_rows"] = dict(kernel="get_rows_dense_kernel (fp64 MFMA)", ms=ms, m=m, n=n, d=d,
                                tflops=flops / ms / 1e9, frac_mfma_peak=flops / ms / 1e9 / FP64_MFMA_PEAK_TFLOPS,
@@ -92,7 +92,7 @@ def kernel_figures(train, params):
                       w.data_ptr(), None)
             capi.call("tsvm_gather_f64", sd.data_ptr(), idx.data_ptr(), m, sdw.data_ptr(), None)
             capi.call("tsvm_get_rows_csr", val_d.data_ptr(), col_d.data_ptr(), ptr_d.data_ptr(), n, sd.data_ptr(),
-                      w.data_ptr(), m, sdw.data_ptr(), kt, gamma, 0.0, 3, k_out.data_ptr(), n, None)
+                      w.data_ptr(), m, sdw.data_ptr(), kt, gamma, 0.0, 3, k_out.data_ptr(), None, n, None)
         ms = event_time(run, 10)
         by = 12.0 * train.nnz + 4.0 * (n + 1) + 8.0 * m * nf + 8.0 * m * n
         out["get_rows"] = dict(kernel="get_rows_csr_kernel", ms=ms, m=m, n=n, d=d, gflops=2.0 * m * train.nnz / ms / 1e6,

@@ -60,8 +60,9 @@ int tsvm_kernel_diag(const double *self_dot, int64_t n, int kernel_type, double 
 int tsvm_csr_to_dense(const double *val, const int *col, const int64_t *row_ptr, int64_t n, double *x, int64_t ld,
                       tsvm_stream stream);
 
-/* Dense get_rows: out[i*ldo + j] = kappa(a_i, x_j), i < m, j < n, where a_i is row a_idx[i] of `a`
- * (a_idx == NULL: row i).  Replaces get_working_set_ins + dns_csr_mul + RBF_kernel/poly_kernel/
+/* Dense get_rows: out[s_i*ldo + j] = kappa(a_i, x_j), i < m, j < n, where a_i is row a_idx[i] of `a`
+ * (a_idx == NULL: row i) and s_i = out_slots[i] (out_slots == NULL: i) is the output row, so new kernel
+ * rows can be written straight into the slots of a row cache.  Replaces get_working_set_ins + dns_csr_mul + RBF_kernel/poly_kernel/
  * sigmoid_kernel (kernelmatrix.cpp:251-312; kernelmatrix_kernel.cpp:9-25,61-108,149-160) in one
  * launch.  x is [n][ldx], a is [*][lda], both row-major fp64 with zero padding up to a multiple of
  * 8 columns (ldx % 8 == 0, lda % 8 == 0, d <= min(ldx, lda)).  The dot product is accumulated over
@@ -69,7 +70,8 @@ int tsvm_csr_to_dense(const double *val, const int *col, const int64_t *row_ptr,
  * products (used by RBF only). */
 int tsvm_get_rows_dense(const double *x, int64_t ldx, int64_t n, int d, const double *sd_x, const double *a,
                         int64_t lda, const int *a_idx, int m, const double *sd_a, int kernel_type, double gamma,
-                        double coef0, int degree, double *out, int64_t ldo, tsvm_stream stream);
+                        double coef0, int degree, double *out, const int *out_slots, int64_t ldo,
+                        tsvm_stream stream);
 
 /* Transposed dense staging of selected CSR rows: w[c*m + i] = value of feature c in row idx[i]
  * (idx == NULL: row i of the given CSR), w is [n_features][m] and is zero-filled first.
@@ -77,13 +79,13 @@ int tsvm_get_rows_dense(const double *x, int64_t ldx, int64_t n, int d, const do
 int tsvm_csr_stage_rows(const double *val, const int *col, const int64_t *row_ptr, const int *idx, int m,
                         int n_features, double *w, tsvm_stream stream);
 
-/* CSR get_rows: out[i*ldo + j] = kappa(w_i, x_j) with x in CSR (n rows) and the m working rows
+/* CSR get_rows: out[s_i*ldo + j] = kappa(w_i, x_j) (s_i as above) with x in CSR (n rows) and the m working rows
  * staged by tsvm_csr_stage_rows.  Accumulates over the stored order of row j's non-zeros
  * (dns_csr_mul, kernelmatrix_kernel.cpp:149-160) and applies the epilogue.  sd_w[i] are the
  * working rows' self dot products (already gathered, length m). */
 int tsvm_get_rows_csr(const double *val, const int *col, const int64_t *row_ptr, int64_t n, const double *sd_x,
                       const double *w, int m, const double *sd_w, int kernel_type, double gamma, double coef0,
-                      int degree, double *out, int64_t ldo, tsvm_stream stream);
+                      int degree, double *out, const int *out_slots, int64_t ldo, tsvm_stream stream);
 
 /* out[i] = in[idx[i]] for doubles (gathers working-set self dots). */
 int tsvm_gather_f64(const double *in, const int *idx, int m, double *out, tsvm_stream stream);

@@ -36,6 +36,7 @@ typedef struct tsvm_param {
     int verbose;
     const int *weight_label;
     const double *weight;
+    int64_t cache_bytes;    /* HBM kernel-row cache budget: -1 = half of the free device memory, 0 = off */
 } tsvm_param;
 
 const char *tsvm_model_last_error(void);
@@ -62,7 +63,8 @@ int tsvm_model_get(void *model, int *label, int *n_sv, double *rho, double *coef
                    int *sv_col, double *sv_val);
 
 /* Solver diagnostics of binary sub-problem k: outer iterations, inner iterations, objective and
- * device milliseconds per phase (select, get_rows, local solve, update_f; zeros unless profiled). */
+ * phase[8]: device milliseconds of select, get_rows, local solve, update_f (zeros unless profiled),
+ * then kernel-row cache lookups, hits, capacity in rows, and 1 if the cache was switched off. */
 int tsvm_model_stats(void *model, int k, int64_t *n_iter, int64_t *local_iter, double *obj, double *phase_ms);
 
 int64_t tsvm_model_binary_size(void *model, int k);
@@ -75,6 +77,16 @@ int tsvm_model_trace(void *model, int *ws_size, const double **diff, const int *
  * [nrows][n_binary_models], labels [nrows] (class label, regression value or +-1). */
 int tsvm_model_predict_csr(void *model, int64_t nrows, const int64_t *row_ptr, const int *col, const double *val,
                            int batch_size, double *dec_values, double *labels);
+
+/* CMDParser::parse_command_line for thundersvm-train (src/thundersvm/cmdparser.cpp:59-166): fills
+ * *param from LibSVM-style flags; argv[0] is the program name.  in/model file names are copied into
+ * the caller's buffers (each `cap` bytes).  Returns -1 with a message for an invalid command line. */
+int tsvm_cmdparser_train(int argc, char **argv, tsvm_param *param, int *gamma_set, int *do_cross_validation,
+                         int *nr_fold, char *input_file, char *model_file, int cap);
+
+/* Frees the device allocation that holds kernel rows between solves (it is otherwise kept until the
+ * process ends, because releasing it costs up to seconds). */
+int tsvm_release_device_cache(void);
 
 int tsvm_model_save(void *model, const char *path);
 int tsvm_model_load(void *model, const char *path);

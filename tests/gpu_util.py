@@ -34,10 +34,11 @@ def dense_padded(data, n_cols=None):
     return data.to_dense(ld), nf, ld
 
 
-def get_rows_dense(x_d, ld, n, d, sd_x, a_d, lda, a_idx, m, sd_a, kernel_type, gamma=0.0, coef0=0.0, degree=3):
-    out = torch.empty((m, n), dtype=torch.float64, device="cuda")
+def get_rows_dense(x_d, ld, n, d, sd_x, a_d, lda, a_idx, m, sd_a, kernel_type, gamma=0.0, coef0=0.0, degree=3,
+                   out_slots=None, out_rows=None):
+    out = torch.empty((out_rows or m, n), dtype=torch.float64, device="cuda")
     capi.call("tsvm_get_rows_dense", ptr(x_d), ld, n, d, ptr(sd_x), ptr(a_d), lda, ptr(a_idx), m, ptr(sd_a),
-              kernel_type, gamma, coef0, degree, ptr(out), n, stream())
+              kernel_type, gamma, coef0, degree, ptr(out), ptr(out_slots), n, stream())
     return out
 
 

@@ -116,7 +116,7 @@ def test_csr_path(name, kt, prm):
     capi.call("tsvm_gather_f64", G.ptr(sd), G.ptr(idx_d), m, G.ptr(sdw), G.stream())
     out = torch.empty((m, n), dtype=torch.float64, device="cuda")
     capi.call("tsvm_get_rows_csr", G.ptr(val_d), G.ptr(col_d), G.ptr(ptr_d), n, G.ptr(sd), G.ptr(w), m, G.ptr(sdw), kt,
-              prm.get("gamma", 0.0), prm.get("coef0", 0.0), prm.get("degree", 3), G.ptr(out), n, G.stream())
+              prm.get("gamma", 0.0), prm.get("coef0", 0.0), prm.get("degree", 3), G.ptr(out), None, n, G.stream())
     _check(name, G.host(out), okm.get_rows(idx))
     # the dense path on the same data gives the same bits (both sum in ascending feature order)
     xh, nf2, ld = G.dense_padded(data)
@@ -166,3 +166,26 @@ def test_sum_kernel_values(n_classes, rows):
     capi.call("tsvm_sum_kernel_values", G.ptr(coef_d), T, G.ptr(start_d), G.ptr(cnt_d), G.ptr(rho_d), G.ptr(k_d), T,
               G.ptr(dec), n_classes, rows, G.stream())
     assert np.abs(G.host(dec) - want).max() < 1e-9
+
+
+def test_output_row_slots():
+    """get_rows writes row i to out[out_slots[i]] (dense and CSR kernels)."""
+    rng = np.random.default_rng(21)
+    n, d, m, pool = 300, 20, 40, 64
+    data = from_dense(rng.standard_normal((n, d)).astype(np.float32))
+    p = O.make_param(kernel_type=O.RBF, gamma=0.2, expf_mode=1)
+    want = O.KernelMatrix(data.ptr, data.col, data.val, p).get_rows(np.arange(m))
+    x_d, nf, ld, sd, diag = _device_km(data, O.RBF, dict(gamma=0.2))
+    slots = rng.permutation(pool)[:m].astype(np.int32)
+    idx_d, slots_d = G.dev(np.arange(m, dtype=np.int32)), G.dev(slots)
+    got = G.host(G.get_rows_dense(x_d, ld, n, nf, sd, x_d, ld, idx_d, m, sd, O.RBF, gamma=0.2, out_slots=slots_d, out_rows=pool))
+    assert np.array_equal(got[slots], want)
+    val_d, col_d, ptr_d = G.dev(data.val), G.dev(data.col), G.dev(data.ptr)
+    w = torch.empty((nf, m), dtype=torch.float64, device="cuda")
+    capi.call("tsvm_csr_stage_rows", G.ptr(val_d), G.ptr(col_d), G.ptr(ptr_d), G.ptr(idx_d), m, nf, G.ptr(w), G.stream())
+    sdw = torch.empty(m, dtype=torch.float64, device="cuda")
+    capi.call("tsvm_gather_f64", G.ptr(sd), G.ptr(idx_d), m, G.ptr(sdw), G.stream())
+    out = torch.zeros((pool, n), dtype=torch.float64, device="cuda")
+    capi.call("tsvm_get_rows_csr", G.ptr(val_d), G.ptr(col_d), G.ptr(ptr_d), n, G.ptr(sd), G.ptr(w), m, G.ptr(sdw), O.RBF,
+              0.2, 0.0, 3, G.ptr(out), G.ptr(slots_d), n, G.stream())
+    assert np.array_equal(G.host(out)[slots], want)

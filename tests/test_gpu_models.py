@@ -127,3 +127,28 @@ def test_max_iter_cap():
     prm.max_iter = 3
     gm, om, _, _ = _compare(w["train"], w["test"], prm)
     assert gm.stats(0)["n_iter"] == 4
+
+
+def test_row_cache_is_value_transparent():
+    """The HBM kernel-row cache only changes which rows get recomputed: with it, without it and with a
+    cache too small to keep everything the trained models are bit-identical."""
+    w = D.workload_c2(scale=0.04)
+    tr = w["train"]
+    ref = None
+    for cache_bytes in (0, -1, 1500 * tr.n * 8):
+        prm = make_param(cache_bytes=cache_bytes, **w["params"])
+        gm = Model(0).train(tr, prm, ws_override=256, keep_binary=True)
+        st = gm.stats(0)
+        if cache_bytes == 0:
+            assert st["cache_rows"] == 0
+        elif cache_bytes == -1:
+            assert st["cache_rows"] == tr.n and st["cache_hits"] > 0
+        else:
+            assert 0 < st["cache_rows"] < tr.n
+        a, f = gm.binary(0)
+        cur = (a, f, gm.rho.copy(), st["n_iter"], st["local_iter"])
+        if ref is None:
+            ref = cur
+        else:
+            assert np.array_equal(cur[0], ref[0]) and np.array_equal(cur[1], ref[1])
+            assert np.array_equal(cur[2], ref[2]) and cur[3:] == ref[3:]

@@ -37,7 +37,7 @@ template <int KT, int TI>
 __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
     const double *__restrict__ x, int64_t ldx, int64_t n, int d, const double *__restrict__ sd_x,
     const double *__restrict__ a, int64_t lda, const int *__restrict__ a_idx, int m, const double *__restrict__ sd_a,
-    KernelParam kp_in, double *__restrict__ out, int64_t ldo, unsigned m_blocks) {
+    KernelParam kp_in, double *__restrict__ out, const int *__restrict__ out_slots, int64_t ldo, unsigned m_blocks) {
     constexpr int BM = 32 * TI;
     __shared__ double As[GR_KT * GR_LS];
     __shared__ double Bs[GR_KT * GR_LS];
@@ -129,7 +129,7 @@ __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
             if (i >= m) continue;
             double sdi = 0.0;
             if (sd_a) sdi = sd_a[a_idx ? a_idx[i] : i];
-            double *orow = out + (int64_t) i * ldo;
+            double *orow = out + (int64_t) (out_slots ? out_slots[i] : i) * ldo;
 #pragma unroll
             for (int tj = 0; tj < 4; ++tj) {
                 if (jj[tj] < n) orow[jj[tj]] = tsvm_epilogue(acc[ti][tj][v], sdi, sdj[tj], kp, exp_tab);
@@ -148,7 +148,7 @@ __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
 __global__ __launch_bounds__(256) void get_rows_csr_kernel(
     const double *__restrict__ val, const int *__restrict__ col, const int64_t *__restrict__ row_ptr, int64_t n,
     const double *__restrict__ sd_x, const double *__restrict__ w, int m, const double *__restrict__ sd_w,
-    KernelParam kp, double *__restrict__ out, int64_t ldo, unsigned i_blocks) {
+    KernelParam kp, double *__restrict__ out, const int *__restrict__ out_slots, int64_t ldo, unsigned i_blocks) {
     __shared__ uint64_t exp_tab[32];
     const int tid = threadIdx.x;
     if (tid < 32) exp_tab[tid] = TSVM_EXP2F_TAB[tid];
@@ -176,7 +176,7 @@ __global__ __launch_bounds__(256) void get_rows_csr_kernel(
     }
     if (!active) return;
     const double sdi = sd_w ? sd_w[i] : 0.0;
-    double *orow = out + (int64_t) i * ldo;
+    double *orow = out + (int64_t) (out_slots ? out_slots[i] : i) * ldo;
 #pragma unroll
     for (int jj = 0; jj < CS_JB; ++jj) {
         const int64_t j = j0 + jj;
@@ -372,7 +372,7 @@ int tsvm_csr_to_dense(const double *val, const int *col, const int64_t *row_ptr,
 
 int tsvm_get_rows_dense(const double *x, int64_t ldx, int64_t n, int d, const double *sd_x, const double *a,
                         int64_t lda, const int *a_idx, int m, const double *sd_a, int kernel_type, double gamma,
-                        double coef0, int degree, double *out, int64_t ldo, tsvm_stream stream) {
+                        double coef0, int degree, double *out, const int *out_slots, int64_t ldo, tsvm_stream stream) {
     TSVM_REQUIRE(x && a && out, "tsvm_get_rows_dense: null pointer");
     TSVM_REQUIRE(n >= 0 && m >= 0 && d >= 0, "tsvm_get_rows_dense: negative size");
     TSVM_REQUIRE(ldx % 8 == 0 && lda % 8 == 0, "tsvm_get_rows_dense: ldx (%lld) and lda (%lld) must be multiples of 8",
@@ -395,10 +395,10 @@ int tsvm_get_rows_dense(const double *x, int64_t ldx, int64_t n, int d, const do
     do {                                                                                                              \
         if (ti == 2)                                                                                                  \
             hipLaunchKernelGGL((get_rows_dense_kernel<KTYPE, 2>), grid, block, 0, tsvm_s(stream), x, ldx, n, d, sd_x, a, \
-                               lda, a_idx, m, sd_a, kp, out, ldo, m_blocks);                                          \
+                               lda, a_idx, m, sd_a, kp, out, out_slots, ldo, m_blocks);                               \
         else                                                                                                          \
             hipLaunchKernelGGL((get_rows_dense_kernel<KTYPE, 4>), grid, block, 0, tsvm_s(stream), x, ldx, n, d, sd_x, a, \
-                               lda, a_idx, m, sd_a, kp, out, ldo, m_blocks);                                          \
+                               lda, a_idx, m, sd_a, kp, out, out_slots, ldo, m_blocks);                               \
     } while (0)
     switch (kernel_type) {
         case TSVM_LINEAR: GR_LAUNCH(TSVM_LINEAR); break;
@@ -425,7 +425,7 @@ int tsvm_csr_stage_rows(const double *val, const int *col, const int64_t *row_pt
 
 int tsvm_get_rows_csr(const double *val, const int *col, const int64_t *row_ptr, int64_t n, const double *sd_x,
                       const double *w, int m, const double *sd_w, int kernel_type, double gamma, double coef0,
-                      int degree, double *out, int64_t ldo, tsvm_stream stream) {
+                      int degree, double *out, const int *out_slots, int64_t ldo, tsvm_stream stream) {
     TSVM_REQUIRE(row_ptr && w && out, "tsvm_get_rows_csr: null pointer");
     TSVM_REQUIRE(n >= 0 && m >= 0 && ldo >= n, "tsvm_get_rows_csr: bad size");
     TSVM_REQUIRE(kernel_type >= 0 && kernel_type <= 4, "tsvm_get_rows_csr: unknown kernel type %d", kernel_type);
@@ -437,7 +437,7 @@ int tsvm_get_rows_csr(const double *val, const int *col, const int64_t *row_ptr,
     const int64_t j_blocks = (n + CS_JB - 1) / CS_JB;
     TSVM_REQUIRE(j_blocks * i_blocks < (int64_t) 0x7fffffff, "tsvm_get_rows_csr: grid too large");
     hipLaunchKernelGGL(get_rows_csr_kernel, dim3((unsigned) (j_blocks * i_blocks)), dim3(256), 0, tsvm_s(stream), val, col,
-                       row_ptr, n, sd_x, w, m, sd_w, kp, out, ldo, i_blocks);
+                       row_ptr, n, sd_x, w, m, sd_w, kp, out, out_slots, ldo, i_blocks);
     TSVM_LAUNCH_CHECK();
     return 0;
 }

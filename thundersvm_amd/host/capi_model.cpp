@@ -5,6 +5,7 @@
 #include <exception>
 #include <new>
 
+#include "cmdparser.h"
 #include "models.h"
 
 namespace {
@@ -73,6 +74,7 @@ static void configure(Handle *h, const tsvm_param *param, int ws_override, int k
     h->model->ws_override = ws_override;
     h->model->keep_binary = keep_binary != 0;
     h->model->profile = profile != 0;
+    h->model->cache_bytes = param->cache_bytes;
     h->trace = SolverTrace();
     h->trace.cap_iters = trace_cap;
     h->model->trace_first = trace_cap > 0 ? &h->trace : nullptr;
@@ -148,6 +150,10 @@ int tsvm_model_stats(void *model, int k, int64_t *n_iter, int64_t *local_iter, d
             phase_ms[1] = s.ms_get_rows;
             phase_ms[2] = s.ms_local;
             phase_ms[3] = s.ms_update_f;
+            phase_ms[4] = (double) s.cache_lookups;
+            phase_ms[5] = (double) s.cache_hits;
+            phase_ms[6] = (double) s.cache_rows;
+            phase_ms[7] = s.cache_disabled ? 1.0 : 0.0;
         }
     })
 }
@@ -183,6 +189,36 @@ int tsvm_model_predict_csr(void *model, int64_t nrows, const int64_t *row_ptr, c
         if (labels) memcpy(labels, out.data(), sizeof(double) * (size_t) nrows);
         if (dec_values) memcpy(dec_values, m.get_dec_value().data(), sizeof(double) * m.get_dec_value().size());
     })
+}
+
+int tsvm_cmdparser_train(int argc, char **argv, tsvm_param *param, int *gamma_set, int *do_cross_validation,
+                         int *nr_fold, char *input_file, char *model_file, int cap) {
+    TSVM_GUARD({
+        CMDParser parser;
+        parser.parse_train(argc, argv, 1);
+        const SvmParam &p = parser.param_cmd;
+        param->svm_type = p.svm_type;
+        param->kernel_type = p.kernel_type;
+        param->degree = p.degree;
+        param->gamma = p.gamma;
+        param->coef0 = p.coef0;
+        param->C = p.C;
+        param->nu = p.nu;
+        param->p = p.p;
+        param->epsilon = p.epsilon;
+        param->max_mem_size = (int64_t) p.max_mem_size;
+        param->nr_weight = p.nr_weight;
+        param->verbose = parser.quiet ? 0 : 1;
+        if (gamma_set) *gamma_set = parser.gamma_set;
+        if (do_cross_validation) *do_cross_validation = parser.do_cross_validation;
+        if (nr_fold) *nr_fold = parser.nr_fold;
+        if (input_file) snprintf(input_file, cap, "%s", parser.svmtrain_input_file_name.c_str());
+        if (model_file) snprintf(model_file, cap, "%s", parser.model_file_name.c_str());
+    })
+}
+
+int tsvm_release_device_cache(void) {
+    TSVM_GUARD({ tsvm::RowArena::instance().release(); })
 }
 
 int tsvm_model_save(void *model, const char *path) {

@@ -30,6 +30,25 @@ inline void abi_check(int rc) {
 
 size_t &device_bytes_in_use();   // running total of DeviceBuffer allocations (the SyncMem byte counter's role)
 
+// One grow-only device allocation that outlives individual solves and holds the kernel rows (working-set
+// rows plus the row cache).  Releasing a multi-gigabyte allocation costs up to seconds on this platform,
+// so the 21 one-vs-one solves of a 7-class problem must not each allocate and free their own pool.
+// Not counted in device_bytes_in_use().
+class RowArena {
+public:
+    static RowArena &instance();
+    // bytes a solve may use when the caller gave no explicit budget: the arena's size once it exists,
+    // otherwise half of the free device memory
+    size_t auto_budget();
+    void *acquire(size_t bytes, bool auto_sized);
+    void release();
+    size_t capacity() const { return cap_; }
+
+private:
+    void *ptr_ = nullptr;
+    size_t cap_ = 0;
+};
+
 template <typename T>
 class DeviceBuffer {
 public:

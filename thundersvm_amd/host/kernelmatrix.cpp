@@ -9,6 +9,34 @@ size_t &device_bytes_in_use() {
     static size_t bytes = 0;
     return bytes;
 }
+
+RowArena &RowArena::instance() {
+    static RowArena arena;
+    return arena;
+}
+
+size_t RowArena::auto_budget() {
+    if (cap_) return cap_;
+    size_t free_b = 0, total_b = 0;
+    TSVM_HIP_CHECK(hipMemGetInfo(&free_b, &total_b));
+    return free_b / 2;
+}
+
+void *RowArena::acquire(size_t bytes, bool auto_sized) {
+    if (bytes <= cap_) return ptr_;
+    size_t want = bytes;
+    if (auto_sized) want = std::max(want, auto_budget());   // take the whole automatic budget once
+    release();
+    TSVM_HIP_CHECK(hipMalloc(&ptr_, want));
+    cap_ = want;
+    return ptr_;
+}
+
+void RowArena::release() {
+    if (ptr_) (void) hipFree(ptr_);
+    ptr_ = nullptr;
+    cap_ = 0;
+}
 }  // namespace tsvm
 
 // Dense rows cost d_pad MFMA k-steps per output, CSR rows cost one L2 gather per stored non-zero;
@@ -76,12 +104,12 @@ void KernelMatrix::build(const DataSet::node2d &all, const int *rows, size_t n_r
     }
 }
 
-void KernelMatrix::get_rows(const int *d_idx, int m, kernel_type *d_out, int64_t ld) const {
+void KernelMatrix::get_rows(const int *d_idx, int m, kernel_type *d_out, int64_t ld, const int *d_out_slots) const {
     const int n = (int) n_instances_;
     if (dense_) {
         abi_check(tsvm_get_rows_dense(x_.data(), ld_, n, (int) n_features_, self_dot_.data(), x_.data(), ld_, d_idx, m,
                                       self_dot_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
-                                      d_out, ld, nullptr));
+                                      d_out, d_out_slots, ld, nullptr));
         return;
     }
     if (stage_.size() < (size_t) m * n_features_) stage_.resize((size_t) m * n_features_);
@@ -91,7 +119,7 @@ void KernelMatrix::get_rows(const int *d_idx, int m, kernel_type *d_out, int64_t
     abi_check(tsvm_gather_f64(self_dot_.data(), d_idx, m, stage_sd_.data(), nullptr));
     abi_check(tsvm_get_rows_csr(val_.data(), col_ind_.data(), row_ptr_.data(), n, self_dot_.data(), stage_.data(), m,
                                 stage_sd_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree, d_out,
-                                ld, nullptr));
+                                d_out_slots, ld, nullptr));
 }
 
 // External batch (kernelmatrix.cpp:281-312, 385-406): features with id >= n_features_ are left out of
@@ -123,13 +151,13 @@ void KernelMatrix::get_rows(const DataSet::node2d &instances, kernel_type *d_out
         abi_check(tsvm_csr_to_dense(b_val_.data(), b_col_.data(), b_ptr_.data(), m, stage_.data(), ld_, nullptr));
         abi_check(tsvm_get_rows_dense(x_.data(), ld_, n, (int) n_features_, self_dot_.data(), stage_.data(), ld_, nullptr, m,
                                       stage_sd_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
-                                      d_out, ld, nullptr));
+                                      d_out, nullptr, ld, nullptr));
     } else {
         if (stage_.size() < (size_t) m * n_features_) stage_.resize((size_t) m * n_features_);
         abi_check(tsvm_csr_stage_rows(b_val_.data(), b_col_.data(), b_ptr_.data(), nullptr, m, (int) n_features_,
                                       stage_.data(), nullptr));
         abi_check(tsvm_get_rows_csr(val_.data(), col_ind_.data(), row_ptr_.data(), n, self_dot_.data(), stage_.data(), m,
                                     stage_sd_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
-                                    d_out, ld, nullptr));
+                                    d_out, nullptr, ld, nullptr));
     }
 }

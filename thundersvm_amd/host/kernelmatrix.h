@@ -16,8 +16,8 @@ public:
     // Rows `rows[0..n_rows)` of `all`, without materialising a node2d copy.
     KernelMatrix(const DataSet::node2d &all, const int *rows, size_t n_rows, SvmParam param, int repeat = 1);
 
-    // kernel rows of stored instances d_idx[0..m) (device ids) -> d_out[i*ld + j]
-    void get_rows(const int *d_idx, int m, kernel_type *d_out, int64_t ld) const;
+    // kernel rows of stored instances d_idx[0..m) (device ids) -> d_out[s_i*ld + j], s_i = d_out_slots[i] (or i)
+    void get_rows(const int *d_idx, int m, kernel_type *d_out, int64_t ld, const int *d_out_slots = nullptr) const;
     // kernel rows of an external batch -> d_out[i*ld + j]
     void get_rows(const DataSet::node2d &instances, kernel_type *d_out, int64_t ld) const;
 

@@ -50,6 +50,7 @@ public:
     int ws_override = 0;                  // > 0 forces the working-set size
     bool profile = false;
     bool keep_binary = false;             // keep binary_alpha / binary_f (tests)
+    long long cache_bytes = -1;           // kernel-row cache budget handed to the solver (-1 auto, 0 off)
 
 protected:
     virtual void model_setup(const DataSet &dataset, SvmParam &param);

@@ -13,6 +13,53 @@ inline bool up_set(float_type a, float_type y, float_type Cp, float_type Cn) { r
 inline bool low_set(float_type a, float_type y, float_type Cp, float_type Cn) { return (y > 0 && a > 0) || (y < 0 && a < Cn); }
 inline bool free_sv(float_type a, float_type y, float_type Cp, float_type Cn) { return a > 0 && (y > 0 ? a < Cp : a < Cn); }
 
+// Kernel-row cache bookkeeping (host side).  Rows of the kernel matrix live in slots of one HBM pool;
+// slot_of maps an instance id to its slot, an intrusive doubly linked list keeps the slots in
+// least-recently-used order.  The device only ever sees slot numbers.  The reference keeps no rows
+// beyond the previous working set's second half (csmosolver.cpp:33-42,65-77); cached rows are the
+// rows get_rows would recompute, so the cache cannot change a result.
+struct RowCache {
+    int cap = 0, used = 0, head = -1, tail = -1;
+    std::vector<int> slot_of, id_of, prev, next;
+    void init(int n, int capacity) {
+        cap = capacity;
+        slot_of.assign(n, -1);
+        id_of.assign(cap, -1);
+        prev.assign(cap, -1);
+        next.assign(cap, -1);
+    }
+    void unlink(int s) {
+        if (prev[s] >= 0) next[prev[s]] = next[s]; else head = next[s];
+        if (next[s] >= 0) prev[next[s]] = prev[s]; else tail = prev[s];
+    }
+    void push_front(int s) {
+        prev[s] = -1;
+        next[s] = head;
+        if (head >= 0) prev[head] = s;
+        head = s;
+        if (tail < 0) tail = s;
+    }
+    int lookup(int id) {                 // slot of a cached row (marked most recently used) or -1
+        const int s = slot_of[id];
+        if (s >= 0) { unlink(s); push_front(s); }
+        return s;
+    }
+    int insert(int id) {                 // slot for a new row: a free one, else the least recently used
+        int s;
+        if (used < cap) {
+            s = used++;
+        } else {
+            s = tail;
+            unlink(s);
+            slot_of[id_of[s]] = -1;
+        }
+        id_of[s] = id;
+        slot_of[id] = s;
+        push_front(s);
+        return s;
+    }
+};
+
 struct PhaseTimer {
     bool on;
     hipEvent_t e0 = nullptr, e1 = nullptr;
@@ -42,9 +89,8 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
     const bool nu = is_nu();
     stats = SolverStats();
 
-    DeviceBuffer<int> d_y(n), d_ws(ws_size), d_slots_even(ws_size), d_slots_odd(ws_size);
+    DeviceBuffer<int> d_y(n), d_ws(ws_size), d_slots_a(ws_size), d_slots_b(ws_size), d_miss_ids(ws_size), d_miss_slots(ws_size);
     DeviceBuffer<float_type> d_alpha(n), d_f(n), d_alpha_diff(ws_size), d_diff(2);
-    DeviceBuffer<kernel_type> d_k_rows((size_t) ws_size * ld);
     DeviceBuffer<unsigned char> d_sel_ws(tsvm_select_workspace(n));
     DeviceBuffer<unsigned char> d_smo_ws(tsvm_smo_solve_workspace(ws_size));
     d_y.upload(y.data(), n);
@@ -52,17 +98,46 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
     d_f.upload(f_val.data(), n);
     d_diff.zero();
     d_alpha_diff.zero();
-    {
-        // Rows kept from the previous working set are re-addressed, not copied (csmosolver.cpp:69,75):
-        // logical row t of the working set lives in physical row slot[t]; the two halves swap every iteration.
-        std::vector<int> even(ws_size), odd(ws_size);
-        for (int t = 0; t < ws_size; ++t) { even[t] = t; odd[t] = (t + q) % ws_size; }
-        d_slots_even.upload(even.data(), ws_size);
-        d_slots_odd.upload(odd.data(), ws_size);
+
+    // Kernel rows live in slots of one pool.  With a cache the pool holds up to pool_rows rows and the
+    // host tracks which instance sits in which slot; without one it holds exactly ws rows.
+    long long pool_rows = ws_size;
+    tsvm::RowArena &arena = tsvm::RowArena::instance();
+    if (cache_bytes != 0 && n > ws_size) {
+        const long long budget = cache_bytes > 0 ? cache_bytes : (long long) arena.auto_budget();
+        const long long fit = budget / (long long) (ld * sizeof(kernel_type));
+        // an LRU that can hold only a small part of the matrix does not hit: require a quarter of the rows
+        if (fit >= 4LL * ws_size && fit >= n / 4) pool_rows = std::min<long long>(n, fit);
     }
+    bool caching = pool_rows > ws_size;
+    kernel_type *const k_rows = (kernel_type *) arena.acquire((size_t) pool_rows * ld * sizeof(kernel_type), cache_bytes < 0);
+    RowCache cache;
+    if (caching) {
+        cache.init(n, (int) pool_rows);
+        stats.cache_rows = pool_rows;
+    }
+    std::vector<int> cur_slots(ws_size), cur_ids(ws_size), miss_ids, miss_slots;
+    int *h_ids = nullptr, *h_slots = nullptr;
     double *h_diff = nullptr;
     TSVM_HIP_CHECK(hipHostMalloc((void **) &h_diff, 2 * sizeof(double)));
+    TSVM_HIP_CHECK(hipHostMalloc((void **) &h_ids, ws_size * sizeof(int)));
+    TSVM_HIP_CHECK(hipHostMalloc((void **) &h_slots, 3 * ws_size * sizeof(int)));
     h_diff[0] = h_diff[1] = 0;
+    // without a cache the slot tables just alternate: the two halves of the working set swap places
+    // every iteration, so the rows kept from the previous iteration are re-addressed, never copied
+    // (the reference copies q*n values per iteration, csmosolver.cpp:75)
+    auto upload_rotation = [&](const std::vector<int> &slots_now) {
+        std::vector<int> other(ws_size);
+        for (int t = 0; t < ws_size; ++t) other[t] = slots_now[(t + q) % ws_size];
+        d_slots_a.upload(slots_now.data(), ws_size);
+        d_slots_b.upload(other.data(), ws_size);
+    };
+    int rotation_base = 0;   // iteration at which d_slots_a was valid
+    long long window_lookups = 0, window_hits = 0;
+    if (!caching) {
+        for (int t = 0; t < ws_size; ++t) cur_slots[t] = t;
+        upload_rotation(cur_slots);
+    }
 
     init_f(alpha, y, k_mat, d_f.data());
 
@@ -78,7 +153,8 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
     }
 
     for (int iter = 0;; ++iter) {
-        const int *slots = (iter % 2 == 0) ? d_slots_even.data() : d_slots_odd.data();
+        const int n_new = iter == 0 ? ws_size : q;
+        const int first_new = iter == 0 ? 0 : q;
         timer.begin();
         if (iter == 0) {
             abi_check(tsvm_select_working_set(d_f.data(), d_y.data(), d_alpha.data(), n, Cp, Cn, nullptr, 0, d_ws.data(),
@@ -90,27 +166,78 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
         }
         timer.end(stats.ms_select);
         timer.begin();
-        if (iter == 0) {
-            k_mat.get_rows(d_ws.data(), ws_size, d_k_rows.data(), ld);
+        const int *slots;
+        if (caching) {
+            // read the new ids back, look them up, and compute only the rows that are not cached
+            TSVM_HIP_CHECK(hipMemcpyAsync(h_ids, d_ws.data() + first_new, sizeof(int) * n_new, hipMemcpyDeviceToHost, nullptr));
+            TSVM_HIP_CHECK(hipStreamSynchronize(nullptr));
+            if (iter > 0) {
+                for (int t = 0; t < q; ++t) {   // rows kept from the previous working set stay most recently used
+                    cur_ids[t] = cur_ids[t + q];
+                    cur_slots[t] = cache.lookup(cur_ids[t]);
+                }
+            }
+            miss_ids.clear();
+            miss_slots.clear();
+            for (int t = 0; t < n_new; ++t) {
+                const int id = h_ids[t];
+                int s = cache.lookup(id);
+                stats.cache_lookups++;
+                if (s >= 0) {
+                    stats.cache_hits++;
+                } else {
+                    s = cache.insert(id);
+                    miss_ids.push_back(id);
+                    miss_slots.push_back(s);
+                }
+                cur_ids[first_new + t] = id;
+                cur_slots[first_new + t] = s;
+            }
+            int *h_miss_ids = h_slots + ws_size, *h_miss_slots = h_slots + 2 * ws_size;
+            std::copy(cur_slots.begin(), cur_slots.end(), h_slots);
+            std::copy(miss_ids.begin(), miss_ids.end(), h_miss_ids);
+            std::copy(miss_slots.begin(), miss_slots.end(), h_miss_slots);
+            const int n_miss = (int) miss_ids.size();
+            TSVM_HIP_CHECK(hipMemcpyAsync(d_slots_a.data(), h_slots, sizeof(int) * ws_size, hipMemcpyHostToDevice, nullptr));
+            if (n_miss) {
+                TSVM_HIP_CHECK(hipMemcpyAsync(d_miss_ids.data(), h_miss_ids, sizeof(int) * n_miss, hipMemcpyHostToDevice, nullptr));
+                TSVM_HIP_CHECK(hipMemcpyAsync(d_miss_slots.data(), h_miss_slots, sizeof(int) * n_miss, hipMemcpyHostToDevice, nullptr));
+                k_mat.get_rows(d_miss_ids.data(), n_miss, k_rows, ld, d_miss_slots.data());
+            }
+            slots = d_slots_a.data();
+            // A cache that has started evicting and still does not hit only costs the id read-back:
+            // every 64 iterations, if fewer than 5 % of the window's lookups hit, fall back to rotation.
+            // (A cache that can hold every row is never switched off: its misses are first touches.)
+            if (cache.cap < n && cache.used == cache.cap && iter % 64 == 63) {
+                const long long dl = stats.cache_lookups - window_lookups, dh = stats.cache_hits - window_hits;
+                if (dh * 20 < dl) {
+                    caching = false;
+                    stats.cache_disabled = true;
+                    upload_rotation(cur_slots);
+                    rotation_base = iter;
+                }
+            }
+            if (iter % 64 == 63) { window_lookups = stats.cache_lookups; window_hits = stats.cache_hits; }
         } else {
-            // new rows go to the physical half that the dropped rows occupied
-            const int phys0 = (iter % 2 == 0) ? q : 0;
-            k_mat.get_rows(d_ws.data() + q, q, d_k_rows.data() + (size_t) phys0 * ld, ld);
+            const bool on_a = ((iter - rotation_base) % 2) == 0;
+            slots = on_a ? d_slots_a.data() : d_slots_b.data();
+            // new rows go to the slots the dropped rows occupied
+            k_mat.get_rows(d_ws.data() + first_new, n_new, k_rows, ld, slots + first_new);
         }
         timer.end(stats.ms_get_rows);
         timer.begin();
         if (nu) {
             abi_check(tsvm_nu_smo_solve(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), d_ws.data(), ws_size, Cp,
-                                        d_k_rows.data(), slots, ld, k_mat.diag(), eps, d_diff.data(), max_iter,
+                                        k_rows, slots, ld, k_mat.diag(), eps, d_diff.data(), max_iter,
                                         d_smo_ws.data(), nullptr));
         } else {
             abi_check(tsvm_c_smo_solve(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), d_ws.data(), ws_size, Cp,
-                                       Cn, d_k_rows.data(), slots, ld, k_mat.diag(), eps, d_diff.data(), max_iter,
+                                       Cn, k_rows, slots, ld, k_mat.diag(), eps, d_diff.data(), max_iter,
                                        d_smo_ws.data(), nullptr));
         }
         timer.end(stats.ms_local);
         timer.begin();
-        abi_check(tsvm_update_f(d_f.data(), d_alpha_diff.data(), ws_size, d_k_rows.data(), slots, ld, n, nullptr));
+        abi_check(tsvm_update_f(d_f.data(), d_alpha_diff.data(), ws_size, k_rows, slots, ld, n, nullptr));
         timer.end(stats.ms_update_f);
         TSVM_HIP_CHECK(hipMemcpyAsync(h_diff, d_diff.data(), 2 * sizeof(double), hipMemcpyDeviceToHost, nullptr));
         TSVM_HIP_CHECK(hipStreamSynchronize(nullptr));
@@ -145,11 +272,13 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
             stats.local_iter = local_iter;
             stats.obj = calculate_obj(f_val, alpha, y);
             TSVM_LOG << "global iter = " << iter << ", total local iter = " << local_iter << ", diff = " << diff0
-                     << ", obj = " << stats.obj;
+                     << ", obj = " << stats.obj << ", cache hits " << stats.cache_hits << "/" << stats.cache_lookups;
             break;
         }
     }
     (void) hipHostFree(h_diff);
+    (void) hipHostFree(h_ids);
+    (void) hipHostFree(h_slots);
 }
 
 // csmosolver.cpp:189-214: f starts from a non-zero alpha in batches of 101 rows.

@@ -17,6 +17,10 @@ struct SolverStats {
     double obj = 0;
     // accumulated device time per phase in ms (only filled when profile == true)
     double ms_select = 0, ms_get_rows = 0, ms_local = 0, ms_update_f = 0;
+    // kernel-row cache
+    long long cache_lookups = 0, cache_hits = 0;
+    long long cache_rows = 0;     // capacity in rows (0: cache not used)
+    bool cache_disabled = false;  // switched off after the warm-up because it was not hitting
 };
 
 class CSMOSolver {
@@ -29,6 +33,8 @@ public:
     mutable SolverStats stats;
     SolverTrace *trace = nullptr;
     bool profile = false;
+    // Budget of the HBM kernel-row cache in bytes: -1 = half of the free device memory, 0 = no cache.
+    long long cache_bytes = -1;
 
 protected:
     virtual bool is_nu() const { return false; }

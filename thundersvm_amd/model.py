@@ -20,16 +20,17 @@ class TsvmParam(C.Structure):
     _fields_ = [("svm_type", C.c_int), ("kernel_type", C.c_int), ("degree", C.c_int), ("max_iter", C.c_int),
                 ("gamma", C.c_double), ("coef0", C.c_double), ("C", C.c_double), ("nu", C.c_double),
                 ("p", C.c_double), ("epsilon", C.c_double), ("max_mem_size", C.c_int64), ("nr_weight", C.c_int),
-                ("verbose", C.c_int), ("weight_label", _ip), ("weight", _dp)]
+                ("verbose", C.c_int), ("weight_label", _ip), ("weight", _dp), ("cache_bytes", C.c_int64)]
 
 
 def make_param(svm_type=0, kernel_type=2, degree=3, gamma=0.0, coef0=0.0, C=1.0, nu=0.5, p=0.1, epsilon=0.001,
-               max_mem_size=8192 << 20, max_iter=-1, verbose=0):
+               max_mem_size=8192 << 20, max_iter=-1, verbose=0, cache_bytes=-1):
     """Defaults of include/thundersvm/svmparam.h:14-29."""
     prm = TsvmParam()
     prm.svm_type, prm.kernel_type, prm.degree, prm.max_iter = svm_type, kernel_type, degree, max_iter
     prm.gamma, prm.coef0, prm.C, prm.nu, prm.p, prm.epsilon = gamma, coef0, C, nu, p, epsilon
     prm.max_mem_size, prm.nr_weight, prm.verbose = max_mem_size, 0, verbose
+    prm.cache_bytes = cache_bytes
     return prm
 
 
@@ -121,10 +122,11 @@ class Model:
 
     def stats(self, k=0):
         ni, li, obj = C.c_int64(), C.c_int64(), C.c_double()
-        ms = np.zeros(4)
+        ms = np.zeros(8)
         _check(host_lib().tsvm_model_stats(self.h, k, C.byref(ni), C.byref(li), C.byref(obj), _p(ms, _dp)))
         return dict(n_iter=ni.value, local_iter=li.value, obj=obj.value, ms_select=ms[0], ms_get_rows=ms[1],
-                    ms_local=ms[2], ms_update_f=ms[3])
+                    ms_local=ms[2], ms_update_f=ms[3], cache_lookups=int(ms[4]), cache_hits=int(ms[5]), cache_rows=int(ms[6]),
+                    cache_disabled=bool(ms[7]))
 
     def binary(self, k):
         n = host_lib().tsvm_model_binary_size(self.h, k)
