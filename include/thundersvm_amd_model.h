@@ -52,6 +52,18 @@ int tsvm_model_train_csr(void *model, int64_t n, const int64_t *row_ptr, const i
                          const double *y, const tsvm_param *param, int ws_override, int keep_binary, int trace_cap,
                          int profile);
 
+/* DataSet handles: rows converted once into the host layer's DataSet (DataSet::load_from_sparse's
+ * role, src/thundersvm/dataset.cpp:124-148, with float64 values and the caller's feature ids), so that
+ * a timed train / predict call covers what the reference's `model->train(dataset, param)` covers and
+ * not the conversion.  y may be NULL for prediction-only data. */
+void *tsvm_dataset_new_csr(int64_t n, const int64_t *row_ptr, const int *col, const double *val, const double *y);
+void *tsvm_dataset_load(const char *libsvm_file);
+void tsvm_dataset_free(void *dataset);
+int64_t tsvm_dataset_rows(void *dataset);
+int tsvm_model_train(void *model, void *dataset, const tsvm_param *param, int ws_override, int keep_binary,
+                     int trace_cap, int profile);
+int tsvm_model_predict(void *model, void *dataset, int batch_size, double *dec_values, double *labels);
+
 /* SvmModel::train on a LibSVM text file (DataSet::load_from_file). */
 int tsvm_model_train_file(void *model, const char *path, const tsvm_param *param);
 

@@ -13,7 +13,7 @@ import pytest
 
 import oracle_lib as O
 from thundersvm_amd import data as D
-from thundersvm_amd.model import Model, make_param
+from thundersvm_amd.model import Dataset, Model, make_param
 
 pytestmark = pytest.mark.gpu
 FIXTURE = os.path.join(os.path.dirname(__file__), "golden", "test_dataset.txt")
@@ -152,3 +152,20 @@ def test_row_cache_is_value_transparent():
         else:
             assert np.array_equal(cur[0], ref[0]) and np.array_equal(cur[1], ref[1])
             assert np.array_equal(cur[2], ref[2]) and cur[3:] == ref[3:]
+
+
+def test_dataset_handle_and_file_loader(tmp_path):
+    """Training from a DataSet handle, from CSR arrays and from a LibSVM text file gives the same model."""
+    w = D.workload_c4(scale=0.004)
+    tr = w["train"]
+    prm = make_param(**w["params"])
+    a = Model(0).train(tr, prm)
+    b = Model(0).train(Dataset(tr), prm)
+    path = str(tmp_path / "c4.txt")
+    D.save_libsvm(path, tr)
+    c = Model(0).train(Dataset(path=path), prm)
+    for m in (b, c):
+        assert np.array_equal(a.coef, m.coef) and np.array_equal(a.rho, m.rho) and np.array_equal(a.sv_indices, m.sv_indices)
+    la, da = a.predict(tr)
+    lb, db = b.predict(Dataset(tr))
+    assert np.array_equal(da, db) and np.array_equal(la, lb)

@@ -22,25 +22,30 @@ typedef double v4d __attribute__((ext_vector_type(4)));
 //
 // Workgroup = 256 threads = 4 wavefronts in a 2x2 grid; each wavefront owns a (16*TI)x64 block of the
 // (32*TI)x128 output tile as TIx4 MFMA tiles (16*TI accumulator doubles per lane).  K is walked in tiles
-// of 8 columns staged through LDS in k-major order [8][130]: the stride of 130 doubles keeps both
-// the staging writes and the operand reads free of bank conflicts.
+// of 8 or 16 columns staged through LDS in k-major order, with the next tile's global loads in flight
+// in registers while the current one is multiplied.
 // ------------------------------------------------------------------------------------------------
 #define GR_BN 128
-#define GR_KT 8
-#define GR_LS 130
 
 // KT: kernel type (compile-time so that only one epilogue is instantiated); TI: 16-row MFMA tiles
-// per wavefront in the working-row direction (4 -> 128-row workgroup tile, 2 -> 64-row tile with
-// half the accumulators and twice the resident wavefronts, used when d is small and the epilogue
-// and stores dominate).
+// per wavefront in the working-row direction.  Two shapes are used:
+//   TI = 4, K tile 8:  128x128 workgroup tile, 2 wavefronts per SIMD (large d, MFMA-bound);
+//   TI = 2, K tile 16: 64x128 workgroup tile, half the accumulators, 3 wavefronts per SIMD (small d,
+//                      where the epilogue and the stores weigh as much as the MFMAs).
+// Either way a wavefront issues 32 MFMAs between two barriers.  LDS tiles are k-major [KTILE][LS];
+// LS (130 / 129 doubles) makes the staging writes and the operand reads bank-conflict free.
 template <int KT, int TI>
 __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
     const double *__restrict__ x, int64_t ldx, int64_t n, int d, const double *__restrict__ sd_x,
     const double *__restrict__ a, int64_t lda, const int *__restrict__ a_idx, int m, const double *__restrict__ sd_a,
     KernelParam kp_in, double *__restrict__ out, const int *__restrict__ out_slots, int64_t ldo, unsigned m_blocks) {
     constexpr int BM = 32 * TI;
-    __shared__ double As[GR_KT * GR_LS];
-    __shared__ double Bs[GR_KT * GR_LS];
+    constexpr int KTILE = TI == 2 ? 16 : 8;
+    constexpr int LS = TI == 2 ? 129 : 130;
+    constexpr int A_TPR = KTILE / 4;          // threads per A row (one 4-double vector each)
+    constexpr int B_VEC = KTILE / 8;          // 4-double vectors per thread for the B tile (2 threads per row)
+    __shared__ double As[KTILE * LS];
+    __shared__ double Bs[KTILE * LS];
     __shared__ uint64_t exp_tab[32];
     KernelParam kp = kp_in;
     kp.kernel_type = KT;
@@ -56,19 +61,19 @@ __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
     const int64_t j0 = (int64_t) (logical / m_blocks) * GR_BN;
     const int i0 = (int) (logical % m_blocks) * BM;
 
-    // staging assignment: thread -> (row = tid/2, 4 consecutive k at 4*(tid&1)); the A tile has BM rows
-    const int srow = tid >> 1;
-    const int skh = (tid & 1) * 4;
+    // staging assignment
+    const int a_row = tid / A_TPR, a_k = (tid % A_TPR) * 4;
+    const int b_row = tid >> 1, b_k = (tid & 1) * (4 * B_VEC);
     const double *a_ptr = nullptr;
     const double *x_ptr = nullptr;
     {
-        int ai = i0 + srow;
-        if (srow < BM && ai < m) {
-            int64_t r = a_idx ? (int64_t) a_idx[ai] : (int64_t) ai;
-            a_ptr = a + r * lda + skh;
+        const int ai = i0 + a_row;
+        if (ai < m) {
+            const int64_t r = a_idx ? (int64_t) a_idx[ai] : (int64_t) ai;
+            a_ptr = a + r * lda + a_k;
         }
-        int64_t xj = j0 + srow;
-        if (xj < n) x_ptr = x + xj * ldx + skh;
+        const int64_t xj = j0 + b_row;
+        if (xj < n) x_ptr = x + xj * ldx + b_k;
     }
 
     v4d acc[TI][4];
@@ -77,62 +82,93 @@ __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
 #pragma unroll
         for (int tj = 0; tj < 4; ++tj) acc[ti][tj] = (v4d){0.0, 0.0, 0.0, 0.0};
 
-    const int n_kt = (d + GR_KT - 1) / GR_KT;
-    v4d ra = (v4d){0.0, 0.0, 0.0, 0.0}, rb = (v4d){0.0, 0.0, 0.0, 0.0};
-    if (a_ptr) ra = *(const v4d *) a_ptr;
-    if (x_ptr) rb = *(const v4d *) x_ptr;
-
+    // Per-row / per-column data of the epilogue (self dot products, output row offsets) is fetched
+    // here, ahead of the K loop, so that its dependent loads are off the critical path by the time the
+    // accumulators are ready.
     const int lrow = lane & 15;
     const int lk = lane >> 4;
+    const int64_t jb = j0 + wj * 64 + lrow;
+    const bool full = (i0 + BM <= m) && (j0 + GR_BN <= n);
+    double sdj[4], sdi[TI * 4];
+    int64_t orow_off[TI * 4];
+#pragma unroll
+    for (int tj = 0; tj < 4; ++tj) sdj[tj] = (sd_x && jb + tj * 16 < n) ? sd_x[jb + tj * 16] : 0.0;
+#pragma unroll
+    for (int u = 0; u < TI * 4; ++u) {
+        const int i = i0 + wi * (16 * TI) + (u >> 2) * 16 + 4 * (u & 3) + lk;
+        const bool ok = i < m;
+        sdi[u] = (sd_a && ok) ? sd_a[a_idx ? a_idx[i] : i] : 0.0;
+        orow_off[u] = (int64_t) ((out_slots && ok) ? out_slots[i] : i) * ldo;
+    }
+
+    // rows are padded with zeros up to ldx / lda (multiples of 8), so a vector may be read whenever
+    // its first column is inside the padded row
+    const int kmax_a = (int) lda, kmax_x = (int) ldx;
+    const int n_kt = (d + KTILE - 1) / KTILE;
+    const v4d zero4 = (v4d){0.0, 0.0, 0.0, 0.0};
+    v4d ra = zero4, rb[B_VEC];
+    auto load_tile = [&](int kt) {
+        const int k0 = kt * KTILE;
+        ra = (a_ptr && (KTILE == 8 || k0 + a_k < kmax_a)) ? *(const v4d *) (a_ptr + k0) : zero4;
+#pragma unroll
+        for (int q = 0; q < B_VEC; ++q)
+            rb[q] = (x_ptr && (KTILE == 8 || k0 + b_k + 4 * q < kmax_x)) ? *(const v4d *) (x_ptr + k0 + 4 * q) : zero4;
+    };
+    load_tile(0);
 
     for (int kt = 0; kt < n_kt; ++kt) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            if (srow < BM) As[(skh + e) * GR_LS + srow] = ra[e];
-            Bs[(skh + e) * GR_LS + srow] = rb[e];
+            As[(a_k + e) * LS + a_row] = ra[e];
+#pragma unroll
+            for (int q = 0; q < B_VEC; ++q) Bs[(b_k + 4 * q + e) * LS + b_row] = rb[q][e];
         }
         __syncthreads();
-        if (kt + 1 < n_kt) {
-            if (a_ptr) ra = *(const v4d *) (a_ptr + (kt + 1) * GR_KT);
-            if (x_ptr) rb = *(const v4d *) (x_ptr + (kt + 1) * GR_KT);
-        }
+        if (kt + 1 < n_kt) load_tile(kt + 1);
+        const int k_left = d - kt * KTILE;               // columns still to multiply (uniform)
+        const int n_ks = k_left >= KTILE ? KTILE / 4 : (k_left + 3) / 4;
 #pragma unroll
-        for (int ks = 0; ks < GR_KT / 4; ++ks) {
-            double af[TI], bf[4];
-            const int kk = (ks * 4 + lk) * GR_LS;
+        for (int ks = 0; ks < KTILE / 4; ++ks) {
+            if (KTILE == 8 || ks < n_ks) {   // 8-column tiles are always whole (rows are padded to 8)
+                double af[TI], bf[4];
+                const int kk = (ks * 4 + lk) * LS;
 #pragma unroll
-            for (int t = 0; t < TI; ++t) af[t] = As[kk + wi * (16 * TI) + t * 16 + lrow];
+                for (int t = 0; t < TI; ++t) af[t] = As[kk + wi * (16 * TI) + t * 16 + lrow];
 #pragma unroll
-            for (int t = 0; t < 4; ++t) bf[t] = Bs[kk + wj * 64 + t * 16 + lrow];
+                for (int t = 0; t < 4; ++t) bf[t] = Bs[kk + wj * 64 + t * 16 + lrow];
 #pragma unroll
-            for (int ti = 0; ti < TI; ++ti)
+                for (int ti = 0; ti < TI; ++ti)
 #pragma unroll
-                for (int tj = 0; tj < 4; ++tj)
-                    acc[ti][tj] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[ti], bf[tj], acc[ti][tj], 0, 0, 0);
+                    for (int tj = 0; tj < 4; ++tj)
+                        acc[ti][tj] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[ti], bf[tj], acc[ti][tj], 0, 0, 0);
+            }
         }
         __syncthreads();
     }
 
-    // epilogue + store
-    double sdj[4];
-    int64_t jj[4];
+    // epilogue + store.  Interior tiles take the unguarded path; edge tiles test every element.
+    if (full) {
 #pragma unroll
-    for (int tj = 0; tj < 4; ++tj) {
-        jj[tj] = j0 + wj * 64 + tj * 16 + lrow;
-        sdj[tj] = (jj[tj] < n && sd_x) ? sd_x[jj[tj]] : 0.0;
-    }
+        for (int ti = 0; ti < TI; ++ti) {
 #pragma unroll
-    for (int ti = 0; ti < TI; ++ti) {
+            for (int v = 0; v < 4; ++v) {
+                double *orow = out + orow_off[ti * 4 + v] + jb;
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            const int i = i0 + wi * (16 * TI) + ti * 16 + 4 * v + lk;
-            if (i >= m) continue;
-            double sdi = 0.0;
-            if (sd_a) sdi = sd_a[a_idx ? a_idx[i] : i];
-            double *orow = out + (int64_t) (out_slots ? out_slots[i] : i) * ldo;
+                for (int tj = 0; tj < 4; ++tj)
+                    orow[tj * 16] = tsvm_epilogue(acc[ti][tj][v], sdi[ti * 4 + v], sdj[tj], kp, exp_tab);
+            }
+        }
+    } else {
 #pragma unroll
-            for (int tj = 0; tj < 4; ++tj) {
-                if (jj[tj] < n) orow[jj[tj]] = tsvm_epilogue(acc[ti][tj][v], sdi, sdj[tj], kp, exp_tab);
+        for (int ti = 0; ti < TI; ++ti) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int i = i0 + wi * (16 * TI) + ti * 16 + 4 * v + lk;
+                if (i >= m) continue;
+                double *orow = out + orow_off[ti * 4 + v] + jb;
+#pragma unroll
+                for (int tj = 0; tj < 4; ++tj)
+                    if (jb + tj * 16 < n) orow[tj * 16] = tsvm_epilogue(acc[ti][tj][v], sdi[ti * 4 + v], sdj[tj], kp, exp_tab);
             }
         }
     }

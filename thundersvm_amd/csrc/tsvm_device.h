@@ -31,14 +31,13 @@ __constant__ const uint64_t TSVM_EXP2F_TAB[32] = {
 // algorithm glibc (>= 2.27) uses for expf.  `tab` points at the 32-entry table (LDS or constant).
 // The reference's kernels call libm expf on the host (kernelmatrix_kernel.cpp:71-72,87-89).
 __device__ __forceinline__ float tsvm_expf(float x, const uint64_t *tab) {
-    if (x != x) return x;
-    if (x > 0x1.62e42ep6f) return __builtin_inff();
-    if (x < -0x1.9fe368p6f) return 0.0f;
     const double InvLn2N = 0x1.71547652b82fep+0 * 32;
     const double SHIFT = 0x1.8p+52;
     const double C0 = 0x1.c6af84b912394p-5 / 32 / 32 / 32;
     const double C1 = 0x1.ebfce50fac4f3p-3 / 32 / 32;
     const double C2 = 0x1.62e42ff0c52d6p-1 / 32;
+    // The main path runs unconditionally and the out-of-range cases are selected afterwards (no
+    // branches in the epilogue); a NaN argument comes out as NaN through the arithmetic itself.
     double xd = (double) x;
     double z = InvLn2N * xd;
     double kd = z + SHIFT;
@@ -53,7 +52,10 @@ __device__ __forceinline__ float tsvm_expf(float x, const uint64_t *tab) {
     double y = __builtin_fma(C2, r, 1.0);
     y = __builtin_fma(zz, r2, y);
     y = y * s;
-    return (float) y;
+    float res = (float) y;
+    res = x > 0x1.62e42ep6f ? __builtin_inff() : res;   // > log(2^128)
+    res = x < -0x1.9fe368p6f ? 0.0f : res;              // < log(2^-150)
+    return res;
 }
 
 // Kernel epilogues (kernelmatrix_kernel.cpp:61-108).  sd0/sd1 are the two rows' self dot products.

@@ -92,6 +92,50 @@ int tsvm_model_train_csr(void *model, int64_t n, const int64_t *row_ptr, const i
     })
 }
 
+void *tsvm_dataset_new_csr(int64_t n, const int64_t *row_ptr, const int *col, const double *val, const double *y) {
+    try {
+        DataSet *ds = new DataSet();
+        ds->load_from_csr(n, row_ptr, col, val, y);
+        return ds;
+    } catch (const std::exception &e) {
+        fail(e);
+        return nullptr;
+    }
+}
+
+void *tsvm_dataset_load(const char *libsvm_file) {
+    try {
+        DataSet *ds = new DataSet();
+        ds->load_from_file(libsvm_file);
+        return ds;
+    } catch (const std::exception &e) {
+        fail(e);
+        return nullptr;
+    }
+}
+
+void tsvm_dataset_free(void *dataset) { delete (DataSet *) dataset; }
+int64_t tsvm_dataset_rows(void *dataset) { return (int64_t) ((DataSet *) dataset)->n_instances(); }
+
+int tsvm_model_train(void *model, void *dataset, const tsvm_param *param, int ws_override, int keep_binary,
+                     int trace_cap, int profile) {
+    TSVM_GUARD({
+        Handle *h = (Handle *) model;
+        configure(h, param, ws_override, keep_binary, trace_cap, profile);
+        h->model->train(*(DataSet *) dataset, to_param(*param));
+    })
+}
+
+int tsvm_model_predict(void *model, void *dataset, int batch_size, double *dec_values, double *labels) {
+    TSVM_GUARD({
+        SvmModel &m = *((Handle *) model)->model;
+        const DataSet &ds = *(DataSet *) dataset;
+        std::vector<float_type> out = m.predict(ds.instances(), batch_size);
+        if (labels) memcpy(labels, out.data(), sizeof(double) * out.size());
+        if (dec_values) memcpy(dec_values, m.get_dec_value().data(), sizeof(double) * m.get_dec_value().size());
+    })
+}
+
 int tsvm_model_train_file(void *model, const char *path, const tsvm_param *param) {
     TSVM_GUARD({
         Handle *h = (Handle *) model;

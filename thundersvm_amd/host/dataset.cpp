@@ -117,7 +117,7 @@ void DataSet::group_classes(bool classification) {
     count_.clear();
     label_.clear();
     perm_.clear();
-    const size_t n = instances_.size();
+    const size_t n = instances().size();
     if (!classification) {
         perm_.resize(n);
         for (size_t i = 0; i < n; ++i) perm_[i] = (int) i;
@@ -143,10 +143,20 @@ void DataSet::group_classes(bool classification) {
     for (size_t i = 0; i < n; ++i) perm_[cursor[cls[i]]++] = (int) i;
 }
 
+DataSet DataSet::grouped_view() const {
+    DataSet v;
+    v.y_ = y_;
+    v.n_features_ = n_features_;
+    v.zero_based_ = zero_based_;
+    v.base_ = base_ ? base_ : &instances_;
+    v.group_classes(true);
+    return v;
+}
+
 const DataSet::node2d DataSet::instances(int y_i) const {
     node2d out;
     out.reserve(count_[y_i]);
-    for (int i = start_[y_i]; i < start_[y_i] + count_[y_i]; ++i) out.push_back(instances_[perm_[i]]);
+    for (int i = start_[y_i]; i < start_[y_i] + count_[y_i]; ++i) out.push_back(instances()[perm_[i]]);
     return out;
 }
 

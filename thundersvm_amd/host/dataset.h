@@ -24,14 +24,16 @@ public:
     void load_from_csr(int64_t n, const int64_t *row_ptr, const int *col, const double *val, const double *y);
 
     void group_classes(bool classification = true);
-    size_t n_instances() const { return instances_.size(); }
+    // A grouped DataSet that refers to this one's instances instead of copying them.
+    DataSet grouped_view() const;
+    size_t n_instances() const { return instances().size(); }
     size_t n_features() const { return n_features_; }
     size_t n_classes() const { return start_.size(); }
     const std::vector<int> &count() const { return count_; }
     const std::vector<int> &start() const { return start_; }
     const std::vector<int> &label() const { return label_; }
     const std::vector<float_type> &y() const { return y_; }
-    const node2d &instances() const { return instances_; }
+    const node2d &instances() const { return base_ ? *base_ : instances_; }
     const node2d instances(int y_i) const;
     const node2d instances(int y_i, int y_j) const;
     const std::vector<int> original_index() const { return perm_; }
@@ -42,6 +44,7 @@ public:
 private:
     std::vector<float_type> y_;
     node2d instances_;
+    const node2d *base_ = nullptr;   // set by grouped_view(): instances live in another DataSet
     size_t n_features_ = 0;
     std::vector<int> start_, count_, label_, perm_;
     bool zero_based_ = false;

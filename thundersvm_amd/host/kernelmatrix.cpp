@@ -64,24 +64,30 @@ KernelMatrix::KernelMatrix(const DataSet::node2d &all, const int *rows, size_t n
 void KernelMatrix::build(const DataSet::node2d &all, const int *rows, size_t n_rows, int repeat) {
     n_instances_ = n_rows * repeat;
     std::vector<int64_t> ptr(n_instances_ + 1, 0);
-    size_t total = 0;
     int max_index = 0;
+#pragma omp parallel for reduction(max : max_index) schedule(static)
     for (size_t r = 0; r < n_rows; ++r) {
         const auto &row = all[rows ? rows[r] : r];
-        total += row.size();
+        ptr[r + 1] = (int64_t) row.size();
         for (const auto &nd : row) max_index = std::max(max_index, nd.index);
     }
+    for (size_t r = 0; r < n_rows; ++r) ptr[r + 1] += ptr[r];
+    const size_t total = (size_t) ptr[n_rows];
+    for (int rep = 1; rep < repeat; ++rep)
+        for (size_t r = 0; r < n_rows; ++r) ptr[rep * n_rows + r + 1] = ptr[r + 1] + (int64_t) (rep * total);
     nnz_ = total * repeat;
     n_features_ = (size_t) max_index + 1;
     std::vector<kernel_type> val(nnz_);
     std::vector<int> col(nnz_);
-    size_t e = 0;
-    for (int rep = 0; rep < repeat; ++rep) {
-        for (size_t r = 0; r < n_rows; ++r) {
-            const auto &row = all[rows ? rows[r] : r];
-            for (const auto &nd : row) { val[e] = nd.value; col[e] = nd.index; ++e; }
-            ptr[rep * n_rows + r + 1] = (int64_t) e;
-        }
+#pragma omp parallel for schedule(static)
+    for (size_t r = 0; r < n_rows; ++r) {
+        const auto &row = all[rows ? rows[r] : r];
+        size_t e = (size_t) ptr[r];
+        for (const auto &nd : row) { val[e] = nd.value; col[e] = nd.index; ++e; }
+    }
+    for (int rep = 1; rep < repeat; ++rep) {
+        std::copy(val.begin(), val.begin() + total, val.begin() + rep * total);
+        std::copy(col.begin(), col.begin() + total, col.begin() + rep * total);
     }
     val_.upload(val);
     col_ind_.upload(col);

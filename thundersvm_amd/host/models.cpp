@@ -304,8 +304,9 @@ void SVC::model_setup(const DataSet &dataset, SvmParam &p) {   // svc.cpp:16-39
 }
 
 void SVC::train(const DataSet &dataset, SvmParam p) {   // svc.cpp:41-145
-    DataSet grouped = dataset;
-    grouped.group_classes();
+    // the reference groups a copy of the data set (svc.cpp:42-43); grouping only reads y, so the copy
+    // here shares nothing but the labels and the instances are referenced in place
+    DataSet grouped = dataset.grouped_view();
     model_setup(grouped, p);
     const int n = (int) grouped.n_instances();
     std::vector<std::vector<float_type>> alpha(n_binary_models);

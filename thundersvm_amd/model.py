@@ -50,6 +50,15 @@ def host_lib():
         L.tsvm_model_free.argtypes = [C.c_void_p]
         L.tsvm_model_train_csr.argtypes = [C.c_void_p, C.c_int64, _i64p, _ip, _dp, _dp, C.POINTER(TsvmParam), C.c_int,
                                            C.c_int, C.c_int, C.c_int]
+        L.tsvm_dataset_new_csr.restype = C.c_void_p
+        L.tsvm_dataset_new_csr.argtypes = [C.c_int64, _i64p, _ip, _dp, _dp]
+        L.tsvm_dataset_load.restype = C.c_void_p
+        L.tsvm_dataset_load.argtypes = [C.c_char_p]
+        L.tsvm_dataset_free.argtypes = [C.c_void_p]
+        L.tsvm_dataset_rows.restype = C.c_int64
+        L.tsvm_dataset_rows.argtypes = [C.c_void_p]
+        L.tsvm_model_train.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(TsvmParam), C.c_int, C.c_int, C.c_int, C.c_int]
+        L.tsvm_model_predict.argtypes = [C.c_void_p, C.c_void_p, C.c_int, _dp, _dp]
         L.tsvm_model_train_file.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(TsvmParam)]
         L.tsvm_model_info.argtypes = [C.c_void_p, _ip, _ip, _ip, _i64p]
         L.tsvm_model_get.argtypes = [C.c_void_p, _ip, _ip, _dp, _dp, _ip, _i64p, _ip, _dp]
@@ -77,6 +86,27 @@ def _p(a, t):
     return None if a is None else a.ctypes.data_as(t)
 
 
+class Dataset:
+    """Rows held by the host layer's DataSet (converted once, reusable across train / predict calls)."""
+
+    def __init__(self, data=None, path=None):
+        L = host_lib()
+        if path is not None:
+            self.h = C.c_void_p(L.tsvm_dataset_load(path.encode()))
+        else:
+            y = None if data.y is None else np.ascontiguousarray(data.y, dtype=np.float64)
+            self.h = C.c_void_p(L.tsvm_dataset_new_csr(data.n, _p(data.ptr, _i64p), _p(data.col, _ip), _p(data.val, _dp),
+                                                       _p(y, _dp)))
+        if not self.h:
+            raise capi.TsvmError(L.tsvm_model_last_error().decode())
+        self.n = L.tsvm_dataset_rows(self.h)
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            host_lib().tsvm_dataset_free(self.h)
+            self.h = None
+
+
 class Model:
     def __init__(self, svm_type=0):
         self.svm_type = svm_type
@@ -90,6 +120,11 @@ class Model:
             self.h = None
 
     def train(self, data, param, ws_override=0, keep_binary=False, trace_cap=0, profile=False):
+        if isinstance(data, Dataset):
+            _check(host_lib().tsvm_model_train(self.h, data.h, C.byref(param), ws_override, int(keep_binary), trace_cap,
+                                               int(profile)))
+            self._fetch()
+            return self
         y = data.y if data.y is not None else np.zeros(data.n)
         _check(host_lib().tsvm_model_train_csr(self.h, data.n, _p(data.ptr, _i64p), _p(data.col, _ip), _p(data.val, _dp),
                                                _p(np.ascontiguousarray(y, dtype=np.float64), _dp), C.byref(param),
@@ -147,6 +182,9 @@ class Model:
         """Returns (labels / values, decision values [n, n_binary])."""
         dec = np.zeros((data.n, self.n_binary))
         lab = np.zeros(data.n)
+        if isinstance(data, Dataset):
+            _check(host_lib().tsvm_model_predict(self.h, data.h, batch_size, _p(dec, _dp), _p(lab, _dp)))
+            return lab, dec
         _check(host_lib().tsvm_model_predict_csr(self.h, data.n, _p(data.ptr, _i64p), _p(data.col, _ip),
                                                  _p(data.val, _dp), batch_size, _p(dec, _dp), _p(lab, _dp)))
         return lab, dec
