@@ -32,7 +32,7 @@ def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=3)
-    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--scale", type=float, default=1.0, help="row-count scale of the workload (1.0 = benchmark shape)")
     ap.add_argument("--cpu-iters", type=int, default=-1, help="outer iterations of the CPU baseline sample (-1 = auto, 0 = skip)")
@@ -76,7 +76,7 @@ def kernel_figures(train, params):
     if dense_ok:
         x = torch.empty((n, ld), dtype=torch.float64, device="cuda")
         capi.call("tsvm_csr_to_dense", val_d.data_ptr(), col_d.data_ptr(), ptr_d.data_ptr(), n, x.data_ptr(), ld, None)
-        ms = event_time(lambda: capi.call("tsvm_get_rows_dense", x.data_ptr(), ld, n, nf, sd.data_ptr(), x.data_ptr(), ld,
+        ms = event_time(lambda: capi.call("tsvm_get_rows_dense", x.data_ptr(), ld, None, n, nf, sd.data_ptr(), x.data_ptr(), ld,
                                           idx.data_ptr(), m, sd.data_ptr(), kt, gamma, 0.0, 3, k_out.data_ptr(), None, n, None), 20)
         flops = 2.0 * m * n * d
         out["get_rows"] = dict(kernel="get_rows_dense_kernel (fp64 MFMA)", ms=ms, m=m, n=n, d=d,
@@ -91,7 +91,7 @@ def kernel_figures(train, params):
             capi.call("tsvm_csr_stage_rows", val_d.data_ptr(), col_d.data_ptr(), ptr_d.data_ptr(), idx.data_ptr(), m, nf,
                       w.data_ptr(), None)
             capi.call("tsvm_gather_f64", sd.data_ptr(), idx.data_ptr(), m, sdw.data_ptr(), None)
-            capi.call("tsvm_get_rows_csr", val_d.data_ptr(), col_d.data_ptr(), ptr_d.data_ptr(), n, sd.data_ptr(),
+            capi.call("tsvm_get_rows_csr", val_d.data_ptr(), col_d.data_ptr(), ptr_d.data_ptr(), None, n, sd.data_ptr(),
                       w.data_ptr(), m, sdw.data_ptr(), kt, gamma, 0.0, 3, k_out.data_ptr(), None, n, None)
         ms = event_time(run, 10)
         by = 12.0 * train.nnz + 4.0 * (n + 1) + 8.0 * m * nf + 8.0 * m * n

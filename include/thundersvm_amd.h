@@ -62,13 +62,15 @@ int tsvm_csr_to_dense(const double *val, const int *col, const int64_t *row_ptr,
 
 /* Dense get_rows: out[s_i*ldo + j] = kappa(a_i, x_j), i < m, j < n, where a_i is row a_idx[i] of `a`
  * (a_idx == NULL: row i) and s_i = out_slots[i] (out_slots == NULL: i) is the output row, so new kernel
- * rows can be written straight into the slots of a row cache.  Replaces get_working_set_ins + dns_csr_mul + RBF_kernel/poly_kernel/
+ * rows can be written straight into the slots of a row cache.  x_idx != NULL restricts the columns to
+ * the rows x_idx[0..n) of x (x_j = row x_idx[j]); with x_idx = a_idx = the working set this yields the
+ * ws x ws block the local solver needs without touching the other n - ws rows.  Replaces get_working_set_ins + dns_csr_mul + RBF_kernel/poly_kernel/
  * sigmoid_kernel (kernelmatrix.cpp:251-312; kernelmatrix_kernel.cpp:9-25,61-108,149-160) in one
  * launch.  x is [n][ldx], a is [*][lda], both row-major fp64 with zero padding up to a multiple of
  * 8 columns (ldx % 8 == 0, lda % 8 == 0, d <= min(ldx, lda)).  The dot product is accumulated over
  * ascending column index with fused multiply-adds.  sd_x[j] / sd_a[a_idx[i]] are the self dot
  * products (used by RBF only). */
-int tsvm_get_rows_dense(const double *x, int64_t ldx, int64_t n, int d, const double *sd_x, const double *a,
+int tsvm_get_rows_dense(const double *x, int64_t ldx, const int *x_idx, int64_t n, int d, const double *sd_x, const double *a,
                         int64_t lda, const int *a_idx, int m, const double *sd_a, int kernel_type, double gamma,
                         double coef0, int degree, double *out, const int *out_slots, int64_t ldo,
                         tsvm_stream stream);
@@ -82,8 +84,8 @@ int tsvm_csr_stage_rows(const double *val, const int *col, const int64_t *row_pt
 /* CSR get_rows: out[s_i*ldo + j] = kappa(w_i, x_j) (s_i as above) with x in CSR (n rows) and the m working rows
  * staged by tsvm_csr_stage_rows.  Accumulates over the stored order of row j's non-zeros
  * (dns_csr_mul, kernelmatrix_kernel.cpp:149-160) and applies the epilogue.  sd_w[i] are the
- * working rows' self dot products (already gathered, length m). */
-int tsvm_get_rows_csr(const double *val, const int *col, const int64_t *row_ptr, int64_t n, const double *sd_x,
+ * working rows' self dot products (already gathered, length m).  x_idx as in tsvm_get_rows_dense. */
+int tsvm_get_rows_csr(const double *val, const int *col, const int64_t *row_ptr, const int *x_idx, int64_t n, const double *sd_x,
                       const double *w, int m, const double *sd_w, int kernel_type, double gamma, double coef0,
                       int degree, double *out, const int *out_slots, int64_t ldo, tsvm_stream stream);
 
@@ -111,6 +113,20 @@ int tsvm_c_smo_solve(const int *y, const double *f_val, double *alpha, double *a
                      int ws_size, double Cp, double Cn, const double *k_rows, const int *slots, int64_t ld,
                      const double *k_diag, double eps, double *diff, int max_iter, void *workspace,
                      tsvm_stream stream);
+
+/* Row stride (in doubles) of the ws x ws block the solver kernels read: ws rounded up to 256, 512 or 1024. */
+int tsvm_smo_solve_block_ld(int ws_size);
+
+/* c_smo_solve / nu_smo_solve on a precomputed block kws[r*ldk + t] = K(x_ws[r], x_ws[t]) (ldk from
+ * tsvm_smo_solve_block_ld, columns t >= ws zero or arbitrary finite values): the solver touches nothing
+ * else of the kernel matrix, so it can run while the full rows are still being computed on another
+ * stream.  C is passed as Cp for the nu variant (Cn unused). */
+int tsvm_c_smo_solve_block(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
+                           int ws_size, double Cp, double Cn, const double *kws, const double *k_diag, double eps,
+                           double *diff, int max_iter, tsvm_stream stream);
+int tsvm_nu_smo_solve_block(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
+                            int ws_size, double C, const double *kws, const double *k_diag, double eps, double *diff,
+                            int max_iter, tsvm_stream stream);
 
 /* nu_smo_solve (smo_kernel.cpp:127-298), same conventions; diff[1] is left untouched as in the
  * reference's CPU code. */

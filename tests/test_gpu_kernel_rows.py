@@ -115,7 +115,7 @@ def test_csr_path(name, kt, prm):
     sdw = torch.empty(m, dtype=torch.float64, device="cuda")
     capi.call("tsvm_gather_f64", G.ptr(sd), G.ptr(idx_d), m, G.ptr(sdw), G.stream())
     out = torch.empty((m, n), dtype=torch.float64, device="cuda")
-    capi.call("tsvm_get_rows_csr", G.ptr(val_d), G.ptr(col_d), G.ptr(ptr_d), n, G.ptr(sd), G.ptr(w), m, G.ptr(sdw), kt,
+    capi.call("tsvm_get_rows_csr", G.ptr(val_d), G.ptr(col_d), G.ptr(ptr_d), None, n, G.ptr(sd), G.ptr(w), m, G.ptr(sdw), kt,
               prm.get("gamma", 0.0), prm.get("coef0", 0.0), prm.get("degree", 3), G.ptr(out), None, n, G.stream())
     _check(name, G.host(out), okm.get_rows(idx))
     # the dense path on the same data gives the same bits (both sum in ascending feature order)
@@ -186,6 +186,6 @@ def test_output_row_slots():
     sdw = torch.empty(m, dtype=torch.float64, device="cuda")
     capi.call("tsvm_gather_f64", G.ptr(sd), G.ptr(idx_d), m, G.ptr(sdw), G.stream())
     out = torch.zeros((pool, n), dtype=torch.float64, device="cuda")
-    capi.call("tsvm_get_rows_csr", G.ptr(val_d), G.ptr(col_d), G.ptr(ptr_d), n, G.ptr(sd), G.ptr(w), m, G.ptr(sdw), O.RBF,
+    capi.call("tsvm_get_rows_csr", G.ptr(val_d), G.ptr(col_d), G.ptr(ptr_d), None, n, G.ptr(sd), G.ptr(w), m, G.ptr(sdw), O.RBF,
               0.2, 0.0, 3, G.ptr(out), G.ptr(slots_d), n, G.stream())
     assert np.array_equal(G.host(out)[slots], want)

@@ -36,9 +36,10 @@ typedef double v4d __attribute__((ext_vector_type(4)));
 // LS (130 / 129 doubles) makes the staging writes and the operand reads bank-conflict free.
 template <int KT, int TI>
 __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
-    const double *__restrict__ x, int64_t ldx, int64_t n, int d, const double *__restrict__ sd_x,
-    const double *__restrict__ a, int64_t lda, const int *__restrict__ a_idx, int m, const double *__restrict__ sd_a,
-    KernelParam kp_in, double *__restrict__ out, const int *__restrict__ out_slots, int64_t ldo, unsigned m_blocks) {
+    const double *__restrict__ x, int64_t ldx, const int *__restrict__ x_idx, int64_t n, int d,
+    const double *__restrict__ sd_x, const double *__restrict__ a, int64_t lda, const int *__restrict__ a_idx, int m,
+    const double *__restrict__ sd_a, KernelParam kp_in, double *__restrict__ out, const int *__restrict__ out_slots,
+    int64_t ldo, unsigned m_blocks) {
     constexpr int BM = 32 * TI;
     constexpr int KTILE = TI == 2 ? 16 : 8;
     constexpr int LS = TI == 2 ? 129 : 130;
@@ -73,7 +74,7 @@ __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
             a_ptr = a + r * lda + a_k;
         }
         const int64_t xj = j0 + b_row;
-        if (xj < n) x_ptr = x + xj * ldx + b_k;
+        if (xj < n) x_ptr = x + (x_idx ? (int64_t) x_idx[xj] : xj) * ldx + b_k;
     }
 
     v4d acc[TI][4];
@@ -92,7 +93,10 @@ __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
     double sdj[4], sdi[TI * 4];
     int64_t orow_off[TI * 4];
 #pragma unroll
-    for (int tj = 0; tj < 4; ++tj) sdj[tj] = (sd_x && jb + tj * 16 < n) ? sd_x[jb + tj * 16] : 0.0;
+    for (int tj = 0; tj < 4; ++tj) {
+        const int64_t j = jb + tj * 16;
+        sdj[tj] = (sd_x && j < n) ? sd_x[x_idx ? (int64_t) x_idx[j] : j] : 0.0;
+    }
 #pragma unroll
     for (int u = 0; u < TI * 4; ++u) {
         const int i = i0 + wi * (16 * TI) + (u >> 2) * 16 + 4 * (u & 3) + lk;
@@ -182,9 +186,10 @@ __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
 #define CS_JB 16
 
 __global__ __launch_bounds__(256) void get_rows_csr_kernel(
-    const double *__restrict__ val, const int *__restrict__ col, const int64_t *__restrict__ row_ptr, int64_t n,
-    const double *__restrict__ sd_x, const double *__restrict__ w, int m, const double *__restrict__ sd_w,
-    KernelParam kp, double *__restrict__ out, const int *__restrict__ out_slots, int64_t ldo, unsigned i_blocks) {
+    const double *__restrict__ val, const int *__restrict__ col, const int64_t *__restrict__ row_ptr,
+    const int *__restrict__ x_idx, int64_t n, const double *__restrict__ sd_x, const double *__restrict__ w, int m,
+    const double *__restrict__ sd_w, KernelParam kp, double *__restrict__ out, const int *__restrict__ out_slots,
+    int64_t ldo, unsigned i_blocks) {
     __shared__ uint64_t exp_tab[32];
     const int tid = threadIdx.x;
     if (tid < 32) exp_tab[tid] = TSVM_EXP2F_TAB[tid];
@@ -200,7 +205,8 @@ __global__ __launch_bounds__(256) void get_rows_csr_kernel(
         acc[jj] = 0.0;
         const int64_t j = j0 + jj;
         if (j < n) {
-            const int64_t e0 = row_ptr[j], e1 = row_ptr[j + 1];
+            const int64_t rj = x_idx ? (int64_t) x_idx[j] : j;
+            const int64_t e0 = row_ptr[rj], e1 = row_ptr[rj + 1];
             double s = 0.0;
             for (int64_t e = e0; e < e1; ++e) {
                 const double v = val[e];
@@ -216,7 +222,7 @@ __global__ __launch_bounds__(256) void get_rows_csr_kernel(
 #pragma unroll
     for (int jj = 0; jj < CS_JB; ++jj) {
         const int64_t j = j0 + jj;
-        if (j < n) orow[j] = tsvm_epilogue(acc[jj], sdi, sd_x ? sd_x[j] : 0.0, kp, exp_tab);
+        if (j < n) orow[j] = tsvm_epilogue(acc[jj], sdi, sd_x ? sd_x[x_idx ? (int64_t) x_idx[j] : j] : 0.0, kp, exp_tab);
     }
 }
 
@@ -406,7 +412,7 @@ int tsvm_csr_to_dense(const double *val, const int *col, const int64_t *row_ptr,
     return 0;
 }
 
-int tsvm_get_rows_dense(const double *x, int64_t ldx, int64_t n, int d, const double *sd_x, const double *a,
+int tsvm_get_rows_dense(const double *x, int64_t ldx, const int *x_idx, int64_t n, int d, const double *sd_x, const double *a,
                         int64_t lda, const int *a_idx, int m, const double *sd_a, int kernel_type, double gamma,
                         double coef0, int degree, double *out, const int *out_slots, int64_t ldo, tsvm_stream stream) {
     TSVM_REQUIRE(x && a && out, "tsvm_get_rows_dense: null pointer");
@@ -430,10 +436,10 @@ int tsvm_get_rows_dense(const double *x, int64_t ldx, int64_t n, int d, const do
 #define GR_LAUNCH(KTYPE)                                                                                              \
     do {                                                                                                              \
         if (ti == 2)                                                                                                  \
-            hipLaunchKernelGGL((get_rows_dense_kernel<KTYPE, 2>), grid, block, 0, tsvm_s(stream), x, ldx, n, d, sd_x, a, \
+            hipLaunchKernelGGL((get_rows_dense_kernel<KTYPE, 2>), grid, block, 0, tsvm_s(stream), x, ldx, x_idx, n, d, sd_x, a, \
                                lda, a_idx, m, sd_a, kp, out, out_slots, ldo, m_blocks);                               \
         else                                                                                                          \
-            hipLaunchKernelGGL((get_rows_dense_kernel<KTYPE, 4>), grid, block, 0, tsvm_s(stream), x, ldx, n, d, sd_x, a, \
+            hipLaunchKernelGGL((get_rows_dense_kernel<KTYPE, 4>), grid, block, 0, tsvm_s(stream), x, ldx, x_idx, n, d, sd_x, a, \
                                lda, a_idx, m, sd_a, kp, out, out_slots, ldo, m_blocks);                               \
     } while (0)
     switch (kernel_type) {
@@ -459,7 +465,7 @@ int tsvm_csr_stage_rows(const double *val, const int *col, const int64_t *row_pt
     return 0;
 }
 
-int tsvm_get_rows_csr(const double *val, const int *col, const int64_t *row_ptr, int64_t n, const double *sd_x,
+int tsvm_get_rows_csr(const double *val, const int *col, const int64_t *row_ptr, const int *x_idx, int64_t n, const double *sd_x,
                       const double *w, int m, const double *sd_w, int kernel_type, double gamma, double coef0,
                       int degree, double *out, const int *out_slots, int64_t ldo, tsvm_stream stream) {
     TSVM_REQUIRE(row_ptr && w && out, "tsvm_get_rows_csr: null pointer");
@@ -473,7 +479,7 @@ int tsvm_get_rows_csr(const double *val, const int *col, const int64_t *row_ptr,
     const int64_t j_blocks = (n + CS_JB - 1) / CS_JB;
     TSVM_REQUIRE(j_blocks * i_blocks < (int64_t) 0x7fffffff, "tsvm_get_rows_csr: grid too large");
     hipLaunchKernelGGL(get_rows_csr_kernel, dim3((unsigned) (j_blocks * i_blocks)), dim3(256), 0, tsvm_s(stream), val, col,
-                       row_ptr, n, sd_x, w, m, sd_w, kp, out, out_slots, ldo, i_blocks);
+                       row_ptr, x_idx, n, sd_x, w, m, sd_w, kp, out, out_slots, ldo, i_blocks);
     TSVM_LAUNCH_CHECK();
     return 0;
 }

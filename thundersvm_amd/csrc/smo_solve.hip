@@ -70,6 +70,9 @@ __global__ __launch_bounds__(SV_T) void c_smo_solve_kernel(
     __shared__ double sA_v[SV_W], sA_l[SV_W], sB_v[SV_W];
     __shared__ int sA_i[SV_W], sB_i[SV_W];
 
+    // This workgroup is a chain of dependent operations; when a chip-wide kernel runs next to it on
+    // another stream its wavefronts must not wait behind that kernel's for issue slots.
+    __builtin_amdgcn_s_setprio(3);
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     double f[E], a[E], a_old[E], y[E], kd[E], kI[E];
@@ -199,6 +202,7 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
     __shared__ double sA_vp[SV_W], sA_vn[SV_W], sA_lp[SV_W], sA_ln[SV_W], sB_vp[SV_W], sB_vn[SV_W];
     __shared__ int sA_ip[SV_W], sA_in[SV_W], sB_ip[SV_W], sB_in[SV_W];
 
+    __builtin_amdgcn_s_setprio(3);
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     double f[E], a[E], a_old[E], y[E], kd[E], kIp[E], kIn[E];
@@ -331,6 +335,16 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
     }
 }
 
+// The solver workgroup asks for the rest of the CU's 160 KB of LDS as (unused) dynamic shared memory:
+// no other workgroup can then be placed on its CU, so a kernel running concurrently on another
+// stream cannot take issue slots, LDS bandwidth or L1 space away from the latency-bound solver.
+template <typename K>
+static hipError_t reserve_cu(K kernel, size_t static_lds, size_t *dyn) {
+    const size_t cu_lds = 160 * 1024;
+    *dyn = cu_lds > static_lds + 1024 ? cu_lds - static_lds - 1024 : 0;
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int) *dyn);
+}
+
 extern "C" {
 
 static int solver_ldk(int ws_size) { return ws_size <= SV_T ? SV_T : (ws_size <= 2 * SV_T ? 2 * SV_T : 4 * SV_T); }
@@ -348,11 +362,20 @@ static int launch_gather(const double *k_rows, const int *slots, int64_t ld, con
     return 0;
 }
 
+#define TSVM_LAUNCH_SOLVER(KERNEL, EVAL, ...)                                                       \
+    do {                                                                                            \
+        hipFuncAttributes fa_;                                                                      \
+        TSVM_HIP(hipFuncGetAttributes(&fa_, reinterpret_cast<const void *>(KERNEL<EVAL>)));         \
+        size_t dyn_ = 0;                                                                            \
+        TSVM_HIP(reserve_cu(KERNEL<EVAL>, fa_.sharedSizeBytes, &dyn_));                              \
+        hipLaunchKernelGGL(KERNEL<EVAL>, dim3(1), dim3(SV_T), dyn_, s, __VA_ARGS__);                 \
+    } while (0)
+
 #define TSVM_DISPATCH_E(KERNEL, ...)                                                            \
     do {                                                                                        \
-        if (ws_size <= SV_T) hipLaunchKernelGGL(KERNEL<1>, dim3(1), dim3(SV_T), 0, s, __VA_ARGS__);      \
-        else if (ws_size <= 2 * SV_T) hipLaunchKernelGGL(KERNEL<2>, dim3(1), dim3(SV_T), 0, s, __VA_ARGS__); \
-        else hipLaunchKernelGGL(KERNEL<4>, dim3(1), dim3(SV_T), 0, s, __VA_ARGS__);                      \
+        if (ws_size <= SV_T) TSVM_LAUNCH_SOLVER(KERNEL, 1, __VA_ARGS__);                        \
+        else if (ws_size <= 2 * SV_T) TSVM_LAUNCH_SOLVER(KERNEL, 2, __VA_ARGS__);               \
+        else TSVM_LAUNCH_SOLVER(KERNEL, 4, __VA_ARGS__);                                        \
     } while (0)
 
 int tsvm_c_smo_solve(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
@@ -367,6 +390,32 @@ int tsvm_c_smo_solve(const int *y, const double *f_val, double *alpha, double *a
     if (rc) return rc;
     const double *kws = (const double *) workspace;
     TSVM_DISPATCH_E(c_smo_solve_kernel, y, f_val, alpha, alpha_diff, working_set, ws_size, Cp, Cn, kws, k_diag, eps, diff,
+                    max_iter);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+int tsvm_smo_solve_block_ld(int ws_size) { return ws_size < 1 ? 0 : solver_ldk(ws_size); }
+
+int tsvm_c_smo_solve_block(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
+                           int ws_size, double Cp, double Cn, const double *kws, const double *k_diag, double eps,
+                           double *diff, int max_iter, tsvm_stream stream) {
+    TSVM_REQUIRE(y && f_val && alpha && alpha_diff && working_set && kws && k_diag && diff, "tsvm_c_smo_solve_block: null pointer");
+    TSVM_REQUIRE(ws_size >= 1 && ws_size <= MAX_WS, "tsvm_c_smo_solve_block: ws_size %d outside [1, %d]", ws_size, MAX_WS);
+    hipStream_t s = tsvm_s(stream);
+    TSVM_DISPATCH_E(c_smo_solve_kernel, y, f_val, alpha, alpha_diff, working_set, ws_size, Cp, Cn, kws, k_diag, eps, diff,
+                    max_iter);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+int tsvm_nu_smo_solve_block(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
+                            int ws_size, double C, const double *kws, const double *k_diag, double eps, double *diff,
+                            int max_iter, tsvm_stream stream) {
+    TSVM_REQUIRE(y && f_val && alpha && alpha_diff && working_set && kws && k_diag && diff, "tsvm_nu_smo_solve_block: null pointer");
+    TSVM_REQUIRE(ws_size >= 1 && ws_size <= MAX_WS, "tsvm_nu_smo_solve_block: ws_size %d outside [1, %d]", ws_size, MAX_WS);
+    hipStream_t s = tsvm_s(stream);
+    TSVM_DISPATCH_E(nu_smo_solve_kernel, y, f_val, alpha, alpha_diff, working_set, ws_size, C, kws, k_diag, eps, diff,
                     max_iter);
     TSVM_LAUNCH_CHECK();
     return 0;

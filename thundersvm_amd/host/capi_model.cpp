@@ -198,6 +198,8 @@ int tsvm_model_stats(void *model, int k, int64_t *n_iter, int64_t *local_iter, d
             phase_ms[5] = (double) s.cache_hits;
             phase_ms[6] = (double) s.cache_rows;
             phase_ms[7] = s.cache_disabled ? 1.0 : 0.0;
+            phase_ms[8] = s.ms_wall;
+            phase_ms[9] = s.ms_setup;
         }
     })
 }

@@ -37,8 +37,7 @@ size_t &device_bytes_in_use();   // running total of DeviceBuffer allocations (t
 class RowArena {
 public:
     static RowArena &instance();
-    // bytes a solve may use when the caller gave no explicit budget: the arena's size once it exists,
-    // otherwise half of the free device memory
+    // bytes a solve may use when the caller gave no explicit budget: half of what is free or already held
     size_t auto_budget();
     void *acquire(size_t bytes, bool auto_sized);
     void release();
@@ -47,6 +46,7 @@ public:
 private:
     void *ptr_ = nullptr;
     size_t cap_ = 0;
+    bool full_budget_ = false;
 };
 
 template <typename T>

@@ -1,6 +1,8 @@
 #include "kernelmatrix.h"
 
 #include <algorithm>
+#include <cstdio>
+#include <cstdlib>
 
 using tsvm::abi_check;
 
@@ -16,19 +18,36 @@ RowArena &RowArena::instance() {
 }
 
 size_t RowArena::auto_budget() {
-    if (cap_) return cap_;
+    if (full_budget_) return cap_;   // the arena already is the budget: never chase small changes in free memory
     size_t free_b = 0, total_b = 0;
     TSVM_HIP_CHECK(hipMemGetInfo(&free_b, &total_b));
-    return free_b / 2;
+    return (free_b + cap_) / 2;   // what the arena already holds counts as available to it
 }
 
+// The arena only ever grows.  Small requests (tests, small problems) get twice what they ask for, so
+// that little is held and little has to be scrubbed by the driver when the process ends (giving back
+// ~140 GB was measured to stall the next process on the device for 2-3 s).  A request above a quarter
+// of the automatic budget takes the whole budget at once: a multi-class run then allocates a single
+// time instead of releasing and re-allocating tens of gigabytes between its sub-problems, each release
+// costing up to a second.
 void *RowArena::acquire(size_t bytes, bool auto_sized) {
     if (bytes <= cap_) return ptr_;
     size_t want = bytes;
-    if (auto_sized) want = std::max(want, auto_budget());   // take the whole automatic budget once
+    bool take_all = false;
+    if (auto_sized) {
+        const size_t budget = auto_budget();
+        take_all = bytes > budget / 4;
+        want = take_all ? std::max(bytes, budget) : std::max(bytes * 2, cap_ + cap_ / 2);
+    }
     release();
     TSVM_HIP_CHECK(hipMalloc(&ptr_, want));
     cap_ = want;
+    full_budget_ = take_all;
+    static bool registered = false;
+    if (!registered) {
+        registered = true;
+        atexit([] { RowArena::instance().release(); });
+    }
     return ptr_;
 }
 
@@ -36,6 +55,7 @@ void RowArena::release() {
     if (ptr_) (void) hipFree(ptr_);
     ptr_ = nullptr;
     cap_ = 0;
+    full_budget_ = false;
 }
 }  // namespace tsvm
 
@@ -110,22 +130,42 @@ void KernelMatrix::build(const DataSet::node2d &all, const int *rows, size_t n_r
     }
 }
 
-void KernelMatrix::get_rows(const int *d_idx, int m, kernel_type *d_out, int64_t ld, const int *d_out_slots) const {
+void KernelMatrix::get_rows(const int *d_idx, int m, kernel_type *d_out, int64_t ld, const int *d_out_slots,
+                            hipStream_t stream) const {
     const int n = (int) n_instances_;
     if (dense_) {
-        abi_check(tsvm_get_rows_dense(x_.data(), ld_, n, (int) n_features_, self_dot_.data(), x_.data(), ld_, d_idx, m,
-                                      self_dot_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
-                                      d_out, d_out_slots, ld, nullptr));
+        abi_check(tsvm_get_rows_dense(x_.data(), ld_, nullptr, n, (int) n_features_, self_dot_.data(), x_.data(), ld_, d_idx,
+                                      m, self_dot_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
+                                      d_out, d_out_slots, ld, stream));
         return;
     }
     if (stage_.size() < (size_t) m * n_features_) stage_.resize((size_t) m * n_features_);
     if (stage_sd_.size() < (size_t) m) stage_sd_.resize(m);
     abi_check(tsvm_csr_stage_rows(val_.data(), col_ind_.data(), row_ptr_.data(), d_idx, m, (int) n_features_,
-                                  stage_.data(), nullptr));
-    abi_check(tsvm_gather_f64(self_dot_.data(), d_idx, m, stage_sd_.data(), nullptr));
-    abi_check(tsvm_get_rows_csr(val_.data(), col_ind_.data(), row_ptr_.data(), n, self_dot_.data(), stage_.data(), m,
-                                stage_sd_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree, d_out,
-                                d_out_slots, ld, nullptr));
+                                  stage_.data(), stream));
+    abi_check(tsvm_gather_f64(self_dot_.data(), d_idx, m, stage_sd_.data(), stream));
+    abi_check(tsvm_get_rows_csr(val_.data(), col_ind_.data(), row_ptr_.data(), nullptr, n, self_dot_.data(), stage_.data(),
+                                m, stage_sd_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree, d_out,
+                                d_out_slots, ld, stream));
+}
+
+// K(x_idx[r], x_idx[t]) for r, t < m: the same kernels with the column set restricted to the m rows,
+// so every value is bit-identical to the corresponding entry of a full kernel row.
+void KernelMatrix::get_block(const int *d_idx, int m, kernel_type *d_out, int64_t ld, hipStream_t stream) const {
+    if (dense_) {
+        abi_check(tsvm_get_rows_dense(x_.data(), ld_, d_idx, m, (int) n_features_, self_dot_.data(), x_.data(), ld_, d_idx, m,
+                                      self_dot_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
+                                      d_out, nullptr, ld, stream));
+        return;
+    }
+    if (stage_blk_.size() < (size_t) m * n_features_) stage_blk_.resize((size_t) m * n_features_);
+    if (stage_blk_sd_.size() < (size_t) m) stage_blk_sd_.resize(m);
+    abi_check(tsvm_csr_stage_rows(val_.data(), col_ind_.data(), row_ptr_.data(), d_idx, m, (int) n_features_,
+                                  stage_blk_.data(), stream));
+    abi_check(tsvm_gather_f64(self_dot_.data(), d_idx, m, stage_blk_sd_.data(), stream));
+    abi_check(tsvm_get_rows_csr(val_.data(), col_ind_.data(), row_ptr_.data(), d_idx, m, self_dot_.data(), stage_blk_.data(),
+                                m, stage_blk_sd_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
+                                d_out, nullptr, ld, stream));
 }
 
 // External batch (kernelmatrix.cpp:281-312, 385-406): features with id >= n_features_ are left out of
@@ -155,14 +195,14 @@ void KernelMatrix::get_rows(const DataSet::node2d &instances, kernel_type *d_out
         if (stage_.size() < (size_t) m * ld_) stage_.resize((size_t) m * ld_);
         // columns >= n_features_ are dropped: the staging matrix is only n_features_ wide
         abi_check(tsvm_csr_to_dense(b_val_.data(), b_col_.data(), b_ptr_.data(), m, stage_.data(), ld_, nullptr));
-        abi_check(tsvm_get_rows_dense(x_.data(), ld_, n, (int) n_features_, self_dot_.data(), stage_.data(), ld_, nullptr, m,
+        abi_check(tsvm_get_rows_dense(x_.data(), ld_, nullptr, n, (int) n_features_, self_dot_.data(), stage_.data(), ld_, nullptr, m,
                                       stage_sd_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
                                       d_out, nullptr, ld, nullptr));
     } else {
         if (stage_.size() < (size_t) m * n_features_) stage_.resize((size_t) m * n_features_);
         abi_check(tsvm_csr_stage_rows(b_val_.data(), b_col_.data(), b_ptr_.data(), nullptr, m, (int) n_features_,
                                       stage_.data(), nullptr));
-        abi_check(tsvm_get_rows_csr(val_.data(), col_ind_.data(), row_ptr_.data(), n, self_dot_.data(), stage_.data(), m,
+        abi_check(tsvm_get_rows_csr(val_.data(), col_ind_.data(), row_ptr_.data(), nullptr, n, self_dot_.data(), stage_.data(), m,
                                     stage_sd_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
                                     d_out, nullptr, ld, nullptr));
     }

@@ -17,7 +17,10 @@ public:
     KernelMatrix(const DataSet::node2d &all, const int *rows, size_t n_rows, SvmParam param, int repeat = 1);
 
     // kernel rows of stored instances d_idx[0..m) (device ids) -> d_out[s_i*ld + j], s_i = d_out_slots[i] (or i)
-    void get_rows(const int *d_idx, int m, kernel_type *d_out, int64_t ld, const int *d_out_slots = nullptr) const;
+    void get_rows(const int *d_idx, int m, kernel_type *d_out, int64_t ld, const int *d_out_slots = nullptr,
+                  hipStream_t stream = nullptr) const;
+    // the m x m block K(x_idx[r], x_idx[t]) -> d_out[r*ld + t] (what the local solver reads)
+    void get_block(const int *d_idx, int m, kernel_type *d_out, int64_t ld, hipStream_t stream = nullptr) const;
     // kernel rows of an external batch -> d_out[i*ld + j]
     void get_rows(const DataSet::node2d &instances, kernel_type *d_out, int64_t ld) const;
 
@@ -46,6 +49,7 @@ private:
     tsvm::DeviceBuffer<kernel_type> diag_;
     // reusable staging for the sparse path and for external batches
     mutable tsvm::DeviceBuffer<kernel_type> stage_;
+    mutable tsvm::DeviceBuffer<kernel_type> stage_blk_, stage_blk_sd_;   // staging of get_block (its own stream)
     mutable tsvm::DeviceBuffer<kernel_type> stage_sd_;
     mutable tsvm::DeviceBuffer<kernel_type> b_val_;
     mutable tsvm::DeviceBuffer<int> b_col_;

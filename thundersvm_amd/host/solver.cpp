@@ -1,5 +1,6 @@
 #include "solver.h"
 
+#include <chrono>
 #include <climits>
 #include <cmath>
 #include <algorithm>
@@ -67,10 +68,11 @@ struct PhaseTimer {
         if (on) { TSVM_HIP_CHECK(hipEventCreate(&e0)); TSVM_HIP_CHECK(hipEventCreate(&e1)); }
     }
     ~PhaseTimer() { if (on) { (void) hipEventDestroy(e0); (void) hipEventDestroy(e1); } }
-    void begin() { if (on) TSVM_HIP_CHECK(hipEventRecord(e0, nullptr)); }
+    hipStream_t stream = nullptr;
+    void begin() { if (on) TSVM_HIP_CHECK(hipEventRecord(e0, stream)); }
     void end(double &acc) {
         if (!on) return;
-        TSVM_HIP_CHECK(hipEventRecord(e1, nullptr));
+        TSVM_HIP_CHECK(hipEventRecord(e1, stream));
         TSVM_HIP_CHECK(hipEventSynchronize(e1));
         float ms = 0;
         TSVM_HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
@@ -88,16 +90,43 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
     const int64_t ld = ((int64_t) n + 1) / 2 * 2;   // even row stride keeps every kernel row 16-byte aligned
     const bool nu = is_nu();
     stats = SolverStats();
+    const auto wall0 = std::chrono::steady_clock::now();
 
     DeviceBuffer<int> d_y(n), d_ws(ws_size), d_slots_a(ws_size), d_slots_b(ws_size), d_miss_ids(ws_size), d_miss_slots(ws_size);
     DeviceBuffer<float_type> d_alpha(n), d_f(n), d_alpha_diff(ws_size), d_diff(2);
     DeviceBuffer<unsigned char> d_sel_ws(tsvm_select_workspace(n));
-    DeviceBuffer<unsigned char> d_smo_ws(tsvm_smo_solve_workspace(ws_size));
+    const int ldk = tsvm_smo_solve_block_ld(ws_size);
+    DeviceBuffer<kernel_type> d_kws((size_t) ws_size * ldk);
     d_y.upload(y.data(), n);
     d_alpha.upload(alpha.data(), n);
     d_f.upload(f_val.data(), n);
     d_diff.zero();
     d_alpha_diff.zero();
+    d_kws.zero();
+
+    // The local solver needs only the ws x ws block of the kernel matrix, which is computed first by a
+    // small launch; the full rows of the new working-set members are needed by update_f only.  With
+    // overlap_streams the solver runs on stream `sa` while get_rows runs on stream `sb` and update_f
+    // waits for both; by default (and always when profiling) everything is enqueued on one stream.
+    struct Streams {
+        hipStream_t a = nullptr, b = nullptr;
+        hipEvent_t selected = nullptr, rows_ready = nullptr;
+        bool two;
+        explicit Streams(bool two_streams) : two(two_streams) {
+            TSVM_HIP_CHECK(hipStreamCreateWithFlags(&a, hipStreamNonBlocking));
+            if (two) TSVM_HIP_CHECK(hipStreamCreateWithFlags(&b, hipStreamNonBlocking)); else b = a;
+            TSVM_HIP_CHECK(hipEventCreateWithFlags(&selected, hipEventDisableTiming));
+            TSVM_HIP_CHECK(hipEventCreateWithFlags(&rows_ready, hipEventDisableTiming));
+        }
+        ~Streams() {
+            (void) hipStreamSynchronize(a);
+            if (two) { (void) hipStreamSynchronize(b); (void) hipStreamDestroy(b); }
+            (void) hipStreamDestroy(a);
+            (void) hipEventDestroy(selected);
+            (void) hipEventDestroy(rows_ready);
+        }
+    } st(overlap_streams && !profile);
+    const hipStream_t sa = st.a, sb = st.b;
 
     // Kernel rows live in slots of one pool.  With a cache the pool holds up to pool_rows rows and the
     // host tracks which instance sits in which slot; without one it holds exactly ws rows.
@@ -140,37 +169,56 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
     }
 
     init_f(alpha, y, k_mat, d_f.data());
+    TSVM_HIP_CHECK(hipDeviceSynchronize());   // uploads, fills and init_f ran on the default stream
 
     const int max_iter = std::max(100000, ws_size > INT_MAX / 100 ? INT_MAX : 100 * ws_size);
     long long local_iter = 0;
     int same_local_diff_cnt = 0, swap_local_diff_cnt = 0;
     float_type previous_local_diff = INFINITY, last_local_diff = INFINITY, second_last_local_diff = INFINITY;
     PhaseTimer timer(profile);
+    timer.stream = sa;
     if (trace) {
         trace->ws_size = ws_size;
         trace->diff.clear();
         trace->ws.clear();
     }
 
+    stats.ms_setup = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - wall0).count();
     for (int iter = 0;; ++iter) {
         const int n_new = iter == 0 ? ws_size : q;
         const int first_new = iter == 0 ? 0 : q;
         timer.begin();
         if (iter == 0) {
             abi_check(tsvm_select_working_set(d_f.data(), d_y.data(), d_alpha.data(), n, Cp, Cn, nullptr, 0, d_ws.data(),
-                                              ws_size, nu, d_sel_ws.data(), nullptr));
+                                              ws_size, nu, d_sel_ws.data(), sa));
         } else {
-            TSVM_HIP_CHECK(hipMemcpyAsync(d_ws.data(), d_ws.data() + q, sizeof(int) * q, hipMemcpyDeviceToDevice, nullptr));
+            TSVM_HIP_CHECK(hipMemcpyAsync(d_ws.data(), d_ws.data() + q, sizeof(int) * q, hipMemcpyDeviceToDevice, sa));
             abi_check(tsvm_select_working_set(d_f.data(), d_y.data(), d_alpha.data(), n, Cp, Cn, d_ws.data(), q,
-                                              d_ws.data() + q, q, nu, d_sel_ws.data(), nullptr));
+                                              d_ws.data() + q, q, nu, d_sel_ws.data(), sa));
         }
         timer.end(stats.ms_select);
-        timer.begin();
         const int *slots;
         if (caching) {
             // read the new ids back, look them up, and compute only the rows that are not cached
-            TSVM_HIP_CHECK(hipMemcpyAsync(h_ids, d_ws.data() + first_new, sizeof(int) * n_new, hipMemcpyDeviceToHost, nullptr));
-            TSVM_HIP_CHECK(hipStreamSynchronize(nullptr));
+            TSVM_HIP_CHECK(hipMemcpyAsync(h_ids, d_ws.data() + first_new, sizeof(int) * n_new, hipMemcpyDeviceToHost, sa));
+            TSVM_HIP_CHECK(hipStreamSynchronize(sa));
+        } else {
+            TSVM_HIP_CHECK(hipEventRecord(st.selected, sa));
+        }
+        // the solver's ws x ws block and the solver itself go first on stream a ...
+        timer.begin();
+        k_mat.get_block(d_ws.data(), ws_size, d_kws.data(), ldk, sa);
+        if (nu) {
+            abi_check(tsvm_nu_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), d_ws.data(), ws_size,
+                                              Cp, d_kws.data(), k_mat.diag(), eps, d_diff.data(), max_iter, sa));
+        } else {
+            abi_check(tsvm_c_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), d_ws.data(), ws_size,
+                                             Cp, Cn, d_kws.data(), k_mat.diag(), eps, d_diff.data(), max_iter, sa));
+        }
+        timer.end(stats.ms_local);
+        // ... while the full rows of the new working-set members are produced on stream b
+        timer.begin();
+        if (caching) {
             if (iter > 0) {
                 for (int t = 0; t < q; ++t) {   // rows kept from the previous working set stay most recently used
                     cur_ids[t] = cur_ids[t + q];
@@ -198,11 +246,11 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
             std::copy(miss_ids.begin(), miss_ids.end(), h_miss_ids);
             std::copy(miss_slots.begin(), miss_slots.end(), h_miss_slots);
             const int n_miss = (int) miss_ids.size();
-            TSVM_HIP_CHECK(hipMemcpyAsync(d_slots_a.data(), h_slots, sizeof(int) * ws_size, hipMemcpyHostToDevice, nullptr));
+            TSVM_HIP_CHECK(hipMemcpyAsync(d_slots_a.data(), h_slots, sizeof(int) * ws_size, hipMemcpyHostToDevice, sb));
             if (n_miss) {
-                TSVM_HIP_CHECK(hipMemcpyAsync(d_miss_ids.data(), h_miss_ids, sizeof(int) * n_miss, hipMemcpyHostToDevice, nullptr));
-                TSVM_HIP_CHECK(hipMemcpyAsync(d_miss_slots.data(), h_miss_slots, sizeof(int) * n_miss, hipMemcpyHostToDevice, nullptr));
-                k_mat.get_rows(d_miss_ids.data(), n_miss, k_rows, ld, d_miss_slots.data());
+                TSVM_HIP_CHECK(hipMemcpyAsync(d_miss_ids.data(), h_miss_ids, sizeof(int) * n_miss, hipMemcpyHostToDevice, sb));
+                TSVM_HIP_CHECK(hipMemcpyAsync(d_miss_slots.data(), h_miss_slots, sizeof(int) * n_miss, hipMemcpyHostToDevice, sb));
+                k_mat.get_rows(d_miss_ids.data(), n_miss, k_rows, ld, d_miss_slots.data(), sb);
             }
             slots = d_slots_a.data();
             // A cache that has started evicting and still does not hit only costs the id read-back:
@@ -211,6 +259,7 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
             if (cache.cap < n && cache.used == cache.cap && iter % 64 == 63) {
                 const long long dl = stats.cache_lookups - window_lookups, dh = stats.cache_hits - window_hits;
                 if (dh * 20 < dl) {
+                    TSVM_HIP_CHECK(hipStreamSynchronize(sb));
                     caching = false;
                     stats.cache_disabled = true;
                     upload_rotation(cur_slots);
@@ -221,26 +270,20 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
         } else {
             const bool on_a = ((iter - rotation_base) % 2) == 0;
             slots = on_a ? d_slots_a.data() : d_slots_b.data();
+            if (st.two) TSVM_HIP_CHECK(hipStreamWaitEvent(sb, st.selected, 0));
             // new rows go to the slots the dropped rows occupied
-            k_mat.get_rows(d_ws.data() + first_new, n_new, k_rows, ld, slots + first_new);
+            k_mat.get_rows(d_ws.data() + first_new, n_new, k_rows, ld, slots + first_new, sb);
+        }
+        if (st.two) {
+            TSVM_HIP_CHECK(hipEventRecord(st.rows_ready, sb));
+            TSVM_HIP_CHECK(hipStreamWaitEvent(sa, st.rows_ready, 0));
         }
         timer.end(stats.ms_get_rows);
         timer.begin();
-        if (nu) {
-            abi_check(tsvm_nu_smo_solve(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), d_ws.data(), ws_size, Cp,
-                                        k_rows, slots, ld, k_mat.diag(), eps, d_diff.data(), max_iter,
-                                        d_smo_ws.data(), nullptr));
-        } else {
-            abi_check(tsvm_c_smo_solve(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), d_ws.data(), ws_size, Cp,
-                                       Cn, k_rows, slots, ld, k_mat.diag(), eps, d_diff.data(), max_iter,
-                                       d_smo_ws.data(), nullptr));
-        }
-        timer.end(stats.ms_local);
-        timer.begin();
-        abi_check(tsvm_update_f(d_f.data(), d_alpha_diff.data(), ws_size, k_rows, slots, ld, n, nullptr));
+        abi_check(tsvm_update_f(d_f.data(), d_alpha_diff.data(), ws_size, k_rows, slots, ld, n, sa));
         timer.end(stats.ms_update_f);
-        TSVM_HIP_CHECK(hipMemcpyAsync(h_diff, d_diff.data(), 2 * sizeof(double), hipMemcpyDeviceToHost, nullptr));
-        TSVM_HIP_CHECK(hipStreamSynchronize(nullptr));
+        TSVM_HIP_CHECK(hipMemcpyAsync(h_diff, d_diff.data(), 2 * sizeof(double), hipMemcpyDeviceToHost, sa));
+        TSVM_HIP_CHECK(hipStreamSynchronize(sa));
         const double diff0 = h_diff[0], diff1 = h_diff[1];
         local_iter += (long long) diff1;
         if (trace && iter < trace->cap_iters) {
@@ -276,6 +319,7 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
             break;
         }
     }
+    stats.ms_wall = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - wall0).count();
     (void) hipHostFree(h_diff);
     (void) hipHostFree(h_ids);
     (void) hipHostFree(h_slots);

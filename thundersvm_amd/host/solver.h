@@ -17,6 +17,7 @@ struct SolverStats {
     double obj = 0;
     // accumulated device time per phase in ms (only filled when profile == true)
     double ms_select = 0, ms_get_rows = 0, ms_local = 0, ms_update_f = 0;
+    double ms_wall = 0, ms_setup = 0;   // host wall-clock of the whole solve / of everything before the first iteration
     // kernel-row cache
     long long cache_lookups = 0, cache_hits = 0;
     long long cache_rows = 0;     // capacity in rows (0: cache not used)
@@ -35,6 +36,10 @@ public:
     bool profile = false;
     // Budget of the HBM kernel-row cache in bytes: -1 = half of the free device memory, 0 = no cache.
     long long cache_bytes = -1;
+    // Run the local solver and the chip-wide get_rows concurrently on two streams.  Off by default: the
+    // solver is a chain of dependent loads, and measured next to get_rows each of its iterations takes
+    // 3.6x longer (2.4 ms instead of 0.66 ms per call at n = 800,000), which cancels the overlap.
+    bool overlap_streams = false;
 
 protected:
     virtual bool is_nu() const { return false; }
