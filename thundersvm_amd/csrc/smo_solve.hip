@@ -3,19 +3,25 @@
 //
 // Shape of the kernel.  One workgroup of 256 threads (one wavefront per SIMD of the CU) holds the
 // whole working set: element t = e*256 + tid lives in register slot e of thread tid (E = ws/256
-// slots, up to 4), with its f, alpha, y and diagonal.  One inner iteration is
+// slots, up to 4) with its f and diagonal; alpha lives in LDS (only two entries change per
+// iteration) and the I_up / I_low membership of a thread's elements is a bit field in one register.
+// One inner iteration is
 //   1. (i, up) = first argmin of f over I_up and low = max of f over I_low: a per-thread scan of
 //      its E slots, a DPP reduction inside each wavefront, four partial results through LDS;
 //   2. row K[i, .] of the gathered ws x ws block (coalesced);
 //   3. j2 = first argmin of -b^2/a over I_low with f > up: same reduction shape;
 //   4. the two-variable step, row K[j2, .], f -= l * (K[j2, .] - K[i, .]).
-// Two workgroup barriers per iteration.  The loop body is written with selects instead of branches:
-// with one wavefront per SIMD nothing hides a taken branch (the same loop written with if-blocks
-// measured about 1.3x slower per inner iteration).  Reductions are lexicographic (value, element index)
-// minima, so ties go to the lowest index exactly as the reference's serial loops resolve them, and
-// all arithmetic is the reference's expression order in IEEE double (the library is compiled with
-// -ffp-contract=off; the one fused operation, f -= l*(kJ - kI), is an explicit fma as gcc -O3
-// contracts it on an FMA host).
+// Two workgroup barriers per iteration.  With one wavefront per SIMD nothing hides an instruction's
+// issue slot or a taken branch, so the loop body is bound by its instruction count: it is written
+// with selects instead of branches (the same loop with if-blocks measured about 1.3x slower), with
+// v_min_f64 / v_max_f64 for the value reductions, and with everything that concerns only the two
+// chosen elements (their alpha, their set membership) computed once per thread from LDS rather than
+// per element.  Reductions are lexicographic (value, element index) minima, so ties go to the lowest
+// index exactly as the reference's serial loops resolve them, and all arithmetic is the reference's
+// expression order in IEEE double (the library is compiled with -ffp-contract=off; the one fused
+// operation, f -= l*(kJ - kI), is an explicit fma as gcc -O3 contracts it on an FMA host, and
+// kd_i + kd_t - 2*K_it is written as fma(-2, K_it, kd_i + kd_t), which rounds identically because
+// the product by 2 is exact).
 #include "../../include/thundersvm_amd.h"
 #include "tsvm_device.h"
 #include "tsvm_internal.h"
@@ -40,7 +46,7 @@ __global__ void gather_ws_block_kernel(const double *__restrict__ k_rows, const 
 __device__ __forceinline__ void block_argmin(const double *s_v, const int *s_i, double &v, int &i, int none) {
     double m = s_v[0];
 #pragma unroll
-    for (int w = 1; w < SV_W; ++w) m = fmin_sel(m, s_v[w]);
+    for (int w = 1; w < SV_W; ++w) m = fmin_f64(m, s_v[w]);
     int r = none;
 #pragma unroll
     for (int w = 0; w < SV_W; ++w) r = imin_sel(r, s_v[w] == m ? s_i[w] : none);
@@ -50,8 +56,30 @@ __device__ __forceinline__ void block_argmin(const double *s_v, const int *s_i, 
 __device__ __forceinline__ double block_max(const double *s_v) {
     double v = s_v[0];
 #pragma unroll
-    for (int w = 1; w < SV_W; ++w) v = fmax_sel(v, s_v[w]);
+    for (int w = 1; w < SV_W; ++w) v = fmax_f64(v, s_v[w]);
     return v;
+}
+
+// The wavefront's lexicographic minimum of the candidates x[e] (element index e*256 + tid):
+// value pass, then the smallest element index among those equal to the minimum.
+template <int E>
+__device__ __forceinline__ void wave_first_argmin(const double (&x)[E], int tid, double &v, int &idx) {
+    double m = x[0];
+#pragma unroll
+    for (int e = 1; e < E; ++e) m = fmin_f64(m, x[e]);
+    m = wave_min_f64(m);
+    int r = MAX_WS;
+#pragma unroll
+    for (int e = E - 1; e >= 0; --e) r = x[e] == m ? e * SV_T + tid : r;
+    idx = wave_min_i32(r);
+    v = m;
+}
+
+// Replaces the `width` membership bits of element t in the bit field of the thread that owns it.
+__device__ __forceinline__ unsigned set_member_bits(unsigned m, int tid, int t, unsigned bits, int width) {
+    const int sh = (t / SV_T) * width;
+    const unsigned field = ((1u << width) - 1u) << sh;
+    return tid == (t & (SV_T - 1)) ? ((m & ~field) | (bits << sh)) : m;
 }
 
 // Elements beyond ws are given y = 0, which puts them in neither I_up nor I_low.
@@ -64,9 +92,8 @@ __global__ __launch_bounds__(SV_T) void c_smo_solve_kernel(
     constexpr int LDK = E * SV_T;
     __shared__ double s_kd[LDK];
     __shared__ float s_y[LDK];
-    __shared__ double s_a[2][LDK];
+    __shared__ double s_a[LDK];
     __shared__ double s_f[2][LDK];
-    __shared__ double s_kI[LDK];
     __shared__ double sA_v[SV_W], sA_l[SV_W], sB_v[SV_W];
     __shared__ int sA_i[SV_W], sB_i[SV_W];
 
@@ -75,45 +102,49 @@ __global__ __launch_bounds__(SV_T) void c_smo_solve_kernel(
     __builtin_amdgcn_s_setprio(3);
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    double f[E], a[E], a_old[E], y[E], kd[E], kI[E];
-    bool upm[E], lowm[E];
-    int wsi[E];
+    double f[E], a_old[E], kd[E];
+    unsigned member = 0;   // bit 2e: element e is in I_up; bit 2e+1: in I_low
 #pragma unroll
     for (int e = 0; e < E; ++e) {
         const int t = e * SV_T + tid;
         const bool active = t < ws;
-        wsi[e] = active ? working_set[t] : 0;
-        f[e] = active ? f_val[wsi[e]] : 0.0;
-        a[e] = active ? alpha[wsi[e]] : 0.0;
-        a_old[e] = a[e];
-        y[e] = active ? (double) label[wsi[e]] : 0.0;
-        kd[e] = active ? k_diag[wsi[e]] : 1.0;
+        const int w = active ? working_set[t] : 0;
+        f[e] = active ? f_val[w] : 0.0;
+        a_old[e] = active ? alpha[w] : 0.0;
+        const double y = active ? (double) label[w] : 0.0;
+        kd[e] = active ? k_diag[w] : 1.0;
         s_kd[t] = kd[e];
-        s_y[t] = (float) y[e];
-        upm[e] = is_I_up(a[e], y[e], Cp, Cn);
-        lowm[e] = is_I_low(a[e], y[e], Cp, Cn);
+        s_y[t] = (float) y;
+        s_a[t] = a_old[e];
+        member |= ((is_I_up(a_old[e], y, Cp, Cn) ? 1u : 0u) | (is_I_low(a_old[e], y, Cp, Cn) ? 2u : 0u)) << (2 * e);
     }
+    // The alpha of the two elements changed by an iteration is written to LDS by thread 0 after the
+    // next iteration's first barrier, when no wavefront can still be reading the old values.
+    int pend_i = 0, pend_j = 0;
+    double pend_ai = a_old[0], pend_aj = a_old[0];   // for thread 0 this is s_a[0]: the first write changes nothing
     double local_eps = 0.0;
     int numOfIter = 0;
     while (true) {
         const int par = numOfIter & 1;
         // i = first argmin of f over I_up; low = max of f over I_low (smo_kernel.cpp:41-59)
-        double v = TSVM_INF, lw = -TSVM_INF;
-        int vi = MAX_WS;
+        double fu[E];
+        double lw = -TSVM_INF;
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            const int t = e * SV_T + tid;
-            s_a[par][t] = a[e];
-            s_f[par][t] = f[e];
-            const bool c = upm[e] & (f[e] < v);
-            v = c ? f[e] : v;
-            vi = c ? t : vi;
-            lw = (lowm[e] & (f[e] > lw)) ? f[e] : lw;
+            s_f[par][e * SV_T + tid] = f[e];
+            fu[e] = (member >> (2 * e)) & 1u ? f[e] : TSVM_INF;
+            lw = fmax_f64(lw, (member >> (2 * e + 1)) & 1u ? f[e] : -TSVM_INF);
         }
-        wave_argmin(v, vi, MAX_WS);
+        double v;
+        int vi;
+        wave_first_argmin<E>(fu, tid, v, vi);
         lw = wave_max_f64(lw);
         if (lane == 0) { sA_v[wave] = v; sA_i[wave] = vi; sA_l[wave] = lw; }
         __syncthreads();
+        if (tid == 0) {
+            s_a[pend_i] = pend_ai;
+            s_a[pend_j] = pend_aj;   // after pend_i: if both name one element the second value is the final one
+        }
         double up_value;
         int i;
         block_argmin(sA_v, sA_i, up_value, i, MAX_WS);
@@ -126,60 +157,62 @@ __global__ __launch_bounds__(SV_T) void c_smo_solve_kernel(
             if (tid == 0) diff[0] = local_diff;
         }
         if (numOfIter > max_iter || local_diff < local_eps) break;
-        const double *row_i = kws + (int64_t) i * LDK + tid;
+        const double *row_i = kws + (int64_t) i * LDK;
+        double kI[E];
 #pragma unroll
-        for (int e = 0; e < E; ++e) kI[e] = row_i[e * SV_T];
+        for (int e = 0; e < E; ++e) kI[e] = row_i[e * SV_T + tid];
         const double kd_i = s_kd[i];
         // j2 = first argmin of -b^2/a over I_low with f > up (smo_kernel.cpp:77-90)
-        double ft = TSVM_INF;
-        int fi = MAX_WS;
+        double qs[E];
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            const int t = e * SV_T + tid;
-            s_kI[t] = kI[e];
-            const double aIJ = kd_i + kd[e] - 2 * kI[e];
+            const double aIJ = __builtin_fma(-2.0, kI[e], kd_i + kd[e]);
             const double bIJ = -up_value + f[e];
             const double q = -bIJ * bIJ / aIJ;
-            const bool c = lowm[e] & (-up_value > -f[e]) & (q < ft);
-            ft = c ? q : ft;
-            fi = c ? t : fi;
+            qs[e] = ((member >> (2 * e + 1)) & 1u) && (-up_value > -f[e]) ? q : TSVM_INF;
         }
-        wave_argmin(ft, fi, MAX_WS);
+        double ft;
+        int fi;
+        wave_first_argmin<E>(qs, tid, ft, fi);
         if (lane == 0) { sB_v[wave] = ft; sB_i[wave] = fi; }
         __syncthreads();
         double min_t;
         int j2;
         block_argmin(sB_v, sB_i, min_t, j2, MAX_WS);
         j2 = min_t < TSVM_INF ? j2 : 0;
-        const double *row_j = kws + (int64_t) j2 * LDK + tid;
+        const double *row_j = kws + (int64_t) j2 * LDK;
         double kJ[E];
 #pragma unroll
-        for (int e = 0; e < E; ++e) kJ[e] = row_j[e * SV_T];
+        for (int e = 0; e < E; ++e) kJ[e] = row_j[e * SV_T + tid];
+        const double kIj = row_i[j2];
         // two-variable step (smo_kernel.cpp:92-103)
-        const double a_i = s_a[par][i], y_i = (double) s_y[i];
-        const double a_j = s_a[par][j2], y_j = (double) s_y[j2];
+        const double a_i = s_a[i], y_i = (double) s_y[i];
+        const double a_j0 = s_a[j2], y_j = (double) s_y[j2];
         const double alpha_i_diff = y_i > 0 ? Cp - a_i : a_i;
-        const double q1 = y_j > 0 ? a_j : Cn - a_j;
-        const double q2 = (-up_value + s_f[par][j2]) / (kd_i + s_kd[j2] - 2 * s_kI[j2]);
+        const double q1 = y_j > 0 ? a_j0 : Cn - a_j0;
+        const double q2 = (-up_value + s_f[par][j2]) / (kd_i + s_kd[j2] - 2 * kIj);
         const double alpha_j_diff = q1 < q2 ? q1 : q2;
         const double l = alpha_i_diff < alpha_j_diff ? alpha_i_diff : alpha_j_diff;
+        const double na_i = a_i + l * y_i;
+        const double na_j = (j2 == i ? na_i : a_j0) - l * y_j;
+        member = set_member_bits(member, tid, i, (is_I_up(na_i, y_i, Cp, Cn) ? 1u : 0u) | (is_I_low(na_i, y_i, Cp, Cn) ? 2u : 0u), 2);
+        member = set_member_bits(member, tid, j2, (is_I_up(na_j, y_j, Cp, Cn) ? 1u : 0u) | (is_I_low(na_j, y_j, Cp, Cn) ? 2u : 0u), 2);
+        pend_i = i;
+        pend_j = j2;
+        pend_ai = na_i;
+        pend_aj = na_j;
 #pragma unroll
-        for (int e = 0; e < E; ++e) {
-            const int t = e * SV_T + tid;
-            a[e] = t == i ? a[e] + l * y[e] : a[e];
-            a[e] = t == j2 ? a[e] - l * y[e] : a[e];
-            upm[e] = is_I_up(a[e], y[e], Cp, Cn);
-            lowm[e] = is_I_low(a[e], y[e], Cp, Cn);
-            f[e] = __builtin_fma(-l, kJ[e] - kI[e], f[e]);
-        }
+        for (int e = 0; e < E; ++e) f[e] = __builtin_fma(-l, kJ[e] - kI[e], f[e]);
         ++numOfIter;
     }
+    __syncthreads();   // the pending alpha writes of the last step were made before the loop's exit test
 #pragma unroll
     for (int e = 0; e < E; ++e) {
         const int t = e * SV_T + tid;
         if (t < ws) {
-            alpha_diff[t] = -(a[e] - a_old[e]) * y[e];
-            alpha[wsi[e]] = a[e];
+            const double a = s_a[t];
+            alpha_diff[t] = -(a - a_old[e]) * (double) s_y[t];
+            alpha[working_set[t]] = a;
         }
     }
     if (tid == 0) diff[1] = (double) numOfIter;
@@ -187,6 +220,12 @@ __global__ __launch_bounds__(SV_T) void c_smo_solve_kernel(
 
 // nu variant (smo_kernel.cpp:127-287): four extrema, two second-order candidates.  Keeps the CPU
 // code's j2n score, which uses kd[ip] and K[ip, .] (smo_kernel.cpp:239), and leaves diff[1] alone.
+// Membership bits per element: 0 = y>0 & a<C (I_up, positive), 1 = y<0 & a>0 (I_up, negative),
+// 2 = y>0 & a>0 (I_low, positive), 3 = y<0 & a<C (I_low, negative).
+__device__ __forceinline__ unsigned nu_member_bits(double a, double y, double C) {
+    return (y > 0 && a < C ? 1u : 0u) | (y < 0 && a > 0 ? 2u : 0u) | (y > 0 && a > 0 ? 4u : 0u) | (y < 0 && a < C ? 8u : 0u);
+}
+
 template <int E>
 __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
     const int *__restrict__ label, const double *__restrict__ f_val, double *__restrict__ alpha,
@@ -196,53 +235,51 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
     constexpr int LDK = E * SV_T;
     __shared__ double s_kd[LDK];
     __shared__ float s_y[LDK];
-    __shared__ double s_a[2][LDK];
+    __shared__ double s_a[LDK];
     __shared__ double s_f[2][LDK];
-    __shared__ double s_kIp[LDK], s_kIn[LDK];
     __shared__ double sA_vp[SV_W], sA_vn[SV_W], sA_lp[SV_W], sA_ln[SV_W], sB_vp[SV_W], sB_vn[SV_W];
     __shared__ int sA_ip[SV_W], sA_in[SV_W], sB_ip[SV_W], sB_in[SV_W];
 
     __builtin_amdgcn_s_setprio(3);
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    double f[E], a[E], a_old[E], y[E], kd[E], kIp[E], kIn[E];
-    int wsi[E];
+    double f[E], a_old[E], kd[E];
+    unsigned member = 0;
 #pragma unroll
     for (int e = 0; e < E; ++e) {
         const int t = e * SV_T + tid;
         const bool active = t < ws;
-        wsi[e] = active ? working_set[t] : 0;
-        f[e] = active ? f_val[wsi[e]] : 0.0;
-        a[e] = active ? alpha[wsi[e]] : 0.0;
-        a_old[e] = a[e];
-        y[e] = active ? (double) label[wsi[e]] : 0.0;
-        kd[e] = active ? k_diag[wsi[e]] : 1.0;
+        const int w = active ? working_set[t] : 0;
+        f[e] = active ? f_val[w] : 0.0;
+        a_old[e] = active ? alpha[w] : 0.0;
+        const double y = active ? (double) label[w] : 0.0;
+        kd[e] = active ? k_diag[w] : 1.0;
         s_kd[t] = kd[e];
-        s_y[t] = (float) y[e];
+        s_y[t] = (float) y;
+        s_a[t] = a_old[e];
+        member |= nu_member_bits(a_old[e], y, C) << (4 * e);
     }
+    int pend_i = 0, pend_j = 0;
+    double pend_ai = a_old[0], pend_aj = a_old[0];
     double local_eps = 0.0;
     int numOfIter = 0;
     while (true) {
         const int par = numOfIter & 1;
-        double vp = TSVM_INF, vn = TSVM_INF, lp = -TSVM_INF, ln = -TSVM_INF;
-        int ipi = MAX_WS, ini = MAX_WS;
+        double fup[E], fun[E];
+        double lp = -TSVM_INF, ln = -TSVM_INF;
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            const int t = e * SV_T + tid;
-            s_a[par][t] = a[e];
-            s_f[par][t] = f[e];
-            const bool pos = y[e] > 0, neg = y[e] < 0;
-            const bool cp = pos & (a[e] < C) & (f[e] < vp);
-            vp = cp ? f[e] : vp;
-            ipi = cp ? t : ipi;
-            const bool cn = neg & (a[e] > 0) & (f[e] < vn);
-            vn = cn ? f[e] : vn;
-            ini = cn ? t : ini;
-            lp = (pos & (a[e] > 0) & (f[e] > lp)) ? f[e] : lp;
-            ln = (neg & (a[e] < C) & (f[e] > ln)) ? f[e] : ln;
+            s_f[par][e * SV_T + tid] = f[e];
+            const unsigned b = member >> (4 * e);
+            fup[e] = b & 1u ? f[e] : TSVM_INF;
+            fun[e] = b & 2u ? f[e] : TSVM_INF;
+            lp = fmax_f64(lp, b & 4u ? f[e] : -TSVM_INF);
+            ln = fmax_f64(ln, b & 8u ? f[e] : -TSVM_INF);
         }
-        wave_argmin(vp, ipi, MAX_WS);
-        wave_argmin(vn, ini, MAX_WS);
+        double vp, vn;
+        int ipi, ini;
+        wave_first_argmin<E>(fup, tid, vp, ipi);
+        wave_first_argmin<E>(fun, tid, vn, ini);
         lp = wave_max_f64(lp);
         ln = wave_max_f64(ln);
         if (lane == 0) {
@@ -250,6 +287,10 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
             sA_lp[wave] = lp; sA_ln[wave] = ln;
         }
         __syncthreads();
+        if (tid == 0) {
+            s_a[pend_i] = pend_ai;
+            s_a[pend_j] = pend_aj;
+        }
         double up_value_p, up_value_n;
         int ip, in;
         block_argmin(sA_vp, sA_ip, up_value_p, ip, MAX_WS);
@@ -265,33 +306,28 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
             if (tid == 0) diff[0] = local_diff;
         }
         if (numOfIter > max_iter || local_diff < local_eps) break;
-        const double *row_p = kws + (int64_t) ip * LDK + tid;
-        const double *row_n = kws + (int64_t) in * LDK + tid;
+        const double *row_p = kws + (int64_t) ip * LDK;
+        const double *row_n = kws + (int64_t) in * LDK;
+        double kIp[E], kIn[E];
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            kIp[e] = row_p[e * SV_T];
-            kIn[e] = row_n[e * SV_T];
+            kIp[e] = row_p[e * SV_T + tid];
+            kIn[e] = row_n[e * SV_T + tid];
         }
         const double kd_ip = s_kd[ip];
-        double ftp = TSVM_INF, ftn = TSVM_INF;
-        int jpi = MAX_WS, jni = MAX_WS;
+        double qp[E], qn[E];
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            const int t = e * SV_T + tid;
-            s_kIp[t] = kIp[e];
-            s_kIn[t] = kIn[e];
-            const double aIJ = kd_ip + kd[e] - 2 * kIp[e];
+            const unsigned b = member >> (4 * e);
+            const double aIJ = __builtin_fma(-2.0, kIp[e], kd_ip + kd[e]);
             const double bp = -up_value_p + f[e], bn = -up_value_n + f[e];
-            const double qp = -bp * bp / aIJ, qn = -bn * bn / aIJ;
-            const bool cp = (-up_value_p > -f[e]) & (y[e] > 0) & (a[e] > 0) & (qp < ftp);
-            ftp = cp ? qp : ftp;
-            jpi = cp ? t : jpi;
-            const bool cn = (-up_value_n > -f[e]) & (y[e] < 0) & (a[e] < C) & (qn < ftn);
-            ftn = cn ? qn : ftn;
-            jni = cn ? t : jni;
+            qp[e] = (b & 4u) && (-up_value_p > -f[e]) ? -bp * bp / aIJ : TSVM_INF;
+            qn[e] = (b & 8u) && (-up_value_n > -f[e]) ? -bn * bn / aIJ : TSVM_INF;
         }
-        wave_argmin(ftp, jpi, MAX_WS);
-        wave_argmin(ftn, jni, MAX_WS);
+        double ftp, ftn;
+        int jpi, jni;
+        wave_first_argmin<E>(qp, tid, ftp, jpi);
+        wave_first_argmin<E>(qn, tid, ftn, jni);
         if (lane == 0) { sB_vp[wave] = ftp; sB_ip[wave] = jpi; sB_vn[wave] = ftn; sB_in[wave] = jni; }
         __syncthreads();
         double f_val_j2p, f_val_j2n;
@@ -304,33 +340,39 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
         const int i = take_p ? ip : in;
         const int j2 = take_p ? j2p : j2n;
         const double up_value = take_p ? up_value_p : up_value_n;
-        const double *row_j = kws + (int64_t) j2 * LDK + tid;
+        const double *row_i = take_p ? row_p : row_n;
+        const double *row_j = kws + (int64_t) j2 * LDK;
         double kJ[E];
 #pragma unroll
-        for (int e = 0; e < E; ++e) kJ[e] = row_j[e * SV_T];
-        const double kIj2 = take_p ? s_kIp[j2] : s_kIn[j2];
-        const double a_i = s_a[par][i], y_i = (double) s_y[i];
-        const double a_j = s_a[par][j2], y_j = (double) s_y[j2];
+        for (int e = 0; e < E; ++e) kJ[e] = row_j[e * SV_T + tid];
+        const double kIj = row_i[j2];
+        const double a_i = s_a[i], y_i = (double) s_y[i];
+        const double a_j0 = s_a[j2], y_j = (double) s_y[j2];
         const double alpha_i_diff = y_i > 0 ? C - a_i : a_i;
-        const double q1 = y_j > 0 ? a_j : C - a_j;
-        const double q2 = (-up_value + s_f[par][j2]) / (s_kd[i] + s_kd[j2] - 2 * kIj2);
+        const double q1 = y_j > 0 ? a_j0 : C - a_j0;
+        const double q2 = (-up_value + s_f[par][j2]) / (s_kd[i] + s_kd[j2] - 2 * kIj);
         const double alpha_j_diff = q1 < q2 ? q1 : q2;
         const double l = alpha_i_diff < alpha_j_diff ? alpha_i_diff : alpha_j_diff;
+        const double na_i = a_i + l * y_i;
+        const double na_j = (j2 == i ? na_i : a_j0) - l * y_j;
+        member = set_member_bits(member, tid, i, nu_member_bits(na_i, y_i, C), 4);
+        member = set_member_bits(member, tid, j2, nu_member_bits(na_j, y_j, C), 4);
+        pend_i = i;
+        pend_j = j2;
+        pend_ai = na_i;
+        pend_aj = na_j;
 #pragma unroll
-        for (int e = 0; e < E; ++e) {
-            const int t = e * SV_T + tid;
-            a[e] = t == i ? a[e] + l * y[e] : a[e];
-            a[e] = t == j2 ? a[e] - l * y[e] : a[e];
-            f[e] = __builtin_fma(-l, kJ[e] - (take_p ? kIp[e] : kIn[e]), f[e]);
-        }
+        for (int e = 0; e < E; ++e) f[e] = __builtin_fma(-l, kJ[e] - (take_p ? kIp[e] : kIn[e]), f[e]);
         ++numOfIter;
     }
+    __syncthreads();
 #pragma unroll
     for (int e = 0; e < E; ++e) {
         const int t = e * SV_T + tid;
         if (t < ws) {
-            alpha_diff[t] = -(a[e] - a_old[e]) * y[e];
-            alpha[wsi[e]] = a[e];
+            const double a = s_a[t];
+            alpha_diff[t] = -(a - a_old[e]) * (double) s_y[t];
+            alpha[working_set[t]] = a;
         }
     }
 }

@@ -96,21 +96,27 @@ __device__ __forceinline__ double shfl_xor_f64(double v, int mask) {
     return __hiloint2double(hi, lo);
 }
 
-// Cross-lane moves on the VALU (DPP) instead of the LDS crossbar: quad_perm xor-1 / xor-2,
-// row_half_mirror and row_mirror make every lane of a 16-lane row see the row's result in four
-// steps; the four row results are then read with v_readlane and combined uniformly.
+// Cross-lane moves on the VALU (DPP) instead of the LDS crossbar.  Inside a 16-lane row, quad_perm
+// xor-1 / xor-2, row_half_mirror and row_mirror make every lane see the row's result in four steps;
+// row_bcast:15 into rows 1 and 3, then row_bcast:31 into rows 2 and 3, carry the row results across,
+// so that lane 63 ends up with the wavefront's result, which v_readlane makes uniform.  The full-mask
+// moves name no previous value (old = 0 with bound_ctrl), which lets the compiler fold them into the
+// consuming 32-bit instruction (v_min_i32 ... quad_perm) instead of copying the source first.
 #define TSVM_DPP_XOR1 0xB1          /* quad_perm [1,0,3,2] */
 #define TSVM_DPP_XOR2 0x4E          /* quad_perm [2,3,0,1] */
 #define TSVM_DPP_HALF_MIRROR 0x141
 #define TSVM_DPP_MIRROR 0x140
+#define TSVM_DPP_BCAST15 0x142
+#define TSVM_DPP_BCAST31 0x143
 
-template <int CTRL>
+template <int CTRL, int ROW_MASK = 0xf>
 __device__ __forceinline__ int dpp_i32(int x) {
-    return __builtin_amdgcn_update_dpp(x, x, CTRL, 0xf, 0xf, false);
+    if (ROW_MASK == 0xf) return __builtin_amdgcn_update_dpp(0, x, CTRL, 0xf, 0xf, true);
+    return __builtin_amdgcn_update_dpp(x, x, CTRL, ROW_MASK, 0xf, false);   // rows outside the mask keep x
 }
-template <int CTRL>
+template <int CTRL, int ROW_MASK = 0xf>
 __device__ __forceinline__ double dpp_f64(double v) {
-    int lo = dpp_i32<CTRL>(__double2loint(v)), hi = dpp_i32<CTRL>(__double2hiint(v));
+    int lo = dpp_i32<CTRL, ROW_MASK>(__double2loint(v)), hi = dpp_i32<CTRL, ROW_MASK>(__double2hiint(v));
     return __hiloint2double(hi, lo);
 }
 __device__ __forceinline__ double readlane_f64(double v, int lane) {
@@ -121,42 +127,51 @@ __device__ __forceinline__ double readlane_f64(double v, int lane) {
 // Wavefront reductions used by the local solvers.  A (value, index) lexicographic minimum -- the
 // smallest value wins and, among equal values, the smallest index: the serial loops' "first strict
 // improvement" rule (smo_kernel.cpp:43-49,80-89) -- is taken in two branch-free passes: the minimum
-// value (v_min_f64 over DPP moves), then the minimum index among the lanes that hold that value.
-// Every lane returns the wavefront's result.  Callers never pass NaN.
-__device__ __forceinline__ double fmin_sel(double a, double b) { return b < a ? b : a; }
-__device__ __forceinline__ double fmax_sel(double a, double b) { return b > a ? b : a; }
+// value, then the minimum index among the elements that hold that value.  Every lane returns the
+// wavefront's result.  Callers never pass NaN.
+//
+// v_min_f64 / v_max_f64 are written out because the compiler turns `b < a ? b : a` into a compare
+// and two 32-bit selects, three issue slots instead of one, and the solvers are bound by issue slots.
+// The instructions may return either zero for min(+0, -0); the solvers only compare and subtract
+// these values, where the sign of a zero changes nothing.
+__device__ __forceinline__ double fmin_f64(double a, double b) {
+    double r;
+    asm("v_min_f64 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+__device__ __forceinline__ double fmax_f64(double a, double b) {
+    double r;
+    asm("v_max_f64 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
 __device__ __forceinline__ int imin_sel(int a, int b) { return b < a ? b : a; }
 
 __device__ __forceinline__ double wave_min_f64(double v) {
-    v = fmin_sel(v, dpp_f64<TSVM_DPP_XOR1>(v));
-    v = fmin_sel(v, dpp_f64<TSVM_DPP_XOR2>(v));
-    v = fmin_sel(v, dpp_f64<TSVM_DPP_HALF_MIRROR>(v));
-    v = fmin_sel(v, dpp_f64<TSVM_DPP_MIRROR>(v));
-    const double r0 = readlane_f64(v, 0), r1 = readlane_f64(v, 16), r2 = readlane_f64(v, 32), r3 = readlane_f64(v, 48);
-    return fmin_sel(fmin_sel(r0, r1), fmin_sel(r2, r3));
+    v = fmin_f64(v, dpp_f64<TSVM_DPP_XOR1>(v));
+    v = fmin_f64(v, dpp_f64<TSVM_DPP_XOR2>(v));
+    v = fmin_f64(v, dpp_f64<TSVM_DPP_HALF_MIRROR>(v));
+    v = fmin_f64(v, dpp_f64<TSVM_DPP_MIRROR>(v));
+    v = fmin_f64(v, dpp_f64<TSVM_DPP_BCAST15, 0xa>(v));
+    v = fmin_f64(v, dpp_f64<TSVM_DPP_BCAST31, 0xc>(v));
+    return readlane_f64(v, 63);
 }
 __device__ __forceinline__ double wave_max_f64(double v) {
-    v = fmax_sel(v, dpp_f64<TSVM_DPP_XOR1>(v));
-    v = fmax_sel(v, dpp_f64<TSVM_DPP_XOR2>(v));
-    v = fmax_sel(v, dpp_f64<TSVM_DPP_HALF_MIRROR>(v));
-    v = fmax_sel(v, dpp_f64<TSVM_DPP_MIRROR>(v));
-    const double r0 = readlane_f64(v, 0), r1 = readlane_f64(v, 16), r2 = readlane_f64(v, 32), r3 = readlane_f64(v, 48);
-    return fmax_sel(fmax_sel(r0, r1), fmax_sel(r2, r3));
+    v = fmax_f64(v, dpp_f64<TSVM_DPP_XOR1>(v));
+    v = fmax_f64(v, dpp_f64<TSVM_DPP_XOR2>(v));
+    v = fmax_f64(v, dpp_f64<TSVM_DPP_HALF_MIRROR>(v));
+    v = fmax_f64(v, dpp_f64<TSVM_DPP_MIRROR>(v));
+    v = fmax_f64(v, dpp_f64<TSVM_DPP_BCAST15, 0xa>(v));
+    v = fmax_f64(v, dpp_f64<TSVM_DPP_BCAST31, 0xc>(v));
+    return readlane_f64(v, 63);
 }
 __device__ __forceinline__ int wave_min_i32(int v) {
     v = imin_sel(v, dpp_i32<TSVM_DPP_XOR1>(v));
     v = imin_sel(v, dpp_i32<TSVM_DPP_XOR2>(v));
     v = imin_sel(v, dpp_i32<TSVM_DPP_HALF_MIRROR>(v));
     v = imin_sel(v, dpp_i32<TSVM_DPP_MIRROR>(v));
-    const int r0 = __builtin_amdgcn_readlane(v, 0), r1 = __builtin_amdgcn_readlane(v, 16);
-    const int r2 = __builtin_amdgcn_readlane(v, 32), r3 = __builtin_amdgcn_readlane(v, 48);
-    return imin_sel(imin_sel(r0, r1), imin_sel(r2, r3));
-}
-// v, i: this lane's candidate; on return the wavefront's lexicographic minimum.
-__device__ __forceinline__ void wave_argmin(double &v, int &i, int none) {
-    const double m = wave_min_f64(v);
-    i = wave_min_i32(v == m ? i : none);
-    v = m;
+    v = imin_sel(v, dpp_i32<TSVM_DPP_BCAST15, 0xa>(v));
+    v = imin_sel(v, dpp_i32<TSVM_DPP_BCAST31, 0xc>(v));
+    return __builtin_amdgcn_readlane(v, 63);
 }
 
 // Maps the launch's linear workgroup id to a logical one so that logical neighbours run on the
