@@ -68,20 +68,28 @@ def kernel_figures(train, params):
     dense_ok = ld * n * 8 < 40e9 and ld <= 32 * max(train.nnz / n, 1)
     m = 512
     idx = torch.from_numpy(np.random.default_rng(0).permutation(n)[:m].astype(np.int32)).cuda()
-    k_out = torch.empty((m, n), dtype=torch.float64, device="cuda")
+    kt, gamma = params.get("kernel_type", 2), params.get("gamma", 0.0)
+    # rows are stored as float for the RBF / polynomial / sigmoid kernels (their values are float-rounded by
+    # definition), as double for the linear kernel: the same choice KernelMatrix makes during training
+    row_type = capi.ROW_F64 if kt == 0 else capi.ROW_F32
+    esz = 8 if row_type == capi.ROW_F64 else 4
+    row_dtype = torch.float64 if row_type == capi.ROW_F64 else torch.float32
+    ldo = (n + 7) // 8 * 8
+    k_out = torch.empty((m, ldo), dtype=row_dtype, device="cuda")
     val_d, col_d, ptr_d = (torch.from_numpy(a).cuda() for a in (train.val, train.col, train.ptr))
     sd = torch.empty(n, dtype=torch.float64, device="cuda")
     capi.call("tsvm_csr_self_dot", val_d.data_ptr(), ptr_d.data_ptr(), n, sd.data_ptr(), None)
-    kt, gamma = params.get("kernel_type", 2), params.get("gamma", 0.0)
     if dense_ok:
         x = torch.empty((n, ld), dtype=torch.float64, device="cuda")
         capi.call("tsvm_csr_to_dense", val_d.data_ptr(), col_d.data_ptr(), ptr_d.data_ptr(), n, x.data_ptr(), ld, None)
         ms = event_time(lambda: capi.call("tsvm_get_rows_dense", x.data_ptr(), ld, None, n, nf, sd.data_ptr(), x.data_ptr(), ld,
-                                          idx.data_ptr(), m, sd.data_ptr(), kt, gamma, 0.0, 3, k_out.data_ptr(), None, n, None), 20)
+                                          idx.data_ptr(), m, sd.data_ptr(), kt, gamma, 0.0, 3, k_out.data_ptr(), row_type, None, ldo,
+                                          None), 20)
         flops = 2.0 * m * n * d
         out["get_rows"] = dict(kernel="get_rows_dense_kernel (fp64 MFMA)", ms=ms, m=m, n=n, d=d,
                                tflops=flops / ms / 1e9, frac_mfma_peak=flops / ms / 1e9 / FP64_MFMA_PEAK_TFLOPS,
-                               useful_tflops=2.0 * m * train.nnz / ms / 1e9, write_gbs=8.0 * m * n / ms / 1e6)
+                               useful_tflops=2.0 * m * train.nnz / ms / 1e9, row_bytes_per_value=esz,
+                               write_gbs=esz * m * n / ms / 1e6)
         del x
     else:
         w = torch.empty((nf, m), dtype=torch.float64, device="cuda")
@@ -92,20 +100,21 @@ def kernel_figures(train, params):
                       w.data_ptr(), None)
             capi.call("tsvm_gather_f64", sd.data_ptr(), idx.data_ptr(), m, sdw.data_ptr(), None)
             capi.call("tsvm_get_rows_csr", val_d.data_ptr(), col_d.data_ptr(), ptr_d.data_ptr(), None, n, sd.data_ptr(),
-                      w.data_ptr(), m, sdw.data_ptr(), kt, gamma, 0.0, 3, k_out.data_ptr(), None, n, None)
+                      w.data_ptr(), m, sdw.data_ptr(), kt, gamma, 0.0, 3, k_out.data_ptr(), row_type, None, ldo, None)
         ms = event_time(run, 10)
-        by = 12.0 * train.nnz + 4.0 * (n + 1) + 8.0 * m * nf + 8.0 * m * n
+        by = 12.0 * train.nnz + 4.0 * (n + 1) + 8.0 * m * nf + esz * m * n
         out["get_rows"] = dict(kernel="get_rows_csr_kernel", ms=ms, m=m, n=n, d=d, gflops=2.0 * m * train.nnz / ms / 1e6,
-                               gbs=by / ms / 1e6, frac_hbm_peak=by / ms / 1e6 / HBM_PEAK_GBS)
+                               gbs=by / ms / 1e6, frac_hbm_peak=by / ms / 1e6 / HBM_PEAK_GBS, row_bytes_per_value=esz)
         del w
     del k_out
     ws = 1024
-    k_rows = torch.rand((ws, n), dtype=torch.float64, device="cuda")
+    k_rows = torch.rand((ws, ldo), dtype=row_dtype, device="cuda")
     f = torch.zeros(n, dtype=torch.float64, device="cuda")
     ad = torch.randn(ws, dtype=torch.float64, device="cuda")
-    ms = event_time(lambda: capi.call("tsvm_update_f", f.data_ptr(), ad.data_ptr(), ws, k_rows.data_ptr(), None, n, n, None), 20)
-    by = 8.0 * ws * n + 16.0 * n + 8.0 * ws
-    out["update_f"] = dict(kernel="update_f_kernel", ms=ms, ws=ws, n=n, gbs=by / ms / 1e6,
+    ms = event_time(lambda: capi.call("tsvm_update_f", f.data_ptr(), ad.data_ptr(), ws, k_rows.data_ptr(), row_type, None,
+                                      ldo, n, 1, None), 20)
+    by = float(esz) * ws * n + 16.0 * n + 8.0 * ws   # bytes this kernel has to move with rows of esz-byte values
+    out["update_f"] = dict(kernel="update_f_kernel", ms=ms, ws=ws, n=n, row_bytes_per_value=esz, gbs=by / ms / 1e6,
                            frac_hbm_peak=by / ms / 1e6 / HBM_PEAK_GBS)
     return out
 
@@ -224,7 +233,7 @@ def main():
     else:
         roofline = dict(kernel=gr["kernel"], bound="hbm", achieved=gr["gbs"], peak=HBM_PEAK_GBS, unit="GB/s",
                         frac=gr["frac_hbm_peak"], traffic=None, launch_ms=gr["ms"],
-                        algorithmic="12*nnz + 4*(n+1) + 8*m*d + 8*m*n bytes per launch")
+                        algorithmic="12*nnz + 4*(n+1) + 8*m*d + %d*m*n bytes per launch" % gr["row_bytes_per_value"])
 
     cpu = None
     if args.cpu_iters != 0:

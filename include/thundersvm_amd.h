@@ -33,6 +33,12 @@ extern "C" {
 /* SvmParam::KERNEL_TYPE (include/thundersvm/svmparam.h:36-38) */
 enum tsvm_kernel_type { TSVM_K_LINEAR = 0, TSVM_K_POLY = 1, TSVM_K_RBF = 2, TSVM_K_SIGMOID = 3, TSVM_K_PRECOMPUTED = 4 };
 
+/* Element type of stored kernel rows.  RBF, polynomial and sigmoid kernel values are float-rounded by
+ * definition (expf / powf / tanhf in kernelmatrix_kernel.cpp:77-108, widened to kernel_type afterwards), so a
+ * float row holds exactly the reference's values in half the bytes; linear kernel values are full doubles and
+ * must use TSVM_ROW_F64 (the calls reject TSVM_ROW_F32 with a linear kernel).  Row strides (ld*) count elements. */
+enum tsvm_row_type { TSVM_ROW_F64 = 0, TSVM_ROW_F32 = 1 };
+
 typedef void *tsvm_stream;
 
 const char *tsvm_last_error(void);
@@ -69,10 +75,10 @@ int tsvm_csr_to_dense(const double *val, const int *col, const int64_t *row_ptr,
  * launch.  x is [n][ldx], a is [*][lda], both row-major fp64 with zero padding up to a multiple of
  * 8 columns (ldx % 8 == 0, lda % 8 == 0, d <= min(ldx, lda)).  The dot product is accumulated over
  * ascending column index with fused multiply-adds.  sd_x[j] / sd_a[a_idx[i]] are the self dot
- * products (used by RBF only). */
+ * products (used by RBF only).  out holds double or float elements as row_type says. */
 int tsvm_get_rows_dense(const double *x, int64_t ldx, const int *x_idx, int64_t n, int d, const double *sd_x, const double *a,
                         int64_t lda, const int *a_idx, int m, const double *sd_a, int kernel_type, double gamma,
-                        double coef0, int degree, double *out, const int *out_slots, int64_t ldo,
+                        double coef0, int degree, void *out, int row_type, const int *out_slots, int64_t ldo,
                         tsvm_stream stream);
 
 /* Transposed dense staging of selected CSR rows: w[c*m + i] = value of feature c in row idx[i]
@@ -87,7 +93,12 @@ int tsvm_csr_stage_rows(const double *val, const int *col, const int64_t *row_pt
  * working rows' self dot products (already gathered, length m).  x_idx as in tsvm_get_rows_dense. */
 int tsvm_get_rows_csr(const double *val, const int *col, const int64_t *row_ptr, const int *x_idx, int64_t n, const double *sd_x,
                       const double *w, int m, const double *sd_w, int kernel_type, double gamma, double coef0,
-                      int degree, double *out, const int *out_slots, int64_t ldo, tsvm_stream stream);
+                      int degree, void *out, int row_type, const int *out_slots, int64_t ldo, tsvm_stream stream);
+
+/* out[t] = ids[t] % period.  The 2n-variable problem of SVR (svr.cpp:14-15) stacks the same n rows twice:
+ * instance id i and i + n share one kernel row, so rows are computed, cached and stored once under the
+ * folded id and are n (not 2n) columns wide. */
+int tsvm_fold_ids(const int *ids, int count, int period, int *out, tsvm_stream stream);
 
 /* out[i] = in[idx[i]] for doubles (gathers working-set self dots). */
 int tsvm_gather_f64(const double *in, const int *idx, int m, double *out, tsvm_stream stream);
@@ -97,11 +108,15 @@ int tsvm_gather_f64(const double *in, const int *idx, int m, double *out, tsvm_s
  * ------------------------------------------------------------------------------------------- */
 
 /* update_f (smo_kernel.cpp:300-319): f[j] -= sum_{t<ws, alpha_diff[t]!=0} alpha_diff[t]*K_t[j], the
- * sum taken in ascending t with fused multiply-adds.  Kernel row t starts at
- * k_rows + slots[t]*ld (slots == NULL: slot t), so rows kept from the previous working set are
- * addressed in place instead of being copied (csmosolver.cpp:75). */
-int tsvm_update_f(double *f, const double *alpha_diff, int ws_size, const double *k_rows, const int *slots,
-                  int64_t ld, int64_t n, tsvm_stream stream);
+ * sum taken in ascending t with fused multiply-adds.  Kernel row t starts at element
+ * slots[t]*ld of k_rows (slots == NULL: slot t), so rows kept from the previous working set are
+ * addressed in place instead of being copied (csmosolver.cpp:75).  Rows are n_cols wide and f has
+ * n_cols*repeat entries: f[j + r*n_cols] -= (the same sum) for r < repeat, which is the reference's
+ * result when its kernel matrix consists of repeat x repeat copies of one n_cols x n_cols block
+ * (repeat = 2 for SVR, else 1).  ld >= n_cols rounded up to a multiple of 4 lets the kernel use
+ * 16-byte loads. */
+int tsvm_update_f(double *f, const double *alpha_diff, int ws_size, const void *k_rows, int row_type, const int *slots,
+                  int64_t ld, int64_t n_cols, int repeat, tsvm_stream stream);
 
 /* Bytes of device workspace tsvm_c_smo_solve / tsvm_nu_smo_solve need for a working set of ws_size. */
 size_t tsvm_smo_solve_workspace(int ws_size);
@@ -110,7 +125,7 @@ size_t tsvm_smo_solve_workspace(int ws_size);
  * diff[0] = initial low-up gap, diff[1] = number of inner iterations.  k_rows/slots/ld as in
  * tsvm_update_f; workspace from tsvm_smo_solve_workspace. */
 int tsvm_c_smo_solve(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
-                     int ws_size, double Cp, double Cn, const double *k_rows, const int *slots, int64_t ld,
+                     int ws_size, double Cp, double Cn, const void *k_rows, int row_type, const int *slots, int64_t ld,
                      const double *k_diag, double eps, double *diff, int max_iter, void *workspace,
                      tsvm_stream stream);
 
@@ -131,7 +146,7 @@ int tsvm_nu_smo_solve_block(const int *y, const double *f_val, double *alpha, do
 /* nu_smo_solve (smo_kernel.cpp:127-298), same conventions; diff[1] is left untouched as in the
  * reference's CPU code. */
 int tsvm_nu_smo_solve(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
-                      int ws_size, double C, const double *k_rows, const int *slots, int64_t ld,
+                      int ws_size, double C, const void *k_rows, int row_type, const int *slots, int64_t ld,
                       const double *k_diag, double eps, double *diff, int max_iter, void *workspace,
                       tsvm_stream stream);
 
@@ -152,10 +167,10 @@ int tsvm_select_working_set(const double *f, const int *y, const double *alpha, 
 
 /* sum_kernel_values: dec[r*P + p] = sum_{l in SV_i} coef[(j-1)*T + l]*K[r][l]
  *                                  + sum_{l in SV_j} coef[i*T + l]*K[r][l] - rho[p]
- * for every class pair p = (i<j), P = k(k-1)/2, T = total_sv, K is [n_instances][ldk]. */
+ * for every class pair p = (i<j), P = k(k-1)/2, T = total_sv, K is [n_instances][ldk] of row_type elements. */
 int tsvm_sum_kernel_values(const double *coef, int total_sv, const int *sv_start, const int *sv_count,
-                           const double *rho, const double *k_mat, int64_t ldk, double *dec_values, int n_classes,
-                           int64_t n_instances, tsvm_stream stream);
+                           const double *rho, const void *k_mat, int row_type, int64_t ldk, double *dec_values,
+                           int n_classes, int64_t n_instances, tsvm_stream stream);
 
 #ifdef __cplusplus
 }

@@ -35,10 +35,12 @@ def dense_padded(data, n_cols=None):
 
 
 def get_rows_dense(x_d, ld, n, d, sd_x, a_d, lda, a_idx, m, sd_a, kernel_type, gamma=0.0, coef0=0.0, degree=3,
-                   out_slots=None, out_rows=None, x_idx=None):
-    out = torch.empty((out_rows or m, n), dtype=torch.float64, device="cuda")
+                   out_slots=None, out_rows=None, x_idx=None, row_type=capi.ROW_F64):
+    """Rows come back as float64 (row_type F64) or float32 (F32) torch tensors."""
+    dt = torch.float32 if row_type == capi.ROW_F32 else torch.float64
+    out = torch.empty((out_rows or m, n), dtype=dt, device="cuda")
     capi.call("tsvm_get_rows_dense", ptr(x_d), ld, ptr(x_idx), n, d, ptr(sd_x), ptr(a_d), lda, ptr(a_idx), m, ptr(sd_a),
-              kernel_type, gamma, coef0, degree, ptr(out), ptr(out_slots), n, stream())
+              kernel_type, gamma, coef0, degree, ptr(out), row_type, ptr(out_slots), n, stream())
     return out
 
 

@@ -37,9 +37,9 @@ def test_model_library_exports():
 
 def test_argument_checks_do_not_need_a_gpu():
     lib = capi.kernel_lib()
-    rc = lib.tsvm_update_f(None, None, 4, None, None, 8, 8, None)
+    rc = lib.tsvm_update_f(None, None, 4, None, 0, None, 8, 8, 1, None)
     assert rc == -1 and b"null pointer" in lib.tsvm_last_error()
-    rc = lib.tsvm_get_rows_dense(8, 12, None, 4, 4, 8, 8, 12, None, 1, 8, 2, 0.5, 0.0, 3, 8, None, 4, None)
+    rc = lib.tsvm_get_rows_dense(8, 12, None, 4, 4, 8, 8, 12, None, 1, 8, 2, 0.5, 0.0, 3, 8, 0, None, 4, None)
     assert rc == -1 and b"multiples of 8" in lib.tsvm_last_error()
     assert lib.tsvm_select_workspace(1000) > 1000 * 10
     assert lib.tsvm_smo_solve_workspace(1024) >= 8 * 1024 * 1024

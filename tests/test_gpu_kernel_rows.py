@@ -59,6 +59,9 @@ def test_fixture_rows_and_diag(name, kt, prm):
     rows_d = G.dev(rows)
     got = G.get_rows_dense(x_d, ld, data.n, nf, sd, x_d, ld, rows_d, len(rows), sd, kt, **prm)
     _check(name, G.host(got), okm.get_rows(rows))
+    if kt != O.LINEAR:   # float rows are the same values in half the bytes
+        got32 = G.get_rows_dense(x_d, ld, data.n, nf, sd, x_d, ld, rows_d, len(rows), sd, kt, row_type=capi.ROW_F32, **prm)
+        assert np.array_equal(G.host(got32).astype(np.float64), G.host(got))
     # get_rows(instances): first 10 rows as an external batch (test_kernelmatrix.cpp:108-118)
     batch = data.rows(np.arange(10))
     bh = batch.to_dense(ld)
@@ -86,6 +89,17 @@ def test_random_dense(name, kt, prm, n, d, m, density):
     idx_d = G.dev(idx)
     got = G.get_rows_dense(x_d, ld, n, nf, sd, x_d, ld, idx_d, m, sd, kt, **prm)
     _check(name, G.host(got), okm.get_rows(idx))
+    if kt != O.LINEAR:
+        got32 = G.get_rows_dense(x_d, ld, n, nf, sd, x_d, ld, idx_d, m, sd, kt, row_type=capi.ROW_F32, **prm)
+        assert got32.dtype == torch.float32 and np.array_equal(G.host(got32).astype(np.float64), G.host(got))
+
+
+def test_float_rows_rejected_for_linear_kernel():
+    x_d = torch.zeros((8, 8), dtype=torch.float64, device="cuda")
+    out = torch.zeros((8, 8), dtype=torch.float32, device="cuda")
+    with pytest.raises(capi.TsvmError):
+        capi.call("tsvm_get_rows_dense", G.ptr(x_d), 8, None, 8, 8, None, G.ptr(x_d), 8, None, 8, None, O.LINEAR, 0.0, 0.0, 3,
+                  G.ptr(out), capi.ROW_F32, None, 8, G.stream())
 
 
 @pytest.mark.parametrize("name,kt,prm", KERNELS)
@@ -116,8 +130,15 @@ def test_csr_path(name, kt, prm):
     capi.call("tsvm_gather_f64", G.ptr(sd), G.ptr(idx_d), m, G.ptr(sdw), G.stream())
     out = torch.empty((m, n), dtype=torch.float64, device="cuda")
     capi.call("tsvm_get_rows_csr", G.ptr(val_d), G.ptr(col_d), G.ptr(ptr_d), None, n, G.ptr(sd), G.ptr(w), m, G.ptr(sdw), kt,
-              prm.get("gamma", 0.0), prm.get("coef0", 0.0), prm.get("degree", 3), G.ptr(out), None, n, G.stream())
+              prm.get("gamma", 0.0), prm.get("coef0", 0.0), prm.get("degree", 3), G.ptr(out), capi.ROW_F64, None, n,
+              G.stream())
     _check(name, G.host(out), okm.get_rows(idx))
+    if kt != O.LINEAR:   # float rows hold the same values
+        out32 = torch.empty((m, n), dtype=torch.float32, device="cuda")
+        capi.call("tsvm_get_rows_csr", G.ptr(val_d), G.ptr(col_d), G.ptr(ptr_d), None, n, G.ptr(sd), G.ptr(w), m, G.ptr(sdw),
+                  kt, prm.get("gamma", 0.0), prm.get("coef0", 0.0), prm.get("degree", 3), G.ptr(out32), capi.ROW_F32, None,
+                  n, G.stream())
+        assert np.array_equal(G.host(out32).astype(np.float64), G.host(out))
     # the dense path on the same data gives the same bits (both sum in ascending feature order)
     xh, nf2, ld = G.dense_padded(data)
     x_d = G.dev(xh)
@@ -163,9 +184,16 @@ def test_sum_kernel_values(n_classes, rows):
     want = O.sum_kernel_values(coef, T, start, cnt, rho, k, n_classes, rows)
     dec = torch.empty((rows, nb), dtype=torch.float64, device="cuda")
     coef_d, start_d, cnt_d, rho_d, k_d = G.dev(coef), G.dev(start), G.dev(cnt), G.dev(rho), G.dev(k)
-    capi.call("tsvm_sum_kernel_values", G.ptr(coef_d), T, G.ptr(start_d), G.ptr(cnt_d), G.ptr(rho_d), G.ptr(k_d), T,
-              G.ptr(dec), n_classes, rows, G.stream())
+    capi.call("tsvm_sum_kernel_values", G.ptr(coef_d), T, G.ptr(start_d), G.ptr(cnt_d), G.ptr(rho_d), G.ptr(k_d),
+              capi.ROW_F64, T, G.ptr(dec), n_classes, rows, G.stream())
     assert np.abs(G.host(dec) - want).max() < 1e-9
+    # float kernel values: same reduction on the float-rounded matrix
+    k32 = k.astype(np.float32)
+    want32 = O.sum_kernel_values(coef, T, start, cnt, rho, k32.astype(np.float64), n_classes, rows)
+    k32_d = G.dev(k32)
+    capi.call("tsvm_sum_kernel_values", G.ptr(coef_d), T, G.ptr(start_d), G.ptr(cnt_d), G.ptr(rho_d), G.ptr(k32_d),
+              capi.ROW_F32, T, G.ptr(dec), n_classes, rows, G.stream())
+    assert np.abs(G.host(dec) - want32).max() < 1e-9
 
 
 def test_output_row_slots():
@@ -187,5 +215,5 @@ def test_output_row_slots():
     capi.call("tsvm_gather_f64", G.ptr(sd), G.ptr(idx_d), m, G.ptr(sdw), G.stream())
     out = torch.zeros((pool, n), dtype=torch.float64, device="cuda")
     capi.call("tsvm_get_rows_csr", G.ptr(val_d), G.ptr(col_d), G.ptr(ptr_d), None, n, G.ptr(sd), G.ptr(w), m, G.ptr(sdw), O.RBF,
-              0.2, 0.0, 3, G.ptr(out), G.ptr(slots_d), n, G.stream())
+              0.2, 0.0, 3, G.ptr(out), capi.ROW_F64, G.ptr(slots_d), n, G.stream())
     assert np.array_equal(G.host(out)[slots], want)

@@ -23,23 +23,55 @@ def _problem(n, d, seed, gamma=0.5):
 
 
 @pytest.mark.parametrize("n,ws,zero_frac", [(1, 1, 0.0), (1000, 1024, 0.5), (1537, 512, 0.0), (4099, 37, 0.9), (513, 2050, 0.3)])
-def test_update_f(n, ws, zero_frac):
+@pytest.mark.parametrize("row_type", [capi.ROW_F64, capi.ROW_F32])
+def test_update_f(n, ws, zero_frac, row_type):
     rng = np.random.default_rng(n + ws)
     ld = n + 3
     k = rng.random((ws + 5, ld))
+    if row_type == capi.ROW_F32:
+        k = k.astype(np.float32)
+    k64 = k.astype(np.float64)
     ad = rng.standard_normal(ws)
     ad[rng.random(ws) < zero_frac] = 0
     f = rng.standard_normal(n)
     slots = rng.permutation(ws + 5)[:ws].astype(np.int32)
-    want = O.update_f(f, ad, np.ascontiguousarray(k[slots][:, :n]), n)
+    want = O.update_f(f, ad, np.ascontiguousarray(k64[slots][:, :n]), n)
     f_d, ad_d, k_d, s_d = G.dev(f), G.dev(ad), G.dev(k), G.dev(slots)
-    capi.call("tsvm_update_f", G.ptr(f_d), G.ptr(ad_d), ws, G.ptr(k_d), G.ptr(s_d), ld, n, G.stream())
+    capi.call("tsvm_update_f", G.ptr(f_d), G.ptr(ad_d), ws, G.ptr(k_d), row_type, G.ptr(s_d), ld, n, 1, G.stream())
     assert np.array_equal(G.host(f_d), want)
     # slots == NULL: identity
-    want = O.update_f(f, ad, np.ascontiguousarray(k[:ws, :n]), n)
+    want = O.update_f(f, ad, np.ascontiguousarray(k64[:ws, :n]), n)
     f_d = G.dev(f)
-    capi.call("tsvm_update_f", G.ptr(f_d), G.ptr(ad_d), ws, G.ptr(k_d), None, ld, n, G.stream())
+    capi.call("tsvm_update_f", G.ptr(f_d), G.ptr(ad_d), ws, G.ptr(k_d), row_type, None, ld, n, 1, G.stream())
     assert np.array_equal(G.host(f_d), want)
+
+
+@pytest.mark.parametrize("n,ws,ld_pad", [(300001, 64, 7), (262144, 33, 0), (270000, 40, 4)])
+@pytest.mark.parametrize("row_type", [capi.ROW_F64, capi.ROW_F32])
+def test_update_f_wide_and_repeated(n, ws, ld_pad, row_type):
+    """Large n takes the 16-byte-load path (also with a ragged last vector); with repeat = 2 the kernel
+    rows are n wide and f has 2n entries, which must equal the reference's update_f on [K K] rows."""
+    rng = np.random.default_rng(n)
+    ld = n + ld_pad
+    k = rng.random((ws, ld))
+    if row_type == capi.ROW_F32:
+        k = k.astype(np.float32)
+    k64 = k.astype(np.float64)[:, :n]
+    ad = rng.standard_normal(ws)
+    ad[::3] = 0
+    f = rng.standard_normal(2 * n)
+    want = O.update_f(f, ad, np.ascontiguousarray(np.concatenate([k64, k64], axis=1)), 2 * n)
+    f_d, ad_d, k_d = G.dev(f), G.dev(ad), G.dev(k)
+    capi.call("tsvm_update_f", G.ptr(f_d), G.ptr(ad_d), ws, G.ptr(k_d), row_type, None, ld, n, 2, G.stream())
+    assert np.array_equal(G.host(f_d), want)
+
+
+def test_fold_ids():
+    ids = np.array([0, 5, 9, 10, 19, 7], dtype=np.int32)
+    out = torch.zeros(6, dtype=torch.int32, device="cuda")
+    ids_d = G.dev(ids)
+    capi.call("tsvm_fold_ids", G.ptr(ids_d), 6, 10, G.ptr(out), G.stream())
+    assert np.array_equal(G.host(out), ids % 10)
 
 
 def _solver_inputs(n, d, ws, seed, C, nu=False):
@@ -69,7 +101,15 @@ def test_c_smo_solve(n, ws, max_iter):
     diff_d = torch.zeros(2, dtype=torch.float64, device="cuda")
     wsp = torch.empty(capi.kernel_lib().tsvm_smo_solve_workspace(ws), dtype=torch.uint8, device="cuda")
     capi.call("tsvm_c_smo_solve", G.ptr(y_d), G.ptr(f_d), G.ptr(a_d), G.ptr(ad_d), G.ptr(ws_d), ws, Cp, Cn, G.ptr(k_d),
-              G.ptr(s_d), n, G.ptr(dg_d), eps, G.ptr(diff_d), max_iter, G.ptr(wsp), G.stream())
+              capi.ROW_F64, G.ptr(s_d), n, G.ptr(dg_d), eps, G.ptr(diff_d), max_iter, G.ptr(wsp), G.stream())
+    assert np.array_equal(G.host(diff_d), diff_want)
+    assert np.array_equal(G.host(a_d), a_want)
+    assert np.array_equal(G.host(ad_d), ad_want)
+    # the same rows held as float (RBF values are float-exact): identical result
+    a_d, k32_d = G.dev(alpha), G.dev(k_phys.astype(np.float32))
+    assert np.array_equal(k_phys.astype(np.float32).astype(np.float64), k_phys)
+    capi.call("tsvm_c_smo_solve", G.ptr(y_d), G.ptr(f_d), G.ptr(a_d), G.ptr(ad_d), G.ptr(ws_d), ws, Cp, Cn, G.ptr(k32_d),
+              capi.ROW_F32, G.ptr(s_d), n, G.ptr(dg_d), eps, G.ptr(diff_d), max_iter, G.ptr(wsp), G.stream())
     assert np.array_equal(G.host(diff_d), diff_want)
     assert np.array_equal(G.host(a_d), a_want)
     assert np.array_equal(G.host(ad_d), ad_want)
@@ -85,8 +125,8 @@ def test_nu_smo_solve(n, ws):
     ad_d = torch.zeros(ws, dtype=torch.float64, device="cuda")
     diff_d = torch.zeros(2, dtype=torch.float64, device="cuda")
     wsp = torch.empty(capi.kernel_lib().tsvm_smo_solve_workspace(ws), dtype=torch.uint8, device="cuda")
-    capi.call("tsvm_nu_smo_solve", G.ptr(y_d), G.ptr(f_d), G.ptr(a_d), G.ptr(ad_d), G.ptr(ws_d), ws, Cc, G.ptr(k_d), None,
-              n, G.ptr(dg_d), eps, G.ptr(diff_d), 100000, G.ptr(wsp), G.stream())
+    capi.call("tsvm_nu_smo_solve", G.ptr(y_d), G.ptr(f_d), G.ptr(a_d), G.ptr(ad_d), G.ptr(ws_d), ws, Cc, G.ptr(k_d),
+              capi.ROW_F64, None, n, G.ptr(dg_d), eps, G.ptr(diff_d), 100000, G.ptr(wsp), G.stream())
     assert G.host(diff_d)[0] == diff_want[0]
     assert np.array_equal(G.host(a_d), a_want)
     assert np.array_equal(G.host(ad_d), ad_want)

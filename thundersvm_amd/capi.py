@@ -12,6 +12,7 @@ HOST_LIB = os.path.join(_HERE, "libthundersvm.so")
 
 LINEAR, POLY, RBF, SIGMOID, PRECOMPUTED = range(5)
 C_SVC, NU_SVC, ONE_CLASS, EPSILON_SVR, NU_SVR = range(5)
+ROW_F64, ROW_F32 = 0, 1
 
 _p = C.c_void_p
 _i64 = C.c_int64
@@ -25,20 +26,21 @@ SIGNATURES = {
     "tsvm_dense_self_dot": (_int, [_p, _i64, _i64, _int, _p, _p]),
     "tsvm_kernel_diag": (_int, [_p, _i64, _int, _dbl, _dbl, _int, _p, _p]),
     "tsvm_csr_to_dense": (_int, [_p, _p, _p, _i64, _p, _i64, _p]),
-    "tsvm_get_rows_dense": (_int, [_p, _i64, _p, _i64, _int, _p, _p, _i64, _p, _int, _p, _int, _dbl, _dbl, _int, _p, _p, _i64, _p]),
+    "tsvm_get_rows_dense": (_int, [_p, _i64, _p, _i64, _int, _p, _p, _i64, _p, _int, _p, _int, _dbl, _dbl, _int, _p, _int, _p, _i64, _p]),
     "tsvm_csr_stage_rows": (_int, [_p, _p, _p, _p, _int, _int, _p, _p]),
-    "tsvm_get_rows_csr": (_int, [_p, _p, _p, _p, _i64, _p, _p, _int, _p, _int, _dbl, _dbl, _int, _p, _p, _i64, _p]),
+    "tsvm_get_rows_csr": (_int, [_p, _p, _p, _p, _i64, _p, _p, _int, _p, _int, _dbl, _dbl, _int, _p, _int, _p, _i64, _p]),
+    "tsvm_fold_ids": (_int, [_p, _int, _int, _p, _p]),
     "tsvm_gather_f64": (_int, [_p, _p, _int, _p, _p]),
-    "tsvm_update_f": (_int, [_p, _p, _int, _p, _p, _i64, _i64, _p]),
+    "tsvm_update_f": (_int, [_p, _p, _int, _p, _int, _p, _i64, _i64, _int, _p]),
     "tsvm_smo_solve_workspace": (C.c_size_t, [_int]),
-    "tsvm_c_smo_solve": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _dbl, _p, _p, _i64, _p, _dbl, _p, _int, _p, _p]),
-    "tsvm_nu_smo_solve": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _p, _p, _i64, _p, _dbl, _p, _int, _p, _p]),
+    "tsvm_c_smo_solve": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _dbl, _p, _int, _p, _i64, _p, _dbl, _p, _int, _p, _p]),
+    "tsvm_nu_smo_solve": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _p, _int, _p, _i64, _p, _dbl, _p, _int, _p, _p]),
     "tsvm_smo_solve_block_ld": (_int, [_int]),
     "tsvm_c_smo_solve_block": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _dbl, _p, _p, _dbl, _p, _int, _p]),
     "tsvm_nu_smo_solve_block": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _p, _p, _dbl, _p, _int, _p]),
     "tsvm_select_workspace": (C.c_size_t, [_i64]),
     "tsvm_select_working_set": (_int, [_p, _p, _p, _i64, _dbl, _dbl, _p, _int, _p, _int, _int, _p, _p]),
-    "tsvm_sum_kernel_values": (_int, [_p, _int, _p, _p, _p, _p, _i64, _p, _int, _i64, _p]),
+    "tsvm_sum_kernel_values": (_int, [_p, _int, _p, _p, _p, _p, _int, _i64, _p, _int, _i64, _p]),
 }
 
 _LIB = None

@@ -34,11 +34,14 @@ typedef double v4d __attribute__((ext_vector_type(4)));
 //                      where the epilogue and the stores weigh as much as the MFMAs).
 // Either way a wavefront issues 32 MFMAs between two barriers.  LDS tiles are k-major [KTILE][LS];
 // LS (130 / 129 doubles) makes the staging writes and the operand reads bank-conflict free.
-template <int KT, int TI>
+// TO: element type of the output rows.  The RBF / polynomial / sigmoid values are float-rounded by
+// definition (kernelmatrix_kernel.cpp:77-108 calls expf / powf / tanhf), so storing them as float
+// loses nothing and halves the bytes written here and read back by update_f.
+template <int KT, int TI, typename TO>
 __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
     const double *__restrict__ x, int64_t ldx, const int *__restrict__ x_idx, int64_t n, int d,
     const double *__restrict__ sd_x, const double *__restrict__ a, int64_t lda, const int *__restrict__ a_idx, int m,
-    const double *__restrict__ sd_a, KernelParam kp_in, double *__restrict__ out, const int *__restrict__ out_slots,
+    const double *__restrict__ sd_a, KernelParam kp_in, TO *__restrict__ out, const int *__restrict__ out_slots,
     int64_t ldo, unsigned m_blocks) {
     constexpr int BM = 32 * TI;
     constexpr int KTILE = TI == 2 ? 16 : 8;
@@ -156,10 +159,10 @@ __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
         for (int ti = 0; ti < TI; ++ti) {
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
-                double *orow = out + orow_off[ti * 4 + v] + jb;
+                TO *orow = out + orow_off[ti * 4 + v] + jb;
 #pragma unroll
                 for (int tj = 0; tj < 4; ++tj)
-                    orow[tj * 16] = tsvm_epilogue(acc[ti][tj][v], sdi[ti * 4 + v], sdj[tj], kp, exp_tab);
+                    orow[tj * 16] = (TO) tsvm_epilogue(acc[ti][tj][v], sdi[ti * 4 + v], sdj[tj], kp, exp_tab);
             }
         }
     } else {
@@ -169,10 +172,10 @@ __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
             for (int v = 0; v < 4; ++v) {
                 const int i = i0 + wi * (16 * TI) + ti * 16 + 4 * v + lk;
                 if (i >= m) continue;
-                double *orow = out + orow_off[ti * 4 + v] + jb;
+                TO *orow = out + orow_off[ti * 4 + v] + jb;
 #pragma unroll
                 for (int tj = 0; tj < 4; ++tj)
-                    if (jb + tj * 16 < n) orow[tj * 16] = tsvm_epilogue(acc[ti][tj][v], sdi[ti * 4 + v], sdj[tj], kp, exp_tab);
+                    if (jb + tj * 16 < n) orow[tj * 16] = (TO) tsvm_epilogue(acc[ti][tj][v], sdi[ti * 4 + v], sdj[tj], kp, exp_tab);
             }
         }
     }
@@ -185,10 +188,11 @@ __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
 // ------------------------------------------------------------------------------------------------
 #define CS_JB 16
 
+template <typename TO>
 __global__ __launch_bounds__(256) void get_rows_csr_kernel(
     const double *__restrict__ val, const int *__restrict__ col, const int64_t *__restrict__ row_ptr,
     const int *__restrict__ x_idx, int64_t n, const double *__restrict__ sd_x, const double *__restrict__ w, int m,
-    const double *__restrict__ sd_w, KernelParam kp, double *__restrict__ out, const int *__restrict__ out_slots,
+    const double *__restrict__ sd_w, KernelParam kp, TO *__restrict__ out, const int *__restrict__ out_slots,
     int64_t ldo, unsigned i_blocks) {
     __shared__ uint64_t exp_tab[32];
     const int tid = threadIdx.x;
@@ -218,12 +222,17 @@ __global__ __launch_bounds__(256) void get_rows_csr_kernel(
     }
     if (!active) return;
     const double sdi = sd_w ? sd_w[i] : 0.0;
-    double *orow = out + (int64_t) (out_slots ? out_slots[i] : i) * ldo;
+    TO *orow = out + (int64_t) (out_slots ? out_slots[i] : i) * ldo;
 #pragma unroll
     for (int jj = 0; jj < CS_JB; ++jj) {
         const int64_t j = j0 + jj;
-        if (j < n) orow[j] = tsvm_epilogue(acc[jj], sdi, sd_x ? sd_x[x_idx ? (int64_t) x_idx[j] : j] : 0.0, kp, exp_tab);
+        if (j < n) orow[j] = (TO) tsvm_epilogue(acc[jj], sdi, sd_x ? sd_x[x_idx ? (int64_t) x_idx[j] : j] : 0.0, kp, exp_tab);
     }
+}
+
+__global__ void fold_ids_kernel(const int *__restrict__ ids, int count, int period, int *__restrict__ out) {
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t < count) out[t] = ids[t] % period;
 }
 
 __global__ void fill_f64_kernel(double *p, int64_t count, double v) {
@@ -308,9 +317,10 @@ __global__ void gather_f64_kernel(const double *__restrict__ in, const int *__re
 #define SK_R 4
 #define SK_T 256
 
+template <typename TK>
 __global__ __launch_bounds__(SK_T) void sum_kernel_values_kernel(
     const double *__restrict__ coef, int total_sv, const int *__restrict__ sv_start, const int *__restrict__ sv_count,
-    const double *__restrict__ rho, const double *__restrict__ k_mat, int64_t ldk, double *__restrict__ dec,
+    const double *__restrict__ rho, const TK *__restrict__ k_mat, int64_t ldk, double *__restrict__ dec,
     int n_classes, int64_t n_instances) {
     extern __shared__ double sm[];  // [SK_R][(k-1)*k] segment sums, then reduction scratch [SK_T/64][SK_R]
     const int tid = threadIdx.x;
@@ -333,7 +343,7 @@ __global__ __launch_bounds__(SK_T) void sum_kernel_values_kernel(
 #pragma unroll
                 for (int rr = 0; rr < SK_R; ++rr) {
                     const int64_t r = r0 + rr;
-                    if (r < n_instances) part[rr] = __builtin_fma(cv, k_mat[r * ldk + st + l], part[rr]);
+                    if (r < n_instances) part[rr] = __builtin_fma(cv, (double) k_mat[r * ldk + st + l], part[rr]);
                 }
             }
 #pragma unroll
@@ -412,9 +422,15 @@ int tsvm_csr_to_dense(const double *val, const int *col, const int64_t *row_ptr,
     return 0;
 }
 
+static bool row_type_ok(int row_type, int kernel_type) {
+    // float rows are exact only where the reference's value is a float to begin with
+    return row_type == TSVM_ROW_F64 || (row_type == TSVM_ROW_F32 && kernel_type != TSVM_LINEAR);
+}
+
 int tsvm_get_rows_dense(const double *x, int64_t ldx, const int *x_idx, int64_t n, int d, const double *sd_x, const double *a,
                         int64_t lda, const int *a_idx, int m, const double *sd_a, int kernel_type, double gamma,
-                        double coef0, int degree, double *out, const int *out_slots, int64_t ldo, tsvm_stream stream) {
+                        double coef0, int degree, void *out, int row_type, const int *out_slots, int64_t ldo,
+                        tsvm_stream stream) {
     TSVM_REQUIRE(x && a && out, "tsvm_get_rows_dense: null pointer");
     TSVM_REQUIRE(n >= 0 && m >= 0 && d >= 0, "tsvm_get_rows_dense: negative size");
     TSVM_REQUIRE(ldx % 8 == 0 && lda % 8 == 0, "tsvm_get_rows_dense: ldx (%lld) and lda (%lld) must be multiples of 8",
@@ -423,6 +439,8 @@ int tsvm_get_rows_dense(const double *x, int64_t ldx, const int *x_idx, int64_t 
     TSVM_REQUIRE(ldo >= n, "tsvm_get_rows_dense: ldo (%lld) < n (%lld)", (long long) ldo, (long long) n);
     TSVM_REQUIRE(((uintptr_t) x % 32 == 0) && ((uintptr_t) a % 32 == 0), "tsvm_get_rows_dense: x and a must be 32-byte aligned");
     TSVM_REQUIRE(kernel_type >= 0 && kernel_type <= 4, "tsvm_get_rows_dense: unknown kernel type %d", kernel_type);
+    TSVM_REQUIRE(row_type_ok(row_type, kernel_type), "tsvm_get_rows_dense: row type %d not valid for kernel type %d", row_type,
+                 kernel_type);
     TSVM_REQUIRE((kernel_type != TSVM_RBF && kernel_type != TSVM_PRECOMPUTED) || (sd_x && sd_a),
                  "tsvm_get_rows_dense: RBF needs self dot products");
     if (n == 0 || m == 0) return 0;
@@ -433,22 +451,28 @@ int tsvm_get_rows_dense(const double *x, int64_t ldx, const int *x_idx, int64_t 
     const int64_t n_blocks = (n + GR_BN - 1) / GR_BN;
     TSVM_REQUIRE(n_blocks * m_blocks < (int64_t) 0x7fffffff, "tsvm_get_rows_dense: grid too large");
     const dim3 grid((unsigned) (n_blocks * m_blocks)), block(256);
-#define GR_LAUNCH(KTYPE)                                                                                              \
+#define GR_LAUNCH_T(KTYPE, TO)                                                                                        \
     do {                                                                                                              \
         if (ti == 2)                                                                                                  \
-            hipLaunchKernelGGL((get_rows_dense_kernel<KTYPE, 2>), grid, block, 0, tsvm_s(stream), x, ldx, x_idx, n, d, sd_x, a, \
-                               lda, a_idx, m, sd_a, kp, out, out_slots, ldo, m_blocks);                               \
+            hipLaunchKernelGGL((get_rows_dense_kernel<KTYPE, 2, TO>), grid, block, 0, tsvm_s(stream), x, ldx, x_idx, n, d, sd_x, \
+                               a, lda, a_idx, m, sd_a, kp, (TO *) out, out_slots, ldo, m_blocks);                     \
         else                                                                                                          \
-            hipLaunchKernelGGL((get_rows_dense_kernel<KTYPE, 4>), grid, block, 0, tsvm_s(stream), x, ldx, x_idx, n, d, sd_x, a, \
-                               lda, a_idx, m, sd_a, kp, out, out_slots, ldo, m_blocks);                               \
+            hipLaunchKernelGGL((get_rows_dense_kernel<KTYPE, 4, TO>), grid, block, 0, tsvm_s(stream), x, ldx, x_idx, n, d, sd_x, \
+                               a, lda, a_idx, m, sd_a, kp, (TO *) out, out_slots, ldo, m_blocks);                     \
+    } while (0)
+#define GR_LAUNCH(KTYPE)                                        \
+    do {                                                        \
+        if (row_type == TSVM_ROW_F32) GR_LAUNCH_T(KTYPE, float); \
+        else GR_LAUNCH_T(KTYPE, double);                        \
     } while (0)
     switch (kernel_type) {
-        case TSVM_LINEAR: GR_LAUNCH(TSVM_LINEAR); break;
+        case TSVM_LINEAR: GR_LAUNCH_T(TSVM_LINEAR, double); break;
         case TSVM_POLY: GR_LAUNCH(TSVM_POLY); break;
         case TSVM_SIGMOID: GR_LAUNCH(TSVM_SIGMOID); break;
         default: GR_LAUNCH(TSVM_RBF); break;
     }
 #undef GR_LAUNCH
+#undef GR_LAUNCH_T
     TSVM_LAUNCH_CHECK();
     return 0;
 }
@@ -467,10 +491,12 @@ int tsvm_csr_stage_rows(const double *val, const int *col, const int64_t *row_pt
 
 int tsvm_get_rows_csr(const double *val, const int *col, const int64_t *row_ptr, const int *x_idx, int64_t n, const double *sd_x,
                       const double *w, int m, const double *sd_w, int kernel_type, double gamma, double coef0,
-                      int degree, double *out, const int *out_slots, int64_t ldo, tsvm_stream stream) {
+                      int degree, void *out, int row_type, const int *out_slots, int64_t ldo, tsvm_stream stream) {
     TSVM_REQUIRE(row_ptr && w && out, "tsvm_get_rows_csr: null pointer");
     TSVM_REQUIRE(n >= 0 && m >= 0 && ldo >= n, "tsvm_get_rows_csr: bad size");
     TSVM_REQUIRE(kernel_type >= 0 && kernel_type <= 4, "tsvm_get_rows_csr: unknown kernel type %d", kernel_type);
+    TSVM_REQUIRE(row_type_ok(row_type, kernel_type), "tsvm_get_rows_csr: row type %d not valid for kernel type %d", row_type,
+                 kernel_type);
     TSVM_REQUIRE((kernel_type != TSVM_RBF && kernel_type != TSVM_PRECOMPUTED) || (sd_x && sd_w),
                  "tsvm_get_rows_csr: RBF needs self dot products");
     if (n == 0 || m == 0) return 0;
@@ -478,8 +504,20 @@ int tsvm_get_rows_csr(const double *val, const int *col, const int64_t *row_ptr,
     const unsigned i_blocks = (unsigned) ((m + 255) / 256);
     const int64_t j_blocks = (n + CS_JB - 1) / CS_JB;
     TSVM_REQUIRE(j_blocks * i_blocks < (int64_t) 0x7fffffff, "tsvm_get_rows_csr: grid too large");
-    hipLaunchKernelGGL(get_rows_csr_kernel, dim3((unsigned) (j_blocks * i_blocks)), dim3(256), 0, tsvm_s(stream), val, col,
-                       row_ptr, x_idx, n, sd_x, w, m, sd_w, kp, out, out_slots, ldo, i_blocks);
+    if (row_type == TSVM_ROW_F32)
+        hipLaunchKernelGGL(get_rows_csr_kernel<float>, dim3((unsigned) (j_blocks * i_blocks)), dim3(256), 0, tsvm_s(stream), val,
+                           col, row_ptr, x_idx, n, sd_x, w, m, sd_w, kp, (float *) out, out_slots, ldo, i_blocks);
+    else
+        hipLaunchKernelGGL(get_rows_csr_kernel<double>, dim3((unsigned) (j_blocks * i_blocks)), dim3(256), 0, tsvm_s(stream), val,
+                           col, row_ptr, x_idx, n, sd_x, w, m, sd_w, kp, (double *) out, out_slots, ldo, i_blocks);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+int tsvm_fold_ids(const int *ids, int count, int period, int *out, tsvm_stream stream) {
+    TSVM_REQUIRE(ids && out && count >= 0 && period > 0, "tsvm_fold_ids: bad argument");
+    if (count == 0) return 0;
+    hipLaunchKernelGGL(fold_ids_kernel, dim3(grid_for(count, 256)), dim3(256), 0, tsvm_s(stream), ids, count, period, out);
     TSVM_LAUNCH_CHECK();
     return 0;
 }
@@ -493,15 +531,22 @@ int tsvm_gather_f64(const double *in, const int *idx, int m, double *out, tsvm_s
 }
 
 int tsvm_sum_kernel_values(const double *coef, int total_sv, const int *sv_start, const int *sv_count,
-                           const double *rho, const double *k_mat, int64_t ldk, double *dec_values, int n_classes,
-                           int64_t n_instances, tsvm_stream stream) {
+                           const double *rho, const void *k_mat, int row_type, int64_t ldk, double *dec_values,
+                           int n_classes, int64_t n_instances, tsvm_stream stream) {
     TSVM_REQUIRE(sv_start && sv_count && rho && dec_values, "tsvm_sum_kernel_values: null pointer");
     TSVM_REQUIRE(n_classes >= 2 && n_classes <= 32, "tsvm_sum_kernel_values: n_classes %d outside [2, 32]", n_classes);
     TSVM_REQUIRE(total_sv >= 0 && ldk >= total_sv && n_instances >= 0, "tsvm_sum_kernel_values: bad size");
+    TSVM_REQUIRE(row_type == TSVM_ROW_F64 || row_type == TSVM_ROW_F32, "tsvm_sum_kernel_values: unknown row type %d", row_type);
     if (n_instances == 0) return 0;
     const size_t shm = sizeof(double) * ((size_t) SK_R * (n_classes - 1) * n_classes + (SK_T / 64) * SK_R);
-    hipLaunchKernelGGL(sum_kernel_values_kernel, dim3(grid_for(n_instances, SK_R)), dim3(SK_T), shm, tsvm_s(stream), coef,
-                       total_sv, sv_start, sv_count, rho, k_mat, ldk, dec_values, n_classes, n_instances);
+    if (row_type == TSVM_ROW_F32)
+        hipLaunchKernelGGL(sum_kernel_values_kernel<float>, dim3(grid_for(n_instances, SK_R)), dim3(SK_T), shm, tsvm_s(stream),
+                           coef, total_sv, sv_start, sv_count, rho, (const float *) k_mat, ldk, dec_values, n_classes,
+                           n_instances);
+    else
+        hipLaunchKernelGGL(sum_kernel_values_kernel<double>, dim3(grid_for(n_instances, SK_R)), dim3(SK_T), shm, tsvm_s(stream),
+                           coef, total_sv, sv_start, sv_count, rho, (const double *) k_mat, ldk, dec_values, n_classes,
+                           n_instances);
     TSVM_LAUNCH_CHECK();
     return 0;
 }

@@ -20,19 +20,21 @@
 #define UF_T 256
 #define UF_CHUNK 1024
 
-// COLS columns per thread (consecutive, loaded as one 8*COLS-byte vector), UNROLL rows in flight.
-template <int COLS, int UNROLL>
+// TK: element type of the kernel rows; COLS columns per thread (consecutive, loaded as one vector of
+// COLS elements); UNROLL rows in flight.  Rows are n columns wide and f holds `repeat` stacked copies
+// of the n columns, each of which receives the same sum.
+template <typename TK, int COLS, int UNROLL>
 __global__ __launch_bounds__(UF_T) void update_f_kernel(double *__restrict__ f, const double *__restrict__ alpha_diff,
-                                                        int ws, const double *__restrict__ k_rows,
-                                                        const int *__restrict__ slots, int64_t ld, int64_t n) {
-    typedef double vec_t __attribute__((ext_vector_type(COLS)));
+                                                        int ws, const TK *__restrict__ k_rows,
+                                                        const int *__restrict__ slots, int64_t ld, int64_t n, int repeat) {
+    typedef TK vec_t __attribute__((ext_vector_type(COLS)));
     __shared__ double s_ad[UF_CHUNK];
     __shared__ int64_t s_off[UF_CHUNK];
     __shared__ int s_wave_cnt[UF_T / 64];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int64_t j = ((int64_t) blockIdx.x * UF_T + tid) * COLS;
-    const bool act = j < n;   // n is a multiple of COLS whenever COLS > 1 (checked by the launcher)
+    const bool act = j < n;   // a vector may reach past n, but never past the padded row (checked by the launcher)
     double sum[COLS];
 #pragma unroll
     for (int c = 0; c < COLS; ++c) sum[c] = 0.0;
@@ -81,21 +83,24 @@ __global__ __launch_bounds__(UF_T) void update_f_kernel(double *__restrict__ f, 
                 for (int e = 0; e < UNROLL; ++e) {
                     const double ad = s_ad[u + e];
 #pragma unroll
-                    for (int c = 0; c < COLS; ++c) sum[c] = __builtin_fma(ad, k[e][c], sum[c]);
+                    for (int c = 0; c < COLS; ++c) sum[c] = __builtin_fma(ad, (double) k[e][c], sum[c]);
                 }
             }
             for (; u < total; ++u) {
                 const vec_t k = *(const vec_t *) (k_rows + s_off[u] + j);
                 const double ad = s_ad[u];
 #pragma unroll
-                for (int c = 0; c < COLS; ++c) sum[c] = __builtin_fma(ad, k[c], sum[c]);
+                for (int c = 0; c < COLS; ++c) sum[c] = __builtin_fma(ad, (double) k[c], sum[c]);
             }
         }
         __syncthreads();
     }
     if (act) {
+        for (int r = 0; r < repeat; ++r) {
 #pragma unroll
-        for (int c = 0; c < COLS; ++c) f[j + c] -= sum[c];
+            for (int c = 0; c < COLS; ++c)
+                if (j + c < n) f[(int64_t) r * n + j + c] -= sum[c];
+        }
     }
 }
 
@@ -509,25 +514,35 @@ __global__ __launch_bounds__(MAX_WS) void sel_final_kernel(SelWorkspace w, SelGe
 // ------------------------------------------------------------------------------------------------
 // C ABI
 // ------------------------------------------------------------------------------------------------
+template <typename TK, int COLS, int UNROLL>
+static void launch_update_f(double *f, const double *alpha_diff, int ws_size, const void *k_rows, const int *slots,
+                            int64_t ld, int64_t n, int repeat, hipStream_t s) {
+    const unsigned grid = (unsigned) (((n + COLS - 1) / COLS + UF_T - 1) / UF_T);
+    hipLaunchKernelGGL((update_f_kernel<TK, COLS, UNROLL>), dim3(grid), dim3(UF_T), 0, s, f, alpha_diff, ws_size,
+                       (const TK *) k_rows, slots, ld, n, repeat);
+}
+
 extern "C" {
 
-int tsvm_update_f(double *f, const double *alpha_diff, int ws_size, const double *k_rows, const int *slots,
-                  int64_t ld, int64_t n, tsvm_stream stream) {
+int tsvm_update_f(double *f, const double *alpha_diff, int ws_size, const void *k_rows, int row_type, const int *slots,
+                  int64_t ld, int64_t n_cols, int repeat, tsvm_stream stream) {
     TSVM_REQUIRE(f && alpha_diff && k_rows, "tsvm_update_f: null pointer");
-    TSVM_REQUIRE(ws_size >= 0 && n >= 0 && ld >= n, "tsvm_update_f: bad size (ws=%d n=%lld ld=%lld)", ws_size,
-                 (long long) n, (long long) ld);
-    if (n == 0 || ws_size == 0) return 0;
-    // 16-byte loads need every row start and f itself 16-byte aligned and an even column count
-    const bool vec2 = n % 2 == 0 && ld % 2 == 0 && ((uintptr_t) k_rows % 16 == 0) && ((uintptr_t) f % 16 == 0) &&
-                      n >= (int64_t) UF_T * 2 * 512;
-    if (vec2) {
-        const unsigned grid = (unsigned) ((n / 2 + UF_T - 1) / UF_T);
-        hipLaunchKernelGGL((update_f_kernel<2, 8>), dim3(grid), dim3(UF_T), 0, tsvm_s(stream), f, alpha_diff, ws_size,
-                           k_rows, slots, ld, n);
+    TSVM_REQUIRE(ws_size >= 0 && n_cols >= 0 && ld >= n_cols && repeat >= 1, "tsvm_update_f: bad size (ws=%d n=%lld ld=%lld)",
+                 ws_size, (long long) n_cols, (long long) ld);
+    TSVM_REQUIRE(row_type == TSVM_ROW_F64 || row_type == TSVM_ROW_F32, "tsvm_update_f: unknown row type %d", row_type);
+    if (n_cols == 0 || ws_size == 0) return 0;
+    const int64_t n = n_cols;
+    hipStream_t s = tsvm_s(stream);
+    // 16-byte loads need every row start 16-byte aligned and the last vector inside the padded row; with few
+    // columns one column per thread and more rows in flight keeps more of the chip busy
+    const bool big = n >= (int64_t) UF_T * 1024;
+    const bool aligned = (uintptr_t) k_rows % 16 == 0;
+    if (row_type == TSVM_ROW_F32) {
+        if (big && aligned && ld % 4 == 0 && ld >= (n + 3) / 4 * 4) launch_update_f<float, 4, 8>(f, alpha_diff, ws_size, k_rows, slots, ld, n, repeat, s);
+        else launch_update_f<float, 1, 32>(f, alpha_diff, ws_size, k_rows, slots, ld, n, repeat, s);
     } else {
-        const unsigned grid = (unsigned) ((n + UF_T - 1) / UF_T);
-        hipLaunchKernelGGL((update_f_kernel<1, 16>), dim3(grid), dim3(UF_T), 0, tsvm_s(stream), f, alpha_diff, ws_size,
-                           k_rows, slots, ld, n);
+        if (big && aligned && ld % 2 == 0 && ld >= (n + 1) / 2 * 2) launch_update_f<double, 2, 8>(f, alpha_diff, ws_size, k_rows, slots, ld, n, repeat, s);
+        else launch_update_f<double, 1, 16>(f, alpha_diff, ws_size, k_rows, slots, ld, n, repeat, s);
     }
     TSVM_LAUNCH_CHECK();
     return 0;

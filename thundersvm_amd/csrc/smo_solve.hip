@@ -35,11 +35,12 @@
 // reads, gathered once per call so that the two row reads per inner iteration
 // (smo_kernel.cpp:50-52,107-110) are contiguous; rows are padded to the solver's thread x slot grid
 // so every thread can load without a bounds test.
-__global__ void gather_ws_block_kernel(const double *__restrict__ k_rows, const int *__restrict__ slots, int64_t ld,
+template <typename TK>
+__global__ void gather_ws_block_kernel(const TK *__restrict__ k_rows, const int *__restrict__ slots, int64_t ld,
                                        const int *__restrict__ working_set, int ws, int ldk, double *__restrict__ kws) {
     const int r = blockIdx.x;
-    const double *row = k_rows + (int64_t) (slots ? slots[r] : r) * ld;
-    for (int t = threadIdx.x; t < ldk; t += blockDim.x) kws[(int64_t) r * ldk + t] = t < ws ? row[working_set[t]] : 0.0;
+    const TK *row = k_rows + (int64_t) (slots ? slots[r] : r) * ld;
+    for (int t = threadIdx.x; t < ldk; t += blockDim.x) kws[(int64_t) r * ldk + t] = t < ws ? (double) row[working_set[t]] : 0.0;
 }
 
 // Cross-wavefront combination of the per-wavefront (value, index) minima held in LDS.
@@ -415,20 +416,32 @@ size_t tsvm_smo_solve_workspace(int ws_size) {
     return sizeof(double) * (size_t) ws_size * (size_t) solver_ldk(ws_size) + 256;
 }
 
-static int launch_gather(const double *k_rows, const int *slots, int64_t ld, const int *working_set, int ws,
+static int launch_gather(const void *k_rows, int row_type, const int *slots, int64_t ld, const int *working_set, int ws,
                          void *workspace, hipStream_t s) {
-    hipLaunchKernelGGL(gather_ws_block_kernel, dim3(ws), dim3(256), 0, s, k_rows, slots, ld, working_set, ws,
-                       solver_ldk(ws), (double *) workspace);
+    TSVM_REQUIRE(row_type == TSVM_ROW_F64 || row_type == TSVM_ROW_F32, "smo_solve: unknown row type %d", row_type);
+    if (row_type == TSVM_ROW_F32)
+        hipLaunchKernelGGL(gather_ws_block_kernel<float>, dim3(ws), dim3(256), 0, s, (const float *) k_rows, slots, ld,
+                           working_set, ws, solver_ldk(ws), (double *) workspace);
+    else
+        hipLaunchKernelGGL(gather_ws_block_kernel<double>, dim3(ws), dim3(256), 0, s, (const double *) k_rows, slots, ld,
+                           working_set, ws, solver_ldk(ws), (double *) workspace);
     TSVM_LAUNCH_CHECK();
     return 0;
 }
 
+// The attribute query and the dynamic-LDS opt-in are made once per kernel and device, not per launch.
 #define TSVM_LAUNCH_SOLVER(KERNEL, EVAL, ...)                                                       \
     do {                                                                                            \
-        hipFuncAttributes fa_;                                                                      \
-        TSVM_HIP(hipFuncGetAttributes(&fa_, reinterpret_cast<const void *>(KERNEL<EVAL>)));         \
-        size_t dyn_ = 0;                                                                            \
-        TSVM_HIP(reserve_cu(KERNEL<EVAL>, fa_.sharedSizeBytes, &dyn_));                              \
+        static thread_local int dev_done_ = -1;                                                     \
+        static thread_local size_t dyn_ = 0;                                                        \
+        int dev_ = 0;                                                                               \
+        TSVM_HIP(hipGetDevice(&dev_));                                                              \
+        if (dev_done_ != dev_) {                                                                    \
+            hipFuncAttributes fa_;                                                                  \
+            TSVM_HIP(hipFuncGetAttributes(&fa_, reinterpret_cast<const void *>(KERNEL<EVAL>)));     \
+            TSVM_HIP(reserve_cu(KERNEL<EVAL>, fa_.sharedSizeBytes, &dyn_));                          \
+            dev_done_ = dev_;                                                                       \
+        }                                                                                           \
         hipLaunchKernelGGL(KERNEL<EVAL>, dim3(1), dim3(SV_T), dyn_, s, __VA_ARGS__);                 \
     } while (0)
 
@@ -440,14 +453,14 @@ static int launch_gather(const double *k_rows, const int *slots, int64_t ld, con
     } while (0)
 
 int tsvm_c_smo_solve(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
-                     int ws_size, double Cp, double Cn, const double *k_rows, const int *slots, int64_t ld,
+                     int ws_size, double Cp, double Cn, const void *k_rows, int row_type, const int *slots, int64_t ld,
                      const double *k_diag, double eps, double *diff, int max_iter, void *workspace,
                      tsvm_stream stream) {
     TSVM_REQUIRE(y && f_val && alpha && alpha_diff && working_set && k_rows && k_diag && diff && workspace,
                  "tsvm_c_smo_solve: null pointer");
     TSVM_REQUIRE(ws_size >= 1 && ws_size <= MAX_WS, "tsvm_c_smo_solve: ws_size %d outside [1, %d]", ws_size, MAX_WS);
     hipStream_t s = tsvm_s(stream);
-    int rc = launch_gather(k_rows, slots, ld, working_set, ws_size, workspace, s);
+    int rc = launch_gather(k_rows, row_type, slots, ld, working_set, ws_size, workspace, s);
     if (rc) return rc;
     const double *kws = (const double *) workspace;
     TSVM_DISPATCH_E(c_smo_solve_kernel, y, f_val, alpha, alpha_diff, working_set, ws_size, Cp, Cn, kws, k_diag, eps, diff,
@@ -483,14 +496,14 @@ int tsvm_nu_smo_solve_block(const int *y, const double *f_val, double *alpha, do
 }
 
 int tsvm_nu_smo_solve(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
-                      int ws_size, double C, const double *k_rows, const int *slots, int64_t ld,
+                      int ws_size, double C, const void *k_rows, int row_type, const int *slots, int64_t ld,
                       const double *k_diag, double eps, double *diff, int max_iter, void *workspace,
                       tsvm_stream stream) {
     TSVM_REQUIRE(y && f_val && alpha && alpha_diff && working_set && k_rows && k_diag && diff && workspace,
                  "tsvm_nu_smo_solve: null pointer");
     TSVM_REQUIRE(ws_size >= 1 && ws_size <= MAX_WS, "tsvm_nu_smo_solve: ws_size %d outside [1, %d]", ws_size, MAX_WS);
     hipStream_t s = tsvm_s(stream);
-    int rc = launch_gather(k_rows, slots, ld, working_set, ws_size, workspace, s);
+    int rc = launch_gather(k_rows, row_type, slots, ld, working_set, ws_size, workspace, s);
     if (rc) return rc;
     const double *kws = (const double *) workspace;
     TSVM_DISPATCH_E(nu_smo_solve_kernel, y, f_val, alpha, alpha_diff, working_set, ws_size, C, kws, k_diag, eps, diff,

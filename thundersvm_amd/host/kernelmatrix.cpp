@@ -80,10 +80,12 @@ KernelMatrix::KernelMatrix(const DataSet::node2d &all, const int *rows, size_t n
 }
 
 // CSR assembly on the host (kernelmatrix.cpp:183-207): n_features_ = largest feature id + 1, ids kept
-// as given.  `repeat` stacks the same rows several times (the 2n-row problem of SVR, svr.cpp:14-15).
+// as given.  With repeat > 1 the reference stacks the same rows several times (the 2n-row problem of
+// SVR, svr.cpp:14-15); here the rows are stored once.
 void KernelMatrix::build(const DataSet::node2d &all, const int *rows, size_t n_rows, int repeat) {
-    n_instances_ = n_rows * repeat;
-    std::vector<int64_t> ptr(n_instances_ + 1, 0);
+    n_unique_ = n_rows;
+    repeat_ = repeat;
+    std::vector<int64_t> ptr(n_rows + 1, 0);
     int max_index = 0;
 #pragma omp parallel for reduction(max : max_index) schedule(static)
     for (size_t r = 0; r < n_rows; ++r) {
@@ -92,10 +94,7 @@ void KernelMatrix::build(const DataSet::node2d &all, const int *rows, size_t n_r
         for (const auto &nd : row) max_index = std::max(max_index, nd.index);
     }
     for (size_t r = 0; r < n_rows; ++r) ptr[r + 1] += ptr[r];
-    const size_t total = (size_t) ptr[n_rows];
-    for (int rep = 1; rep < repeat; ++rep)
-        for (size_t r = 0; r < n_rows; ++r) ptr[rep * n_rows + r + 1] = ptr[r + 1] + (int64_t) (rep * total);
-    nnz_ = total * repeat;
+    nnz_ = (size_t) ptr[n_rows];
     n_features_ = (size_t) max_index + 1;
     std::vector<kernel_type> val(nnz_);
     std::vector<int> col(nnz_);
@@ -105,23 +104,22 @@ void KernelMatrix::build(const DataSet::node2d &all, const int *rows, size_t n_r
         size_t e = (size_t) ptr[r];
         for (const auto &nd : row) { val[e] = nd.value; col[e] = nd.index; ++e; }
     }
-    for (int rep = 1; rep < repeat; ++rep) {
-        std::copy(val.begin(), val.begin() + total, val.begin() + rep * total);
-        std::copy(col.begin(), col.begin() + total, col.begin() + rep * total);
-    }
     val_.upload(val);
     col_ind_.upload(col);
     row_ptr_.upload(ptr);
-    self_dot_.resize(n_instances_);
-    diag_.resize(n_instances_);
-    abi_check(tsvm_csr_self_dot(val_.data(), row_ptr_.data(), (int64_t) n_instances_, self_dot_.data(), nullptr));
-    abi_check(tsvm_kernel_diag(self_dot_.data(), (int64_t) n_instances_, (int) param.kernel_type, param.gamma, param.coef0,
+    self_dot_.resize(n_unique_);
+    diag_.resize(n_unique_ * repeat_);
+    abi_check(tsvm_csr_self_dot(val_.data(), row_ptr_.data(), (int64_t) n_unique_, self_dot_.data(), nullptr));
+    abi_check(tsvm_kernel_diag(self_dot_.data(), (int64_t) n_unique_, (int) param.kernel_type, param.gamma, param.coef0,
                                param.degree, diag_.data(), nullptr));
-    dense_ = choose_dense(n_instances_, n_features_, nnz_);
+    for (int rep = 1; rep < repeat_; ++rep)
+        TSVM_HIP_CHECK(hipMemcpyAsync(diag_.data() + rep * n_unique_, diag_.data(), n_unique_ * sizeof(kernel_type),
+                                      hipMemcpyDeviceToDevice, nullptr));
+    dense_ = choose_dense(n_unique_, n_features_, nnz_);
     if (dense_) {
         ld_ = (int64_t) ((n_features_ + 7) / 8 * 8);
-        x_.resize(n_instances_ * (size_t) ld_);
-        abi_check(tsvm_csr_to_dense(val_.data(), col_ind_.data(), row_ptr_.data(), (int64_t) n_instances_, x_.data(), ld_,
+        x_.resize(n_unique_ * (size_t) ld_);
+        abi_check(tsvm_csr_to_dense(val_.data(), col_ind_.data(), row_ptr_.data(), (int64_t) n_unique_, x_.data(), ld_,
                                     nullptr));
         TSVM_HIP_CHECK(hipDeviceSynchronize());
         val_.release();
@@ -130,13 +128,13 @@ void KernelMatrix::build(const DataSet::node2d &all, const int *rows, size_t n_r
     }
 }
 
-void KernelMatrix::get_rows(const int *d_idx, int m, kernel_type *d_out, int64_t ld, const int *d_out_slots,
+void KernelMatrix::get_rows(const int *d_idx, int m, void *d_out, int64_t ld, const int *d_out_slots,
                             hipStream_t stream) const {
-    const int n = (int) n_instances_;
+    const int n = (int) n_unique_;
     if (dense_) {
         abi_check(tsvm_get_rows_dense(x_.data(), ld_, nullptr, n, (int) n_features_, self_dot_.data(), x_.data(), ld_, d_idx,
                                       m, self_dot_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
-                                      d_out, d_out_slots, ld, stream));
+                                      d_out, row_type(), d_out_slots, ld, stream));
         return;
     }
     if (stage_.size() < (size_t) m * n_features_) stage_.resize((size_t) m * n_features_);
@@ -146,7 +144,7 @@ void KernelMatrix::get_rows(const int *d_idx, int m, kernel_type *d_out, int64_t
     abi_check(tsvm_gather_f64(self_dot_.data(), d_idx, m, stage_sd_.data(), stream));
     abi_check(tsvm_get_rows_csr(val_.data(), col_ind_.data(), row_ptr_.data(), nullptr, n, self_dot_.data(), stage_.data(),
                                 m, stage_sd_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree, d_out,
-                                d_out_slots, ld, stream));
+                                row_type(), d_out_slots, ld, stream));
 }
 
 // K(x_idx[r], x_idx[t]) for r, t < m: the same kernels with the column set restricted to the m rows,
@@ -155,7 +153,7 @@ void KernelMatrix::get_block(const int *d_idx, int m, kernel_type *d_out, int64_
     if (dense_) {
         abi_check(tsvm_get_rows_dense(x_.data(), ld_, d_idx, m, (int) n_features_, self_dot_.data(), x_.data(), ld_, d_idx, m,
                                       self_dot_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
-                                      d_out, nullptr, ld, stream));
+                                      d_out, TSVM_ROW_F64, nullptr, ld, stream));
         return;
     }
     if (stage_blk_.size() < (size_t) m * n_features_) stage_blk_.resize((size_t) m * n_features_);
@@ -165,12 +163,12 @@ void KernelMatrix::get_block(const int *d_idx, int m, kernel_type *d_out, int64_
     abi_check(tsvm_gather_f64(self_dot_.data(), d_idx, m, stage_blk_sd_.data(), stream));
     abi_check(tsvm_get_rows_csr(val_.data(), col_ind_.data(), row_ptr_.data(), d_idx, m, self_dot_.data(), stage_blk_.data(),
                                 m, stage_blk_sd_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
-                                d_out, nullptr, ld, stream));
+                                d_out, TSVM_ROW_F64, nullptr, ld, stream));
 }
 
 // External batch (kernelmatrix.cpp:281-312, 385-406): features with id >= n_features_ are left out of
 // the dot product but stay in the batch row's self dot.
-void KernelMatrix::get_rows(const DataSet::node2d &instances, kernel_type *d_out, int64_t ld) const {
+void KernelMatrix::get_rows(const DataSet::node2d &instances, void *d_out, int64_t ld) const {
     const int m = (int) instances.size();
     if (m == 0) return;
     std::vector<int64_t> ptr(m + 1, 0);
@@ -190,20 +188,20 @@ void KernelMatrix::get_rows(const DataSet::node2d &instances, kernel_type *d_out
     b_ptr_.upload(ptr.data(), m + 1);
     if (stage_sd_.size() < (size_t) m) stage_sd_.resize(m);
     abi_check(tsvm_csr_self_dot(b_val_.data(), b_ptr_.data(), m, stage_sd_.data(), nullptr));
-    const int n = (int) n_instances_;
+    const int n = (int) n_unique_;
     if (dense_) {
         if (stage_.size() < (size_t) m * ld_) stage_.resize((size_t) m * ld_);
         // columns >= n_features_ are dropped: the staging matrix is only n_features_ wide
         abi_check(tsvm_csr_to_dense(b_val_.data(), b_col_.data(), b_ptr_.data(), m, stage_.data(), ld_, nullptr));
         abi_check(tsvm_get_rows_dense(x_.data(), ld_, nullptr, n, (int) n_features_, self_dot_.data(), stage_.data(), ld_, nullptr, m,
                                       stage_sd_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
-                                      d_out, nullptr, ld, nullptr));
+                                      d_out, row_type(), nullptr, ld, nullptr));
     } else {
         if (stage_.size() < (size_t) m * n_features_) stage_.resize((size_t) m * n_features_);
         abi_check(tsvm_csr_stage_rows(b_val_.data(), b_col_.data(), b_ptr_.data(), nullptr, m, (int) n_features_,
                                       stage_.data(), nullptr));
         abi_check(tsvm_get_rows_csr(val_.data(), col_ind_.data(), row_ptr_.data(), nullptr, n, self_dot_.data(), stage_.data(), m,
                                     stage_sd_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
-                                    d_out, nullptr, ld, nullptr));
+                                    d_out, row_type(), nullptr, ld, nullptr));
     }
 }

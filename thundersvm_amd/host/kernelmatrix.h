@@ -5,6 +5,14 @@
 // Layout in HBM: either dense row-major fp64 [n][ld] (ld = n_features rounded up to 8, column c =
 // feature id c) for the MFMA path, or CSR (fp64 values, int32 columns, int64 row offsets) for the
 // sparse path.  The layout is chosen from the average row fill (see choose_dense()).
+//
+// A matrix built with repeat = r stands for the reference's r*n-row matrix made of the same n rows
+// stacked r times (SVR, svr.cpp:14-15).  Instance id i and i + n then have the same kernel row, and
+// that row consists of r identical n-column pieces: only the n unique rows are stored, and kernel
+// rows are produced under the folded id i % n, n columns wide.
+//
+// Kernel rows are produced as float for the RBF, polynomial and sigmoid kernels, whose values are
+// float-rounded by definition, and as double for the linear kernel (row_type()).
 #pragma once
 #include "dataset.h"
 #include "device.h"
@@ -16,17 +24,22 @@ public:
     // Rows `rows[0..n_rows)` of `all`, without materialising a node2d copy.
     KernelMatrix(const DataSet::node2d &all, const int *rows, size_t n_rows, SvmParam param, int repeat = 1);
 
-    // kernel rows of stored instances d_idx[0..m) (device ids) -> d_out[s_i*ld + j], s_i = d_out_slots[i] (or i)
-    void get_rows(const int *d_idx, int m, kernel_type *d_out, int64_t ld, const int *d_out_slots = nullptr,
+    // kernel rows of stored rows d_idx[0..m) (device, folded ids) -> element s_i*ld + j of d_out,
+    // s_i = d_out_slots[i] (or i), j < n_columns(); elements are row_type() wide
+    void get_rows(const int *d_idx, int m, void *d_out, int64_t ld, const int *d_out_slots = nullptr,
                   hipStream_t stream = nullptr) const;
-    // the m x m block K(x_idx[r], x_idx[t]) -> d_out[r*ld + t] (what the local solver reads)
+    // the m x m block K(x_idx[r], x_idx[t]) -> d_out[r*ld + t] (what the local solver reads; always double)
     void get_block(const int *d_idx, int m, kernel_type *d_out, int64_t ld, hipStream_t stream = nullptr) const;
-    // kernel rows of an external batch -> d_out[i*ld + j]
-    void get_rows(const DataSet::node2d &instances, kernel_type *d_out, int64_t ld) const;
+    // kernel rows of an external batch -> element i*ld + j of d_out (row_type() elements)
+    void get_rows(const DataSet::node2d &instances, void *d_out, int64_t ld) const;
 
-    const kernel_type *diag() const { return diag_.data(); }          // device
-    const kernel_type *self_dot() const { return self_dot_.data(); }  // device
-    size_t n_instances() const { return n_instances_; }
+    const kernel_type *diag() const { return diag_.data(); }          // device, n_instances() entries
+    const kernel_type *self_dot() const { return self_dot_.data(); }  // device, n_columns() entries
+    size_t n_instances() const { return n_unique_ * repeat_; }        // rows of the matrix the solver sees
+    size_t n_columns() const { return n_unique_; }                    // stored rows = columns of a kernel row
+    int repeat() const { return repeat_; }
+    int row_type() const { return param.kernel_type == SvmParam::LINEAR ? TSVM_ROW_F64 : TSVM_ROW_F32; }
+    size_t row_elem_size() const { return row_type() == TSVM_ROW_F32 ? sizeof(float) : sizeof(double); }
     size_t n_features() const { return n_features_; }
     size_t nnz() const { return nnz_; }
     bool dense_layout() const { return dense_; }
@@ -38,7 +51,8 @@ private:
     void build(const DataSet::node2d &all, const int *rows, size_t n_rows, int repeat);
 
     SvmParam param;
-    size_t n_instances_ = 0, n_features_ = 0, nnz_ = 0;
+    size_t n_unique_ = 0, n_features_ = 0, nnz_ = 0;
+    int repeat_ = 1;
     bool dense_ = false;
     int64_t ld_ = 0;
     tsvm::DeviceBuffer<kernel_type> x_;          // dense layout

@@ -86,13 +86,21 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
                        float_type &rho, std::vector<float_type> &f_val, float_type eps, float_type Cp, float_type Cn,
                        int ws_size, int out_max_iter) const {
     const int n = (int) k_mat.n_instances();
+    // Kernel rows are stored once per distinct data row: n_u columns wide, addressed by the folded id
+    // (id % n_u); f, alpha and y keep the reference's n = rep * n_u entries.
+    const int n_u = (int) k_mat.n_columns();
+    const int rep = k_mat.repeat();
+    const int row_type = k_mat.row_type();
+    const size_t row_esz = k_mat.row_elem_size();
     const int q = ws_size / 2;
-    const int64_t ld = ((int64_t) n + 1) / 2 * 2;   // even row stride keeps every kernel row 16-byte aligned
+    const int64_t ld = ((int64_t) n_u + 7) / 8 * 8;   // row stride in elements: rows stay 32-byte aligned
     const bool nu = is_nu();
     stats = SolverStats();
     const auto wall0 = std::chrono::steady_clock::now();
 
     DeviceBuffer<int> d_y(n), d_ws(ws_size), d_slots_a(ws_size), d_slots_b(ws_size), d_miss_ids(ws_size), d_miss_slots(ws_size);
+    DeviceBuffer<int> d_ws_folded(rep > 1 ? ws_size : 0);
+    const int *const ws_u = rep > 1 ? d_ws_folded.data() : d_ws.data();   // working set as folded ids
     DeviceBuffer<float_type> d_alpha(n), d_f(n), d_alpha_diff(ws_size), d_diff(2);
     DeviceBuffer<unsigned char> d_sel_ws(tsvm_select_workspace(n));
     const int ldk = tsvm_smo_solve_block_ld(ws_size);
@@ -108,22 +116,29 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
     // small launch; the full rows of the new working-set members are needed by update_f only.  With
     // overlap_streams the solver runs on stream `sa` while get_rows runs on stream `sb` and update_f
     // waits for both; by default (and always when profiling) everything is enqueued on one stream.
+    // A third stream only carries the read-back of the newly selected ids for the host-side cache
+    // bookkeeping, so that the host does that work while the local solver is already running.
     struct Streams {
-        hipStream_t a = nullptr, b = nullptr;
-        hipEvent_t selected = nullptr, rows_ready = nullptr;
+        hipStream_t a = nullptr, b = nullptr, ids = nullptr;
+        hipEvent_t selected = nullptr, rows_ready = nullptr, ids_ready = nullptr;
         bool two;
         explicit Streams(bool two_streams) : two(two_streams) {
             TSVM_HIP_CHECK(hipStreamCreateWithFlags(&a, hipStreamNonBlocking));
             if (two) TSVM_HIP_CHECK(hipStreamCreateWithFlags(&b, hipStreamNonBlocking)); else b = a;
+            TSVM_HIP_CHECK(hipStreamCreateWithFlags(&ids, hipStreamNonBlocking));
             TSVM_HIP_CHECK(hipEventCreateWithFlags(&selected, hipEventDisableTiming));
             TSVM_HIP_CHECK(hipEventCreateWithFlags(&rows_ready, hipEventDisableTiming));
+            TSVM_HIP_CHECK(hipEventCreateWithFlags(&ids_ready, hipEventDisableTiming));
         }
         ~Streams() {
             (void) hipStreamSynchronize(a);
             if (two) { (void) hipStreamSynchronize(b); (void) hipStreamDestroy(b); }
+            (void) hipStreamSynchronize(ids);
+            (void) hipStreamDestroy(ids);
             (void) hipStreamDestroy(a);
             (void) hipEventDestroy(selected);
             (void) hipEventDestroy(rows_ready);
+            (void) hipEventDestroy(ids_ready);
         }
     } st(overlap_streams && !profile);
     const hipStream_t sa = st.a, sb = st.b;
@@ -132,17 +147,17 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
     // host tracks which instance sits in which slot; without one it holds exactly ws rows.
     long long pool_rows = ws_size;
     tsvm::RowArena &arena = tsvm::RowArena::instance();
-    if (cache_bytes != 0 && n > ws_size) {
+    if (cache_bytes != 0 && n_u > ws_size) {
         const long long budget = cache_bytes > 0 ? cache_bytes : (long long) arena.auto_budget();
-        const long long fit = budget / (long long) (ld * sizeof(kernel_type));
+        const long long fit = budget / (long long) (ld * row_esz);
         // an LRU that can hold only a small part of the matrix does not hit: require a quarter of the rows
-        if (fit >= 4LL * ws_size && fit >= n / 4) pool_rows = std::min<long long>(n, fit);
+        if (fit >= 4LL * ws_size && fit >= n_u / 4) pool_rows = std::min<long long>(n_u, fit);
     }
     bool caching = pool_rows > ws_size;
-    kernel_type *const k_rows = (kernel_type *) arena.acquire((size_t) pool_rows * ld * sizeof(kernel_type), cache_bytes < 0);
+    void *const k_rows = arena.acquire((size_t) pool_rows * ld * row_esz, cache_bytes < 0);
     RowCache cache;
     if (caching) {
-        cache.init(n, (int) pool_rows);
+        cache.init(n_u, (int) pool_rows);
         stats.cache_rows = pool_rows;
     }
     std::vector<int> cur_slots(ws_size), cur_ids(ws_size), miss_ids, miss_slots;
@@ -183,12 +198,10 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
         trace->ws.clear();
     }
 
-    stats.ms_setup = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - wall0).count();
-    for (int iter = 0;; ++iter) {
-        const int n_new = iter == 0 ? ws_size : q;
-        const int first_new = iter == 0 ? 0 : q;
-        timer.begin();
-        if (iter == 0) {
+    // Working-set selection of iteration `it`: the first one picks ws_size ids, later ones keep the last
+    // half of the previous set and pick q new ids (csmosolver.cpp:63-77).
+    auto enqueue_select = [&](int it) {
+        if (it == 0) {
             abi_check(tsvm_select_working_set(d_f.data(), d_y.data(), d_alpha.data(), n, Cp, Cn, nullptr, 0, d_ws.data(),
                                               ws_size, nu, d_sel_ws.data(), sa));
         } else {
@@ -196,18 +209,35 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
             abi_check(tsvm_select_working_set(d_f.data(), d_y.data(), d_alpha.data(), n, Cp, Cn, d_ws.data(), q,
                                               d_ws.data() + q, q, nu, d_sel_ws.data(), sa));
         }
+        if (rep > 1) abi_check(tsvm_fold_ids(d_ws.data(), ws_size, n_u, d_ws_folded.data(), sa));
+    };
+    // The next selection is enqueued before the host has seen this iteration's diff, so the device goes
+    // straight from update_f into it; if the diff then says stop, that selection was simply not needed.
+    // (Not when tracing, which reads the working set back after each iteration, nor when profiling.)
+    const bool select_ahead = !trace && !profile;
+    bool select_enqueued = false;
+    hipEvent_t diff_ready = nullptr;
+    TSVM_HIP_CHECK(hipEventCreateWithFlags(&diff_ready, hipEventDisableTiming));
+
+    stats.ms_setup = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - wall0).count();
+    for (int iter = 0;; ++iter) {
+        const int n_new = iter == 0 ? ws_size : q;
+        const int first_new = iter == 0 ? 0 : q;
+        timer.begin();
+        if (!select_enqueued) enqueue_select(iter);
+        select_enqueued = false;
         timer.end(stats.ms_select);
         const int *slots;
+        TSVM_HIP_CHECK(hipEventRecord(st.selected, sa));
         if (caching) {
-            // read the new ids back, look them up, and compute only the rows that are not cached
-            TSVM_HIP_CHECK(hipMemcpyAsync(h_ids, d_ws.data() + first_new, sizeof(int) * n_new, hipMemcpyDeviceToHost, sa));
-            TSVM_HIP_CHECK(hipStreamSynchronize(sa));
-        } else {
-            TSVM_HIP_CHECK(hipEventRecord(st.selected, sa));
+            // the new ids travel to the host on their own stream while the solver below is enqueued and runs
+            TSVM_HIP_CHECK(hipStreamWaitEvent(st.ids, st.selected, 0));
+            TSVM_HIP_CHECK(hipMemcpyAsync(h_ids, d_ws.data() + first_new, sizeof(int) * n_new, hipMemcpyDeviceToHost, st.ids));
+            TSVM_HIP_CHECK(hipEventRecord(st.ids_ready, st.ids));
         }
         // the solver's ws x ws block and the solver itself go first on stream a ...
         timer.begin();
-        k_mat.get_block(d_ws.data(), ws_size, d_kws.data(), ldk, sa);
+        k_mat.get_block(ws_u, ws_size, d_kws.data(), ldk, sa);
         if (nu) {
             abi_check(tsvm_nu_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), d_ws.data(), ws_size,
                                               Cp, d_kws.data(), k_mat.diag(), eps, d_diff.data(), max_iter, sa));
@@ -219,6 +249,8 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
         // ... while the full rows of the new working-set members are produced on stream b
         timer.begin();
         if (caching) {
+            // look the new ids up and compute only the rows that are not cached
+            TSVM_HIP_CHECK(hipEventSynchronize(st.ids_ready));
             if (iter > 0) {
                 for (int t = 0; t < q; ++t) {   // rows kept from the previous working set stay most recently used
                     cur_ids[t] = cur_ids[t + q];
@@ -228,7 +260,7 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
             miss_ids.clear();
             miss_slots.clear();
             for (int t = 0; t < n_new; ++t) {
-                const int id = h_ids[t];
+                const int id = h_ids[t] % n_u;   // a second member with the same folded id hits the slot just assigned
                 int s = cache.lookup(id);
                 stats.cache_lookups++;
                 if (s >= 0) {
@@ -256,7 +288,7 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
             // A cache that has started evicting and still does not hit only costs the id read-back:
             // every 64 iterations, if fewer than 5 % of the window's lookups hit, fall back to rotation.
             // (A cache that can hold every row is never switched off: its misses are first touches.)
-            if (cache.cap < n && cache.used == cache.cap && iter % 64 == 63) {
+            if (cache.cap < n_u && cache.used == cache.cap && iter % 64 == 63) {
                 const long long dl = stats.cache_lookups - window_lookups, dh = stats.cache_hits - window_hits;
                 if (dh * 20 < dl) {
                     TSVM_HIP_CHECK(hipStreamSynchronize(sb));
@@ -272,7 +304,7 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
             slots = on_a ? d_slots_a.data() : d_slots_b.data();
             if (st.two) TSVM_HIP_CHECK(hipStreamWaitEvent(sb, st.selected, 0));
             // new rows go to the slots the dropped rows occupied
-            k_mat.get_rows(d_ws.data() + first_new, n_new, k_rows, ld, slots + first_new, sb);
+            k_mat.get_rows(ws_u + first_new, n_new, k_rows, ld, slots + first_new, sb);
         }
         if (st.two) {
             TSVM_HIP_CHECK(hipEventRecord(st.rows_ready, sb));
@@ -280,10 +312,15 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
         }
         timer.end(stats.ms_get_rows);
         timer.begin();
-        abi_check(tsvm_update_f(d_f.data(), d_alpha_diff.data(), ws_size, k_rows, slots, ld, n, sa));
+        abi_check(tsvm_update_f(d_f.data(), d_alpha_diff.data(), ws_size, k_rows, row_type, slots, ld, n_u, rep, sa));
         timer.end(stats.ms_update_f);
         TSVM_HIP_CHECK(hipMemcpyAsync(h_diff, d_diff.data(), 2 * sizeof(double), hipMemcpyDeviceToHost, sa));
-        TSVM_HIP_CHECK(hipStreamSynchronize(sa));
+        TSVM_HIP_CHECK(hipEventRecord(diff_ready, sa));
+        if (select_ahead) {
+            enqueue_select(iter + 1);
+            select_enqueued = true;
+        }
+        TSVM_HIP_CHECK(hipEventSynchronize(diff_ready));
         const double diff0 = h_diff[0], diff1 = h_diff[1];
         local_iter += (long long) diff1;
         if (trace && iter < trace->cap_iters) {
@@ -319,6 +356,8 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
             break;
         }
     }
+    TSVM_HIP_CHECK(hipStreamSynchronize(sa));   // a selection enqueued ahead may still be running
+    (void) hipEventDestroy(diff_ready);
     stats.ms_wall = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - wall0).count();
     (void) hipHostFree(h_diff);
     (void) hipHostFree(h_ids);
@@ -329,16 +368,16 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
 void CSMOSolver::init_f(const std::vector<float_type> &alpha, const std::vector<int> &y, const KernelMatrix &k_mat,
                         float_type *d_f) const {
     const size_t batch_size = 100;
-    const int n = (int) k_mat.n_instances();
-    const int64_t ld = ((int64_t) n + 1) / 2 * 2;
+    const int n_u = (int) k_mat.n_columns();
+    const int64_t ld = ((int64_t) n_u + 7) / 8 * 8;
     std::vector<int> idx_vec;
     std::vector<float_type> alpha_diff_vec;
     DeviceBuffer<int> d_idx;
     DeviceBuffer<float_type> d_ad;
-    DeviceBuffer<kernel_type> d_rows;
+    DeviceBuffer<unsigned char> d_rows;
     for (size_t i = 0; i < alpha.size(); ++i) {
         if (alpha[i] != 0) {
-            idx_vec.push_back((int) i);
+            idx_vec.push_back((int) (i % (size_t) n_u));
             alpha_diff_vec.push_back(-alpha[i] * y[i]);
         }
         if (idx_vec.size() > batch_size || (i == alpha.size() - 1 && !idx_vec.empty())) {
@@ -346,12 +385,12 @@ void CSMOSolver::init_f(const std::vector<float_type> &alpha, const std::vector<
             if (d_rows.size() == 0) {
                 d_idx.resize(batch_size + 1);
                 d_ad.resize(batch_size + 1);
-                d_rows.resize((batch_size + 1) * (size_t) ld);
+                d_rows.resize((batch_size + 1) * (size_t) ld * k_mat.row_elem_size());
             }
             d_idx.upload(idx_vec.data(), m);
             d_ad.upload(alpha_diff_vec.data(), m);
             k_mat.get_rows(d_idx.data(), m, d_rows.data(), ld);
-            abi_check(tsvm_update_f(d_f, d_ad.data(), m, d_rows.data(), nullptr, ld, n, nullptr));
+            abi_check(tsvm_update_f(d_f, d_ad.data(), m, d_rows.data(), k_mat.row_type(), nullptr, ld, n_u, k_mat.repeat(), nullptr));
             TSVM_HIP_CHECK(hipStreamSynchronize(nullptr));
             idx_vec.clear();
             alpha_diff_vec.clear();
