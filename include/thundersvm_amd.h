@@ -132,6 +132,12 @@ int tsvm_c_smo_solve(const int *y, const double *f_val, double *alpha, double *a
 /* Row stride (in doubles) of the ws x ws block the solver kernels read: ws rounded up to 256, 512 or 1024. */
 int tsvm_smo_solve_block_ld(int ws_size);
 
+/* The block from stored kernel rows: kws[r*ldk + t] = element cols[t] of the row in slot slots[r] (slots == NULL:
+ * slot r), r, t < ws_size, ldk = tsvm_smo_solve_block_ld(ws_size), columns t >= ws_size zero-filled; the gather that
+ * replaces the strided reads k_mat_rows[row_len*i + working_set[t]] of smo_kernel.cpp:50-52,107-110. */
+int tsvm_smo_gather_block(const void *k_rows, int row_type, const int *slots, int64_t ld, const int *cols, int ws_size,
+                          double *kws, tsvm_stream stream);
+
 /* c_smo_solve / nu_smo_solve on a precomputed block kws[r*ldk + t] = K(x_ws[r], x_ws[t]) (ldk from
  * tsvm_smo_solve_block_ld, columns t >= ws zero or arbitrary finite values): the solver touches nothing
  * else of the kernel matrix, so it can run while the full rows are still being computed on another

@@ -36,6 +36,7 @@ SIGNATURES = {
     "tsvm_c_smo_solve": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _dbl, _p, _int, _p, _i64, _p, _dbl, _p, _int, _p, _p]),
     "tsvm_nu_smo_solve": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _p, _int, _p, _i64, _p, _dbl, _p, _int, _p, _p]),
     "tsvm_smo_solve_block_ld": (_int, [_int]),
+    "tsvm_smo_gather_block": (_int, [_p, _int, _p, _i64, _p, _int, _p, _p]),
     "tsvm_c_smo_solve_block": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _dbl, _p, _p, _dbl, _p, _int, _p]),
     "tsvm_nu_smo_solve_block": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _p, _p, _dbl, _p, _int, _p]),
     "tsvm_select_workspace": (C.c_size_t, [_i64]),

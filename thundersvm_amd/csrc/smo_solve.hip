@@ -471,6 +471,13 @@ int tsvm_c_smo_solve(const int *y, const double *f_val, double *alpha, double *a
 
 int tsvm_smo_solve_block_ld(int ws_size) { return ws_size < 1 ? 0 : solver_ldk(ws_size); }
 
+int tsvm_smo_gather_block(const void *k_rows, int row_type, const int *slots, int64_t ld, const int *cols, int ws_size,
+                          double *kws, tsvm_stream stream) {
+    TSVM_REQUIRE(k_rows && cols && kws, "tsvm_smo_gather_block: null pointer");
+    TSVM_REQUIRE(ws_size >= 1 && ws_size <= MAX_WS, "tsvm_smo_gather_block: ws_size %d outside [1, %d]", ws_size, MAX_WS);
+    return launch_gather(k_rows, row_type, slots, ld, cols, ws_size, kws, tsvm_s(stream));
+}
+
 int tsvm_c_smo_solve_block(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
                            int ws_size, double Cp, double Cn, const double *kws, const double *k_diag, double eps,
                            double *diff, int max_iter, tsvm_stream stream) {

@@ -215,6 +215,7 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
     // straight from update_f into it; if the diff then says stop, that selection was simply not needed.
     // (Not when tracing, which reads the working set back after each iteration, nor when profiling.)
     const bool select_ahead = !trace && !profile;
+    const bool block_first = st.two || k_mat.n_features() < 256;
     bool select_enqueued = false;
     hipEvent_t diff_ready = nullptr;
     TSVM_HIP_CHECK(hipEventCreateWithFlags(&diff_ready, hipEventDisableTiming));
@@ -235,18 +236,28 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
             TSVM_HIP_CHECK(hipMemcpyAsync(h_ids, d_ws.data() + first_new, sizeof(int) * n_new, hipMemcpyDeviceToHost, st.ids));
             TSVM_HIP_CHECK(hipEventRecord(st.ids_ready, st.ids));
         }
-        // the solver's ws x ws block and the solver itself go first on stream a ...
-        timer.begin();
-        k_mat.get_block(ws_u, ws_size, d_kws.data(), ldk, sa);
-        if (nu) {
-            abi_check(tsvm_nu_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), d_ws.data(), ws_size,
-                                              Cp, d_kws.data(), k_mat.diag(), eps, d_diff.data(), max_iter, sa));
-        } else {
-            abi_check(tsvm_c_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), d_ws.data(), ws_size,
-                                             Cp, Cn, d_kws.data(), k_mat.diag(), eps, d_diff.data(), max_iter, sa));
-        }
-        timer.end(stats.ms_local);
-        // ... while the full rows of the new working-set members are produced on stream b
+        // The solver reads the ws x ws block of the kernel matrix.  With few features the block is cheap to
+        // compute on its own, ahead of the rows: the solver then already runs while the host does the cache
+        // bookkeeping (and, with two streams, while get_rows runs).  With many features that small launch
+        // (64 workgroups walking the whole feature range) costs more than it hides, and the block is
+        // gathered from the stored rows once they are complete.
+        auto enqueue_local = [&](const int *gather_slots, bool from_rows) {
+            timer.begin();
+            if (from_rows)
+                abi_check(tsvm_smo_gather_block(k_rows, row_type, gather_slots, ld, ws_u, ws_size, d_kws.data(), sa));
+            else
+                k_mat.get_block(ws_u, ws_size, d_kws.data(), ldk, sa);
+            if (nu) {
+                abi_check(tsvm_nu_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), d_ws.data(),
+                                                  ws_size, Cp, d_kws.data(), k_mat.diag(), eps, d_diff.data(), max_iter, sa));
+            } else {
+                abi_check(tsvm_c_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), d_ws.data(),
+                                                 ws_size, Cp, Cn, d_kws.data(), k_mat.diag(), eps, d_diff.data(), max_iter, sa));
+            }
+            timer.end(stats.ms_local);
+        };
+        if (block_first) enqueue_local(nullptr, false);
+        // the full rows of the new working-set members (on stream b when two streams are used)
         timer.begin();
         if (caching) {
             // look the new ids up and compute only the rows that are not cached
@@ -311,6 +322,7 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
             TSVM_HIP_CHECK(hipStreamWaitEvent(sa, st.rows_ready, 0));
         }
         timer.end(stats.ms_get_rows);
+        if (!block_first) enqueue_local(slots, true);
         timer.begin();
         abi_check(tsvm_update_f(d_f.data(), d_alpha_diff.data(), ws_size, k_rows, row_type, slots, ld, n_u, rep, sa));
         timer.end(stats.ms_update_f);
