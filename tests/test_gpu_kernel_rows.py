@@ -217,3 +217,27 @@ def test_output_row_slots():
     capi.call("tsvm_get_rows_csr", G.ptr(val_d), G.ptr(col_d), G.ptr(ptr_d), None, n, G.ptr(sd), G.ptr(w), m, G.ptr(sdw), O.RBF,
               0.2, 0.0, 3, G.ptr(out), capi.ROW_F64, G.ptr(slots_d), n, G.stream())
     assert np.array_equal(G.host(out)[slots], want)
+
+
+def test_row_subsets_on_device():
+    """tsvm_gather_rows_f64 / tsvm_csr_gather_rows: a class pair's rows taken from the resident data set."""
+    rng = np.random.default_rng(5)
+    n, d, m = 300, 21, 120
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    x[rng.random((n, d)) < 0.6] = 0
+    x[7] = 0                                     # an empty row
+    data = from_dense(x)
+    idx = rng.permutation(n)[:m].astype(np.int32)
+    idx[3] = 7
+    xh, nf, ld = G.dense_padded(data)
+    x_d, idx_d = G.dev(xh), G.dev(idx)
+    out = torch.empty((m, ld), dtype=torch.float64, device="cuda")
+    capi.call("tsvm_gather_rows_f64", G.ptr(x_d), ld, G.ptr(idx_d), m, G.ptr(out), G.stream())
+    assert np.array_equal(G.host(out), xh[idx])
+    sub = data.rows(idx)
+    val_d, col_d, ptr_d, optr_d = G.dev(data.val), G.dev(data.col), G.dev(data.ptr), G.dev(sub.ptr)
+    oval = torch.empty(sub.nnz, dtype=torch.float64, device="cuda")
+    ocol = torch.empty(sub.nnz, dtype=torch.int32, device="cuda")
+    capi.call("tsvm_csr_gather_rows", G.ptr(val_d), G.ptr(col_d), G.ptr(ptr_d), G.ptr(idx_d), m, G.ptr(optr_d), G.ptr(oval),
+              G.ptr(ocol), G.stream())
+    assert np.array_equal(G.host(oval), sub.val) and np.array_equal(G.host(ocol), sub.col)

@@ -164,7 +164,10 @@ def test_dataset_handle_and_file_loader(tmp_path):
     path = str(tmp_path / "c4.txt")
     D.save_libsvm(path, tr)
     c = Model(0).train(Dataset(path=path), prm)
-    for m in (b, c):
+    ds = Dataset(tr).to_device()          # rows uploaded once; both trainings below take them from HBM
+    d = Model(0).train(ds, prm)
+    e = Model(0).train(ds, prm)
+    for m in (b, c, d, e):
         assert np.array_equal(a.coef, m.coef) and np.array_equal(a.rho, m.rho) and np.array_equal(a.sv_indices, m.sv_indices)
     la, da = a.predict(tr)
     lb, db = b.predict(Dataset(tr))

@@ -30,6 +30,8 @@ SIGNATURES = {
     "tsvm_csr_stage_rows": (_int, [_p, _p, _p, _p, _int, _int, _p, _p]),
     "tsvm_get_rows_csr": (_int, [_p, _p, _p, _p, _i64, _p, _p, _int, _p, _int, _dbl, _dbl, _int, _p, _int, _p, _i64, _p]),
     "tsvm_fold_ids": (_int, [_p, _int, _int, _p, _p]),
+    "tsvm_gather_rows_f64": (_int, [_p, _i64, _p, _i64, _p, _p]),
+    "tsvm_csr_gather_rows": (_int, [_p, _p, _p, _p, _i64, _p, _p, _p, _p]),
     "tsvm_gather_f64": (_int, [_p, _p, _int, _p, _p]),
     "tsvm_update_f": (_int, [_p, _p, _int, _p, _int, _p, _i64, _i64, _int, _p]),
     "tsvm_smo_solve_workspace": (C.c_size_t, [_int]),

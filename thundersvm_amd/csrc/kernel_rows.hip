@@ -6,6 +6,8 @@
 #include "tsvm_device.h"
 #include "tsvm_internal.h"
 
+#include <algorithm>
+
 typedef double v4d __attribute__((ext_vector_type(4)));
 
 // ------------------------------------------------------------------------------------------------
@@ -227,6 +229,31 @@ __global__ __launch_bounds__(256) void get_rows_csr_kernel(
     for (int jj = 0; jj < CS_JB; ++jj) {
         const int64_t j = j0 + jj;
         if (j < n) orow[j] = (TO) tsvm_epilogue(acc[jj], sdi, sd_x ? sd_x[x_idx ? (int64_t) x_idx[j] : j] : 0.0, kp, exp_tab);
+    }
+}
+
+// out row r = x row idx[r]; rows are ld doubles long, ld a multiple of 4, moved as 32-byte vectors
+__global__ void gather_rows_f64_kernel(const v4d *__restrict__ x, int64_t ld4, const int *__restrict__ idx, int64_t m,
+                                       v4d *__restrict__ out) {
+    const int64_t total = m * ld4;
+    for (int64_t e = (int64_t) blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (int64_t) gridDim.x * blockDim.x) {
+        const int64_t r = e / ld4, c = e % ld4;
+        out[e] = x[(int64_t) idx[r] * ld4 + c];
+    }
+}
+
+// CSR rows idx[0..m) copied to a new CSR whose row offsets out_ptr are already known; one wavefront per row
+__global__ void csr_gather_rows_kernel(const double *__restrict__ val, const int *__restrict__ col,
+                                       const int64_t *__restrict__ row_ptr, const int *__restrict__ idx, int64_t m,
+                                       const int64_t *__restrict__ out_ptr, double *__restrict__ out_val,
+                                       int *__restrict__ out_col) {
+    const int64_t r = ((int64_t) blockIdx.x * blockDim.x + threadIdx.x) / 64;
+    const int lane = threadIdx.x & 63;
+    if (r >= m) return;
+    const int64_t src = row_ptr[idx[r]], dst = out_ptr[r], len = out_ptr[r + 1] - dst;
+    for (int64_t e = lane; e < len; e += 64) {
+        out_val[dst + e] = val[src + e];
+        out_col[dst + e] = col[src + e];
     }
 }
 
@@ -510,6 +537,27 @@ int tsvm_get_rows_csr(const double *val, const int *col, const int64_t *row_ptr,
     else
         hipLaunchKernelGGL(get_rows_csr_kernel<double>, dim3((unsigned) (j_blocks * i_blocks)), dim3(256), 0, tsvm_s(stream), val,
                            col, row_ptr, x_idx, n, sd_x, w, m, sd_w, kp, (double *) out, out_slots, ldo, i_blocks);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+int tsvm_gather_rows_f64(const double *x, int64_t ld, const int *idx, int64_t m, double *out, tsvm_stream stream) {
+    TSVM_REQUIRE(x && idx && out && m >= 0 && ld > 0 && ld % 4 == 0, "tsvm_gather_rows_f64: bad argument");
+    TSVM_REQUIRE(((uintptr_t) x % 32 == 0) && ((uintptr_t) out % 32 == 0), "tsvm_gather_rows_f64: x and out must be 32-byte aligned");
+    if (m == 0) return 0;
+    const int64_t total = m * (ld / 4);
+    const unsigned grid = (unsigned) std::min<int64_t>((total + 255) / 256, 65536);
+    hipLaunchKernelGGL(gather_rows_f64_kernel, dim3(grid), dim3(256), 0, tsvm_s(stream), (const v4d *) x, ld / 4, idx, m, (v4d *) out);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+int tsvm_csr_gather_rows(const double *val, const int *col, const int64_t *row_ptr, const int *idx, int64_t m,
+                         const int64_t *out_ptr, double *out_val, int *out_col, tsvm_stream stream) {
+    TSVM_REQUIRE(row_ptr && idx && out_ptr && m >= 0, "tsvm_csr_gather_rows: bad argument");
+    if (m == 0) return 0;
+    hipLaunchKernelGGL(csr_gather_rows_kernel, dim3(grid_for(m * 64, 256)), dim3(256), 0, tsvm_s(stream), val, col, row_ptr, idx,
+                       m, out_ptr, out_val, out_col);
     TSVM_LAUNCH_CHECK();
     return 0;
 }

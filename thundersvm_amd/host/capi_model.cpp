@@ -114,6 +114,15 @@ void *tsvm_dataset_load(const char *libsvm_file) {
     }
 }
 
+int tsvm_dataset_to_device(void *dataset) {
+    try {
+        (void) DeviceRows::of(*(DataSet *) dataset);
+        return 0;
+    } catch (const std::exception &e) {
+        return fail(e);
+    }
+}
+
 void tsvm_dataset_free(void *dataset) { delete (DataSet *) dataset; }
 int64_t tsvm_dataset_rows(void *dataset) { return (int64_t) ((DataSet *) dataset)->n_instances(); }
 

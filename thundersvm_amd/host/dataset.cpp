@@ -12,6 +12,7 @@ DataSet::DataSet(const node2d &instances, int n_features, const std::vector<floa
 // One pass over the file text.  Each token "i:v" is parsed the way the reference's sscanf("%d:%f")
 // does: v goes through float (src/thundersvm/dataset.cpp:72-80).  Row order is file order.
 void DataSet::load_from_file(std::string file_name) {
+    device_slot_ = std::make_shared<std::shared_ptr<void>>();   // new instances: any device copy is stale
     y_.clear();
     instances_.clear();
     n_features_ = 0;
@@ -51,6 +52,7 @@ void DataSet::load_from_file(std::string file_name) {
 }
 
 void DataSet::load_from_python(float *y, char **x, int len) {
+    device_slot_ = std::make_shared<std::shared_ptr<void>>();   // new instances: any device copy is stale
     y_.clear();
     instances_.clear();
     n_features_ = 0;
@@ -70,6 +72,7 @@ void DataSet::load_from_python(float *y, char **x, int len) {
 }
 
 void DataSet::load_from_sparse(int row_size, float *val, int *row_ptr, int *col_ptr, float *label) {
+    device_slot_ = std::make_shared<std::shared_ptr<void>>();   // new instances: any device copy is stale
     y_.clear();
     instances_.assign(row_size, {});
     n_features_ = 0;
@@ -84,6 +87,7 @@ void DataSet::load_from_sparse(int row_size, float *val, int *row_ptr, int *col_
 }
 
 void DataSet::load_from_dense(int row_size, int features, float *data, float *label) {
+    device_slot_ = std::make_shared<std::shared_ptr<void>>();   // new instances: any device copy is stale
     y_.clear();
     instances_.assign(row_size, {});
     for (int r = 0; r < row_size; ++r) {
@@ -95,6 +99,7 @@ void DataSet::load_from_dense(int row_size, int features, float *data, float *la
 }
 
 void DataSet::load_from_csr(int64_t n, const int64_t *row_ptr, const int *col, const double *val, const double *y) {
+    device_slot_ = std::make_shared<std::shared_ptr<void>>();   // new instances: any device copy is stale
     y_.clear();
     instances_.assign(n, {});
     n_features_ = 0;
@@ -149,6 +154,7 @@ DataSet DataSet::grouped_view() const {
     v.n_features_ = n_features_;
     v.zero_based_ = zero_based_;
     v.base_ = base_ ? base_ : &instances_;
+    v.device_slot_ = device_slot_;   // same instances, same device copy
     v.group_classes(true);
     return v;
 }

@@ -2,6 +2,8 @@
 // Same public surface as include/thundersvm/dataset.h; values are float32-rounded on load
 // (src/thundersvm/dataset.cpp:76-79) and held as kernel_type.
 #pragma once
+#include <memory>
+
 #include "thundersvm.h"
 
 class DataSet {
@@ -40,6 +42,10 @@ public:
     const std::vector<int> original_index(int y_i) const;
     const std::vector<int> original_index(int y_i, int y_j) const;
     bool is_zero_based() const { return zero_based_; }
+    // Slot for a device-resident copy of instances(), filled by the first KernelMatrix built from this
+    // DataSet (or by whoever wants the upload to happen early) and shared with its grouped views.  It is
+    // dropped when the instances are reloaded.
+    std::shared_ptr<void> &device_cache() const { return *device_slot_; }
 
 private:
     std::vector<float_type> y_;
@@ -48,4 +54,5 @@ private:
     size_t n_features_ = 0;
     std::vector<int> start_, count_, label_, perm_;
     bool zero_based_ = false;
+    mutable std::shared_ptr<std::shared_ptr<void>> device_slot_ = std::make_shared<std::shared_ptr<void>>();
 };

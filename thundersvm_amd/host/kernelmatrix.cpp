@@ -70,79 +70,136 @@ bool KernelMatrix::choose_dense(size_t n, size_t n_features, size_t nnz) {
     return (double) ld <= 32.0 * std::max(avg, 1.0);
 }
 
+// CSR assembly on the host (kernelmatrix.cpp:183-207): n_features = largest feature id + 1, ids kept
+// as given; self dot products from the CSR values in stored order; then the layout is chosen.
+std::shared_ptr<DeviceRows> DeviceRows::from_host(const DataSet::node2d &all, const int *rows, size_t n_rows) {
+    auto out = std::make_shared<DeviceRows>();
+    DeviceRows &r = *out;
+    r.n = n_rows;
+    std::vector<int64_t> ptr(n_rows + 1, 0);
+    int max_index = 0;
+#pragma omp parallel for reduction(max : max_index) schedule(static)
+    for (size_t i = 0; i < n_rows; ++i) {
+        const auto &row = all[rows ? rows[i] : i];
+        ptr[i + 1] = (int64_t) row.size();
+        for (const auto &nd : row) max_index = std::max(max_index, nd.index);
+    }
+    for (size_t i = 0; i < n_rows; ++i) ptr[i + 1] += ptr[i];
+    r.nnz = (size_t) ptr[n_rows];
+    r.n_features = (size_t) max_index + 1;
+    std::vector<kernel_type> val(r.nnz);
+    std::vector<int> col(r.nnz);
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < n_rows; ++i) {
+        const auto &row = all[rows ? rows[i] : i];
+        size_t e = (size_t) ptr[i];
+        for (const auto &nd : row) { val[e] = nd.value; col[e] = nd.index; ++e; }
+    }
+    r.val.upload(val);
+    r.col.upload(col);
+    r.row_ptr.upload(ptr);
+    r.self_dot.resize(r.n);
+    abi_check(tsvm_csr_self_dot(r.val.data(), r.row_ptr.data(), (int64_t) r.n, r.self_dot.data(), nullptr));
+    r.dense = KernelMatrix::choose_dense(r.n, r.n_features, r.nnz);
+    if (r.dense) {
+        r.ld = (int64_t) ((r.n_features + 7) / 8 * 8);
+        r.x.resize(r.n * (size_t) r.ld);
+        abi_check(tsvm_csr_to_dense(r.val.data(), r.col.data(), r.row_ptr.data(), (int64_t) r.n, r.x.data(), r.ld, nullptr));
+        TSVM_HIP_CHECK(hipDeviceSynchronize());
+        r.val.release();
+        r.col.release();
+        r.row_ptr.release();
+    } else {
+        r.host_row_ptr = std::move(ptr);
+    }
+    return out;
+}
+
+std::shared_ptr<DeviceRows> DeviceRows::subset(const DeviceRows &base, const int *rows, size_t n_rows) {
+    auto out = std::make_shared<DeviceRows>();
+    DeviceRows &r = *out;
+    r.n = n_rows;
+    r.n_features = base.n_features;
+    r.dense = base.dense;
+    r.ld = base.ld;
+    tsvm::DeviceBuffer<int> d_rows(n_rows);
+    d_rows.upload(rows, n_rows);
+    r.self_dot.resize(n_rows);
+    abi_check(tsvm_gather_f64(base.self_dot.data(), d_rows.data(), (int) n_rows, r.self_dot.data(), nullptr));
+    if (base.dense) {
+        r.x.resize(n_rows * (size_t) r.ld);
+        abi_check(tsvm_gather_rows_f64(base.x.data(), base.ld, d_rows.data(), (int64_t) n_rows, r.x.data(), nullptr));
+        r.nnz = n_rows ? base.nnz / std::max<size_t>(base.n, 1) * n_rows : 0;   // estimate, informational only
+    } else {
+        r.host_row_ptr.assign(n_rows + 1, 0);
+        for (size_t i = 0; i < n_rows; ++i)
+            r.host_row_ptr[i + 1] = r.host_row_ptr[i] + base.host_row_ptr[rows[i] + 1] - base.host_row_ptr[rows[i]];
+        r.nnz = (size_t) r.host_row_ptr[n_rows];
+        r.row_ptr.upload(r.host_row_ptr);
+        r.val.resize(r.nnz);
+        r.col.resize(r.nnz);
+        abi_check(tsvm_csr_gather_rows(base.val.data(), base.col.data(), base.row_ptr.data(), d_rows.data(), (int64_t) n_rows,
+                                       r.row_ptr.data(), r.val.data(), r.col.data(), nullptr));
+    }
+    TSVM_HIP_CHECK(hipDeviceSynchronize());   // d_rows is released on return
+    return out;
+}
+
+std::shared_ptr<DeviceRows> DeviceRows::of(const DataSet &dataset) {
+    std::shared_ptr<void> &slot = dataset.device_cache();
+    if (!slot) slot = from_host(dataset.instances(), nullptr, dataset.instances().size());
+    return std::static_pointer_cast<DeviceRows>(slot);
+}
+
 KernelMatrix::KernelMatrix(const DataSet::node2d &instances, SvmParam param) : param(param) {
-    build(instances, nullptr, instances.size(), 1);
+    rows_ = DeviceRows::from_host(instances, nullptr, instances.size());
+    finish(1);
 }
 
 KernelMatrix::KernelMatrix(const DataSet::node2d &all, const int *rows, size_t n_rows, SvmParam param, int repeat)
     : param(param) {
-    build(all, rows, n_rows, repeat);
+    rows_ = DeviceRows::from_host(all, rows, n_rows);
+    finish(repeat);
 }
 
-// CSR assembly on the host (kernelmatrix.cpp:183-207): n_features_ = largest feature id + 1, ids kept
-// as given.  With repeat > 1 the reference stacks the same rows several times (the 2n-row problem of
-// SVR, svr.cpp:14-15); here the rows are stored once.
-void KernelMatrix::build(const DataSet::node2d &all, const int *rows, size_t n_rows, int repeat) {
-    n_unique_ = n_rows;
+KernelMatrix::KernelMatrix(const DataSet &dataset, const int *rows, size_t n_rows, SvmParam param, int repeat)
+    : param(param) {
+    std::shared_ptr<DeviceRows> all = DeviceRows::of(dataset);
+    rows_ = rows ? DeviceRows::subset(*all, rows, n_rows) : all;
+    finish(repeat);
+}
+
+// diag from the self dot products (kernelmatrix.cpp:225-247).  With repeat > 1 the reference stacks the
+// same rows several times (the 2n-row problem of SVR, svr.cpp:14-15); here the rows are stored once and
+// only the diagonal, which the solver kernels index by instance id, is replicated.
+void KernelMatrix::finish(int repeat) {
+    n_unique_ = rows_->n;
     repeat_ = repeat;
-    std::vector<int64_t> ptr(n_rows + 1, 0);
-    int max_index = 0;
-#pragma omp parallel for reduction(max : max_index) schedule(static)
-    for (size_t r = 0; r < n_rows; ++r) {
-        const auto &row = all[rows ? rows[r] : r];
-        ptr[r + 1] = (int64_t) row.size();
-        for (const auto &nd : row) max_index = std::max(max_index, nd.index);
-    }
-    for (size_t r = 0; r < n_rows; ++r) ptr[r + 1] += ptr[r];
-    nnz_ = (size_t) ptr[n_rows];
-    n_features_ = (size_t) max_index + 1;
-    std::vector<kernel_type> val(nnz_);
-    std::vector<int> col(nnz_);
-#pragma omp parallel for schedule(static)
-    for (size_t r = 0; r < n_rows; ++r) {
-        const auto &row = all[rows ? rows[r] : r];
-        size_t e = (size_t) ptr[r];
-        for (const auto &nd : row) { val[e] = nd.value; col[e] = nd.index; ++e; }
-    }
-    val_.upload(val);
-    col_ind_.upload(col);
-    row_ptr_.upload(ptr);
-    self_dot_.resize(n_unique_);
     diag_.resize(n_unique_ * repeat_);
-    abi_check(tsvm_csr_self_dot(val_.data(), row_ptr_.data(), (int64_t) n_unique_, self_dot_.data(), nullptr));
-    abi_check(tsvm_kernel_diag(self_dot_.data(), (int64_t) n_unique_, (int) param.kernel_type, param.gamma, param.coef0,
+    abi_check(tsvm_kernel_diag(rows_->self_dot.data(), (int64_t) n_unique_, (int) param.kernel_type, param.gamma, param.coef0,
                                param.degree, diag_.data(), nullptr));
     for (int rep = 1; rep < repeat_; ++rep)
         TSVM_HIP_CHECK(hipMemcpyAsync(diag_.data() + rep * n_unique_, diag_.data(), n_unique_ * sizeof(kernel_type),
                                       hipMemcpyDeviceToDevice, nullptr));
-    dense_ = choose_dense(n_unique_, n_features_, nnz_);
-    if (dense_) {
-        ld_ = (int64_t) ((n_features_ + 7) / 8 * 8);
-        x_.resize(n_unique_ * (size_t) ld_);
-        abi_check(tsvm_csr_to_dense(val_.data(), col_ind_.data(), row_ptr_.data(), (int64_t) n_unique_, x_.data(), ld_,
-                                    nullptr));
-        TSVM_HIP_CHECK(hipDeviceSynchronize());
-        val_.release();
-        col_ind_.release();
-        row_ptr_.release();
-    }
+    TSVM_HIP_CHECK(hipDeviceSynchronize());
 }
 
 void KernelMatrix::get_rows(const int *d_idx, int m, void *d_out, int64_t ld, const int *d_out_slots,
                             hipStream_t stream) const {
+    const DeviceRows &R = *rows_;
     const int n = (int) n_unique_;
-    if (dense_) {
-        abi_check(tsvm_get_rows_dense(x_.data(), ld_, nullptr, n, (int) n_features_, self_dot_.data(), x_.data(), ld_, d_idx,
-                                      m, self_dot_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
+    if (R.dense) {
+        abi_check(tsvm_get_rows_dense(R.x.data(), R.ld, nullptr, n, (int) R.n_features, R.self_dot.data(), R.x.data(), R.ld, d_idx,
+                                      m, R.self_dot.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
                                       d_out, row_type(), d_out_slots, ld, stream));
         return;
     }
-    if (stage_.size() < (size_t) m * n_features_) stage_.resize((size_t) m * n_features_);
+    if (stage_.size() < (size_t) m * R.n_features) stage_.resize((size_t) m * R.n_features);
     if (stage_sd_.size() < (size_t) m) stage_sd_.resize(m);
-    abi_check(tsvm_csr_stage_rows(val_.data(), col_ind_.data(), row_ptr_.data(), d_idx, m, (int) n_features_,
+    abi_check(tsvm_csr_stage_rows(R.val.data(), R.col.data(), R.row_ptr.data(), d_idx, m, (int) R.n_features,
                                   stage_.data(), stream));
-    abi_check(tsvm_gather_f64(self_dot_.data(), d_idx, m, stage_sd_.data(), stream));
-    abi_check(tsvm_get_rows_csr(val_.data(), col_ind_.data(), row_ptr_.data(), nullptr, n, self_dot_.data(), stage_.data(),
+    abi_check(tsvm_gather_f64(R.self_dot.data(), d_idx, m, stage_sd_.data(), stream));
+    abi_check(tsvm_get_rows_csr(R.val.data(), R.col.data(), R.row_ptr.data(), nullptr, n, R.self_dot.data(), stage_.data(),
                                 m, stage_sd_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree, d_out,
                                 row_type(), d_out_slots, ld, stream));
 }
@@ -150,25 +207,27 @@ void KernelMatrix::get_rows(const int *d_idx, int m, void *d_out, int64_t ld, co
 // K(x_idx[r], x_idx[t]) for r, t < m: the same kernels with the column set restricted to the m rows,
 // so every value is bit-identical to the corresponding entry of a full kernel row.
 void KernelMatrix::get_block(const int *d_idx, int m, kernel_type *d_out, int64_t ld, hipStream_t stream) const {
-    if (dense_) {
-        abi_check(tsvm_get_rows_dense(x_.data(), ld_, d_idx, m, (int) n_features_, self_dot_.data(), x_.data(), ld_, d_idx, m,
-                                      self_dot_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
+    const DeviceRows &R = *rows_;
+    if (R.dense) {
+        abi_check(tsvm_get_rows_dense(R.x.data(), R.ld, d_idx, m, (int) R.n_features, R.self_dot.data(), R.x.data(), R.ld, d_idx, m,
+                                      R.self_dot.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
                                       d_out, TSVM_ROW_F64, nullptr, ld, stream));
         return;
     }
-    if (stage_blk_.size() < (size_t) m * n_features_) stage_blk_.resize((size_t) m * n_features_);
+    if (stage_blk_.size() < (size_t) m * R.n_features) stage_blk_.resize((size_t) m * R.n_features);
     if (stage_blk_sd_.size() < (size_t) m) stage_blk_sd_.resize(m);
-    abi_check(tsvm_csr_stage_rows(val_.data(), col_ind_.data(), row_ptr_.data(), d_idx, m, (int) n_features_,
+    abi_check(tsvm_csr_stage_rows(R.val.data(), R.col.data(), R.row_ptr.data(), d_idx, m, (int) R.n_features,
                                   stage_blk_.data(), stream));
-    abi_check(tsvm_gather_f64(self_dot_.data(), d_idx, m, stage_blk_sd_.data(), stream));
-    abi_check(tsvm_get_rows_csr(val_.data(), col_ind_.data(), row_ptr_.data(), d_idx, m, self_dot_.data(), stage_blk_.data(),
+    abi_check(tsvm_gather_f64(R.self_dot.data(), d_idx, m, stage_blk_sd_.data(), stream));
+    abi_check(tsvm_get_rows_csr(R.val.data(), R.col.data(), R.row_ptr.data(), d_idx, m, R.self_dot.data(), stage_blk_.data(),
                                 m, stage_blk_sd_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
                                 d_out, TSVM_ROW_F64, nullptr, ld, stream));
 }
 
-// External batch (kernelmatrix.cpp:281-312, 385-406): features with id >= n_features_ are left out of
+// External batch (kernelmatrix.cpp:281-312, 385-406): features with id >= R.n_features are left out of
 // the dot product but stay in the batch row's self dot.
 void KernelMatrix::get_rows(const DataSet::node2d &instances, void *d_out, int64_t ld) const {
+    const DeviceRows &R = *rows_;
     const int m = (int) instances.size();
     if (m == 0) return;
     std::vector<int64_t> ptr(m + 1, 0);
@@ -189,18 +248,18 @@ void KernelMatrix::get_rows(const DataSet::node2d &instances, void *d_out, int64
     if (stage_sd_.size() < (size_t) m) stage_sd_.resize(m);
     abi_check(tsvm_csr_self_dot(b_val_.data(), b_ptr_.data(), m, stage_sd_.data(), nullptr));
     const int n = (int) n_unique_;
-    if (dense_) {
-        if (stage_.size() < (size_t) m * ld_) stage_.resize((size_t) m * ld_);
-        // columns >= n_features_ are dropped: the staging matrix is only n_features_ wide
-        abi_check(tsvm_csr_to_dense(b_val_.data(), b_col_.data(), b_ptr_.data(), m, stage_.data(), ld_, nullptr));
-        abi_check(tsvm_get_rows_dense(x_.data(), ld_, nullptr, n, (int) n_features_, self_dot_.data(), stage_.data(), ld_, nullptr, m,
+    if (R.dense) {
+        if (stage_.size() < (size_t) m * R.ld) stage_.resize((size_t) m * R.ld);
+        // columns >= R.n_features are dropped: the staging matrix is only R.n_features wide
+        abi_check(tsvm_csr_to_dense(b_val_.data(), b_col_.data(), b_ptr_.data(), m, stage_.data(), R.ld, nullptr));
+        abi_check(tsvm_get_rows_dense(R.x.data(), R.ld, nullptr, n, (int) R.n_features, R.self_dot.data(), stage_.data(), R.ld, nullptr, m,
                                       stage_sd_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
                                       d_out, row_type(), nullptr, ld, nullptr));
     } else {
-        if (stage_.size() < (size_t) m * n_features_) stage_.resize((size_t) m * n_features_);
-        abi_check(tsvm_csr_stage_rows(b_val_.data(), b_col_.data(), b_ptr_.data(), nullptr, m, (int) n_features_,
+        if (stage_.size() < (size_t) m * R.n_features) stage_.resize((size_t) m * R.n_features);
+        abi_check(tsvm_csr_stage_rows(b_val_.data(), b_col_.data(), b_ptr_.data(), nullptr, m, (int) R.n_features,
                                       stage_.data(), nullptr));
-        abi_check(tsvm_get_rows_csr(val_.data(), col_ind_.data(), row_ptr_.data(), nullptr, n, self_dot_.data(), stage_.data(), m,
+        abi_check(tsvm_get_rows_csr(R.val.data(), R.col.data(), R.row_ptr.data(), nullptr, n, R.self_dot.data(), stage_.data(), m,
                                     stage_sd_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
                                     d_out, row_type(), nullptr, ld, nullptr));
     }

@@ -18,11 +18,38 @@
 #include "device.h"
 #include "svmparam.h"
 
+// A set of data rows resident in HBM (either layout) with their self dot products; what a KernelMatrix
+// multiplies against.  A DataSet keeps one for all of its instances (DeviceRows::of), so that the
+// one-vs-one sub-problems of a multi-class run take their rows from HBM with a device-side gather
+// instead of being assembled on the host and uploaded once per class pair.
+struct DeviceRows {
+    size_t n = 0, n_features = 0, nnz = 0;
+    bool dense = false;
+    int64_t ld = 0;                              // dense row stride (n_features rounded up to 8)
+    tsvm::DeviceBuffer<kernel_type> x;           // dense layout [n][ld]
+    tsvm::DeviceBuffer<kernel_type> val;         // CSR layout
+    tsvm::DeviceBuffer<int> col;
+    tsvm::DeviceBuffer<int64_t> row_ptr;
+    std::vector<int64_t> host_row_ptr;           // CSR layout only: needed to lay out a subset
+    tsvm::DeviceBuffer<kernel_type> self_dot;    // [n]
+
+    // rows[0..n_rows) of `all` (rows == nullptr: the first n_rows), assembled on the host and uploaded
+    static std::shared_ptr<DeviceRows> from_host(const DataSet::node2d &all, const int *rows, size_t n_rows);
+    // rows[0..n_rows) of `base`, gathered on the device; keeps base's layout and feature count
+    static std::shared_ptr<DeviceRows> subset(const DeviceRows &base, const int *rows, size_t n_rows);
+    // the device copy of all instances of a DataSet, built on first use and kept with the DataSet
+    static std::shared_ptr<DeviceRows> of(const DataSet &dataset);
+};
+
 class KernelMatrix {
 public:
     KernelMatrix(const DataSet::node2d &instances, SvmParam param);
     // Rows `rows[0..n_rows)` of `all`, without materialising a node2d copy.
     KernelMatrix(const DataSet::node2d &all, const int *rows, size_t n_rows, SvmParam param, int repeat = 1);
+    // Rows `rows[0..n_rows)` of the DataSet's device-resident instances (rows == nullptr: all of them, shared
+    // in place).  The feature count is the whole DataSet's, not the subset's: extra all-zero columns add
+    // exact zeros to every dot product.
+    KernelMatrix(const DataSet &dataset, const int *rows, size_t n_rows, SvmParam param, int repeat = 1);
 
     // kernel rows of stored rows d_idx[0..m) (device, folded ids) -> element s_i*ld + j of d_out,
     // s_i = d_out_slots[i] (or i), j < n_columns(); elements are row_type() wide
@@ -34,32 +61,26 @@ public:
     void get_rows(const DataSet::node2d &instances, void *d_out, int64_t ld) const;
 
     const kernel_type *diag() const { return diag_.data(); }          // device, n_instances() entries
-    const kernel_type *self_dot() const { return self_dot_.data(); }  // device, n_columns() entries
+    const kernel_type *self_dot() const { return rows_->self_dot.data(); }  // device, n_columns() entries
     size_t n_instances() const { return n_unique_ * repeat_; }        // rows of the matrix the solver sees
     size_t n_columns() const { return n_unique_; }                    // stored rows = columns of a kernel row
     int repeat() const { return repeat_; }
     int row_type() const { return param.kernel_type == SvmParam::LINEAR ? TSVM_ROW_F64 : TSVM_ROW_F32; }
     size_t row_elem_size() const { return row_type() == TSVM_ROW_F32 ? sizeof(float) : sizeof(double); }
-    size_t n_features() const { return n_features_; }
-    size_t nnz() const { return nnz_; }
-    bool dense_layout() const { return dense_; }
+    size_t n_features() const { return rows_->n_features; }
+    size_t nnz() const { return rows_->nnz; }
+    bool dense_layout() const { return rows_->dense; }
     const SvmParam &get_param() const { return param; }
 
     static bool choose_dense(size_t n, size_t n_features, size_t nnz);
 
 private:
-    void build(const DataSet::node2d &all, const int *rows, size_t n_rows, int repeat);
+    void finish(int repeat);
 
     SvmParam param;
-    size_t n_unique_ = 0, n_features_ = 0, nnz_ = 0;
+    std::shared_ptr<DeviceRows> rows_;
+    size_t n_unique_ = 0;
     int repeat_ = 1;
-    bool dense_ = false;
-    int64_t ld_ = 0;
-    tsvm::DeviceBuffer<kernel_type> x_;          // dense layout
-    tsvm::DeviceBuffer<kernel_type> val_;        // CSR layout
-    tsvm::DeviceBuffer<int> col_ind_;
-    tsvm::DeviceBuffer<int64_t> row_ptr_;
-    tsvm::DeviceBuffer<kernel_type> self_dot_;
     tsvm::DeviceBuffer<kernel_type> diag_;
     // reusable staging for the sparse path and for external batches
     mutable tsvm::DeviceBuffer<kernel_type> stage_;

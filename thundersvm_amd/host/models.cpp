@@ -56,6 +56,15 @@ int SvmModel::get_working_set_size(int n_instances, int n_features) {
     return ws;
 }
 
+// sv[s] = instances[sv_indices[s]]: the model owns copies of its support vectors (svc.cpp:86-108).  With
+// hundreds of thousands of support vectors the copy is tens of milliseconds of memory traffic, so it is
+// spread over the host cores.
+void SvmModel::copy_support_vectors(const DataSet::node2d &instances) {
+    sv.resize(sv_indices.size());
+#pragma omp parallel for schedule(static)
+    for (size_t s = 0; s < sv_indices.size(); ++s) sv[s] = instances[sv_indices[s]];
+}
+
 void SvmModel::run_solver(CSMOSolver &solver, const KernelMatrix &k_mat, const std::vector<int> &y,
                           std::vector<float_type> &alpha, float_type &rho_out, std::vector<float_type> &f_val,
                           float_type Cp, float_type Cn) {
@@ -325,9 +334,9 @@ void SVC::train(const DataSet &dataset, SvmParam p) {   // svc.cpp:41-145
         for (int id : grouped.original_index(c))
             if (is_sv[id]) {
                 n_sv[c]++;
-                sv.push_back(grouped.instances()[id]);
                 sv_indices.push_back(id);
             }
+    copy_support_vectors(grouped.instances());
     n_total_sv = (int) sv.size();
     TSVM_LOG << "#total unique sv = " << n_total_sv;
     // LibSVM coefficient layout: pair (i<j) stores class i's SVs in row j-1 and class j's SVs in row i
@@ -373,7 +382,7 @@ void SVC::train_binary(const DataSet &dataset, int i, int j, std::vector<float_t
         y[l] = l < ci ? +1 : -1;
         f_val[l] = l < ci ? -1 : +1;
     }
-    KernelMatrix k_mat(dataset.instances(), ids.data(), ids.size(), param);
+    KernelMatrix k_mat(dataset, ids.data(), ids.size(), param);
     CSMOSolver solver;
     run_solver(solver, k_mat, y, alpha, rho_out, f_val, param.C * c_weight[i], param.C * c_weight[j]);
     int count = 0;
@@ -427,7 +436,7 @@ void NuSVC::train_binary(const DataSet &dataset, int i, int j, std::vector<float
         alpha[l] = std::min(1., budget);
         budget -= alpha[l];
     }
-    KernelMatrix k_mat(dataset.instances(), ids.data(), ids.size(), param);
+    KernelMatrix k_mat(dataset, ids.data(), ids.size(), param);
     NuSMOSolver solver(false);
     run_solver(solver, k_mat, y, alpha, rho_out, f_val, 1, 1);
     for (int l = 0; l < n; ++l) alpha[l] *= y[l];
@@ -445,7 +454,7 @@ void SVR::model_setup(const DataSet &dataset, SvmParam &p) {
 void SVR::train(const DataSet &dataset, SvmParam p) {
     model_setup(dataset, p);
     const int n = (int) dataset.n_instances();
-    KernelMatrix k_mat(dataset.instances(), nullptr, n, param, 2);
+    KernelMatrix k_mat(dataset, nullptr, n, param, 2);
     std::vector<float_type> f_val(2 * (size_t) n), alpha_2(2 * (size_t) n, 0);
     std::vector<int> y(2 * (size_t) n);
     for (int i = 0; i < n; ++i) {
@@ -466,11 +475,11 @@ void SVR::save_svr_coef(const std::vector<float_type> &alpha_2, const DataSet::n
     for (size_t i = 0; i < n; ++i) {
         const float_type a = alpha_2[i] - alpha_2[i + n];
         if (a != 0) {
-            sv.push_back(instances[i]);
             sv_indices.push_back((int) i);
             coef.push_back(a);
         }
     }
+    copy_support_vectors(instances);
     n_sv[0] = (int) sv.size();
     n_sv[1] = 0;
     n_total_sv = (int) sv.size();
@@ -485,7 +494,7 @@ void NuSVR::model_setup(const DataSet &dataset, SvmParam &p) {
 void NuSVR::train(const DataSet &dataset, SvmParam p) {   // nusvr.cpp:7-41
     model_setup(dataset, p);
     const int n = (int) dataset.n_instances();
-    KernelMatrix k_mat(dataset.instances(), nullptr, n, param, 2);
+    KernelMatrix k_mat(dataset, nullptr, n, param, 2);
     std::vector<float_type> f_val(2 * (size_t) n), alpha_2(2 * (size_t) n);
     std::vector<int> y(2 * (size_t) n);
     float_type sum = param.C * param.nu * n / 2;
@@ -515,7 +524,7 @@ void OneClassSVC::model_setup(const DataSet &dataset, SvmParam &p) {
 void OneClassSVC::train(const DataSet &dataset, SvmParam p) {
     model_setup(dataset, p);
     const int n = (int) dataset.n_instances();
-    KernelMatrix k_mat(dataset.instances(), param);
+    KernelMatrix k_mat(dataset, nullptr, n, param);
     std::vector<float_type> alpha(n, 0), f_val(n, 0);
     std::vector<int> y(n, 1);
     const int full = static_cast<int>(param.nu * n);
@@ -526,10 +535,10 @@ void OneClassSVC::train(const DataSet &dataset, SvmParam p) {
     if (keep_binary) binary_alpha.push_back(alpha);
     for (int i = 0; i < n; ++i)
         if (alpha[i] != 0) {
-            sv.push_back(dataset.instances()[i]);
             sv_indices.push_back(i);
             coef.push_back(alpha[i]);
         }
+    copy_support_vectors(dataset.instances());
     n_sv[0] = (int) sv.size();
     n_sv[1] = 0;
     n_total_sv = (int) sv.size();

@@ -54,6 +54,7 @@ public:
 
 protected:
     virtual void model_setup(const DataSet &dataset, SvmParam &param);
+    void copy_support_vectors(const DataSet::node2d &instances);
     void run_solver(CSMOSolver &solver, const KernelMatrix &k_mat, const std::vector<int> &y, std::vector<float_type> &alpha,
                     float_type &rho, std::vector<float_type> &f_val, float_type Cp, float_type Cn);
     void compute_linear_coef_single_model(size_t n_feature, bool zero_based);

@@ -57,6 +57,7 @@ def host_lib():
         L.tsvm_dataset_free.argtypes = [C.c_void_p]
         L.tsvm_dataset_rows.restype = C.c_int64
         L.tsvm_dataset_rows.argtypes = [C.c_void_p]
+        L.tsvm_dataset_to_device.argtypes = [C.c_void_p]
         L.tsvm_model_train.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(TsvmParam), C.c_int, C.c_int, C.c_int, C.c_int]
         L.tsvm_model_predict.argtypes = [C.c_void_p, C.c_void_p, C.c_int, _dp, _dp]
         L.tsvm_model_train_file.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(TsvmParam)]
@@ -100,6 +101,12 @@ class Dataset:
         if not self.h:
             raise capi.TsvmError(L.tsvm_model_last_error().decode())
         self.n = L.tsvm_dataset_rows(self.h)
+
+    def to_device(self):
+        """Uploads the rows to HBM now; training calls on this Dataset then start from device-resident data."""
+        if host_lib().tsvm_dataset_to_device(self.h) != 0:
+            raise capi.TsvmError(host_lib().tsvm_model_last_error().decode())
+        return self
 
     def __del__(self):
         if getattr(self, "h", None):
