@@ -105,7 +105,7 @@ __global__ __launch_bounds__(SV_T) void c_smo_solve_kernel(
     __shared__ double s_a[LDK];
     __shared__ double s_f[2][LDK];
     __shared__ double sA_v[SV_W], sA_l[SV_W], sB_v[SV_W];
-    __shared__ int sA_i[SV_W], sB_i[SV_W];
+    __shared__ int sA_i[SV_W], sB_i[SV_W], sB_go[SV_W];
 
     // This workgroup is a chain of dependent operations; when a chip-wide kernel runs next to it on
     // another stream its wavefronts must not wait behind that kernel's for issue slots.
@@ -132,26 +132,48 @@ __global__ __launch_bounds__(SV_T) void c_smo_solve_kernel(
     // next iteration's first barrier, when no wavefront can still be reading the old values.
     int pend_i = 0, pend_j = 0;
     double pend_ai = a_old[0], pend_aj = a_old[0];   // for thread 0 this is s_a[0]: the first write changes nothing
-    double local_eps = 0.0;
+    // The initial gap fixes the local stopping threshold (smo_kernel.cpp:61-66).  It is the only place
+    // where the value of low = max of f over I_low is needed: inside the loop the stopping test
+    // low - up < local_eps is evaluated per element, as "no I_low element has f - up >= local_eps"
+    // (the same decision, since rounding the subtraction is monotone), which costs a ballot instead of
+    // a second cross-lane reduction per iteration.
+    double local_eps;
+    {
+        double mn = TSVM_INF, mx = -TSVM_INF;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            mn = fmin_f64(mn, (member >> (2 * e)) & 1u ? f[e] : TSVM_INF);
+            mx = fmax_f64(mx, (member >> (2 * e + 1)) & 1u ? f[e] : -TSVM_INF);
+        }
+        mn = wave_min_f64(mn);
+        mx = wave_max_f64(mx);
+        if (lane == 0) { sA_v[wave] = mn; sA_l[wave] = mx; }
+        __syncthreads();
+        double up0 = sA_v[0];
+#pragma unroll
+        for (int w = 1; w < SV_W; ++w) up0 = fmin_f64(up0, sA_v[w]);
+        const double local_diff = block_max(sA_l) - up0;
+        const double t = 0.1f * local_diff;   // float literal, as in the reference (smo_kernel.cpp:64)
+        local_eps = eps > t ? eps : t;
+        if (tid == 0) diff[0] = local_diff;
+        __syncthreads();   // sA_* are written again below
+    }
     int numOfIter = 0;
     unsigned touched = 0;
     while (true) {
         const int par = numOfIter & 1;
-        // i = first argmin of f over I_up; low = max of f over I_low (smo_kernel.cpp:41-59)
+        // i = first argmin of f over I_up (smo_kernel.cpp:41-59)
         double fu[E];
-        double lw = -TSVM_INF;
 #pragma unroll
         for (int e = 0; e < E; ++e) {
             s_f[par][e * SV_T + tid] = f[e];
             fu[e] = (member >> (2 * e)) & 1u ? f[e] : TSVM_INF;
-            lw = fmax_f64(lw, (member >> (2 * e + 1)) & 1u ? f[e] : -TSVM_INF);
         }
         double v;
         int vi;
         wave_first_argmin<E>(fu, tid, v, vi);
         const unsigned pre_i = TSVM_TOUCH_ROW(kws, vi, ws, LDK, lane);
-        lw = wave_max_f64(lw);
-        if (lane == 0) { sA_v[wave] = v; sA_i[wave] = vi; sA_l[wave] = lw; }
+        if (lane == 0) { sA_v[wave] = v; sA_i[wave] = vi; }
         __syncthreads();
         if (tid == 0) {
             s_a[pend_i] = pend_ai;
@@ -160,15 +182,7 @@ __global__ __launch_bounds__(SV_T) void c_smo_solve_kernel(
         double up_value;
         int i;
         block_argmin(sA_v, sA_i, up_value, i, MAX_WS);
-        const double low_value = block_max(sA_l);
         i = up_value < TSVM_INF ? i : 0;
-        const double local_diff = low_value - up_value;
-        if (numOfIter == 0) {
-            const double t = 0.1f * local_diff;   // float literal, as in the reference (smo_kernel.cpp:64)
-            local_eps = eps > t ? eps : t;
-            if (tid == 0) diff[0] = local_diff;
-        }
-        if (numOfIter > max_iter || local_diff < local_eps) break;
         const double *row_i = kws + (int64_t) i * LDK;
         double kI[E];
 #pragma unroll
@@ -176,19 +190,27 @@ __global__ __launch_bounds__(SV_T) void c_smo_solve_kernel(
         const double kd_i = s_kd[i];
         // j2 = first argmin of -b^2/a over I_low with f > up (smo_kernel.cpp:77-90)
         double qs[E];
+        bool go = false;   // some I_low element still violates: low - up >= local_eps (smo_kernel.cpp:68)
 #pragma unroll
         for (int e = 0; e < E; ++e) {
+            const bool low = (member >> (2 * e + 1)) & 1u;
             const double aIJ = __builtin_fma(-2.0, kI[e], kd_i + kd[e]);
             const double bIJ = -up_value + f[e];
             const double q = -bIJ * bIJ / aIJ;
-            qs[e] = ((member >> (2 * e + 1)) & 1u) && (-up_value > -f[e]) ? q : TSVM_INF;
+            qs[e] = low && (-up_value > -f[e]) ? q : TSVM_INF;
+            go |= low && !(f[e] - up_value < local_eps);
         }
         double ft;
         int fi;
         wave_first_argmin<E>(qs, tid, ft, fi);
         const unsigned pre_j = TSVM_TOUCH_ROW(kws, fi, ws, LDK, lane);
-        if (lane == 0) { sB_v[wave] = ft; sB_i[wave] = fi; }
+        const bool wave_go = __builtin_amdgcn_ballot_w64(go) != 0;
+        if (lane == 0) { sB_v[wave] = ft; sB_i[wave] = fi; sB_go[wave] = wave_go; }
         __syncthreads();
+        bool any_go = false;
+#pragma unroll
+        for (int w = 0; w < SV_W; ++w) any_go |= sB_go[w] != 0;
+        if (numOfIter > max_iter || !any_go) break;
         double min_t;
         int j2;
         block_argmin(sB_v, sB_i, min_t, j2, MAX_WS);
@@ -253,7 +275,7 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
     __shared__ double s_a[LDK];
     __shared__ double s_f[2][LDK];
     __shared__ double sA_vp[SV_W], sA_vn[SV_W], sA_lp[SV_W], sA_ln[SV_W], sB_vp[SV_W], sB_vn[SV_W];
-    __shared__ int sA_ip[SV_W], sA_in[SV_W], sB_ip[SV_W], sB_in[SV_W];
+    __shared__ int sA_ip[SV_W], sA_in[SV_W], sB_ip[SV_W], sB_in[SV_W], sB_go[SV_W];
 
     __builtin_amdgcn_s_setprio(3);
     const int tid = threadIdx.x;
@@ -276,33 +298,53 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
     }
     int pend_i = 0, pend_j = 0;
     double pend_ai = a_old[0], pend_aj = a_old[0];
-    double local_eps = 0.0;
+    // initial gap -> local stopping threshold (smo_kernel.cpp:176-183); inside the loop the stopping
+    // test is evaluated per element, as in the C variant
+    double local_eps;
+    {
+        double mnp = TSVM_INF, mnn = TSVM_INF, mxp = -TSVM_INF, mxn = -TSVM_INF;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            const unsigned b = member >> (4 * e);
+            mnp = fmin_f64(mnp, b & 1u ? f[e] : TSVM_INF);
+            mnn = fmin_f64(mnn, b & 2u ? f[e] : TSVM_INF);
+            mxp = fmax_f64(mxp, b & 4u ? f[e] : -TSVM_INF);
+            mxn = fmax_f64(mxn, b & 8u ? f[e] : -TSVM_INF);
+        }
+        mnp = wave_min_f64(mnp);
+        mnn = wave_min_f64(mnn);
+        mxp = wave_max_f64(mxp);
+        mxn = wave_max_f64(mxn);
+        if (lane == 0) { sA_vp[wave] = mnp; sA_vn[wave] = mnn; sA_lp[wave] = mxp; sA_ln[wave] = mxn; }
+        __syncthreads();
+        double up_p0 = sA_vp[0], up_n0 = sA_vn[0];
+#pragma unroll
+        for (int w = 1; w < SV_W; ++w) { up_p0 = fmin_f64(up_p0, sA_vp[w]); up_n0 = fmin_f64(up_n0, sA_vn[w]); }
+        const double dp = block_max(sA_lp) - up_p0, dn = block_max(sA_ln) - up_n0;
+        const double local_diff = dp > dn ? dp : dn;
+        const double t = 0.1 * local_diff;
+        local_eps = eps > t ? eps : t;
+        if (tid == 0) diff[0] = local_diff;
+        __syncthreads();
+    }
     int numOfIter = 0;
     unsigned touched = 0;
     while (true) {
         const int par = numOfIter & 1;
         double fup[E], fun[E];
-        double lp = -TSVM_INF, ln = -TSVM_INF;
 #pragma unroll
         for (int e = 0; e < E; ++e) {
             s_f[par][e * SV_T + tid] = f[e];
             const unsigned b = member >> (4 * e);
             fup[e] = b & 1u ? f[e] : TSVM_INF;
             fun[e] = b & 2u ? f[e] : TSVM_INF;
-            lp = fmax_f64(lp, b & 4u ? f[e] : -TSVM_INF);
-            ln = fmax_f64(ln, b & 8u ? f[e] : -TSVM_INF);
         }
         double vp, vn;
         int ipi, ini;
         wave_first_argmin<E>(fup, tid, vp, ipi);
         wave_first_argmin<E>(fun, tid, vn, ini);
         const unsigned pre_i = TSVM_TOUCH_ROW(kws, ipi, ws, LDK, lane) ^ TSVM_TOUCH_ROW(kws, ini, ws, LDK, lane);
-        lp = wave_max_f64(lp);
-        ln = wave_max_f64(ln);
-        if (lane == 0) {
-            sA_vp[wave] = vp; sA_ip[wave] = ipi; sA_vn[wave] = vn; sA_in[wave] = ini;
-            sA_lp[wave] = lp; sA_ln[wave] = ln;
-        }
+        if (lane == 0) { sA_vp[wave] = vp; sA_ip[wave] = ipi; sA_vn[wave] = vn; sA_in[wave] = ini; }
         __syncthreads();
         if (tid == 0) {
             s_a[pend_i] = pend_ai;
@@ -314,15 +356,6 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
         block_argmin(sA_vn, sA_in, up_value_n, in, MAX_WS);
         ip = up_value_p < TSVM_INF ? ip : 0;
         in = up_value_n < TSVM_INF ? in : 0;
-        const double low_value_p = block_max(sA_lp), low_value_n = block_max(sA_ln);
-        const double dp = low_value_p - up_value_p, dn = low_value_n - up_value_n;
-        const double local_diff = dp > dn ? dp : dn;
-        if (numOfIter == 0) {
-            const double t = 0.1 * local_diff;
-            local_eps = eps > t ? eps : t;
-            if (tid == 0) diff[0] = local_diff;
-        }
-        if (numOfIter > max_iter || local_diff < local_eps) break;
         const double *row_p = kws + (int64_t) ip * LDK;
         const double *row_n = kws + (int64_t) in * LDK;
         double kIp[E], kIn[E];
@@ -333,6 +366,7 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
         }
         const double kd_ip = s_kd[ip];
         double qp[E], qn[E];
+        bool go = false;   // max(low_p - up_p, low_n - up_n) >= local_eps (smo_kernel.cpp:185)
 #pragma unroll
         for (int e = 0; e < E; ++e) {
             const unsigned b = member >> (4 * e);
@@ -340,14 +374,20 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
             const double bp = -up_value_p + f[e], bn = -up_value_n + f[e];
             qp[e] = (b & 4u) && (-up_value_p > -f[e]) ? -bp * bp / aIJ : TSVM_INF;
             qn[e] = (b & 8u) && (-up_value_n > -f[e]) ? -bn * bn / aIJ : TSVM_INF;
+            go |= ((b & 4u) && !(f[e] - up_value_p < local_eps)) || ((b & 8u) && !(f[e] - up_value_n < local_eps));
         }
         double ftp, ftn;
         int jpi, jni;
         wave_first_argmin<E>(qp, tid, ftp, jpi);
         wave_first_argmin<E>(qn, tid, ftn, jni);
         const unsigned pre_j = TSVM_TOUCH_ROW(kws, jpi, ws, LDK, lane) ^ TSVM_TOUCH_ROW(kws, jni, ws, LDK, lane);
-        if (lane == 0) { sB_vp[wave] = ftp; sB_ip[wave] = jpi; sB_vn[wave] = ftn; sB_in[wave] = jni; }
+        const bool wave_go = __builtin_amdgcn_ballot_w64(go) != 0;
+        if (lane == 0) { sB_vp[wave] = ftp; sB_ip[wave] = jpi; sB_vn[wave] = ftn; sB_in[wave] = jni; sB_go[wave] = wave_go; }
         __syncthreads();
+        bool any_go = false;
+#pragma unroll
+        for (int w = 0; w < SV_W; ++w) any_go |= sB_go[w] != 0;
+        if (numOfIter > max_iter || !any_go) break;
         double f_val_j2p, f_val_j2n;
         int j2p, j2n;
         block_argmin(sB_vp, sB_ip, f_val_j2p, j2p, MAX_WS);
