@@ -82,125 +82,163 @@ struct PhaseTimer {
 
 }  // namespace
 
-void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std::vector<float_type> &alpha,
-                       float_type &rho, std::vector<float_type> &f_val, float_type eps, float_type Cp, float_type Cn,
-                       int ws_size, int out_max_iter) const {
-    const int n = (int) k_mat.n_instances();
+struct SolveTask::Impl {
+    const CSMOSolver &solver;
+    const KernelMatrix &k_mat;
+    const std::vector<int> &y;
+    std::vector<float_type> &alpha;
+    float_type &rho;
+    std::vector<float_type> &f_val;
+    const float_type eps, Cp, Cn;
+    const int ws_size, out_max_iter;
+
     // Kernel rows are stored once per distinct data row: n_u columns wide, addressed by the folded id
     // (id % n_u); f, alpha and y keep the reference's n = rep * n_u entries.
-    const int n_u = (int) k_mat.n_columns();
-    const int rep = k_mat.repeat();
-    const int row_type = k_mat.row_type();
-    const size_t row_esz = k_mat.row_elem_size();
-    const int q = ws_size / 2;
-    const int64_t ld = ((int64_t) n_u + 7) / 8 * 8;   // row stride in elements: rows stay 32-byte aligned
-    const bool nu = is_nu();
-    stats = SolverStats();
-    const auto wall0 = std::chrono::steady_clock::now();
+    const int n, n_u, rep, row_type;
+    const size_t row_esz;
+    const int q;
+    const int64_t ld;   // row stride in elements: rows stay 32-byte aligned
+    const bool nu;
+    const int ldk;
+    SolverStats stats;
+    std::chrono::steady_clock::time_point wall0;
 
-    DeviceBuffer<int> d_y(n), d_ws(ws_size), d_slots_a(ws_size), d_slots_b(ws_size), d_miss_ids(ws_size), d_miss_slots(ws_size);
-    DeviceBuffer<int> d_ws_folded(rep > 1 ? ws_size : 0);
-    const int *const ws_u = rep > 1 ? d_ws_folded.data() : d_ws.data();   // working set as folded ids
-    DeviceBuffer<float_type> d_alpha(n), d_f(n), d_alpha_diff(ws_size), d_diff(2);
-    DeviceBuffer<unsigned char> d_sel_ws(tsvm_select_workspace(n));
-    const int ldk = tsvm_smo_solve_block_ld(ws_size);
-    DeviceBuffer<kernel_type> d_kws((size_t) ws_size * ldk);
-    d_y.upload(y.data(), n);
-    d_alpha.upload(alpha.data(), n);
-    d_f.upload(f_val.data(), n);
-    d_diff.zero();
-    d_alpha_diff.zero();
-    d_kws.zero();
+    DeviceBuffer<int> d_y, d_ws, d_slots_a, d_slots_b, d_miss_ids, d_miss_slots, d_ws_folded;
+    DeviceBuffer<float_type> d_alpha, d_f, d_alpha_diff, d_diff;
+    DeviceBuffer<unsigned char> d_sel_ws;
+    DeviceBuffer<kernel_type> d_kws;
+    const int *ws_u = nullptr;   // working set as folded ids
 
-    // The local solver needs only the ws x ws block of the kernel matrix, which is computed first by a
-    // small launch; the full rows of the new working-set members are needed by update_f only.  With
-    // overlap_streams the solver runs on stream `sa` while get_rows runs on stream `sb` and update_f
-    // waits for both; by default (and always when profiling) everything is enqueued on one stream.
-    // A third stream only carries the read-back of the newly selected ids for the host-side cache
-    // bookkeeping, so that the host does that work while the local solver is already running.
-    struct Streams {
-        hipStream_t a = nullptr, b = nullptr, ids = nullptr;
-        hipEvent_t selected = nullptr, rows_ready = nullptr, ids_ready = nullptr;
-        bool two;
-        explicit Streams(bool two_streams) : two(two_streams) {
-            TSVM_HIP_CHECK(hipStreamCreateWithFlags(&a, hipStreamNonBlocking));
-            if (two) TSVM_HIP_CHECK(hipStreamCreateWithFlags(&b, hipStreamNonBlocking)); else b = a;
-            TSVM_HIP_CHECK(hipStreamCreateWithFlags(&ids, hipStreamNonBlocking));
-            TSVM_HIP_CHECK(hipEventCreateWithFlags(&selected, hipEventDisableTiming));
-            TSVM_HIP_CHECK(hipEventCreateWithFlags(&rows_ready, hipEventDisableTiming));
-            TSVM_HIP_CHECK(hipEventCreateWithFlags(&ids_ready, hipEventDisableTiming));
-        }
-        ~Streams() {
-            (void) hipStreamSynchronize(a);
-            if (two) { (void) hipStreamSynchronize(b); (void) hipStreamDestroy(b); }
-            (void) hipStreamSynchronize(ids);
-            (void) hipStreamDestroy(ids);
-            (void) hipStreamDestroy(a);
-            (void) hipEventDestroy(selected);
-            (void) hipEventDestroy(rows_ready);
-            (void) hipEventDestroy(ids_ready);
-        }
-    } st(overlap_streams && !profile);
-    const hipStream_t sa = st.a, sb = st.b;
+    // Everything of a task is enqueued on stream `sa`; `ids` only carries the read-back of the newly
+    // selected ids for the host-side cache bookkeeping, so that it does not wait behind the solver.
+    hipStream_t sa = nullptr, ids = nullptr;
+    hipEvent_t selected = nullptr, ids_ready = nullptr, diff_ready = nullptr;
 
-    // Kernel rows live in slots of one pool.  With a cache the pool holds up to pool_rows rows and the
-    // host tracks which instance sits in which slot; without one it holds exactly ws rows.
-    long long pool_rows = ws_size;
-    tsvm::RowArena &arena = tsvm::RowArena::instance();
-    if (cache_bytes != 0 && n_u > ws_size) {
-        const long long budget = cache_bytes > 0 ? cache_bytes : (long long) arena.auto_budget();
-        const long long fit = budget / (long long) (ld * row_esz);
-        // an LRU that can hold only a small part of the matrix does not hit: require a quarter of the rows
-        if (fit >= 4LL * ws_size && fit >= n_u / 4) pool_rows = std::min<long long>(n_u, fit);
-    }
-    bool caching = pool_rows > ws_size;
-    void *const k_rows = arena.acquire((size_t) pool_rows * ld * row_esz, cache_bytes < 0);
+    void *k_rows = nullptr;
+    bool caching = false;
     RowCache cache;
-    if (caching) {
-        cache.init(n_u, (int) pool_rows);
-        stats.cache_rows = pool_rows;
-    }
-    std::vector<int> cur_slots(ws_size), cur_ids(ws_size), miss_ids, miss_slots;
+    std::vector<int> cur_slots, cur_ids, miss_ids, miss_slots;
     int *h_ids = nullptr, *h_slots = nullptr;
     double *h_diff = nullptr;
-    TSVM_HIP_CHECK(hipHostMalloc((void **) &h_diff, 2 * sizeof(double)));
-    TSVM_HIP_CHECK(hipHostMalloc((void **) &h_ids, ws_size * sizeof(int)));
-    TSVM_HIP_CHECK(hipHostMalloc((void **) &h_slots, 3 * ws_size * sizeof(int)));
-    h_diff[0] = h_diff[1] = 0;
+    int rotation_base = 0;   // iteration at which d_slots_a was valid
+    long long window_lookups = 0, window_hits = 0;
+    const int *slots = nullptr;
+
+    int max_iter = 0;
+    long long local_iter = 0;
+    int same_local_diff_cnt = 0, swap_local_diff_cnt = 0;
+    float_type previous_local_diff = INFINITY, last_local_diff = INFINITY, second_last_local_diff = INFINITY;
+    PhaseTimer timer;
+    bool select_ahead = false, block_first = false, select_enqueued = false;
+    int iter = 0;
+
+    Impl(const CSMOSolver &solver, const KernelMatrix &k_mat, const std::vector<int> &y, std::vector<float_type> &alpha,
+         float_type &rho, std::vector<float_type> &f_val, float_type eps, float_type Cp, float_type Cn, int ws_size,
+         int out_max_iter, void *pool, size_t pool_bytes)
+        : solver(solver), k_mat(k_mat), y(y), alpha(alpha), rho(rho), f_val(f_val), eps(eps), Cp(Cp), Cn(Cn), ws_size(ws_size),
+          out_max_iter(out_max_iter), n((int) k_mat.n_instances()), n_u((int) k_mat.n_columns()), rep(k_mat.repeat()),
+          row_type(k_mat.row_type()), row_esz(k_mat.row_elem_size()), q(ws_size / 2), ld(((int64_t) n_u + 7) / 8 * 8),
+          nu(solver.is_nu()), ldk(tsvm_smo_solve_block_ld(ws_size)), timer(solver.profile) {
+        wall0 = std::chrono::steady_clock::now();
+        d_y.resize(n); d_ws.resize(ws_size); d_slots_a.resize(ws_size); d_slots_b.resize(ws_size);
+        d_miss_ids.resize(ws_size); d_miss_slots.resize(ws_size);
+        if (rep > 1) d_ws_folded.resize(ws_size);
+        ws_u = rep > 1 ? d_ws_folded.data() : d_ws.data();
+        d_alpha.resize(n); d_f.resize(n); d_alpha_diff.resize(ws_size); d_diff.resize(2);
+        d_sel_ws.resize(tsvm_select_workspace(n));
+        d_kws.resize((size_t) ws_size * ldk);
+        d_y.upload(y.data(), n);
+        d_alpha.upload(alpha.data(), n);
+        d_f.upload(f_val.data(), n);
+        d_diff.zero();
+        d_alpha_diff.zero();
+        d_kws.zero();
+        TSVM_HIP_CHECK(hipStreamCreateWithFlags(&sa, hipStreamNonBlocking));
+        TSVM_HIP_CHECK(hipStreamCreateWithFlags(&ids, hipStreamNonBlocking));
+        TSVM_HIP_CHECK(hipEventCreateWithFlags(&selected, hipEventDisableTiming));
+        TSVM_HIP_CHECK(hipEventCreateWithFlags(&ids_ready, hipEventDisableTiming));
+        TSVM_HIP_CHECK(hipEventCreateWithFlags(&diff_ready, hipEventDisableTiming));
+
+        // Kernel rows live in slots of one pool.  With a cache the pool holds up to pool_rows rows and the
+        // host tracks which instance sits in which slot; without one it holds exactly ws rows.
+        long long pool_rows = ws_size;
+        const long long cache_bytes = solver.cache_bytes;
+        tsvm::RowArena &arena = tsvm::RowArena::instance();
+        if (cache_bytes != 0 && n_u > ws_size) {
+            const long long budget = pool ? (long long) pool_bytes : cache_bytes > 0 ? cache_bytes : (long long) arena.auto_budget();
+            const long long fit = budget / (long long) (ld * row_esz);
+            // an LRU that can hold only a small part of the matrix does not hit: require a quarter of the rows
+            if (fit >= 4LL * ws_size && fit >= n_u / 4) pool_rows = std::min<long long>(n_u, fit);
+        }
+        caching = pool_rows > ws_size;
+        const size_t need = (size_t) pool_rows * ld * row_esz;
+        if (pool) {
+            if (need > pool_bytes) throw std::runtime_error("SolveTask: kernel-row pool too small");
+            k_rows = pool;
+        } else {
+            k_rows = arena.acquire(need, cache_bytes < 0);
+        }
+        if (caching) {
+            cache.init(n_u, (int) pool_rows);
+            stats.cache_rows = pool_rows;
+        }
+        cur_slots.resize(ws_size);
+        cur_ids.resize(ws_size);
+        TSVM_HIP_CHECK(hipHostMalloc((void **) &h_diff, 2 * sizeof(double)));
+        TSVM_HIP_CHECK(hipHostMalloc((void **) &h_ids, ws_size * sizeof(int)));
+        TSVM_HIP_CHECK(hipHostMalloc((void **) &h_slots, 3 * ws_size * sizeof(int)));
+        h_diff[0] = h_diff[1] = 0;
+        if (!caching) {
+            for (int t = 0; t < ws_size; ++t) cur_slots[t] = t;
+            upload_rotation(cur_slots);
+        }
+        solver.init_f(alpha, y, k_mat, d_f.data());
+        TSVM_HIP_CHECK(hipDeviceSynchronize());   // uploads, fills and init_f ran on the default stream
+
+        max_iter = std::max(100000, ws_size > INT_MAX / 100 ? INT_MAX : 100 * ws_size);
+        timer.stream = sa;
+        if (solver.trace) {
+            solver.trace->ws_size = ws_size;
+            solver.trace->diff.clear();
+            solver.trace->ws.clear();
+        }
+        // The next selection is enqueued before the host has seen this iteration's diff, so the device goes
+        // straight from update_f into it; if the diff then says stop, that selection was simply not needed.
+        // (Not when tracing, which reads the working set back after each iteration, nor when profiling.)
+        select_ahead = !solver.trace && !solver.profile;
+        // The solver reads the ws x ws block of the kernel matrix.  With few features the block is cheap to
+        // compute on its own, without the stored rows, so it and the solver can be enqueued before the host
+        // does the cache bookkeeping.  With many features that small launch (64 workgroups walking the whole
+        // feature range) costs more than it hides, and the block is gathered from the stored rows instead.
+        block_first = k_mat.n_features() < 256;
+        stats.ms_setup = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - wall0).count();
+    }
+
+    ~Impl() {
+        if (sa) (void) hipStreamSynchronize(sa);   // a selection enqueued ahead may still be running
+        if (ids) { (void) hipStreamSynchronize(ids); (void) hipStreamDestroy(ids); }
+        if (sa) (void) hipStreamDestroy(sa);
+        if (selected) (void) hipEventDestroy(selected);
+        if (ids_ready) (void) hipEventDestroy(ids_ready);
+        if (diff_ready) (void) hipEventDestroy(diff_ready);
+        if (h_diff) (void) hipHostFree(h_diff);
+        if (h_ids) (void) hipHostFree(h_ids);
+        if (h_slots) (void) hipHostFree(h_slots);
+    }
+
     // without a cache the slot tables just alternate: the two halves of the working set swap places
     // every iteration, so the rows kept from the previous iteration are re-addressed, never copied
     // (the reference copies q*n values per iteration, csmosolver.cpp:75)
-    auto upload_rotation = [&](const std::vector<int> &slots_now) {
+    void upload_rotation(const std::vector<int> &slots_now) {
         std::vector<int> other(ws_size);
         for (int t = 0; t < ws_size; ++t) other[t] = slots_now[(t + q) % ws_size];
         d_slots_a.upload(slots_now.data(), ws_size);
         d_slots_b.upload(other.data(), ws_size);
-    };
-    int rotation_base = 0;   // iteration at which d_slots_a was valid
-    long long window_lookups = 0, window_hits = 0;
-    if (!caching) {
-        for (int t = 0; t < ws_size; ++t) cur_slots[t] = t;
-        upload_rotation(cur_slots);
-    }
-
-    init_f(alpha, y, k_mat, d_f.data());
-    TSVM_HIP_CHECK(hipDeviceSynchronize());   // uploads, fills and init_f ran on the default stream
-
-    const int max_iter = std::max(100000, ws_size > INT_MAX / 100 ? INT_MAX : 100 * ws_size);
-    long long local_iter = 0;
-    int same_local_diff_cnt = 0, swap_local_diff_cnt = 0;
-    float_type previous_local_diff = INFINITY, last_local_diff = INFINITY, second_last_local_diff = INFINITY;
-    PhaseTimer timer(profile);
-    timer.stream = sa;
-    if (trace) {
-        trace->ws_size = ws_size;
-        trace->diff.clear();
-        trace->ws.clear();
     }
 
     // Working-set selection of iteration `it`: the first one picks ws_size ids, later ones keep the last
     // half of the previous set and pick q new ids (csmosolver.cpp:63-77).
-    auto enqueue_select = [&](int it) {
+    void launch_select(int it) {
         if (it == 0) {
             abi_check(tsvm_select_working_set(d_f.data(), d_y.data(), d_alpha.data(), n, Cp, Cn, nullptr, 0, d_ws.data(),
                                               ws_size, nu, d_sel_ws.data(), sa));
@@ -210,58 +248,31 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
                                               d_ws.data() + q, q, nu, d_sel_ws.data(), sa));
         }
         if (rep > 1) abi_check(tsvm_fold_ids(d_ws.data(), ws_size, n_u, d_ws_folded.data(), sa));
-    };
-    // The next selection is enqueued before the host has seen this iteration's diff, so the device goes
-    // straight from update_f into it; if the diff then says stop, that selection was simply not needed.
-    // (Not when tracing, which reads the working set back after each iteration, nor when profiling.)
-    const bool select_ahead = !trace && !profile;
-    const bool block_first = st.two || k_mat.n_features() < 256;
-    bool select_enqueued = false;
-    hipEvent_t diff_ready = nullptr;
-    TSVM_HIP_CHECK(hipEventCreateWithFlags(&diff_ready, hipEventDisableTiming));
+    }
 
-    stats.ms_setup = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - wall0).count();
-    for (int iter = 0;; ++iter) {
+    void enqueue_select() {
         const int n_new = iter == 0 ? ws_size : q;
         const int first_new = iter == 0 ? 0 : q;
         timer.begin();
-        if (!select_enqueued) enqueue_select(iter);
+        if (!select_enqueued) launch_select(iter);
         select_enqueued = false;
         timer.end(stats.ms_select);
-        const int *slots;
-        TSVM_HIP_CHECK(hipEventRecord(st.selected, sa));
+        TSVM_HIP_CHECK(hipEventRecord(selected, sa));
         if (caching) {
-            // the new ids travel to the host on their own stream while the solver below is enqueued and runs
-            TSVM_HIP_CHECK(hipStreamWaitEvent(st.ids, st.selected, 0));
-            TSVM_HIP_CHECK(hipMemcpyAsync(h_ids, d_ws.data() + first_new, sizeof(int) * n_new, hipMemcpyDeviceToHost, st.ids));
-            TSVM_HIP_CHECK(hipEventRecord(st.ids_ready, st.ids));
+            // the new ids travel to the host on their own stream
+            TSVM_HIP_CHECK(hipStreamWaitEvent(ids, selected, 0));
+            TSVM_HIP_CHECK(hipMemcpyAsync(h_ids, d_ws.data() + first_new, sizeof(int) * n_new, hipMemcpyDeviceToHost, ids));
+            TSVM_HIP_CHECK(hipEventRecord(ids_ready, ids));
         }
-        // The solver reads the ws x ws block of the kernel matrix.  With few features the block is cheap to
-        // compute on its own, ahead of the rows: the solver then already runs while the host does the cache
-        // bookkeeping (and, with two streams, while get_rows runs).  With many features that small launch
-        // (64 workgroups walking the whole feature range) costs more than it hides, and the block is
-        // gathered from the stored rows once they are complete.
-        auto enqueue_local = [&](const int *gather_slots, bool from_rows) {
-            timer.begin();
-            if (from_rows)
-                abi_check(tsvm_smo_gather_block(k_rows, row_type, gather_slots, ld, ws_u, ws_size, d_kws.data(), sa));
-            else
-                k_mat.get_block(ws_u, ws_size, d_kws.data(), ldk, sa);
-            if (nu) {
-                abi_check(tsvm_nu_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), d_ws.data(),
-                                                  ws_size, Cp, d_kws.data(), k_mat.diag(), eps, d_diff.data(), max_iter, sa));
-            } else {
-                abi_check(tsvm_c_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), d_ws.data(),
-                                                 ws_size, Cp, Cn, d_kws.data(), k_mat.diag(), eps, d_diff.data(), max_iter, sa));
-            }
-            timer.end(stats.ms_local);
-        };
-        if (block_first) enqueue_local(nullptr, false);
-        // the full rows of the new working-set members (on stream b when two streams are used)
+    }
+
+    void enqueue_rows() {
+        const int n_new = iter == 0 ? ws_size : q;
+        const int first_new = iter == 0 ? 0 : q;
         timer.begin();
         if (caching) {
             // look the new ids up and compute only the rows that are not cached
-            TSVM_HIP_CHECK(hipEventSynchronize(st.ids_ready));
+            TSVM_HIP_CHECK(hipEventSynchronize(ids_ready));
             if (iter > 0) {
                 for (int t = 0; t < q; ++t) {   // rows kept from the previous working set stay most recently used
                     cur_ids[t] = cur_ids[t + q];
@@ -289,11 +300,11 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
             std::copy(miss_ids.begin(), miss_ids.end(), h_miss_ids);
             std::copy(miss_slots.begin(), miss_slots.end(), h_miss_slots);
             const int n_miss = (int) miss_ids.size();
-            TSVM_HIP_CHECK(hipMemcpyAsync(d_slots_a.data(), h_slots, sizeof(int) * ws_size, hipMemcpyHostToDevice, sb));
+            TSVM_HIP_CHECK(hipMemcpyAsync(d_slots_a.data(), h_slots, sizeof(int) * ws_size, hipMemcpyHostToDevice, sa));
             if (n_miss) {
-                TSVM_HIP_CHECK(hipMemcpyAsync(d_miss_ids.data(), h_miss_ids, sizeof(int) * n_miss, hipMemcpyHostToDevice, sb));
-                TSVM_HIP_CHECK(hipMemcpyAsync(d_miss_slots.data(), h_miss_slots, sizeof(int) * n_miss, hipMemcpyHostToDevice, sb));
-                k_mat.get_rows(d_miss_ids.data(), n_miss, k_rows, ld, d_miss_slots.data(), sb);
+                TSVM_HIP_CHECK(hipMemcpyAsync(d_miss_ids.data(), h_miss_ids, sizeof(int) * n_miss, hipMemcpyHostToDevice, sa));
+                TSVM_HIP_CHECK(hipMemcpyAsync(d_miss_slots.data(), h_miss_slots, sizeof(int) * n_miss, hipMemcpyHostToDevice, sa));
+                k_mat.get_rows(d_miss_ids.data(), n_miss, k_rows, ld, d_miss_slots.data(), sa);
             }
             slots = d_slots_a.data();
             // A cache that has started evicting and still does not hit only costs the id read-back:
@@ -302,7 +313,7 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
             if (cache.cap < n_u && cache.used == cache.cap && iter % 64 == 63) {
                 const long long dl = stats.cache_lookups - window_lookups, dh = stats.cache_hits - window_hits;
                 if (dh * 20 < dl) {
-                    TSVM_HIP_CHECK(hipStreamSynchronize(sb));
+                    TSVM_HIP_CHECK(hipStreamSynchronize(sa));
                     caching = false;
                     stats.cache_disabled = true;
                     upload_rotation(cur_slots);
@@ -313,35 +324,56 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
         } else {
             const bool on_a = ((iter - rotation_base) % 2) == 0;
             slots = on_a ? d_slots_a.data() : d_slots_b.data();
-            if (st.two) TSVM_HIP_CHECK(hipStreamWaitEvent(sb, st.selected, 0));
             // new rows go to the slots the dropped rows occupied
-            k_mat.get_rows(ws_u + first_new, n_new, k_rows, ld, slots + first_new, sb);
-        }
-        if (st.two) {
-            TSVM_HIP_CHECK(hipEventRecord(st.rows_ready, sb));
-            TSVM_HIP_CHECK(hipStreamWaitEvent(sa, st.rows_ready, 0));
+            k_mat.get_rows(ws_u + first_new, n_new, k_rows, ld, slots + first_new, sa);
         }
         timer.end(stats.ms_get_rows);
-        if (!block_first) enqueue_local(slots, true);
+    }
+
+    void enqueue_block() {
+        timer.begin();
+        if (block_first)
+            k_mat.get_block(ws_u, ws_size, d_kws.data(), ldk, sa);
+        else
+            abi_check(tsvm_smo_gather_block(k_rows, row_type, slots, ld, ws_u, ws_size, d_kws.data(), sa));
+        timer.end(stats.ms_local);
+    }
+
+    void enqueue_solver() {
+        timer.begin();
+        if (nu) {
+            abi_check(tsvm_nu_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), d_ws.data(), ws_size,
+                                              Cp, d_kws.data(), k_mat.diag(), eps, d_diff.data(), max_iter, sa));
+        } else {
+            abi_check(tsvm_c_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), d_ws.data(), ws_size,
+                                             Cp, Cn, d_kws.data(), k_mat.diag(), eps, d_diff.data(), max_iter, sa));
+        }
+        timer.end(stats.ms_local);
+    }
+
+    void enqueue_update() {
         timer.begin();
         abi_check(tsvm_update_f(d_f.data(), d_alpha_diff.data(), ws_size, k_rows, row_type, slots, ld, n_u, rep, sa));
         timer.end(stats.ms_update_f);
         TSVM_HIP_CHECK(hipMemcpyAsync(h_diff, d_diff.data(), 2 * sizeof(double), hipMemcpyDeviceToHost, sa));
         TSVM_HIP_CHECK(hipEventRecord(diff_ready, sa));
         if (select_ahead) {
-            enqueue_select(iter + 1);
+            launch_select(iter + 1);
             select_enqueued = true;
         }
+    }
+
+    bool finish_iteration() {
         TSVM_HIP_CHECK(hipEventSynchronize(diff_ready));
         const double diff0 = h_diff[0], diff1 = h_diff[1];
         local_iter += (long long) diff1;
+        SolverTrace *trace = solver.trace;
         if (trace && iter < trace->cap_iters) {
             trace->diff.push_back(diff0);
             trace->diff.push_back(diff1);
             std::vector<int> w = d_ws.to_host();
             trace->ws.insert(trace->ws.end(), w.begin(), w.end());
         }
-
         // stall guards and stopping rule (csmosolver.cpp:86-111)
         if (fabs(diff0 - previous_local_diff) < eps * 0.001) {
             same_local_diff_cnt++;
@@ -357,23 +389,56 @@ void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std
             TSVM_LOG << "global iter = " << iter << ", total local iter = " << local_iter << ", diff = " << diff0;
         const bool stalled = (same_local_diff_cnt >= 10 || swap_local_diff_cnt >= 10) && fabs(diff0 - 2.0) > eps;
         if (stalled || diff0 < eps || (out_max_iter != -1 && iter == out_max_iter)) {
+            TSVM_HIP_CHECK(hipStreamSynchronize(sa));   // a selection enqueued ahead may still be running
             d_alpha.download(alpha.data(), n);
             d_f.download(f_val.data(), n);
-            rho = calculate_rho(f_val, y, alpha, Cp, Cn);
+            rho = solver.calculate_rho(f_val, y, alpha, Cp, Cn);
             stats.n_iter = iter + 1;
             stats.local_iter = local_iter;
-            stats.obj = calculate_obj(f_val, alpha, y);
+            stats.obj = solver.calculate_obj(f_val, alpha, y);
             TSVM_LOG << "global iter = " << iter << ", total local iter = " << local_iter << ", diff = " << diff0
                      << ", obj = " << stats.obj << ", cache hits " << stats.cache_hits << "/" << stats.cache_lookups;
-            break;
+            stats.ms_wall = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - wall0).count();
+            return true;
         }
+        ++iter;
+        return false;
     }
-    TSVM_HIP_CHECK(hipStreamSynchronize(sa));   // a selection enqueued ahead may still be running
-    (void) hipEventDestroy(diff_ready);
-    stats.ms_wall = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - wall0).count();
-    (void) hipHostFree(h_diff);
-    (void) hipHostFree(h_ids);
-    (void) hipHostFree(h_slots);
+};
+
+SolveTask::SolveTask(const CSMOSolver &solver, const KernelMatrix &k_mat, const std::vector<int> &y, std::vector<float_type> &alpha,
+                     float_type &rho, std::vector<float_type> &f_val, float_type eps, float_type Cp, float_type Cn, int ws_size,
+                     int out_max_iter, void *pool, size_t pool_bytes)
+    : impl_(new Impl(solver, k_mat, y, alpha, rho, f_val, eps, Cp, Cn, ws_size, out_max_iter, pool, pool_bytes)) {}
+SolveTask::~SolveTask() { delete impl_; }
+void SolveTask::enqueue_select() { impl_->enqueue_select(); }
+void SolveTask::enqueue_rows() { impl_->enqueue_rows(); }
+void SolveTask::enqueue_block() { impl_->enqueue_block(); }
+void SolveTask::enqueue_solver() { impl_->enqueue_solver(); }
+void SolveTask::enqueue_update() { impl_->enqueue_update(); }
+bool SolveTask::finish_iteration() { return impl_->finish_iteration(); }
+bool SolveTask::block_needs_rows() const { return !impl_->block_first; }
+hipStream_t SolveTask::stream() const { return impl_->sa; }
+const SolverStats &SolveTask::stats() const { return impl_->stats; }
+size_t SolveTask::min_pool_bytes(const KernelMatrix &k_mat, int ws_size) {
+    const size_t ld = (k_mat.n_columns() + 7) / 8 * 8;
+    return (size_t) ws_size * ld * k_mat.row_elem_size();
+}
+
+void CSMOSolver::solve(const KernelMatrix &k_mat, const std::vector<int> &y, std::vector<float_type> &alpha,
+                       float_type &rho, std::vector<float_type> &f_val, float_type eps, float_type Cp, float_type Cn,
+                       int ws_size, int out_max_iter) const {
+    SolveTask task(*this, k_mat, y, alpha, rho, f_val, eps, Cp, Cn, ws_size, out_max_iter);
+    const bool rows_first = task.block_needs_rows();
+    do {
+        task.enqueue_select();
+        if (rows_first) task.enqueue_rows();
+        task.enqueue_block();
+        task.enqueue_solver();
+        if (!rows_first) task.enqueue_rows();   // the host's cache bookkeeping runs while the solver does
+        task.enqueue_update();
+    } while (!task.finish_iteration());
+    stats = task.stats();
 }
 
 // csmosolver.cpp:189-214: f starts from a non-zero alpha in batches of 101 rows.

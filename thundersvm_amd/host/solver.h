@@ -24,6 +24,8 @@ struct SolverStats {
     bool cache_disabled = false;  // switched off after the warm-up because it was not hitting
 };
 
+class SolveTask;
+
 class CSMOSolver {
 public:
     virtual ~CSMOSolver() = default;
@@ -36,12 +38,9 @@ public:
     bool profile = false;
     // Budget of the HBM kernel-row cache in bytes: -1 = half of the free device memory, 0 = no cache.
     long long cache_bytes = -1;
-    // Run the local solver and the chip-wide get_rows concurrently on two streams.  Off by default: the
-    // solver is a chain of dependent loads, and measured next to get_rows each of its iterations takes
-    // 3.6x longer (2.4 ms instead of 0.66 ms per call at n = 800,000), which cancels the overlap.
-    bool overlap_streams = false;
 
 protected:
+    friend class SolveTask;
     virtual bool is_nu() const { return false; }
     virtual float_type calculate_rho(const std::vector<float_type> &f_val, const std::vector<int> &y,
                                      std::vector<float_type> &alpha, float_type Cp, float_type Cn) const;
@@ -62,4 +61,39 @@ protected:
 
 private:
     bool for_svr;
+};
+
+// One SMO solve as a resumable sequence of enqueue steps on its own stream.  CSMOSolver::solve runs one
+// task to completion; a one-vs-one run advances several tasks (class pairs) in lockstep, so that their
+// local solvers -- each a single workgroup bound by latency, and half of a multi-class run's device
+// time -- occupy different CUs at the same time, while the chip-wide steps (selection, get_rows,
+// update_f) of the pairs follow one another.  The steps of one outer iteration, in order:
+//   enqueue_select, enqueue_rows, enqueue_block, enqueue_solver, enqueue_update, finish_iteration
+// (a task whose block does not need the stored rows may run enqueue_block / enqueue_solver before
+// enqueue_rows, which hides the host's cache bookkeeping behind the solver).
+class SolveTask {
+public:
+    // pool / pool_bytes: device memory for the kernel rows (nullptr: taken from the process-wide arena
+    // according to solver.cache_bytes)
+    SolveTask(const CSMOSolver &solver, const KernelMatrix &k_mat, const std::vector<int> &y, std::vector<float_type> &alpha,
+              float_type &rho, std::vector<float_type> &f_val, float_type eps, float_type Cp, float_type Cn, int ws_size,
+              int out_max_iter, void *pool = nullptr, size_t pool_bytes = 0);
+    ~SolveTask();
+    SolveTask(const SolveTask &) = delete;
+    SolveTask &operator=(const SolveTask &) = delete;
+
+    void enqueue_select();
+    void enqueue_rows();
+    void enqueue_block();
+    void enqueue_solver();
+    void enqueue_update();
+    bool finish_iteration();   // waits for this iteration's diff; true once the solve is complete and its results are written
+    bool block_needs_rows() const;
+    hipStream_t stream() const;
+    const SolverStats &stats() const;
+    static size_t min_pool_bytes(const KernelMatrix &k_mat, int ws_size);
+
+private:
+    struct Impl;
+    Impl *impl_;
 };
