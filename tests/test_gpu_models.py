@@ -172,3 +172,20 @@ def test_dataset_handle_and_file_loader(tmp_path):
     la, da = a.predict(tr)
     lb, db = b.predict(Dataset(tr))
     assert np.array_equal(da, db) and np.array_equal(la, lb)
+
+
+def test_class_pairs_in_lockstep_give_the_same_model():
+    """The pairs of a one-vs-one run are advanced one at a time or several in lockstep: identical models."""
+    w = D.workload_c4(scale=0.01)
+    tr = w["train"]
+    ref = None
+    for lanes, cache in ((1, -1), (2, -1), (3, 0), (5, 64 << 20)):
+        m = Model(0).train(tr, make_param(pair_lanes=lanes, cache_bytes=cache, **w["params"]))
+        cur = (m.coef.copy(), m.rho.copy(), m.sv_indices.copy(), [m.stats(b)["n_iter"] for b in range(m.n_binary)],
+               [m.stats(b)["local_iter"] for b in range(m.n_binary)])
+        if ref is None:
+            ref = cur
+            assert m.n_binary == 21
+        else:
+            assert np.array_equal(cur[0], ref[0]) and np.array_equal(cur[1], ref[1]) and np.array_equal(cur[2], ref[2])
+            assert cur[3] == ref[3] and cur[4] == ref[4]

@@ -321,9 +321,22 @@ void SVC::train(const DataSet &dataset, SvmParam p) {   // svc.cpp:41-145
     std::vector<std::vector<float_type>> alpha(n_binary_models);
     std::vector<char> is_sv(n, 0);
     int k = 0;
+    const int lanes = std::min(pair_lanes, n_binary_models);
+    if (lanes > 1 && !profile && !trace_first) {
+        train_pairs_in_lockstep(grouped, lanes, alpha);
+    } else {
+        for (int i = 0; i < n_classes; ++i)
+            for (int j = i + 1; j < n_classes; ++j, ++k) {
+                BinaryProblem p;
+                p.k = k;
+                setup_binary(grouped, i, j, p);
+                run_solver(*p.solver, *p.k_mat, p.y, p.alpha, rho[k], p.f_val, p.Cp, p.Cn);
+                finish_binary(p, alpha[k]);
+            }
+    }
+    k = 0;
     for (int i = 0; i < n_classes; ++i)
         for (int j = i + 1; j < n_classes; ++j, ++k) {
-            train_binary(grouped, i, j, alpha[k], rho[k]);
             const std::vector<int> ids = grouped.original_index(i, j);
             for (size_t l = 0; l < ids.size(); ++l)
                 if (alpha[k][l] != 0) is_sv[ids[l]] = 1;
@@ -372,25 +385,112 @@ void SVC::train(const DataSet &dataset, SvmParam p) {   // svc.cpp:41-145
     if (param.probability == 1) throw std::runtime_error("probability estimates are not part of this build");
 }
 
-void SVC::train_binary(const DataSet &dataset, int i, int j, std::vector<float_type> &alpha, float_type &rho_out) {   // svc.cpp:147-177
+void SVC::setup_binary(const DataSet &dataset, int i, int j, BinaryProblem &p) {   // svc.cpp:147-170
     const std::vector<int> ids = dataset.original_index(i, j);
     const int ci = dataset.count()[i], n = (int) ids.size();
-    std::vector<int> y(n);
-    std::vector<float_type> f_val(n);
-    alpha.assign(n, 0);
+    p.i = i;
+    p.j = j;
+    p.y.resize(n);
+    p.f_val.resize(n);
+    p.alpha.assign(n, 0);
     for (int l = 0; l < n; ++l) {
-        y[l] = l < ci ? +1 : -1;
-        f_val[l] = l < ci ? -1 : +1;
+        p.y[l] = l < ci ? +1 : -1;
+        p.f_val[l] = l < ci ? -1 : +1;
     }
-    KernelMatrix k_mat(dataset, ids.data(), ids.size(), param);
-    CSMOSolver solver;
-    run_solver(solver, k_mat, y, alpha, rho_out, f_val, param.C * c_weight[i], param.C * c_weight[j]);
+    p.k_mat.reset(new KernelMatrix(dataset, ids.data(), ids.size(), param));
+    p.solver.reset(new CSMOSolver());
+    p.Cp = param.C * c_weight[i];
+    p.Cn = param.C * c_weight[j];
+}
+
+void SVC::finish_binary(BinaryProblem &p, std::vector<float_type> &alpha_out) {   // svc.cpp:171-177
     int count = 0;
-    for (int l = 0; l < n; ++l) {
-        alpha[l] *= y[l];
-        if (alpha[l] != 0) count++;
+    for (size_t l = 0; l < p.alpha.size(); ++l) {
+        p.alpha[l] *= p.y[l];
+        if (p.alpha[l] != 0) count++;
     }
-    TSVM_LOG << "rho = " << rho_out << ", #sv = " << count;
+    TSVM_LOG << "rho = " << rho[p.k] << ", #sv = " << count;
+    alpha_out = std::move(p.alpha);
+}
+
+// The class pairs are independent problems.  Up to `lanes` of them are in flight, each a SolveTask on its
+// own stream with its own slice of the kernel-row arena, advanced one outer iteration at a time in three
+// phases separated by events: (1) selection, kernel rows and the solver's block of every pair, (2) the
+// local solvers of all pairs, which are single workgroups and so run side by side on different CUs, (3)
+// update_f of every pair.  A chip-wide kernel never overlaps a local solver: measured next to one, each
+// solver iteration takes 3.3-3.6x longer.  A pair that finishes hands its lane to the next pair.  The
+// result of a pair does not depend on what runs beside it.
+void SVC::train_pairs_in_lockstep(const DataSet &grouped, int lanes, std::vector<std::vector<float_type>> &alpha) {
+    struct PairId { int i, j; };
+    std::vector<PairId> pairs;
+    for (int i = 0; i < n_classes; ++i)
+        for (int j = i + 1; j < n_classes; ++j) pairs.push_back({i, j});
+    // every lane's slice of the arena must hold at least the working-set rows of the largest pair
+    const size_t esz = param.kernel_type == SvmParam::LINEAR ? sizeof(double) : sizeof(float);
+    size_t need_min = 0;
+    for (const auto &pr : pairs) {
+        const size_t cols = (size_t) grouped.count()[pr.i] + grouped.count()[pr.j];
+        need_min = std::max(need_min, (size_t) 1024 * ((cols + 7) / 8 * 8) * esz);
+    }
+    tsvm::RowArena &arena = tsvm::RowArena::instance();
+    const size_t budget = cache_bytes > 0 ? (size_t) cache_bytes : cache_bytes < 0 ? arena.auto_budget() : 0;
+    const size_t slice = std::max(budget / lanes, need_min) / 256 * 256;
+    char *const pool = (char *) arena.acquire(slice * lanes, cache_bytes < 0);
+
+    solver_stats.assign(pairs.size(), SolverStats());
+    if (keep_binary) binary_f.assign(pairs.size(), std::vector<float_type>());
+    std::vector<std::unique_ptr<BinaryProblem>> active;
+    std::vector<int> free_lanes;
+    for (int l = lanes - 1; l >= 0; --l) free_lanes.push_back(l);
+    size_t next = 0;
+    auto start_next = [&]() {
+        std::unique_ptr<BinaryProblem> p(new BinaryProblem());
+        p->k = (int) next;
+        setup_binary(grouped, pairs[next].i, pairs[next].j, *p);
+        ++next;
+        p->lane = free_lanes.back();
+        free_lanes.pop_back();
+        const int ws = get_working_set_size((int) p->k_mat->n_instances(), (int) p->k_mat->n_features());
+        p->solver->cache_bytes = cache_bytes;
+        p->task.reset(new SolveTask(*p->solver, *p->k_mat, p->y, p->alpha, rho[p->k], p->f_val, param.epsilon, p->Cp, p->Cn, ws,
+                                    max_iter, pool + (size_t) p->lane * slice, slice));
+        TSVM_HIP_CHECK(hipEventCreateWithFlags(&p->rows_done, hipEventDisableTiming));
+        TSVM_HIP_CHECK(hipEventCreateWithFlags(&p->solved, hipEventDisableTiming));
+        active.push_back(std::move(p));
+    };
+    while (next < pairs.size() && !free_lanes.empty()) start_next();
+    while (!active.empty()) {
+        for (auto &p : active) p->task->enqueue_select();
+        for (auto &p : active) {
+            p->task->enqueue_rows();
+            p->task->enqueue_block();
+            TSVM_HIP_CHECK(hipEventRecord(p->rows_done, p->task->stream()));
+        }
+        for (auto &p : active) {
+            for (auto &o : active)
+                if (o.get() != p.get()) TSVM_HIP_CHECK(hipStreamWaitEvent(p->task->stream(), o->rows_done, 0));
+            p->task->enqueue_solver();
+            TSVM_HIP_CHECK(hipEventRecord(p->solved, p->task->stream()));
+        }
+        for (auto &p : active) {
+            for (auto &o : active)
+                if (o.get() != p.get()) TSVM_HIP_CHECK(hipStreamWaitEvent(p->task->stream(), o->solved, 0));
+            p->task->enqueue_update();
+        }
+        for (size_t a = 0; a < active.size();) {
+            BinaryProblem &p = *active[a];
+            if (!p.task->finish_iteration()) { ++a; continue; }
+            solver_stats[p.k] = p.task->stats();
+            if (keep_binary) binary_f[p.k] = p.f_val;
+            p.task.reset();   // synchronises and releases the pair's stream before its lane is reused
+            (void) hipEventDestroy(p.rows_done);
+            (void) hipEventDestroy(p.solved);
+            finish_binary(p, alpha[p.k]);
+            free_lanes.push_back(p.lane);
+            active.erase(active.begin() + a);
+        }
+        while (next < pairs.size() && !free_lanes.empty()) start_next();
+    }
 }
 
 std::vector<float_type> SVC::predict(const DataSet::node2d &instances, int batch_size) {   // svc.cpp:179-185
@@ -422,24 +522,26 @@ void NuSVC::model_setup(const DataSet &dataset, SvmParam &p) {
     param.svm_type = SvmParam::NU_SVC;
 }
 
-void NuSVC::train_binary(const DataSet &dataset, int i, int j, std::vector<float_type> &alpha, float_type &rho_out) {
+void NuSVC::setup_binary(const DataSet &dataset, int i, int j, BinaryProblem &p) {   // nusvc.cpp:17-50
     const std::vector<int> ids = dataset.original_index(i, j);
     const int n_pos = dataset.count()[i], n = (int) ids.size();
-    std::vector<int> y(n);
-    std::vector<float_type> f_val(n, 0);
-    alpha.assign(n, 0);
+    p.i = i;
+    p.j = j;
+    p.y.resize(n);
+    p.f_val.assign(n, 0);
+    p.alpha.assign(n, 0);
     float_type sum_pos = param.nu * n / 2;
     float_type sum_neg = sum_pos;
     for (int l = 0; l < n; ++l) {
         float_type &budget = l < n_pos ? sum_pos : sum_neg;
-        y[l] = l < n_pos ? +1 : -1;
-        alpha[l] = std::min(1., budget);
-        budget -= alpha[l];
+        p.y[l] = l < n_pos ? +1 : -1;
+        p.alpha[l] = std::min(1., budget);
+        budget -= p.alpha[l];
     }
-    KernelMatrix k_mat(dataset, ids.data(), ids.size(), param);
-    NuSMOSolver solver(false);
-    run_solver(solver, k_mat, y, alpha, rho_out, f_val, 1, 1);
-    for (int l = 0; l < n; ++l) alpha[l] *= y[l];
+    p.k_mat.reset(new KernelMatrix(dataset, ids.data(), ids.size(), param));
+    p.solver.reset(new NuSMOSolver(false));
+    p.Cp = 1;
+    p.Cn = 1;
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -51,6 +51,7 @@ public:
     bool profile = false;
     bool keep_binary = false;             // keep binary_alpha / binary_f (tests)
     long long cache_bytes = -1;           // kernel-row cache budget handed to the solver (-1 auto, 0 off)
+    int pair_lanes = 3;                   // class pairs of a one-vs-one run advanced in lockstep (1: one at a time)
 
 protected:
     virtual void model_setup(const DataSet &dataset, SvmParam &param);
@@ -84,7 +85,22 @@ public:
 
 protected:
     void model_setup(const DataSet &dataset, SvmParam &param) override;
-    virtual void train_binary(const DataSet &dataset, int i, int j, std::vector<float_type> &alpha, float_type &rho);
+    // One class pair (i, j) of the one-vs-one decomposition: its rows, labels, starting point and solver.
+    struct BinaryProblem {
+        int i = 0, j = 0, k = 0;
+        std::unique_ptr<KernelMatrix> k_mat;
+        std::unique_ptr<CSMOSolver> solver;
+        std::vector<int> y;
+        std::vector<float_type> alpha, f_val;
+        float_type Cp = 0, Cn = 0;
+        // lockstep execution
+        std::unique_ptr<SolveTask> task;
+        hipEvent_t rows_done = nullptr, solved = nullptr;
+        int lane = 0;
+    };
+    virtual void setup_binary(const DataSet &dataset, int i, int j, BinaryProblem &p);   // svc.cpp:147-170
+    void finish_binary(BinaryProblem &p, std::vector<float_type> &alpha_out);            // svc.cpp:171-177
+    void train_pairs_in_lockstep(const DataSet &grouped, int lanes, std::vector<std::vector<float_type>> &alpha);
     std::vector<float_type> predict_label(const std::vector<float_type> &dec_values, int n_instances) const;
     std::vector<float_type> c_weight;
 };
@@ -92,7 +108,7 @@ protected:
 class NuSVC : public SVC {
 protected:
     void model_setup(const DataSet &dataset, SvmParam &param) override;
-    void train_binary(const DataSet &dataset, int i, int j, std::vector<float_type> &alpha, float_type &rho) override;
+    void setup_binary(const DataSet &dataset, int i, int j, BinaryProblem &p) override;
 };
 
 class SVR : public SvmModel {

@@ -154,7 +154,11 @@ struct SolveTask::Impl {
         d_alpha_diff.zero();
         d_kws.zero();
         TSVM_HIP_CHECK(hipStreamCreateWithFlags(&sa, hipStreamNonBlocking));
-        TSVM_HIP_CHECK(hipStreamCreateWithFlags(&ids, hipStreamNonBlocking));
+        // A task that runs alone enqueues its solver before the host looks at the new ids, so their
+        // read-back gets a stream of its own; tasks in lockstep read them back on their one stream (the
+        // device has few hardware queues, and streams that share one wait for each other).
+        if (pool) ids = sa;
+        else TSVM_HIP_CHECK(hipStreamCreateWithFlags(&ids, hipStreamNonBlocking));
         TSVM_HIP_CHECK(hipEventCreateWithFlags(&selected, hipEventDisableTiming));
         TSVM_HIP_CHECK(hipEventCreateWithFlags(&ids_ready, hipEventDisableTiming));
         TSVM_HIP_CHECK(hipEventCreateWithFlags(&diff_ready, hipEventDisableTiming));
@@ -216,7 +220,7 @@ struct SolveTask::Impl {
 
     ~Impl() {
         if (sa) (void) hipStreamSynchronize(sa);   // a selection enqueued ahead may still be running
-        if (ids) { (void) hipStreamSynchronize(ids); (void) hipStreamDestroy(ids); }
+        if (ids && ids != sa) { (void) hipStreamSynchronize(ids); (void) hipStreamDestroy(ids); }
         if (sa) (void) hipStreamDestroy(sa);
         if (selected) (void) hipEventDestroy(selected);
         if (ids_ready) (void) hipEventDestroy(ids_ready);
@@ -259,8 +263,8 @@ struct SolveTask::Impl {
         timer.end(stats.ms_select);
         TSVM_HIP_CHECK(hipEventRecord(selected, sa));
         if (caching) {
-            // the new ids travel to the host on their own stream
-            TSVM_HIP_CHECK(hipStreamWaitEvent(ids, selected, 0));
+            // the new ids travel to the host, on their own stream if there is one
+            if (ids != sa) TSVM_HIP_CHECK(hipStreamWaitEvent(ids, selected, 0));
             TSVM_HIP_CHECK(hipMemcpyAsync(h_ids, d_ws.data() + first_new, sizeof(int) * n_new, hipMemcpyDeviceToHost, ids));
             TSVM_HIP_CHECK(hipEventRecord(ids_ready, ids));
         }

@@ -20,17 +20,18 @@ class TsvmParam(C.Structure):
     _fields_ = [("svm_type", C.c_int), ("kernel_type", C.c_int), ("degree", C.c_int), ("max_iter", C.c_int),
                 ("gamma", C.c_double), ("coef0", C.c_double), ("C", C.c_double), ("nu", C.c_double),
                 ("p", C.c_double), ("epsilon", C.c_double), ("max_mem_size", C.c_int64), ("nr_weight", C.c_int),
-                ("verbose", C.c_int), ("weight_label", _ip), ("weight", _dp), ("cache_bytes", C.c_int64)]
+                ("verbose", C.c_int), ("weight_label", _ip), ("weight", _dp), ("cache_bytes", C.c_int64), ("pair_lanes", C.c_int)]
 
 
 def make_param(svm_type=0, kernel_type=2, degree=3, gamma=0.0, coef0=0.0, C=1.0, nu=0.5, p=0.1, epsilon=0.001,
-               max_mem_size=8192 << 20, max_iter=-1, verbose=0, cache_bytes=-1):
+               max_mem_size=8192 << 20, max_iter=-1, verbose=0, cache_bytes=-1, pair_lanes=0):
     """Defaults of include/thundersvm/svmparam.h:14-29."""
     prm = TsvmParam()
     prm.svm_type, prm.kernel_type, prm.degree, prm.max_iter = svm_type, kernel_type, degree, max_iter
     prm.gamma, prm.coef0, prm.C, prm.nu, prm.p, prm.epsilon = gamma, coef0, C, nu, p, epsilon
     prm.max_mem_size, prm.nr_weight, prm.verbose = max_mem_size, 0, verbose
     prm.cache_bytes = cache_bytes
+    prm.pair_lanes = pair_lanes
     return prm
 
 
