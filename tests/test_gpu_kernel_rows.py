@@ -241,3 +241,27 @@ def test_row_subsets_on_device():
     capi.call("tsvm_csr_gather_rows", G.ptr(val_d), G.ptr(col_d), G.ptr(ptr_d), G.ptr(idx_d), m, G.ptr(optr_d), G.ptr(oval),
               G.ptr(ocol), G.stream())
     assert np.array_equal(G.host(oval), sub.val) and np.array_equal(G.host(ocol), sub.col)
+
+
+@pytest.mark.parametrize("n,d,m", [(131072 + 77, 7, 133), (140001, 54, 512), (131072, 90, 200), (135000, 200, 1024), (133333, 16, 65)])
+def test_dense_rbf_many_columns_few_features(n, d, m):
+    """The shapes of the multi-class and regression workloads (hundreds of thousands of columns, tens of features):
+    float and double rows, output slots, ragged last tiles in both directions."""
+    rng = np.random.default_rng(n + d)
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    x[rng.random((n, d)) < 0.3] = 0
+    data = from_dense(x)
+    prm = dict(gamma=0.7 / d)
+    p = O.make_param(kernel_type=O.RBF, expf_mode=1, **prm)
+    okm = O.KernelMatrix(data.ptr, data.col, data.val, p)
+    x_d, nf, ld, sd, diag = _device_km(data, O.RBF, prm)
+    idx = rng.integers(0, n, size=m).astype(np.int32)
+    idx[-1] = n - 1
+    want = okm.get_rows(idx)
+    idx_d = G.dev(idx)
+    got = G.host(G.get_rows_dense(x_d, ld, n, nf, sd, x_d, ld, idx_d, m, sd, O.RBF, **prm))
+    assert np.array_equal(got, want)
+    slots = rng.permutation(m + 9)[:m].astype(np.int32)
+    got32 = G.host(G.get_rows_dense(x_d, ld, n, nf, sd, x_d, ld, idx_d, m, sd, O.RBF, row_type=capi.ROW_F32,
+                                    out_slots=G.dev(slots), out_rows=m + 9, **prm))
+    assert np.array_equal(got32[slots].astype(np.float64), want)
