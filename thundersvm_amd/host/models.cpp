@@ -32,6 +32,7 @@ void SvmModel::model_setup(const DataSet &, SvmParam &p) {   // svmmodel.cpp:22-
     rho.assign(n_binary_models, 0);
     n_sv.assign(n_classes, 0);
     sv.clear();
+    sv_k_mat.reset();
     sv_indices.clear();
     coef.clear();
     linear_coef.clear();
@@ -90,7 +91,10 @@ void SvmModel::predict_dec_values(const DataSet::node2d &instances, std::vector<
             for (int p = 0; p < n_binary_models; ++p) dec[r * n_binary_models + p] = -rho[p];
         return;
     }
-    KernelMatrix k_mat(sv, param);
+    // the support vectors' device copy is built by the first predict call and kept for the next ones (the
+    // reference rebuilds it per call, svmmodel.cpp:84)
+    if (!sv_k_mat) sv_k_mat.reset(new KernelMatrix(sv, param));
+    const KernelMatrix &k_mat = *sv_k_mat;
     if (batch_size == -1) {
         const size_t used = tsvm::device_bytes_in_use();
         const size_t free_mem = param.max_mem_size > used ? param.max_mem_size - used : 0;
@@ -220,6 +224,7 @@ void SvmModel::load_from_file(std::string path) {
 
 // svmmodel.cpp:280-383
 void SvmModel::load_from_string(std::string data) {
+    sv_k_mat.reset();
     std::stringstream iss(data);
     std::string key;
     while (iss >> key) {

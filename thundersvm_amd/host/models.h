@@ -64,6 +64,7 @@ protected:
     std::vector<float_type> coef;
     std::vector<float_type> linear_coef;
     DataSet::node2d sv;
+    mutable std::shared_ptr<KernelMatrix> sv_k_mat;   // device copy of sv, built by the first predict call
     std::vector<int> sv_indices;
     std::vector<int> n_sv;           // per class
     int n_total_sv = 0;
