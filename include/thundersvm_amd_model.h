@@ -69,6 +69,10 @@ int tsvm_dataset_to_device(void *dataset);
 int tsvm_model_train(void *model, void *dataset, const tsvm_param *param, int ws_override, int keep_binary,
                      int trace_cap, int profile);
 int tsvm_model_predict(void *model, void *dataset, int batch_size, double *dec_values, double *labels);
+/* SvmModel::cross_validation (src/thundersvm/model/svmmodel.cpp:31-71) on a freshly created model: stratified
+ * n_fold folds in class order, predictions[i] = the prediction for instance i by the model trained without its
+ * fold (a label for the classifiers, a value for the regressors). */
+int tsvm_model_cross_validation(void *model, void *dataset, const tsvm_param *param, int n_fold, double *predictions);
 
 /* SvmModel::train on a LibSVM text file (DataSet::load_from_file). */
 int tsvm_model_train_file(void *model, const char *path, const tsvm_param *param);

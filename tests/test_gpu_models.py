@@ -12,7 +12,9 @@ import numpy as np
 import pytest
 
 import oracle_lib as O
+from thundersvm_amd import capi
 from thundersvm_amd import data as D
+from thundersvm_amd.data import load_libsvm
 from thundersvm_amd.model import Dataset, Model, make_param
 
 pytestmark = pytest.mark.gpu
@@ -189,3 +191,19 @@ def test_class_pairs_in_lockstep_give_the_same_model():
         else:
             assert np.array_equal(cur[0], ref[0]) and np.array_equal(cur[1], ref[1]) and np.array_equal(cur[2], ref[2])
             assert cur[3] == ref[3] and cur[4] == ref[4]
+
+
+@pytest.mark.parametrize("svm_type,extra,golden,metric", [
+    (capi.C_SVC, dict(C=10.0), 0.973, "acc"),          # test_cross_validation.cpp:51-59
+    (capi.NU_SVC, dict(), 0.660, "acc"),               # :61-68
+    (capi.NU_SVR, dict(), 0.045, "mse"),               # :70-76
+    (capi.EPSILON_SVR, dict(), 0.044, "mse"),          # :78-84
+])
+def test_cross_validation_goldens(svm_type, extra, golden, metric):
+    """The reference's 5-fold cross-validation scores on its fixture (tolerance 1e-3, as in its tests)."""
+    ds = Dataset(path=FIXTURE)
+    y = load_libsvm(FIXTURE).y
+    prm = make_param(svm_type=svm_type, kernel_type=capi.RBF, gamma=0.125, **extra)
+    pred = Model(svm_type).cross_validation(ds, prm, 5)
+    score = float(np.mean(pred == y)) if metric == "acc" else float(np.mean((pred - y) ** 2))
+    assert abs(score - golden) < 1e-3, score

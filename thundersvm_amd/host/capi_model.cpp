@@ -146,6 +146,16 @@ int tsvm_model_predict(void *model, void *dataset, int batch_size, double *dec_v
     })
 }
 
+int tsvm_model_cross_validation(void *model, void *dataset, const tsvm_param *param, int n_fold, double *predictions) {
+    TSVM_GUARD({
+        Handle *h = (Handle *) model;
+        configure(h, param, 0, 0, 0, 0);
+        const DataSet &ds = *(DataSet *) dataset;
+        std::vector<float_type> out = h->model->cross_validation(ds, to_param(*param), n_fold);
+        memcpy(predictions, out.data(), sizeof(double) * out.size());
+    })
+}
+
 int tsvm_model_train_file(void *model, const char *path, const tsvm_param *param) {
     TSVM_GUARD({
         Handle *h = (Handle *) model;

@@ -197,6 +197,14 @@ class Model:
                                                  _p(data.val, _dp), batch_size, _p(dec, _dp), _p(lab, _dp)))
         return lab, dec
 
+    def cross_validation(self, dataset, prm, n_fold):
+        """SvmModel::cross_validation on a Dataset: the out-of-fold prediction of every instance."""
+        L = host_lib()
+        L.tsvm_model_cross_validation.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(TsvmParam), C.c_int, _dp]
+        out = np.zeros(dataset.n)
+        _check(L.tsvm_model_cross_validation(self.h, dataset.h, C.byref(prm), n_fold, _p(out, _dp)))
+        return out
+
     def save(self, path):
         _check(host_lib().tsvm_model_save(self.h, path.encode()))
 
