@@ -24,11 +24,14 @@
 //     cubic polynomial, all in double), which the HIP epilogue restates too.
 //     tests/test_oracle_expf.py counts how often the two differ on this host.
 //
-// Pinning status of each part is listed in DESIGN.md; the composite solver
-// trajectory (solve + sort_f + select_working_set + c_smo_solve) has no
-// fixture in the reference holding alpha/rho, and the reference CPU build
-// cannot be built here (Eigen absent): that composite is "parity unpinned"
-// beyond the reference's accuracy / MSE / SV-count goldens.
+// Pinning: tests/test_oracle_golden.py (the reference's fixture, row sets and
+// accuracy / MSE / SV-count goldens), tests/test_oracle_expf.py and
+// tests/test_oracle_smo.py (closed forms, brute force, invariants) check every
+// part on its own.  The composite solver trajectory (solve + sort_f +
+// select_working_set + c_smo_solve / nu_smo_solve) has no fixture in the
+// reference holding alpha or rho, and the reference CPU build cannot be built
+// here (Eigen absent): that composite is "parity unpinned" beyond the
+// reference's accuracy / MSE / SV-count / cross-validation goldens.
 #include <algorithm>
 #include <cmath>
 #include <cstdint>
