@@ -48,7 +48,8 @@ __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
     constexpr int BM = 32 * TI;
     constexpr int KTILE = TI == 2 ? 16 : 8;
     constexpr int LS = TI == 2 ? 129 : 130;
-    constexpr int A_TPR = KTILE / 4;          // threads per A row (one 4-double vector each)
+    constexpr int A_TPR = 256 / BM;           // threads per A row
+    constexpr int A_VEC = KTILE / 4 / A_TPR;  // 4-double vectors per thread for the A tile
     constexpr int B_VEC = KTILE / 8;          // 4-double vectors per thread for the B tile (2 threads per row)
     __shared__ double As[KTILE * LS];
     __shared__ double Bs[KTILE * LS];
@@ -67,19 +68,19 @@ __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
     const int64_t j0 = (int64_t) (logical / m_blocks) * GR_BN;
     const int i0 = (int) (logical % m_blocks) * BM;
 
-    // staging assignment
-    const int a_row = tid / A_TPR, a_k = (tid % A_TPR) * 4;
+    // Staging assignment.  Rows beyond the tile's valid range are clamped to the last valid row: what they
+    // stage only reaches outputs that are never stored, and every load stays unconditional.  (Any VALU
+    // instruction, a zero fill included, is issued at the expense of another wavefront's fp64 MFMA.)
+    const int a_row = tid / A_TPR, a_k = (tid % A_TPR) * (4 * A_VEC);
     const int b_row = tid >> 1, b_k = (tid & 1) * (4 * B_VEC);
-    const double *a_ptr = nullptr;
-    const double *x_ptr = nullptr;
+    const double *a_ptr, *x_ptr;   // first column of this thread's row
     {
-        const int ai = i0 + a_row;
-        if (ai < m) {
-            const int64_t r = a_idx ? (int64_t) a_idx[ai] : (int64_t) ai;
-            a_ptr = a + r * lda + a_k;
-        }
-        const int64_t xj = j0 + b_row;
-        if (xj < n) x_ptr = x + (x_idx ? (int64_t) x_idx[xj] : xj) * ldx + b_k;
+        const int ai = min(i0 + a_row, m - 1);
+        const uint32_t r = (uint32_t) (a_idx ? a_idx[ai] : ai);
+        a_ptr = a + (uint64_t) r * (uint32_t) lda;
+        const int64_t xj = min(j0 + b_row, n - 1);
+        const uint32_t xr = (uint32_t) (x_idx ? (int64_t) x_idx[xj] : xj);
+        x_ptr = x + (uint64_t) xr * (uint32_t) ldx;
     }
 
     v4d acc[TI][4];
@@ -99,60 +100,77 @@ __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
     int64_t orow_off[TI * 4];
 #pragma unroll
     for (int tj = 0; tj < 4; ++tj) {
-        const int64_t j = jb + tj * 16;
-        sdj[tj] = (sd_x && j < n) ? sd_x[x_idx ? (int64_t) x_idx[j] : j] : 0.0;
+        const int64_t j = min(jb + tj * 16, n - 1);
+        sdj[tj] = sd_x ? sd_x[x_idx ? (int64_t) x_idx[j] : j] : 0.0;
     }
 #pragma unroll
     for (int u = 0; u < TI * 4; ++u) {
-        const int i = i0 + wi * (16 * TI) + (u >> 2) * 16 + 4 * (u & 3) + lk;
-        const bool ok = i < m;
-        sdi[u] = (sd_a && ok) ? sd_a[a_idx ? a_idx[i] : i] : 0.0;
-        orow_off[u] = (int64_t) ((out_slots && ok) ? out_slots[i] : i) * ldo;
+        const int i = min(i0 + wi * (16 * TI) + (u >> 2) * 16 + 4 * (u & 3) + lk, m - 1);
+        sdi[u] = sd_a ? sd_a[a_idx ? a_idx[i] : i] : 0.0;
+        orow_off[u] = (int64_t) ((uint64_t) (uint32_t) (out_slots ? out_slots[i] : i) * (uint32_t) ldo);
     }
 
-    // rows are padded with zeros up to ldx / lda (multiples of 8), so a vector may be read whenever
-    // its first column is inside the padded row
-    const int kmax_a = (int) lda, kmax_x = (int) ldx;
+    // Rows are padded with zeros up to ldx / lda (multiples of 8).  An 8-column tile therefore always lies
+    // inside the padded row.  The last 16-column tile may reach past it: its vectors that would start beyond
+    // the row re-read the row's last four columns instead; they are staged but never multiplied (n_ks below).
     const int n_kt = (d + KTILE - 1) / KTILE;
-    const v4d zero4 = (v4d){0.0, 0.0, 0.0, 0.0};
-    v4d ra = zero4, rb[B_VEC];
+    v4d ra[A_VEC], rb[B_VEC];
     auto load_tile = [&](int kt) {
         const int k0 = kt * KTILE;
-        ra = (a_ptr && (KTILE == 8 || k0 + a_k < kmax_a)) ? *(const v4d *) (a_ptr + k0) : zero4;
 #pragma unroll
-        for (int q = 0; q < B_VEC; ++q)
-            rb[q] = (x_ptr && (KTILE == 8 || k0 + b_k + 4 * q < kmax_x)) ? *(const v4d *) (x_ptr + k0 + 4 * q) : zero4;
+        for (int q = 0; q < A_VEC; ++q) ra[q] = *(const v4d *) (a_ptr + (k0 + a_k + 4 * q));
+#pragma unroll
+        for (int q = 0; q < B_VEC; ++q) rb[q] = *(const v4d *) (x_ptr + (k0 + b_k + 4 * q));
     };
-    load_tile(0);
-
-    for (int kt = 0; kt < n_kt; ++kt) {
+    auto load_last_tile = [&](int kt) {
+        const int k0 = kt * KTILE;
+#pragma unroll
+        for (int q = 0; q < A_VEC; ++q) ra[q] = *(const v4d *) (a_ptr + min(k0 + a_k + 4 * q, (int) lda - 4));
+#pragma unroll
+        for (int q = 0; q < B_VEC; ++q) rb[q] = *(const v4d *) (x_ptr + min(k0 + b_k + 4 * q, (int) ldx - 4));
+    };
+    auto stage_tile = [&]() {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            As[(a_k + e) * LS + a_row] = ra[e];
+#pragma unroll
+            for (int q = 0; q < A_VEC; ++q) As[(a_k + 4 * q + e) * LS + a_row] = ra[q][e];
 #pragma unroll
             for (int q = 0; q < B_VEC; ++q) Bs[(b_k + 4 * q + e) * LS + b_row] = rb[q][e];
         }
-        __syncthreads();
-        if (kt + 1 < n_kt) load_tile(kt + 1);
-        const int k_left = d - kt * KTILE;               // columns still to multiply (uniform)
-        const int n_ks = k_left >= KTILE ? KTILE / 4 : (k_left + 3) / 4;
+    };
+    auto mma_step = [&](int ks) {   // four columns of the staged tile
+        double af[TI], bf[4];
+        const int kk = (ks * 4 + lk) * LS;
 #pragma unroll
-        for (int ks = 0; ks < KTILE / 4; ++ks) {
-            if (KTILE == 8 || ks < n_ks) {   // 8-column tiles are always whole (rows are padded to 8)
-                double af[TI], bf[4];
-                const int kk = (ks * 4 + lk) * LS;
+        for (int t = 0; t < TI; ++t) af[t] = As[kk + wi * (16 * TI) + t * 16 + lrow];
 #pragma unroll
-                for (int t = 0; t < TI; ++t) af[t] = As[kk + wi * (16 * TI) + t * 16 + lrow];
+        for (int t = 0; t < 4; ++t) bf[t] = Bs[kk + wj * 64 + t * 16 + lrow];
 #pragma unroll
-                for (int t = 0; t < 4; ++t) bf[t] = Bs[kk + wj * 64 + t * 16 + lrow];
+        for (int ti = 0; ti < TI; ++ti)
 #pragma unroll
-                for (int ti = 0; ti < TI; ++ti)
+            for (int tj = 0; tj < 4; ++tj)
+                acc[ti][tj] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[ti], bf[tj], acc[ti][tj], 0, 0, 0);
+    };
+
+    if (n_kt > 0) {
+        if (KTILE == 8 || n_kt > 1) load_tile(0);
+        else load_last_tile(0);
+        // every tile but the last is whole
+        for (int kt = 0; kt + 1 < n_kt; ++kt) {
+            stage_tile();
+            __syncthreads();
+            if (KTILE == 8 || kt + 2 < n_kt) load_tile(kt + 1);
+            else load_last_tile(kt + 1);
 #pragma unroll
-                    for (int tj = 0; tj < 4; ++tj)
-                        acc[ti][tj] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[ti], bf[tj], acc[ti][tj], 0, 0, 0);
-            }
+            for (int ks = 0; ks < KTILE / 4; ++ks) mma_step(ks);
+            __syncthreads();
         }
+        stage_tile();
         __syncthreads();
+        const int n_ks = (d - (n_kt - 1) * KTILE + 3) / 4;   // groups of four columns left, 1 .. KTILE / 4
+#pragma unroll
+        for (int ks = 0; ks < KTILE / 4; ++ks)
+            if (KTILE == 8 || ks < n_ks) mma_step(ks);       // 8-column tiles are always whole (rows are padded to 8)
     }
 
     // epilogue + store.  Interior tiles take the unguarded path; edge tiles test every element.
@@ -164,7 +182,7 @@ __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
                 TO *orow = out + orow_off[ti * 4 + v] + jb;
 #pragma unroll
                 for (int tj = 0; tj < 4; ++tj)
-                    orow[tj * 16] = (TO) tsvm_epilogue(acc[ti][tj][v], sdi[ti * 4 + v], sdj[tj], kp, exp_tab);
+                    orow[tj * 16] = tsvm_epilogue_as<TO>(acc[ti][tj][v], sdi[ti * 4 + v], sdj[tj], kp, exp_tab);
             }
         }
     } else {
@@ -177,7 +195,7 @@ __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
                 TO *orow = out + orow_off[ti * 4 + v] + jb;
 #pragma unroll
                 for (int tj = 0; tj < 4; ++tj)
-                    if (jb + tj * 16 < n) orow[tj * 16] = (TO) tsvm_epilogue(acc[ti][tj][v], sdi[ti * 4 + v], sdj[tj], kp, exp_tab);
+                    if (jb + tj * 16 < n) orow[tj * 16] = tsvm_epilogue_as<TO>(acc[ti][tj][v], sdi[ti * 4 + v], sdj[tj], kp, exp_tab);
             }
         }
     }
@@ -228,7 +246,7 @@ __global__ __launch_bounds__(256) void get_rows_csr_kernel(
 #pragma unroll
     for (int jj = 0; jj < CS_JB; ++jj) {
         const int64_t j = j0 + jj;
-        if (j < n) orow[j] = (TO) tsvm_epilogue(acc[jj], sdi, sd_x ? sd_x[x_idx ? (int64_t) x_idx[j] : j] : 0.0, kp, exp_tab);
+        if (j < n) orow[j] = tsvm_epilogue_as<TO>(acc[jj], sdi, sd_x ? sd_x[x_idx ? (int64_t) x_idx[j] : j] : 0.0, kp, exp_tab);
     }
 }
 
@@ -460,6 +478,8 @@ int tsvm_get_rows_dense(const double *x, int64_t ldx, const int *x_idx, int64_t 
                         tsvm_stream stream) {
     TSVM_REQUIRE(x && a && out, "tsvm_get_rows_dense: null pointer");
     TSVM_REQUIRE(n >= 0 && m >= 0 && d >= 0, "tsvm_get_rows_dense: negative size");
+    TSVM_REQUIRE(n <= 0x7fffffff && ldx <= 0x7fffffff && lda <= 0x7fffffff && ldo <= 0x7fffffff,
+                 "tsvm_get_rows_dense: row counts and leading dimensions must fit 31 bits");
     TSVM_REQUIRE(ldx % 8 == 0 && lda % 8 == 0, "tsvm_get_rows_dense: ldx (%lld) and lda (%lld) must be multiples of 8",
                  (long long) ldx, (long long) lda);
     TSVM_REQUIRE(d <= ldx && d <= lda, "tsvm_get_rows_dense: d (%d) exceeds a leading dimension", d);

@@ -41,12 +41,13 @@ __device__ __forceinline__ float tsvm_expf(float x, const uint64_t *tab) {
     double xd = (double) x;
     double z = InvLn2N * xd;
     double kd = z + SHIFT;
-    uint64_t ki = (uint64_t) __double_as_longlong(kd);
+    const uint32_t ki = (uint32_t) __double2loint(kd);
     kd -= SHIFT;
     double r = z - kd;
-    uint64_t t = tab[ki & 31];
-    t += ki << 47;
-    double s = __longlong_as_double((long long) t);
+    // s = 2^(k/32): table entry with k/32 added into the exponent field.  The published routine adds
+    // ki << 47 to the 64-bit entry; the low word of that term is zero, so only the high word changes.
+    const uint64_t t = tab[ki & 31];
+    double s = __hiloint2double((int) ((uint32_t) (t >> 32) + (ki << 15)), (int) (uint32_t) t);
     double zz = __builtin_fma(C0, r, C1);
     double r2 = r * r;
     double y = __builtin_fma(C2, r, 1.0);
@@ -59,26 +60,39 @@ __device__ __forceinline__ float tsvm_expf(float x, const uint64_t *tab) {
 }
 
 // Kernel epilogues (kernelmatrix_kernel.cpp:61-108).  sd0/sd1 are the two rows' self dot products.
-__device__ __forceinline__ double tsvm_epilogue(double dot, double sd0, double sd1, const KernelParam &p,
-                                                const uint64_t *tab) {
+// The RBF / polynomial / sigmoid values are floats by definition (expf / powf / tanhf); this returns that
+// float, so that a caller storing float rows pays for no round trip through double.
+__device__ __forceinline__ float tsvm_epilogue_f32(double dot, double sd0, double sd1, const KernelParam &p,
+                                                   const uint64_t *tab) {
     switch (p.kernel_type) {
-        case TSVM_RBF:
-        case TSVM_PRECOMPUTED: {
-            double arg = -(sd0 + sd1 - dot * 2) * p.gamma;
-            return (double) tsvm_expf((float) arg, tab);
-        }
         case TSVM_POLY: {
             // powf / tanhf of a float-rounded argument: evaluated in double and rounded once to float
             const float arg = (float) __builtin_fma(p.gamma, dot, p.coef0);
-            return (double) (float) pow((double) arg, (double) p.degree);
+            return (float) pow((double) arg, (double) p.degree);
         }
         case TSVM_SIGMOID: {
             const float arg = (float) __builtin_fma(p.gamma, dot, p.coef0);
-            return (double) (float) tanh((double) arg);
+            return (float) tanh((double) arg);
         }
-        default:
-            return dot;
+        default: {
+            // -(sd0 + sd1 - 2*dot) * gamma; 2*dot is exact, so the fma rounds exactly where the subtraction would
+            const double arg = -__builtin_fma(-2.0, dot, sd0 + sd1) * p.gamma;
+            return tsvm_expf((float) arg, tab);
+        }
     }
+}
+
+__device__ __forceinline__ double tsvm_epilogue(double dot, double sd0, double sd1, const KernelParam &p,
+                                                const uint64_t *tab) {
+    return p.kernel_type == TSVM_LINEAR ? dot : (double) tsvm_epilogue_f32(dot, sd0, sd1, p, tab);
+}
+
+// the value as an element of a kernel row (float rows are never used with the linear kernel)
+template <typename TO>
+__device__ __forceinline__ TO tsvm_epilogue_as(double dot, double sd0, double sd1, const KernelParam &p,
+                                               const uint64_t *tab) {
+    if constexpr (sizeof(TO) == 4) return tsvm_epilogue_f32(dot, sd0, sd1, p, tab);
+    else return tsvm_epilogue(dot, sd0, sd1, p, tab);
 }
 
 // include/thundersvm/kernel/smo_kernel.h:13-23
