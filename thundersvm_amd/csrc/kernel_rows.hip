@@ -65,50 +65,66 @@ __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
     __syncthreads();
 
     const unsigned logical = xcd_remap(blockIdx.x, gridDim.x);
-    const int64_t j0 = (int64_t) (logical / m_blocks) * GR_BN;
+    const int j0 = (int) (logical / m_blocks) * GR_BN;   // n fits 31 bits (checked by the host)
     const int i0 = (int) (logical % m_blocks) * BM;
+    const int n_last = (int) n - 1, m_last = m - 1;
 
     // Staging assignment.  Rows beyond the tile's valid range are clamped to the last valid row: what they
     // stage only reaches outputs that are never stored, and every load stays unconditional.  (Any VALU
     // instruction, a zero fill included, is issued at the expense of another wavefront's fp64 MFMA.)
     const int a_row = tid / A_TPR, a_k = (tid % A_TPR) * (4 * A_VEC);
     const int b_row = tid >> 1, b_k = (tid & 1) * (4 * B_VEC);
-    const double *a_ptr, *x_ptr;   // first column of this thread's row
-    {
-        const int ai = min(i0 + a_row, m - 1);
-        const uint32_t r = (uint32_t) (a_idx ? a_idx[ai] : ai);
-        a_ptr = a + (uint64_t) r * (uint32_t) lda;
-        const int64_t xj = min(j0 + b_row, n - 1);
-        const uint32_t xr = (uint32_t) (x_idx ? (int64_t) x_idx[xj] : xj);
-        x_ptr = x + (uint64_t) xr * (uint32_t) ldx;
+    // Per-row / per-column data of the epilogue (self dot products, output row offsets).  Everything that goes
+    // through an index array is fetched in two batches of independent loads (all indices, then all values),
+    // ahead of the K loop, instead of one dependent pair after the other.
+    const int lrow = lane & 15;
+    const int lk = lane >> 4;
+    const int jb = j0 + wj * 64 + lrow;
+    const bool full = (i0 + BM <= m) && (j0 + GR_BN <= (int) n);
+    int a_r = min(i0 + a_row, m_last), x_r = min(j0 + b_row, n_last);   // staged rows
+    int jr[4], ir[TI * 4], slot[TI * 4];
+#pragma unroll
+    for (int tj = 0; tj < 4; ++tj) jr[tj] = min(jb + tj * 16, n_last);
+#pragma unroll
+    for (int u = 0; u < TI * 4; ++u) ir[u] = slot[u] = min(i0 + wi * (16 * TI) + (u >> 2) * 16 + 4 * (u & 3) + lk, m_last);
+    if (out_slots) {
+#pragma unroll
+        for (int u = 0; u < TI * 4; ++u) slot[u] = out_slots[slot[u]];
     }
+    if (a_idx) {
+        a_r = a_idx[a_r];
+#pragma unroll
+        for (int u = 0; u < TI * 4; ++u) ir[u] = a_idx[ir[u]];
+    }
+    if (x_idx) {
+        x_r = x_idx[x_r];
+#pragma unroll
+        for (int tj = 0; tj < 4; ++tj) jr[tj] = x_idx[jr[tj]];
+    }
+    const double *a_ptr = a + (uint64_t) (uint32_t) a_r * (uint32_t) lda;   // first column of this thread's rows
+    const double *x_ptr = x + (uint64_t) (uint32_t) x_r * (uint32_t) ldx;
+    double sdj[4], sdi[TI * 4];
+#pragma unroll
+    for (int tj = 0; tj < 4; ++tj) sdj[tj] = 0.0;
+#pragma unroll
+    for (int u = 0; u < TI * 4; ++u) sdi[u] = 0.0;
+    if (sd_x) {
+#pragma unroll
+        for (int tj = 0; tj < 4; ++tj) sdj[tj] = sd_x[jr[tj]];
+    }
+    if (sd_a) {
+#pragma unroll
+        for (int u = 0; u < TI * 4; ++u) sdi[u] = sd_a[ir[u]];
+    }
+    int64_t orow_off[TI * 4];
+#pragma unroll
+    for (int u = 0; u < TI * 4; ++u) orow_off[u] = (int64_t) ((uint64_t) (uint32_t) slot[u] * (uint32_t) ldo);
 
     v4d acc[TI][4];
 #pragma unroll
     for (int ti = 0; ti < TI; ++ti)
 #pragma unroll
         for (int tj = 0; tj < 4; ++tj) acc[ti][tj] = (v4d){0.0, 0.0, 0.0, 0.0};
-
-    // Per-row / per-column data of the epilogue (self dot products, output row offsets) is fetched
-    // here, ahead of the K loop, so that its dependent loads are off the critical path by the time the
-    // accumulators are ready.
-    const int lrow = lane & 15;
-    const int lk = lane >> 4;
-    const int64_t jb = j0 + wj * 64 + lrow;
-    const bool full = (i0 + BM <= m) && (j0 + GR_BN <= n);
-    double sdj[4], sdi[TI * 4];
-    int64_t orow_off[TI * 4];
-#pragma unroll
-    for (int tj = 0; tj < 4; ++tj) {
-        const int64_t j = min(jb + tj * 16, n - 1);
-        sdj[tj] = sd_x ? sd_x[x_idx ? (int64_t) x_idx[j] : j] : 0.0;
-    }
-#pragma unroll
-    for (int u = 0; u < TI * 4; ++u) {
-        const int i = min(i0 + wi * (16 * TI) + (u >> 2) * 16 + 4 * (u & 3) + lk, m - 1);
-        sdi[u] = sd_a ? sd_a[a_idx ? a_idx[i] : i] : 0.0;
-        orow_off[u] = (int64_t) ((uint64_t) (uint32_t) (out_slots ? out_slots[i] : i) * (uint32_t) ldo);
-    }
 
     // Rows are padded with zeros up to ldx / lda (multiples of 8).  An 8-column tile therefore always lies
     // inside the padded row.  The last 16-column tile may reach past it: its vectors that would start beyond
@@ -478,7 +494,7 @@ int tsvm_get_rows_dense(const double *x, int64_t ldx, const int *x_idx, int64_t 
                         tsvm_stream stream) {
     TSVM_REQUIRE(x && a && out, "tsvm_get_rows_dense: null pointer");
     TSVM_REQUIRE(n >= 0 && m >= 0 && d >= 0, "tsvm_get_rows_dense: negative size");
-    TSVM_REQUIRE(n <= 0x7fffffff && ldx <= 0x7fffffff && lda <= 0x7fffffff && ldo <= 0x7fffffff,
+    TSVM_REQUIRE(n <= 0x7fff0000 && ldx <= 0x7fffffff && lda <= 0x7fffffff && ldo <= 0x7fffffff,
                  "tsvm_get_rows_dense: row counts and leading dimensions must fit 31 bits");
     TSVM_REQUIRE(ldx % 8 == 0 && lda % 8 == 0, "tsvm_get_rows_dense: ldx (%lld) and lda (%lld) must be multiples of 8",
                  (long long) ldx, (long long) lda);
