@@ -508,8 +508,8 @@ int tsvm_get_rows_dense(const double *x, int64_t ldx, const int *x_idx, int64_t 
                  "tsvm_get_rows_dense: RBF needs self dot products");
     if (n == 0 || m == 0) return 0;
     KernelParam kp{kernel_type, degree, gamma, coef0};
-    // small feature counts: the epilogue and the stores dominate, run the 64-row tile at higher occupancy
-    const int ti = d <= 256 ? 2 : 4;
+    // few features: the epilogue weighs as much as the MFMAs, run the 64-row tile at higher occupancy
+    const int ti = d <= 128 ? 2 : 4;
     const unsigned m_blocks = (unsigned) ((m + 32 * ti - 1) / (32 * ti));
     const int64_t n_blocks = (n + GR_BN - 1) / GR_BN;
     TSVM_REQUIRE(n_blocks * m_blocks < (int64_t) 0x7fffffff, "tsvm_get_rows_dense: grid too large");
