@@ -155,7 +155,8 @@ def _select_case(n, n_select, n_marked, seed, tie_mode, nu):
 @pytest.mark.parametrize("nu", [0, 1])
 @pytest.mark.parametrize("tie_mode", [0, 1, 2])
 @pytest.mark.parametrize("n,n_select,n_marked", [(2, 2, 0), (150, 128, 0), (150, 64, 64), (3200, 1024, 0), (3200, 512, 512),
-                                                 (100000, 512, 512), (70001, 1024, 0), (1100, 1024, 0), (1030, 512, 512)])
+                                                 (100000, 512, 512), (70001, 1024, 0), (1100, 1024, 0), (1030, 512, 512),
+                                                 (1200000, 512, 512)])
 def test_select_working_set(n, n_select, n_marked, tie_mode, nu):
     f, y, alpha, C, marked = _select_case(n, n_select, n_marked, n + n_select + tie_mode, tie_mode, nu)
     want = O.select_working_set(f, y, alpha, C, C, marked, n_select, nu=bool(nu))

@@ -242,51 +242,63 @@ __global__ void sel_mark_kernel(uint8_t *ind, const int *__restrict__ marked, in
 }
 
 // Computes, in LDS, the state after pass p-1's histogram has been consumed (st_out), from the
-// state before it (global state[p-1]) and hist[p-1].  Every workgroup does this redundantly.
+// state before it (global state[p-1]) and hist[p-1].  Every workgroup does this redundantly; the first
+// SEL_T threads of the workgroup do the work, any others only join the barriers.
+//
+// A side is decided as soon as the boundary bucket can be taken whole: when everything up to and including
+// it fits the side's list (MAX_WS entries), the list is a superset of the k smallest candidates, in which
+// every extra entry is larger than all of them, and sel_final_kernel sorts the list and reads it from the
+// front.  With 11-bit digits that is the normal case after the second pass.
 __device__ void sel_advance_state(const SelWorkspace &w, const SelGeom &g, int p, SelState *st_out /* LDS [sides] */,
                                   uint32_t *scratch /* LDS [SEL_T + 8] */) {
     const int tid = threadIdx.x;
+    const bool worker = tid < SEL_T;
     const int lane = tid & 63, wave = tid >> 6;
     for (int s = 0; s < g.n_sides; ++s) {
         SelState st = w.state[(p - 1) * SEL_MAX_SIDES + s];
         if (!st.done) {
             const uint32_t *h = w.hist + ((size_t) (p - 1) * SEL_MAX_SIDES + s) * SEL_BINS;
             uint32_t c[SEL_BINS / SEL_T];
-            uint32_t sum = 0;
+            uint32_t sum = 0, incl = 0;
+            if (worker) {
 #pragma unroll
-            for (int e = 0; e < SEL_BINS / SEL_T; ++e) { c[e] = h[tid * (SEL_BINS / SEL_T) + e]; sum += c[e]; }
-            uint32_t incl = sum;
+                for (int e = 0; e < SEL_BINS / SEL_T; ++e) { c[e] = h[tid * (SEL_BINS / SEL_T) + e]; sum += c[e]; }
+                incl = sum;
 #pragma unroll
-            for (int d = 1; d < 64; d <<= 1) {
-                uint32_t o = __shfl_up(incl, d, 64);
-                if (lane >= d) incl += o;
-            }
-            if (lane == 63) scratch[wave] = incl;
-            __syncthreads();
-            uint32_t wave_base = 0, total = 0;
-            for (int wv = 0; wv < SEL_T / 64; ++wv) {
-                if (wv < wave) wave_base += scratch[wv];
-                total += scratch[wv];
-            }
-            const uint32_t excl = wave_base + incl - sum;
-            if (total < st.k_rem) {
-                // fewer candidates than requested (only possible on the first digit): take them all
-                if (tid == 0) { st.done = 1; st.k_rem = total; st_out[s] = st; }
-            } else if (excl < st.k_rem && st.k_rem <= excl + sum) {
-                uint32_t below = excl;
-                int b = 0;
-                for (int e = 0; e < SEL_BINS / SEL_T; ++e) {
-                    if (below + c[e] >= st.k_rem) { b = tid * (SEL_BINS / SEL_T) + e; break; }
-                    below += c[e];
+                for (int d = 1; d < 64; d <<= 1) {
+                    uint32_t o = __shfl_up(incl, d, 64);
+                    if (lane >= d) incl += o;
                 }
-                const uint32_t cb = h[b];
-                bool is_key; int shift, width;
-                sel_digit_geom(p - 1, g.idx_bits, is_key, shift, width);
-                if (is_key) st.pk |= (uint64_t) b << shift; else st.pi |= (uint32_t) b << shift;
-                st.k_rem -= below;
-                st.pad = (uint32_t) p;
-                if (cb == st.k_rem || p == g.n_pass) st.done = 1;
-                st_out[s] = st;
+                if (lane == 63) scratch[wave] = incl;
+            }
+            __syncthreads();
+            if (worker) {
+                uint32_t wave_base = 0, total = 0;
+                for (int wv = 0; wv < SEL_T / 64; ++wv) {
+                    if (wv < wave) wave_base += scratch[wv];
+                    total += scratch[wv];
+                }
+                const uint32_t excl = wave_base + incl - sum;
+                if (total < st.k_rem) {
+                    // fewer candidates than requested (only possible on the first digit): take them all
+                    if (tid == 0) { st.done = 1; st.k_rem = total; st_out[s] = st; }
+                } else if (excl < st.k_rem && st.k_rem <= excl + sum) {
+                    uint32_t below = excl;
+                    int b = 0;
+                    for (int e = 0; e < SEL_BINS / SEL_T; ++e) {
+                        if (below + c[e] >= st.k_rem) { b = tid * (SEL_BINS / SEL_T) + e; break; }
+                        below += c[e];
+                    }
+                    const uint32_t cb = h[b];
+                    const uint32_t taken = g.k - st.k_rem;   // entries of the buckets decided by earlier digits
+                    bool is_key; int shift, width;
+                    sel_digit_geom(p - 1, g.idx_bits, is_key, shift, width);
+                    if (is_key) st.pk |= (uint64_t) b << shift; else st.pi |= (uint32_t) b << shift;
+                    st.k_rem -= below;
+                    st.pad = (uint32_t) p;
+                    if (cb == st.k_rem || p == g.n_pass || taken + below + cb <= (uint32_t) MAX_WS) st.done = 1;
+                    st_out[s] = st;
+                }
             }
             __syncthreads();
         } else {
@@ -295,6 +307,21 @@ __device__ void sel_advance_state(const SelWorkspace &w, const SelGeom &g, int p
         }
     }
     __syncthreads();
+}
+
+// One candidate's contribution to the histograms of digit p: on every undecided side it belongs to, if it
+// matches that side's prefix.
+__device__ __forceinline__ void sel_count(const SelGeom &g, const SelState *st, uint32_t (*lhist)[SEL_BINS], int p,
+                                          bool is_key, int shift, uint32_t dmask, uint64_t key, uint32_t fl, int64_t j) {
+    for (int s = 0; s < g.n_sides; ++s) {
+        if (!(fl & (1u << s)) || st[s].done) continue;
+        const bool desc = sel_side_descending(s, g.n_sides);
+        const uint64_t k2 = desc ? ~key : key;
+        const uint32_t i2 = desc ? g.idx_mask - (uint32_t) j : (uint32_t) j;
+        if (sel_cmp_prefix(k2, i2, st[s], p, g.idx_bits) != 0) continue;
+        const uint32_t dg = is_key ? (uint32_t) (k2 >> shift) & dmask : (i2 >> shift) & dmask;
+        atomicAdd(&lhist[s][dg], 1u);
+    }
 }
 
 // Pass p: (p == 0: also builds keys/flags) histogram digit p of the not-yet-decided candidates.
@@ -345,21 +372,51 @@ __global__ __launch_bounds__(SEL_T) void sel_pass_kernel(SelWorkspace w, const d
             if (!fl) continue;
             key = w.keys[j];
         }
-        for (int s = 0; s < g.n_sides; ++s) {
-            if (!(fl & (1u << s)) || st[s].done) continue;
-            const bool desc = sel_side_descending(s, g.n_sides);
-            const uint64_t k2 = desc ? ~key : key;
-            const uint32_t i2 = desc ? g.idx_mask - (uint32_t) j : (uint32_t) j;
-            if (sel_cmp_prefix(k2, i2, st[s], p, g.idx_bits) != 0) continue;
-            const uint32_t dg = is_key ? (uint32_t) (k2 >> shift) & dmask : (i2 >> shift) & dmask;
-            atomicAdd(&lhist[s][dg], 1u);
-        }
+        sel_count(g, st, lhist, p, is_key, shift, dmask, key, fl, j);
     }
     __syncthreads();
     uint32_t *gh = w.hist + (size_t) p * SEL_MAX_SIDES * SEL_BINS;
     for (int e = tid; e < g.n_sides * SEL_BINS; e += SEL_T) {
         const uint32_t c = (&lhist[0][0])[e];
         if (c) atomicAdd(&gh[e], c);
+    }
+}
+
+// Passes p_first .. n_pass-1 in one workgroup.  After the grid-wide passes every side is normally decided
+// and this kernel only carries the state forward; when a boundary bucket is still too large (many equal f
+// values, e.g. the first iteration of a training run, where the instance index has to break the ties), the
+// one workgroup walks the candidates once per remaining digit.  That is slow but rare, and it replaces one
+// kernel launch per digit in every call.
+#define SEL_TAIL_T 1024
+__global__ __launch_bounds__(SEL_TAIL_T) void sel_tail_kernel(SelWorkspace w, int64_t n, SelGeom g, int p_first) {
+    __shared__ uint32_t lhist[SEL_MAX_SIDES][SEL_BINS];
+    __shared__ SelState st[SEL_MAX_SIDES];
+    __shared__ uint32_t scratch[SEL_T + 16];
+    const int tid = threadIdx.x;
+    for (int p = p_first; p < g.n_pass; ++p) {
+        sel_advance_state(w, g, p, st, scratch);
+        if (tid < g.n_sides) w.state[p * SEL_MAX_SIDES + tid] = st[tid];
+        bool any = false;
+        for (int s = 0; s < g.n_sides; ++s) any |= !st[s].done;
+        if (!any) {
+            // decided: later states are copies (sel_compact_kernel reads the last one)
+            for (int q = p + 1; q < g.n_pass; ++q)
+                if (tid < g.n_sides) w.state[q * SEL_MAX_SIDES + tid] = st[tid];
+            return;
+        }
+        for (int e = tid; e < SEL_MAX_SIDES * SEL_BINS; e += SEL_TAIL_T) (&lhist[0][0])[e] = 0;
+        __syncthreads();
+        bool is_key; int shift, width;
+        sel_digit_geom(p, g.idx_bits, is_key, shift, width);
+        const uint32_t dmask = (1u << width) - 1;
+        for (int64_t j = tid; j < n; j += SEL_TAIL_T) {
+            const uint32_t fl = w.flags[j];
+            if (fl) sel_count(g, st, lhist, p, is_key, shift, dmask, w.keys[j], fl, j);
+        }
+        __syncthreads();
+        uint32_t *gh = w.hist + (size_t) p * SEL_MAX_SIDES * SEL_BINS;   // zeroed by sel_init_kernel
+        for (int e = tid; e < g.n_sides * SEL_BINS; e += SEL_TAIL_T) gh[e] = (&lhist[0][0])[e];
+        __syncthreads();   // the next digit's sel_advance_state reads state[p] and hist[p] back from memory
     }
 }
 
@@ -581,8 +638,14 @@ int tsvm_select_working_set(const double *f, const int *y, const double *alpha, 
         hipLaunchKernelGGL(sel_mark_kernel, dim3((n_marked + 255) / 256), dim3(256), 0, s, w.ind, marked, n_marked);
         TSVM_LAUNCH_CHECK();
     }
-    for (int p = 0; p < g.n_pass; ++p) {
+    // the first digits are counted by the whole chip, the rest (rarely needed) by one workgroup
+    const int p_full = std::min(g.n_pass, n > ((int64_t) 1 << 20) ? 3 : 2);
+    for (int p = 0; p < p_full; ++p) {
         hipLaunchKernelGGL(sel_pass_kernel, dim3(grid), dim3(SEL_T), 0, s, w, f, y, alpha, n, Cp, Cn, g, p);
+        TSVM_LAUNCH_CHECK();
+    }
+    if (p_full < g.n_pass) {
+        hipLaunchKernelGGL(sel_tail_kernel, dim3(1), dim3(SEL_TAIL_T), 0, s, w, n, g, p_full);
         TSVM_LAUNCH_CHECK();
     }
     hipLaunchKernelGGL(sel_compact_kernel, dim3(grid), dim3(SEL_T), 0, s, w, n, g);
