@@ -483,22 +483,37 @@ __global__ __launch_bounds__(MAX_WS) void sel_final_kernel(SelWorkspace w, SelGe
         }
     }
     __syncthreads();
-    // bitonic sort, ascending composite, all sides at once
-    for (int size = 2; size <= MAX_WS; size <<= 1) {
+    // Bitonic sort, ascending composite, all sides at once.  Thread t owns compare-exchange pair t & 511 of
+    // side t >> 9 (and of side 2 + (t >> 9) when there are four), so every thread works in every stage.  With
+    // strides up to 64 a wavefront's 64 pairs cover one closed block of 128 entries, stage after stage: such
+    // stages only need the wavefront's own LDS accesses kept in order, not a workgroup barrier.
+    int m_sort = 2;
+    for (int s = 0; s < g.n_sides; ++s)
+        while (m_sort < cnt[s]) m_sort <<= 1;   // padding entries are already in place behind the longest list
+    const int pr = tid & (MAX_WS / 2 - 1);
+    for (int size = 2; size <= m_sort; size <<= 1) {
         for (int strd = size >> 1; strd > 0; strd >>= 1) {
-            const int partner = tid ^ strd;
-            if (partner > tid) {
-                const bool asc = (tid & size) == 0;
-                for (int s = 0; s < g.n_sides; ++s) {
-                    const uint64_t ka = sk[s][tid], kb = sk[s][partner];
-                    const uint32_t ia = si[s][tid], ib = si[s][partner];
+            const int lo = ((pr & ~(strd - 1)) << 1) | (pr & (strd - 1));
+            const int hi = lo | strd;
+            const bool asc = (lo & size) == 0;
+            if (hi < m_sort) {
+                for (int s = tid >> 9; s < g.n_sides; s += 2) {
+                    const uint64_t ka = sk[s][lo], kb = sk[s][hi];
+                    const uint32_t ia = si[s][lo], ib = si[s][hi];
                     const bool sw = asc ? comp_less(kb, ib, ka, ia) : comp_less(ka, ia, kb, ib);
-                    if (sw) { sk[s][tid] = kb; sk[s][partner] = ka; si[s][tid] = ib; si[s][partner] = ia; }
+                    if (sw) { sk[s][lo] = kb; sk[s][hi] = ka; si[s][lo] = ib; si[s][hi] = ia; }
                 }
             }
-            __syncthreads();
+            const int next_strd = strd > 1 ? strd >> 1 : (2 * size <= m_sort ? size : 0);
+            if (strd > 64 || next_strd > 64) {
+                __syncthreads();
+            } else {
+                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");   // LDS accesses of a wavefront complete in order
+                __builtin_amdgcn_wave_barrier();
+            }
         }
     }
+    __syncthreads();
     // real instance ids; descending sides stored idx_mask - id
     for (int s = 0; s < g.n_sides; ++s)
         if (tid < cnt[s] && sel_side_descending(s, g.n_sides)) si[s][tid] = g.idx_mask - si[s][tid];
