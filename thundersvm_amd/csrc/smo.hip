@@ -248,7 +248,7 @@ __global__ void sel_mark_kernel(uint8_t *ind, const int *__restrict__ marked, in
 // A side is decided as soon as the boundary bucket can be taken whole: when everything up to and including
 // it fits the side's list (MAX_WS entries), the list is a superset of the k smallest candidates, in which
 // every extra entry is larger than all of them, and sel_final_kernel sorts the list and reads it from the
-// front.  With 11-bit digits that is the normal case after the second pass.
+// front.  With 11-bit digits that is the normal case after the second or third pass.
 __device__ void sel_advance_state(const SelWorkspace &w, const SelGeom &g, int p, SelState *st_out /* LDS [sides] */,
                                   uint32_t *scratch /* LDS [SEL_T + 8] */) {
     const int tid = threadIdx.x;
@@ -653,8 +653,10 @@ int tsvm_select_working_set(const double *f, const int *y, const double *alpha, 
         hipLaunchKernelGGL(sel_mark_kernel, dim3((n_marked + 255) / 256), dim3(256), 0, s, w.ind, marked, n_marked);
         TSVM_LAUNCH_CHECK();
     }
-    // the first digits are counted by the whole chip, the rest (rarely needed) by one workgroup
-    const int p_full = std::min(g.n_pass, n > ((int64_t) 1 << 20) ? 3 : 2);
+    // The first three digits (33 bits of f) are counted by the whole chip, the rest (rarely needed) by one
+    // workgroup.  Near convergence the free support vectors crowd within epsilon of the threshold, so the third
+    // digit is usually the one that separates them.
+    const int p_full = std::min(g.n_pass, n > ((int64_t) 1 << 26) ? 4 : 3);
     for (int p = 0; p < p_full; ++p) {
         hipLaunchKernelGGL(sel_pass_kernel, dim3(grid), dim3(SEL_T), 0, s, w, f, y, alpha, n, Cp, Cn, g, p);
         TSVM_LAUNCH_CHECK();
