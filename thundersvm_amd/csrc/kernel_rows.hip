@@ -509,7 +509,10 @@ int tsvm_get_rows_dense(const double *x, int64_t ldx, const int *x_idx, int64_t 
     if (n == 0 || m == 0) return 0;
     KernelParam kp{kernel_type, degree, gamma, coef0};
     // few features: the epilogue weighs as much as the MFMAs, run the 64-row tile at higher occupancy
-    const int ti = d <= 128 ? 2 : 4;
+    // (also when the 128-row tile would leave most of the chip without a workgroup, as for the solver's
+    // ws x ws block, whose latency is that of one workgroup walking the whole feature range)
+    const int64_t wg4 = ((n + GR_BN - 1) / GR_BN) * ((m + 127) / 128);
+    const int ti = (d <= 128 || wg4 < 512) ? 2 : 4;
     const unsigned m_blocks = (unsigned) ((m + 32 * ti - 1) / (32 * ti));
     const int64_t n_blocks = (n + GR_BN - 1) / GR_BN;
     TSVM_REQUIRE(n_blocks * m_blocks < (int64_t) 0x7fffffff, "tsvm_get_rows_dense: grid too large");

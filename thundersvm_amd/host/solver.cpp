@@ -113,6 +113,13 @@ struct SolveTask::Impl {
     // selected ids for the host-side cache bookkeeping, so that it does not wait behind the solver.
     hipStream_t sa = nullptr, ids = nullptr;
     hipEvent_t selected = nullptr, ids_ready = nullptr, diff_ready = nullptr;
+    // A task that runs alone splits the chip: the local solver (one workgroup, a chain of dependent steps) gets a
+    // stream `ss` restricted to one CU of every XCD, everything else runs on `sa`, restricted to the other CUs.
+    // The solver then runs next to this iteration's get_rows at nearly its stand-alone speed; sharing CUs with a
+    // chip-wide kernel it runs two to three times slower, which is why tasks in lockstep keep the phases apart.
+    hipStream_t ss = nullptr;
+    hipEvent_t block_done = nullptr, solved = nullptr;
+    bool split = false;
 
     void *k_rows = nullptr;
     bool caching = false;
@@ -153,7 +160,11 @@ struct SolveTask::Impl {
         d_diff.zero();
         d_alpha_diff.zero();
         d_kws.zero();
-        TSVM_HIP_CHECK(hipStreamCreateWithFlags(&sa, hipStreamNonBlocking));
+        split = !pool && !solver.profile && create_split_streams();
+        if (!split) {
+            TSVM_HIP_CHECK(hipStreamCreateWithFlags(&sa, hipStreamNonBlocking));
+            ss = sa;
+        }
         // A task that runs alone enqueues its solver before the host looks at the new ids, so their
         // read-back gets a stream of its own; tasks in lockstep read them back on their one stream (the
         // device has few hardware queues, and streams that share one wait for each other).
@@ -162,6 +173,8 @@ struct SolveTask::Impl {
         TSVM_HIP_CHECK(hipEventCreateWithFlags(&selected, hipEventDisableTiming));
         TSVM_HIP_CHECK(hipEventCreateWithFlags(&ids_ready, hipEventDisableTiming));
         TSVM_HIP_CHECK(hipEventCreateWithFlags(&diff_ready, hipEventDisableTiming));
+        TSVM_HIP_CHECK(hipEventCreateWithFlags(&block_done, hipEventDisableTiming));
+        TSVM_HIP_CHECK(hipEventCreateWithFlags(&solved, hipEventDisableTiming));
 
         // Kernel rows live in slots of one pool.  With a cache the pool holds up to pool_rows rows and the
         // host tracks which instance sits in which slot; without one it holds exactly ws rows.
@@ -171,8 +184,8 @@ struct SolveTask::Impl {
         if (cache_bytes != 0 && n_u > ws_size) {
             const long long budget = pool ? (long long) pool_bytes : cache_bytes > 0 ? cache_bytes : (long long) arena.auto_budget();
             const long long fit = budget / (long long) (ld * row_esz);
-            // an LRU that can hold only a small part of the matrix does not hit: require a quarter of the rows
-            if (fit >= 4LL * ws_size && fit >= n_u / 4) pool_rows = std::min<long long>(n_u, fit);
+            // a cache worth having holds a few working sets; one that turns out not to hit is switched off below
+            if (fit >= 4LL * ws_size) pool_rows = std::min<long long>(n_u, fit);
         }
         caching = pool_rows > ws_size;
         const size_t need = (size_t) pool_rows * ld * row_esz;
@@ -214,20 +227,46 @@ struct SolveTask::Impl {
         // compute on its own, without the stored rows, so it and the solver can be enqueued before the host
         // does the cache bookkeeping.  With many features that small launch (64 workgroups walking the whole
         // feature range) costs more than it hides, and the block is gathered from the stored rows instead.
-        block_first = k_mat.n_features() < 256;
+        // (When the solver has CUs of its own the block always comes first: the solver then runs while the rows
+        // are computed.)
+        block_first = split || k_mat.n_features() < 256;
         stats.ms_setup = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - wall0).count();
     }
 
     ~Impl() {
         if (sa) (void) hipStreamSynchronize(sa);   // a selection enqueued ahead may still be running
+        if (ss && ss != sa) { (void) hipStreamSynchronize(ss); (void) hipStreamDestroy(ss); }
         if (ids && ids != sa) { (void) hipStreamSynchronize(ids); (void) hipStreamDestroy(ids); }
         if (sa) (void) hipStreamDestroy(sa);
+        if (block_done) (void) hipEventDestroy(block_done);
+        if (solved) (void) hipEventDestroy(solved);
         if (selected) (void) hipEventDestroy(selected);
         if (ids_ready) (void) hipEventDestroy(ids_ready);
         if (diff_ready) (void) hipEventDestroy(diff_ready);
         if (h_diff) (void) hipHostFree(h_diff);
         if (h_ids) (void) hipHostFree(h_ids);
         if (h_slots) (void) hipHostFree(h_slots);
+    }
+
+    // Two streams with disjoint CU masks.  Bit i of a mask names CU i/8 of XCD i%8 on the 8-XCD, 256-CU part
+    // (a mask has to leave every XCD at least one CU: workgroups are dealt to the XCDs in turn).  Anything
+    // unexpected (another CU count, the call failing, TSVM_NO_CU_SPLIT set) leaves the task on one plain stream.
+    bool create_split_streams() {
+        if (getenv("TSVM_NO_CU_SPLIT")) return false;
+        int dev = 0, n_cu = 0;
+        if (hipGetDevice(&dev) != hipSuccess) return false;
+        if (hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n_cu != 256) return false;
+        uint32_t small[8] = {0xffu, 0, 0, 0, 0, 0, 0, 0};
+        uint32_t big[8];
+        for (int w = 0; w < 8; ++w) big[w] = ~small[w];
+        if (hipExtStreamCreateWithCUMask(&ss, 8, small) != hipSuccess) { (void) hipGetLastError(); ss = nullptr; return false; }
+        if (hipExtStreamCreateWithCUMask(&sa, 8, big) != hipSuccess) {
+            (void) hipGetLastError();
+            (void) hipStreamDestroy(ss);
+            ss = sa = nullptr;
+            return false;
+        }
+        return true;
     }
 
     // without a cache the slot tables just alternate: the two halves of the working set swap places
@@ -341,21 +380,25 @@ struct SolveTask::Impl {
         else
             abi_check(tsvm_smo_gather_block(k_rows, row_type, slots, ld, ws_u, ws_size, d_kws.data(), sa));
         timer.end(stats.ms_local);
+        if (split) TSVM_HIP_CHECK(hipEventRecord(block_done, sa));
     }
 
     void enqueue_solver() {
         timer.begin();
+        if (split) TSVM_HIP_CHECK(hipStreamWaitEvent(ss, block_done, 0));
         if (nu) {
             abi_check(tsvm_nu_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), d_ws.data(), ws_size,
-                                              Cp, d_kws.data(), k_mat.diag(), eps, d_diff.data(), max_iter, sa));
+                                              Cp, d_kws.data(), k_mat.diag(), eps, d_diff.data(), max_iter, ss));
         } else {
             abi_check(tsvm_c_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), d_ws.data(), ws_size,
-                                             Cp, Cn, d_kws.data(), k_mat.diag(), eps, d_diff.data(), max_iter, sa));
+                                             Cp, Cn, d_kws.data(), k_mat.diag(), eps, d_diff.data(), max_iter, ss));
         }
         timer.end(stats.ms_local);
+        if (split) TSVM_HIP_CHECK(hipEventRecord(solved, ss));
     }
 
     void enqueue_update() {
+        if (split) TSVM_HIP_CHECK(hipStreamWaitEvent(sa, solved, 0));   // alpha_diff, alpha and diff come from the solver
         timer.begin();
         abi_check(tsvm_update_f(d_f.data(), d_alpha_diff.data(), ws_size, k_rows, row_type, slots, ld, n_u, rep, sa));
         timer.end(stats.ms_update_f);
