@@ -75,7 +75,7 @@ static void configure(Handle *h, const tsvm_param *param, int ws_override, int k
     h->model->keep_binary = keep_binary != 0;
     h->model->profile = profile != 0;
     h->model->cache_bytes = param->cache_bytes;
-    h->model->pair_lanes = param->pair_lanes > 0 ? param->pair_lanes : 3;
+    h->model->pair_lanes = param->pair_lanes > 0 ? param->pair_lanes : 0;
     h->trace = SolverTrace();
     h->trace.cap_iters = trace_cap;
     h->model->trace_first = trace_cap > 0 ? &h->trace : nullptr;

@@ -326,7 +326,9 @@ void SVC::train(const DataSet &dataset, SvmParam p) {   // svc.cpp:41-145
     std::vector<std::vector<float_type>> alpha(n_binary_models);
     std::vector<char> is_sv(n, 0);
     int k = 0;
-    const int lanes = std::min(pair_lanes, n_binary_models);
+    // pairs in flight: two when every pair's solver gets CUs of its own (more pairs only add queues), three when
+    // the pairs alternate between a solver phase and a chip-wide phase
+    const int lanes = std::min(pair_lanes > 0 ? pair_lanes : SolveTask::cu_split_available() ? 2 : 3, n_binary_models);
     if (lanes > 1 && !profile && !trace_first) {
         train_pairs_in_lockstep(grouped, lanes, alpha);
     } else {
@@ -458,7 +460,7 @@ void SVC::train_pairs_in_lockstep(const DataSet &grouped, int lanes, std::vector
         const int ws = get_working_set_size((int) p->k_mat->n_instances(), (int) p->k_mat->n_features());
         p->solver->cache_bytes = cache_bytes;
         p->task.reset(new SolveTask(*p->solver, *p->k_mat, p->y, p->alpha, rho[p->k], p->f_val, param.epsilon, p->Cp, p->Cn, ws,
-                                    max_iter, pool + (size_t) p->lane * slice, slice));
+                                    max_iter, pool + (size_t) p->lane * slice, slice, p->lane, lanes));
         TSVM_HIP_CHECK(hipEventCreateWithFlags(&p->rows_done, hipEventDisableTiming));
         TSVM_HIP_CHECK(hipEventCreateWithFlags(&p->solved, hipEventDisableTiming));
         active.push_back(std::move(p));
@@ -466,6 +468,13 @@ void SVC::train_pairs_in_lockstep(const DataSet &grouped, int lanes, std::vector
     while (next < pairs.size() && !free_lanes.empty()) start_next();
     while (!active.empty()) {
         for (auto &p : active) p->task->enqueue_select();
+        if (active.front()->task->split_streams()) {
+            // Every pair's solver has CUs of its own: the pairs need no phases, their steps are only enqueued in
+            // an order that lets each solver start before the host turns to the cache bookkeeping.
+            for (auto &p : active) { p->task->enqueue_block(); p->task->enqueue_solver(); }
+            for (auto &p : active) p->task->enqueue_rows();
+            for (auto &p : active) p->task->enqueue_update();
+        } else {
         for (auto &p : active) {
             p->task->enqueue_rows();
             p->task->enqueue_block();
@@ -481,6 +490,7 @@ void SVC::train_pairs_in_lockstep(const DataSet &grouped, int lanes, std::vector
             for (auto &o : active)
                 if (o.get() != p.get()) TSVM_HIP_CHECK(hipStreamWaitEvent(p->task->stream(), o->solved, 0));
             p->task->enqueue_update();
+        }
         }
         for (size_t a = 0; a < active.size();) {
             BinaryProblem &p = *active[a];

@@ -51,7 +51,7 @@ public:
     bool profile = false;
     bool keep_binary = false;             // keep binary_alpha / binary_f (tests)
     long long cache_bytes = -1;           // kernel-row cache budget handed to the solver (-1 auto, 0 off)
-    int pair_lanes = 3;                   // class pairs of a one-vs-one run advanced in lockstep (1: one at a time)
+    int pair_lanes = 0;                   // class pairs of a one-vs-one run in flight (0: automatic, 1: one at a time)
 
 protected:
     virtual void model_setup(const DataSet &dataset, SvmParam &param);

@@ -141,7 +141,7 @@ struct SolveTask::Impl {
 
     Impl(const CSMOSolver &solver, const KernelMatrix &k_mat, const std::vector<int> &y, std::vector<float_type> &alpha,
          float_type &rho, std::vector<float_type> &f_val, float_type eps, float_type Cp, float_type Cn, int ws_size,
-         int out_max_iter, void *pool, size_t pool_bytes)
+         int out_max_iter, void *pool, size_t pool_bytes, int lane, int n_lanes)
         : solver(solver), k_mat(k_mat), y(y), alpha(alpha), rho(rho), f_val(f_val), eps(eps), Cp(Cp), Cn(Cn), ws_size(ws_size),
           out_max_iter(out_max_iter), n((int) k_mat.n_instances()), n_u((int) k_mat.n_columns()), rep(k_mat.repeat()),
           row_type(k_mat.row_type()), row_esz(k_mat.row_elem_size()), q(ws_size / 2), ld(((int64_t) n_u + 7) / 8 * 8),
@@ -160,7 +160,7 @@ struct SolveTask::Impl {
         d_diff.zero();
         d_alpha_diff.zero();
         d_kws.zero();
-        split = !pool && !solver.profile && create_split_streams();
+        split = !solver.profile && create_split_streams(lane, n_lanes);
         if (!split) {
             TSVM_HIP_CHECK(hipStreamCreateWithFlags(&sa, hipStreamNonBlocking));
             ss = sa;
@@ -251,14 +251,12 @@ struct SolveTask::Impl {
     // Two streams with disjoint CU masks.  Bit i of a mask names CU i/8 of XCD i%8 on the 8-XCD, 256-CU part
     // (a mask has to leave every XCD at least one CU: workgroups are dealt to the XCDs in turn).  Anything
     // unexpected (another CU count, the call failing, TSVM_NO_CU_SPLIT set) leaves the task on one plain stream.
-    bool create_split_streams() {
-        if (getenv("TSVM_NO_CU_SPLIT")) return false;
-        int dev = 0, n_cu = 0;
-        if (hipGetDevice(&dev) != hipSuccess) return false;
-        if (hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n_cu != 256) return false;
-        uint32_t small[8] = {0xffu, 0, 0, 0, 0, 0, 0, 0};
-        uint32_t big[8];
-        for (int w = 0; w < 8; ++w) big[w] = ~small[w];
+    // Lane l's solver gets CU l of every XCD; the chip-wide kernels of all lanes get the CUs no lane's solver has.
+    bool create_split_streams(int lane, int n_lanes) {
+        if (!SolveTask::cu_split_available() || n_lanes < 1 || n_lanes > 4 || lane < 0 || lane >= n_lanes) return false;
+        uint32_t small[8] = {0xffu << (8 * lane), 0, 0, 0, 0, 0, 0, 0};
+        uint32_t big[8] = {0, ~0u, ~0u, ~0u, ~0u, ~0u, ~0u, ~0u};
+        big[0] = n_lanes == 4 ? 0u : ~0u << (8 * n_lanes);
         if (hipExtStreamCreateWithCUMask(&ss, 8, small) != hipSuccess) { (void) hipGetLastError(); ss = nullptr; return false; }
         if (hipExtStreamCreateWithCUMask(&sa, 8, big) != hipSuccess) {
             (void) hipGetLastError();
@@ -455,8 +453,8 @@ struct SolveTask::Impl {
 
 SolveTask::SolveTask(const CSMOSolver &solver, const KernelMatrix &k_mat, const std::vector<int> &y, std::vector<float_type> &alpha,
                      float_type &rho, std::vector<float_type> &f_val, float_type eps, float_type Cp, float_type Cn, int ws_size,
-                     int out_max_iter, void *pool, size_t pool_bytes)
-    : impl_(new Impl(solver, k_mat, y, alpha, rho, f_val, eps, Cp, Cn, ws_size, out_max_iter, pool, pool_bytes)) {}
+                     int out_max_iter, void *pool, size_t pool_bytes, int lane, int n_lanes)
+    : impl_(new Impl(solver, k_mat, y, alpha, rho, f_val, eps, Cp, Cn, ws_size, out_max_iter, pool, pool_bytes, lane, n_lanes)) {}
 SolveTask::~SolveTask() { delete impl_; }
 void SolveTask::enqueue_select() { impl_->enqueue_select(); }
 void SolveTask::enqueue_rows() { impl_->enqueue_rows(); }
@@ -465,6 +463,13 @@ void SolveTask::enqueue_solver() { impl_->enqueue_solver(); }
 void SolveTask::enqueue_update() { impl_->enqueue_update(); }
 bool SolveTask::finish_iteration() { return impl_->finish_iteration(); }
 bool SolveTask::block_needs_rows() const { return !impl_->block_first; }
+bool SolveTask::split_streams() const { return impl_->split; }
+bool SolveTask::cu_split_available() {
+    if (getenv("TSVM_NO_CU_SPLIT")) return false;
+    int dev = 0, n_cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return false;
+    return hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n_cu == 256;
+}
 hipStream_t SolveTask::stream() const { return impl_->sa; }
 const SolverStats &SolveTask::stats() const { return impl_->stats; }
 size_t SolveTask::min_pool_bytes(const KernelMatrix &k_mat, int ws_size) {

@@ -74,10 +74,11 @@ private:
 class SolveTask {
 public:
     // pool / pool_bytes: device memory for the kernel rows (nullptr: taken from the process-wide arena
-    // according to solver.cache_bytes)
+    // according to solver.cache_bytes).  lane / n_lanes: which of the tasks advanced side by side this one is;
+    // every lane's local solver gets CUs of its own.
     SolveTask(const CSMOSolver &solver, const KernelMatrix &k_mat, const std::vector<int> &y, std::vector<float_type> &alpha,
               float_type &rho, std::vector<float_type> &f_val, float_type eps, float_type Cp, float_type Cn, int ws_size,
-              int out_max_iter, void *pool = nullptr, size_t pool_bytes = 0);
+              int out_max_iter, void *pool = nullptr, size_t pool_bytes = 0, int lane = 0, int n_lanes = 1);
     ~SolveTask();
     SolveTask(const SolveTask &) = delete;
     SolveTask &operator=(const SolveTask &) = delete;
@@ -89,9 +90,11 @@ public:
     void enqueue_update();
     bool finish_iteration();   // waits for this iteration's diff; true once the solve is complete and its results are written
     bool block_needs_rows() const;
+    bool split_streams() const;   // the local solver runs on CUs of its own, next to this task's (and other tasks') chip-wide kernels
     hipStream_t stream() const;
     const SolverStats &stats() const;
     static size_t min_pool_bytes(const KernelMatrix &k_mat, int ws_size);
+    static bool cu_split_available();   // the device is one whose CUs this code knows how to divide
 
 private:
     struct Impl;
