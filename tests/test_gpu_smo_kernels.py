@@ -167,3 +167,23 @@ def test_select_working_set(n, n_select, n_marked, tie_mode, nu):
               n_marked, G.ptr(out_d), n_select, nu, G.ptr(wsp), G.stream())
     got = G.host(out_d)
     assert np.array_equal(got, want), "first mismatch at %s" % np.flatnonzero(got != want)[:5]
+
+
+@pytest.mark.parametrize("nu", [0, 1])
+@pytest.mark.parametrize("tie_mode", [0, 1, 2])
+def test_longer_selection_starts_with_the_shorter_one(tie_mode, nu):
+    """Asking for more ids appends runners-up: the first n_select ids do not change."""
+    n, n_marked = 50000, 512
+    f, y, alpha, C, marked = _select_case(n, 512, n_marked, 99 + tie_mode, tie_mode, nu)
+    f_d, y_d, a_d, m_d = G.dev(f), G.dev(y), G.dev(alpha), G.dev(marked)
+    wsp = torch.empty(capi.kernel_lib().tsvm_select_workspace(n), dtype=torch.uint8, device="cuda")
+    outs = []
+    for n_select in (512, 768):
+        out_d = torch.full((n_select,), -7, dtype=torch.int32, device="cuda")
+        capi.call("tsvm_select_working_set", G.ptr(f_d), G.ptr(y_d), G.ptr(a_d), n, C, C, G.ptr(m_d), n_marked, G.ptr(out_d),
+                  n_select, nu, G.ptr(wsp), G.stream())
+        outs.append(G.host(out_d))
+    assert np.array_equal(outs[1][:512], outs[0])
+    assert np.array_equal(outs[1], O.select_working_set(f, y, alpha, C, C, marked, 768, nu=bool(nu)))
+    tail = outs[1][512:]
+    assert (tail >= 0).all() and len(set(tail.tolist()) | set(outs[0].tolist()) | set(marked.tolist())) == 768 + n_marked
