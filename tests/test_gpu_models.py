@@ -193,6 +193,25 @@ def test_class_pairs_in_lockstep_give_the_same_model():
             assert cur[3] == ref[3] and cur[4] == ref[4]
 
 
+@pytest.mark.parametrize("wl", ["c1", "c5"])
+def test_split_and_serial_schedules_give_the_same_model(wl, monkeypatch):
+    """A task alone runs its local solver on compute units of its own, next to get_rows; with TSVM_NO_CU_SPLIT it
+    runs every step in order on one stream.  Same trajectory, same model."""
+    w = D.workload_c1(scale=0.5) if wl == "c1" else D.workload_c5(scale=0.005)
+    tr, prm = w["train"], make_param(**w["params"])
+    models = []
+    for serial in (False, True):
+        if serial:
+            monkeypatch.setenv("TSVM_NO_CU_SPLIT", "1")
+        m = Model(prm.svm_type).train(tr, prm, keep_binary=True)
+        models.append((m.coef.copy(), m.rho.copy(), m.sv_indices.copy(), m.stats(0)["n_iter"], m.stats(0)["local_iter"],
+                       m.binary(0)))
+    a, b = models
+    assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1]) and np.array_equal(a[2], b[2])
+    assert a[3] == b[3] and a[4] == b[4]
+    assert np.array_equal(a[5][0], b[5][0]) and np.array_equal(a[5][1], b[5][1])
+
+
 @pytest.mark.parametrize("svm_type,extra,golden,metric", [
     (capi.C_SVC, dict(C=10.0), 0.973, "acc"),          # test_cross_validation.cpp:51-59
     (capi.NU_SVC, dict(), 0.660, "acc"),               # :61-68
