@@ -120,6 +120,9 @@ struct SolveTask::Impl {
     hipStream_t ss = nullptr;
     hipEvent_t block_done = nullptr, solved = nullptr;
     bool split = false;
+    // Once the cache holds every row there is no get_rows left to run next to the solver; the iteration then
+    // stays on `sa` from start to end and saves the two hand-overs between the streams.
+    bool on_one_stream = false, alone = true;   // alone: no other task's kernels on the chip
 
     void *k_rows = nullptr;
     bool caching = false;
@@ -160,6 +163,7 @@ struct SolveTask::Impl {
         d_diff.zero();
         d_alpha_diff.zero();
         d_kws.zero();
+        alone = n_lanes == 1;
         split = !solver.profile && create_split_streams(lane, n_lanes);
         if (!split) {
             TSVM_HIP_CHECK(hipStreamCreateWithFlags(&sa, hipStreamNonBlocking));
@@ -378,25 +382,27 @@ struct SolveTask::Impl {
         else
             abi_check(tsvm_smo_gather_block(k_rows, row_type, slots, ld, ws_u, ws_size, d_kws.data(), sa));
         timer.end(stats.ms_local);
-        if (split) TSVM_HIP_CHECK(hipEventRecord(block_done, sa));
+        on_one_stream = !split || (alone && caching && cache.used == n_u);
+        if (!on_one_stream) TSVM_HIP_CHECK(hipEventRecord(block_done, sa));
     }
 
     void enqueue_solver() {
         timer.begin();
-        if (split) TSVM_HIP_CHECK(hipStreamWaitEvent(ss, block_done, 0));
+        hipStream_t st = on_one_stream ? sa : ss;
+        if (!on_one_stream) TSVM_HIP_CHECK(hipStreamWaitEvent(ss, block_done, 0));
         if (nu) {
             abi_check(tsvm_nu_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), d_ws.data(), ws_size,
-                                              Cp, d_kws.data(), k_mat.diag(), eps, d_diff.data(), max_iter, ss));
+                                              Cp, d_kws.data(), k_mat.diag(), eps, d_diff.data(), max_iter, st));
         } else {
             abi_check(tsvm_c_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), d_ws.data(), ws_size,
-                                             Cp, Cn, d_kws.data(), k_mat.diag(), eps, d_diff.data(), max_iter, ss));
+                                             Cp, Cn, d_kws.data(), k_mat.diag(), eps, d_diff.data(), max_iter, st));
         }
         timer.end(stats.ms_local);
-        if (split) TSVM_HIP_CHECK(hipEventRecord(solved, ss));
+        if (!on_one_stream) TSVM_HIP_CHECK(hipEventRecord(solved, ss));
     }
 
     void enqueue_update() {
-        if (split) TSVM_HIP_CHECK(hipStreamWaitEvent(sa, solved, 0));   // alpha_diff, alpha and diff come from the solver
+        if (!on_one_stream) TSVM_HIP_CHECK(hipStreamWaitEvent(sa, solved, 0));   // alpha_diff, alpha and diff come from the solver
         timer.begin();
         abi_check(tsvm_update_f(d_f.data(), d_alpha_diff.data(), ws_size, k_rows, row_type, slots, ld, n_u, rep, sa));
         timer.end(stats.ms_update_f);
