@@ -420,13 +420,14 @@ void SVC::finish_binary(BinaryProblem &p, std::vector<float_type> &alpha_out) { 
     alpha_out = std::move(p.alpha);
 }
 
-// The class pairs are independent problems.  Up to `lanes` of them are in flight, each a SolveTask on its
-// own stream with its own slice of the kernel-row arena, advanced one outer iteration at a time in three
-// phases separated by events: (1) selection, kernel rows and the solver's block of every pair, (2) the
-// local solvers of all pairs, which are single workgroups and so run side by side on different CUs, (3)
-// update_f of every pair.  A chip-wide kernel never overlaps a local solver: measured next to one, each
-// solver iteration takes 3.3-3.6x longer.  A pair that finishes hands its lane to the next pair.  The
-// result of a pair does not depend on what runs beside it.
+// The class pairs are independent problems.  Up to `lanes` of them are in flight, each a SolveTask with its own
+// slice of the kernel-row arena; a pair that finishes hands its lane to the next pair, and the result of a pair
+// does not depend on what runs beside it.  When every lane's local solver has compute units of its own, the
+// steps of the pairs are simply enqueued in turn.  Otherwise the pairs advance one outer iteration at a time in
+// three phases separated by events: (1) selection, kernel rows and the solver's block of every pair, (2) the
+// local solvers of all pairs, single workgroups that run side by side on different CUs, (3) update_f of every
+// pair, so that no chip-wide kernel shares CUs with a local solver (next to one, each solver iteration takes
+// two to three times longer).
 void SVC::train_pairs_in_lockstep(const DataSet &grouped, int lanes, std::vector<std::vector<float_type>> &alpha) {
     struct PairId { int i, j; };
     std::vector<PairId> pairs;

@@ -63,14 +63,15 @@ private:
     bool for_svr;
 };
 
-// One SMO solve as a resumable sequence of enqueue steps on its own stream.  CSMOSolver::solve runs one
-// task to completion; a one-vs-one run advances several tasks (class pairs) in lockstep, so that their
-// local solvers -- each a single workgroup bound by latency, and half of a multi-class run's device
-// time -- occupy different CUs at the same time, while the chip-wide steps (selection, get_rows,
-// update_f) of the pairs follow one another.  The steps of one outer iteration, in order:
-//   enqueue_select, enqueue_rows, enqueue_block, enqueue_solver, enqueue_update, finish_iteration
-// (a task whose block does not need the stored rows may run enqueue_block / enqueue_solver before
-// enqueue_rows, which hides the host's cache bookkeeping behind the solver).
+// One SMO solve as a resumable sequence of enqueue steps.  CSMOSolver::solve runs one task to completion; a
+// one-vs-one run keeps several tasks (class pairs) in flight and enqueues their steps in turn.  The local
+// solver is a single workgroup bound by latency; it runs on a stream restricted to compute units of its own
+// (one per XCD and lane), everything else of the task on a stream restricted to the remaining ones, so the
+// solver of an iteration runs next to that iteration's get_rows.  Where such streams cannot be had the task
+// uses one ordinary stream, and the driver of several tasks keeps their solver phases apart from their
+// chip-wide phases with events.  The steps of one outer iteration:
+//   enqueue_select, enqueue_block, enqueue_solver, enqueue_rows, enqueue_update, finish_iteration
+// (enqueue_rows before enqueue_block when the block is gathered from the stored rows: block_needs_rows()).
 class SolveTask {
 public:
     // pool / pool_bytes: device memory for the kernel rows (nullptr: taken from the process-wide arena
