@@ -35,6 +35,26 @@ def test_model_library_exports():
         assert hasattr(lib, n), n
 
 
+def test_scikit_interface_exports():
+    """Every function the reference's Python package binds (thundersvm-scikit.cpp) is exported under its name."""
+    lib = model.host_lib()
+    text = open(os.path.join(ROOT, "include", "thundersvm_scikit.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = sorted(set(re.findall(r"\b\*?([a-z_]+)\s*\(", text)) - {"defined"})
+    assert len(names) == 26, names
+    for n in names:
+        assert hasattr(lib, n), n
+    # no GPU needed for these
+    lib.model_new.restype = ctypes.c_void_p
+    m = lib.model_new(0)
+    assert m and lib.model_new(9) is None
+    n_model = (ctypes.c_int * 1)(7)
+    lib.get_n_binary_models(ctypes.c_void_p(m), n_model)
+    assert n_model[0] == 1
+    assert lib.n_sv(ctypes.c_void_p(m)) == 0
+    lib.model_free(ctypes.c_void_p(m))
+
+
 def test_argument_checks_do_not_need_a_gpu():
     lib = capi.kernel_lib()
     rc = lib.tsvm_update_f(None, None, 4, None, 0, None, 8, 8, 1, None)

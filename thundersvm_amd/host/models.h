@@ -30,6 +30,7 @@ public:
     const std::vector<float_type> &get_linear_coef() const { return linear_coef; }
     const std::vector<float_type> &get_rho() const { return rho; }
     int get_n_classes() const { return n_classes; }
+    int get_sv_max_index() const { return sv_max_index; }
     const std::vector<int> &get_sv_ind() const { return sv_indices; }
     const std::vector<int> &get_label() const { return label; }
     void set_max_iter(int iter) { max_iter = iter; }

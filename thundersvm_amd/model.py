@@ -24,14 +24,19 @@ class TsvmParam(C.Structure):
 
 
 def make_param(svm_type=0, kernel_type=2, degree=3, gamma=0.0, coef0=0.0, C=1.0, nu=0.5, p=0.1, epsilon=0.001,
-               max_mem_size=8192 << 20, max_iter=-1, verbose=0, cache_bytes=-1, pair_lanes=0):
-    """Defaults of include/thundersvm/svmparam.h:14-29."""
+               max_mem_size=8192 << 20, max_iter=-1, verbose=0, cache_bytes=-1, pair_lanes=0, weights=None):
+    """Defaults of include/thundersvm/svmparam.h:14-29.  weights: {class label: factor on C} (the CLI's -wi)."""
     prm = TsvmParam()
     prm.svm_type, prm.kernel_type, prm.degree, prm.max_iter = svm_type, kernel_type, degree, max_iter
     prm.gamma, prm.coef0, prm.C, prm.nu, prm.p, prm.epsilon = gamma, coef0, C, nu, p, epsilon
     prm.max_mem_size, prm.nr_weight, prm.verbose = max_mem_size, 0, verbose
     prm.cache_bytes = cache_bytes
     prm.pair_lanes = pair_lanes
+    if weights:
+        prm._keep = (np.array(list(weights.keys()), dtype=np.int32), np.array(list(weights.values()), dtype=np.float64))
+        prm.nr_weight = len(weights)
+        prm.weight_label = prm._keep[0].ctypes.data_as(_ip)
+        prm.weight = prm._keep[1].ctypes.data_as(_dp)
     return prm
 
 
