@@ -25,9 +25,9 @@
 //     tests/test_oracle_expf.py counts how often the two differ on this host.
 //
 // Pinning: tests/test_oracle_golden.py (the reference's fixture, row sets and
-// accuracy / MSE / SV-count goldens), tests/test_oracle_expf.py and
-// tests/test_oracle_smo.py (closed forms, brute force, invariants) check every
-// part on its own.  The composite solver trajectory (solve + sort_f +
+// accuracy / MSE / SV-count goldens), tests/test_oracle_expf.py,
+// tests/test_oracle_smo.py and tests/test_oracle_probability.py (closed forms,
+// brute force, invariants, independent minimisers) check every part on its own.  The composite solver trajectory (solve + sort_f +
 // select_working_set + c_smo_solve / nu_smo_solve) has no fixture in the
 // reference holding alpha or rho, and the reference CPU build cannot be built
 // here (Eigen absent): that composite is "parity unpinned" beyond the
@@ -1148,6 +1148,110 @@ void orc_predict_label(void *mp, const double *dec_values, int nrows, double *ou
         for (int l = 0; l < nrows; ++l) out[l] = dec_values[l] > 0 ? 1 : -1;
     } else {
         for (int l = 0; l < nrows; ++l) out[l] = dec_values[l];
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Probability estimates (svc.cpp:197-430).  The fold loop of SVC::probability_train
+// (svc.cpp:432-491) is driven from tests/oracle_lib.py with the model functions above.
+// ---------------------------------------------------------------------------
+
+// sigmoidPredict (svc.cpp:197-204)
+double orc_sigmoid_predict(double dec_value, double A, double B) {
+    double fApB = dec_value * A + B;
+    if (fApB >= 0) return exp(-fApB) / (1.0 + exp(-fApB));
+    return 1.0 / (1 + exp(fApB));
+}
+
+// sigmoidTrain (svc.cpp:318-430): regularised targets, Newton direction on (A, B) with H + sigma*I,
+// backtracking line search with the 1e-4 sufficient-decrease rule.
+void orc_sigmoid_train(const double *dec, int l, const int *labels, double *A_out, double *B_out) {
+    double prior1 = 0, prior0 = 0;
+    for (int i = 0; i < l; i++) { if (labels[i] > 0) prior1 += 1; else prior0 += 1; }
+    const int max_iter = 100;
+    const double min_step = 1e-10, sigma = 1e-12, eps = 1e-5;
+    const double hiTarget = (prior1 + 1.0) / (prior1 + 2.0), loTarget = 1 / (prior0 + 2.0);
+    vector<double> t(l);
+    double A = 0.0, B = log((prior0 + 1.0) / (prior1 + 1.0)), fval = 0.0;
+    for (int i = 0; i < l; i++) {
+        t[i] = labels[i] > 0 ? hiTarget : loTarget;
+        double fApB = dec[i] * A + B;
+        if (fApB >= 0) fval += t[i] * fApB + log(1 + exp(-fApB));
+        else fval += (t[i] - 1) * fApB + log(1 + exp(fApB));
+    }
+    int iter;
+    for (iter = 0; iter < max_iter; iter++) {
+        double h11 = sigma, h22 = sigma, h21 = 0.0, g1 = 0.0, g2 = 0.0;
+        for (int i = 0; i < l; i++) {
+            double fApB = dec[i] * A + B, p, q;
+            if (fApB >= 0) { p = exp(-fApB) / (1.0 + exp(-fApB)); q = 1.0 / (1.0 + exp(-fApB)); }
+            else { p = 1.0 / (1.0 + exp(fApB)); q = exp(fApB) / (1.0 + exp(fApB)); }
+            double d2 = p * q;
+            h11 += dec[i] * dec[i] * d2;
+            h22 += d2;
+            h21 += dec[i] * d2;
+            double d1 = t[i] - p;
+            g1 += dec[i] * d1;
+            g2 += d1;
+        }
+        if (fabs(g1) < eps && fabs(g2) < eps) break;
+        double det = h11 * h22 - h21 * h21;
+        double dA = -(h22 * g1 - h21 * g2) / det;
+        double dB = -(-h21 * g1 + h11 * g2) / det;
+        double gd = g1 * dA + g2 * dB;
+        double stepsize = 1;
+        while (stepsize >= min_step) {
+            double newA = A + stepsize * dA, newB = B + stepsize * dB, newf = 0.0;
+            for (int i = 0; i < l; i++) {
+                double fApB = dec[i] * newA + newB;
+                if (fApB >= 0) newf += t[i] * fApB + log(1 + exp(-fApB));
+                else newf += (t[i] - 1) * fApB + log(1 + exp(fApB));
+            }
+            if (newf < fval + 0.0001 * stepsize * gd) { A = newA; B = newB; fval = newf; break; }
+            stepsize = stepsize / 2.0;
+        }
+        if (stepsize < min_step) break;
+    }
+    *A_out = A;
+    *B_out = B;
+}
+
+// SVC::multiclass_probability (svc.cpp:206-263); r is k x k row-major, p has k entries.
+void orc_multiclass_probability(const double *r, int k, double *p) {
+    int max_iter = std::max(100, k);
+    vector<double> Q((size_t) k * k, 0.0), Qp(k);
+    double eps = 0.005 / k;
+    for (int t = 0; t < k; t++) {
+        p[t] = 1.0 / k;
+        Q[t * k + t] = 0;
+        for (int j = 0; j < t; j++) {
+            Q[t * k + t] += r[j * k + t] * r[j * k + t];
+            Q[t * k + j] = Q[j * k + t];
+        }
+        for (int j = t + 1; j < k; j++) {
+            Q[t * k + t] += r[j * k + t] * r[j * k + t];
+            Q[t * k + j] = -r[j * k + t] * r[t * k + j];
+        }
+    }
+    for (int iter = 0; iter < max_iter; iter++) {
+        double pQp = 0;
+        for (int t = 0; t < k; t++) {
+            Qp[t] = 0;
+            for (int j = 0; j < k; j++) Qp[t] += Q[t * k + j] * p[j];
+            pQp += p[t] * Qp[t];
+        }
+        double max_error = 0;
+        for (int t = 0; t < k; t++) max_error = std::max(max_error, fabs(Qp[t] - pQp));
+        if (max_error < eps) break;
+        for (int t = 0; t < k; t++) {
+            double diff = (-Qp[t] + pQp) / Q[t * k + t];
+            p[t] += diff;
+            pQp = (pQp + diff * (diff * Q[t * k + t] + 2 * Qp[t])) / (1 + diff) / (1 + diff);
+            for (int j = 0; j < k; j++) {
+                Qp[j] = (Qp[j] + diff * Q[t * k + j]) / (1 + diff);
+                p[j] /= (1 + diff);
+            }
+        }
     }
 }
 

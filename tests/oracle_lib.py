@@ -272,3 +272,86 @@ class Model:
         out = np.zeros(len(dec))
         lib().orc_predict_label(self.h, _ptr(dec, C.c_double), C.c_int(len(dec)), _ptr(out, C.c_double))
         return out, dec
+
+
+# ---------------------------------------------------------------------------------------------
+# Probability estimates (svc.cpp:197-491)
+# ---------------------------------------------------------------------------------------------
+def sigmoid_predict(dec, A, B):
+    L = lib()
+    L.orc_sigmoid_predict.restype = C.c_double
+    return L.orc_sigmoid_predict(C.c_double(dec), C.c_double(A), C.c_double(B))
+
+
+def sigmoid_train(dec, labels):
+    dec = np.ascontiguousarray(dec, dtype=np.float64)
+    labels = np.ascontiguousarray(labels, dtype=np.int32)
+    a, b = C.c_double(), C.c_double()
+    lib().orc_sigmoid_train(_ptr(dec, C.c_double), C.c_int(len(dec)), _ptr(labels, C.c_int), C.byref(a), C.byref(b))
+    return a.value, b.value
+
+
+def multiclass_probability(r):
+    r = np.ascontiguousarray(r, dtype=np.float64)
+    p = np.zeros(len(r))
+    lib().orc_multiclass_probability(_ptr(r, C.c_double), C.c_int(len(r)), _ptr(p, C.c_double))
+    return p
+
+
+def _rows(ptr, col, val, idx):
+    idx = np.asarray(idx, dtype=np.int64)
+    lens = ptr[idx + 1] - ptr[idx]
+    out_ptr = np.zeros(len(idx) + 1, dtype=np.int64)
+    np.cumsum(lens, out=out_ptr[1:])
+    take = np.repeat(ptr[idx] - out_ptr[:-1], lens) + np.arange(out_ptr[-1])
+    return out_ptr, col[take], val[take]
+
+
+def probability_train(ptr, col, val, y, param):
+    """SVC::probability_train (svc.cpp:432-491): decision values of every instance from a 5-fold cross-validation
+    (folds cut class by class in grouped order, class order = first appearance, dataset.cpp:199-214), then
+    sigmoidTrain per class pair.  Returns (probA, probB)."""
+    ptr, col, val = csr_arrays(ptr, col, val)
+    y = np.asarray(y, dtype=np.float64)
+    labels = list(dict.fromkeys(y.astype(np.int64).tolist()))
+    groups = [np.flatnonzero(y.astype(np.int64) == c) for c in labels]
+    k_cls = len(labels)
+    n_binary = k_cls * (k_cls - 1) // 2
+    dec_all = np.zeros((len(y), n_binary))
+    n_fold = 5
+    for fold in range(n_fold):
+        train_idx, test_idx = [], []
+        for ids in groups:
+            per = len(ids) // n_fold
+            b = per * fold
+            e = len(ids) if fold == n_fold - 1 else min(len(ids), b + per)
+            test_idx.extend(ids[b:e])
+            train_idx.extend(np.concatenate([ids[:b], ids[e:]]))
+        tp, tc, tv = _rows(ptr, col, val, train_idx)
+        m = Model(tp, tc, tv, y[train_idx], param)
+        sp_, sc, sv = _rows(ptr, col, val, test_idx)
+        dec_all[test_idx] = m.predict_dec_values(sp_, sc, sv, 1000)
+    prob_a, prob_b = np.zeros(n_binary), np.zeros(n_binary)
+    k = 0
+    for i in range(k_cls):
+        for j in range(i + 1, k_cls):
+            ids = np.concatenate([groups[i], groups[j]])
+            lab = np.concatenate([np.ones(len(groups[i]), dtype=np.int32), -np.ones(len(groups[j]), dtype=np.int32)])
+            prob_a[k], prob_b[k] = sigmoid_train(dec_all[ids, k], lab)
+            k += 1
+    return prob_a, prob_b
+
+
+def predict_probability(dec, prob_a, prob_b, n_classes):
+    """The probability branch of SVC::predict_label (svc.cpp:289-314): per row the coupled class probabilities."""
+    out = np.zeros((len(dec), n_classes))
+    for row in range(len(dec)):
+        r = np.zeros((n_classes, n_classes))
+        k = 0
+        for i in range(n_classes):
+            for j in range(i + 1, n_classes):
+                r[i, j] = min(max(sigmoid_predict(dec[row, k], prob_a[k], prob_b[k]), 1e-7), 1 - 1e-7)
+                r[j, i] = 1 - r[i, j]
+                k += 1
+        out[row] = multiclass_probability(r)
+    return out

@@ -8,6 +8,7 @@ import os
 import numpy as np
 import pytest
 
+import oracle_lib as O
 from thundersvm_amd import data as D
 from thundersvm_amd.model import Model, host_lib, make_param
 
@@ -165,6 +166,49 @@ def test_failures_are_reported_through_succeed():
     m, _, _, ok = _fit(lib, d, 1, 2, True, gamma=0.5, nu=0.999)    # nu infeasible for the smallest class pair
     assert ok == -1
     lib.model_free(C.c_void_p(m))
-    m, _, _, ok = _fit(lib, d, 0, 2, True, gamma=0.5, probability=1)   # probability estimates are not built
+    m, _, _, ok = _fit(lib, d, 0, 7, True, gamma=0.5)    # no such kernel: the kernel-level ABI refuses it
     assert ok == -1
     lib.model_free(C.c_void_p(m))
+
+
+@pytest.mark.parametrize("sparse", [True, False])
+def test_probability_estimates(sparse):
+    """probability = 1 (svc.cpp:137-143, 289-314, 432-491): probA / probB from the 5-fold decision values, coupled
+    class probabilities per predicted row (get_pro), labels by highest probability; against the oracle, whose
+    probability functions tests/test_oracle_probability.py pins."""
+    lib = _lib()
+    d = D.load_libsvm(FIXTURE)
+    m, _, n_classes, ok = _fit(lib, d, 0, 2, sparse, gamma=0.5, cost=100.0, probability=1)
+    assert ok == 1 and n_classes == 3
+    lab, dec = _predict(lib, m, d, sparse, 3)
+    prob = np.zeros(d.n * 3, dtype=np.float32)
+    lib.get_pro(C.c_void_p(m), _fp(prob))
+    prob = prob.reshape(d.n, 3)
+    op = O.make_param(svm_type=0, kernel_type=2, gamma=0.5, C_=100.0, epsilon=float(np.float32(0.001)), expf_mode=1)
+    pa, pb = O.probability_train(d.ptr, d.col, d.val, d.y, op)
+    om = O.Model(d.ptr, d.col, d.val, d.y, op)
+    want = O.predict_probability(om.predict_dec_values(d.ptr, d.col, d.val), pa, pb, 3)
+    assert np.abs(prob - want).max() < 1e-6
+    assert np.abs(prob.sum(axis=1) - 1).max() < 1e-6
+    assert np.array_equal(lab, om.label[np.argmax(want, axis=1)].astype(np.float32))
+    assert (lab == d.y).mean() > 0.95
+    # probA / probB travel in the model text
+    sp = lib.save_to_string_scikit(C.c_void_p(m))
+    text = C.string_at(sp)
+    lib.free_string(C.c_void_p(sp))
+    assert b"probA" in text and b"probB" in text
+    got_a = np.array(text.split(b"probA ")[1].split(b"\n")[0].split(), dtype=np.float64)
+    got_b = np.array(text.split(b"probB ")[1].split(b"\n")[0].split(), dtype=np.float64)
+    np.testing.assert_allclose(got_a, pa, rtol=1e-5)
+    np.testing.assert_allclose(got_b, pb, rtol=1e-5, atol=1e-7)
+    m2 = lib.model_new(0)
+    lib.load_from_string_scikit(C.c_void_p(m2), text)
+    kernel, deg, gam, c0, pr = C.create_string_buffer(20), (C.c_int * 1)(), (C.c_float * 1)(), (C.c_float * 1)(), (C.c_int * 1)()
+    lib.init_model_param(kernel, deg, gam, c0, pr, C.c_void_p(m2))
+    assert pr[0] == 1
+    lab2, _ = _predict(lib, m2, d, sparse, 3)
+    prob2 = np.zeros(d.n * 3, dtype=np.float32)
+    lib.get_pro(C.c_void_p(m2), _fp(prob2))
+    assert np.array_equal(lab2, lab) and np.abs(prob2.reshape(d.n, 3) - prob).max() < 1e-4   # six digits in the text
+    lib.model_free(C.c_void_p(m))
+    lib.model_free(C.c_void_p(m2))

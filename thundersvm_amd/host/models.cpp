@@ -389,7 +389,12 @@ void SVC::train(const DataSet &dataset, SvmParam p) {   // svc.cpp:41-145
                 }
             }
     }
-    if (param.probability == 1) throw std::runtime_error("probability estimates are not part of this build");
+    if (param.probability == 1) {   // svc.cpp:137-143
+        TSVM_LOG << "performing probability train";
+        probA.assign(n_binary_models, 0);
+        probB.assign(n_binary_models, 0);
+        probability_train(grouped);
+    }
 }
 
 void SVC::setup_binary(const DataSet &dataset, int i, int j, BinaryProblem &p) {   // svc.cpp:147-170
@@ -514,18 +519,215 @@ std::vector<float_type> SVC::predict(const DataSet::node2d &instances, int batch
     return predict_label(dec_values, (int) instances.size());
 }
 
-// One-vs-one vote, ties to the lowest class index (svc.cpp:265-288).
-std::vector<float_type> SVC::predict_label(const std::vector<float_type> &dec, int n_instances) const {
+// ------------------------------------------------------------------------------------------------
+// Probability estimates (svc.cpp:197-491): Platt scaling of every pair's decision values, fitted on
+// decision values from a 5-fold cross-validation, and pairwise coupling of the pair probabilities
+// (Lin, Lin, Weng, "A note on Platt's probabilistic outputs for support vector machines", 2007; Wu, Lin,
+// Weng, "Probability estimates for multi-class classification by pairwise coupling", 2004).
+// ------------------------------------------------------------------------------------------------
+namespace {
+
+// P(y = +1 | dec) = 1 / (1 + exp(A*dec + B)), in the form that avoids cancellation (svc.cpp:197-204)
+float_type sigmoid_predict(float_type dec, float_type A, float_type B) {
+    const double v = dec * A + B;
+    return v >= 0 ? exp(-v) / (1.0 + exp(-v)) : 1.0 / (1 + exp(v));
+}
+
+// negative log likelihood of the targets t under the sigmoid with parameters (A, B)
+double sigmoid_objective(const std::vector<float_type> &dec, const std::vector<double> &t, double A, double B) {
+    double f = 0.0;
+    for (size_t i = 0; i < dec.size(); ++i) {
+        const double v = dec[i] * A + B;
+        f += v >= 0 ? t[i] * v + log(1 + exp(-v)) : (t[i] - 1) * v + log(1 + exp(v));
+    }
+    return f;
+}
+
+// Newton's method with backtracking on (A, B) (svc.cpp:318-430)
+void sigmoid_train(const std::vector<float_type> &dec, const std::vector<int> &labels, float_type &A, float_type &B) {
+    const size_t l = dec.size();
+    double prior1 = 0, prior0 = 0;
+    for (size_t i = 0; i < l; ++i) (labels[i] > 0 ? prior1 : prior0) += 1;
+    const int max_iter = 100;
+    const double min_step = 1e-10, sigma = 1e-12, eps = 1e-5;
+    const double hi_target = (prior1 + 1.0) / (prior1 + 2.0), lo_target = 1 / (prior0 + 2.0);
+    std::vector<double> t(l);
+    for (size_t i = 0; i < l; ++i) t[i] = labels[i] > 0 ? hi_target : lo_target;
+    A = 0.0;
+    B = log((prior0 + 1.0) / (prior1 + 1.0));
+    double fval = sigmoid_objective(dec, t, A, B);
+    int iter = 0;
+    for (; iter < max_iter; ++iter) {
+        double h11 = sigma, h22 = sigma, h21 = 0.0, g1 = 0.0, g2 = 0.0;   // H + sigma*I keeps the Hessian positive definite
+        for (size_t i = 0; i < l; ++i) {
+            const double v = dec[i] * A + B;
+            double pp, qq;
+            if (v >= 0) { pp = exp(-v) / (1.0 + exp(-v)); qq = 1.0 / (1.0 + exp(-v)); }
+            else { pp = 1.0 / (1.0 + exp(v)); qq = exp(v) / (1.0 + exp(v)); }
+            const double d2 = pp * qq, d1 = t[i] - pp;
+            h11 += dec[i] * dec[i] * d2;
+            h22 += d2;
+            h21 += dec[i] * d2;
+            g1 += dec[i] * d1;
+            g2 += d1;
+        }
+        if (fabs(g1) < eps && fabs(g2) < eps) break;
+        const double det = h11 * h22 - h21 * h21;
+        const double dA = -(h22 * g1 - h21 * g2) / det, dB = -(-h21 * g1 + h11 * g2) / det;
+        const double gd = g1 * dA + g2 * dB;
+        double step = 1;
+        while (step >= min_step) {
+            const double newA = A + step * dA, newB = B + step * dB;
+            const double newf = sigmoid_objective(dec, t, newA, newB);
+            if (newf < fval + 0.0001 * step * gd) {   // sufficient decrease
+                A = newA;
+                B = newB;
+                fval = newf;
+                break;
+            }
+            step = step / 2.0;
+        }
+        if (step < min_step) {
+            printf("Line search fails in two-class probability estimates\n");
+            break;
+        }
+    }
+    if (iter >= max_iter) printf("Reaching maximal iterations in two-class probability estimates\n");
+}
+
+}  // namespace
+
+// Class probabilities p from the pairwise r[i][j] = P(class i | class i or j): the fixed-point iteration for
+// min sum_{i<j} (r[j][i]*p[i] - r[i][j]*p[j])^2 subject to sum p = 1 (svc.cpp:206-263).
+void SVC::multiclass_probability(const std::vector<std::vector<float_type>> &r, std::vector<float_type> &p) const {
+    const int k = n_classes;
+    const int max_it = std::max(100, k);
+    std::vector<std::vector<double>> Q(k, std::vector<double>(k, 0.0));
+    std::vector<double> Qp(k);
+    const double eps = 0.005 / k;
+    for (int t = 0; t < k; ++t) {
+        p[t] = 1.0 / k;
+        Q[t][t] = 0;
+        for (int j = 0; j < t; ++j) {
+            Q[t][t] += r[j][t] * r[j][t];
+            Q[t][j] = Q[j][t];
+        }
+        for (int j = t + 1; j < k; ++j) {
+            Q[t][t] += r[j][t] * r[j][t];
+            Q[t][j] = -r[j][t] * r[t][j];
+        }
+    }
+    int iter = 0;
+    for (; iter < max_it; ++iter) {
+        double pQp = 0;   // recomputed every sweep for accuracy
+        for (int t = 0; t < k; ++t) {
+            Qp[t] = 0;
+            for (int j = 0; j < k; ++j) Qp[t] += Q[t][j] * p[j];
+            pQp += p[t] * Qp[t];
+        }
+        double max_error = 0;
+        for (int t = 0; t < k; ++t) max_error = std::max(max_error, fabs(Qp[t] - pQp));
+        if (max_error < eps) break;
+        for (int t = 0; t < k; ++t) {
+            const double diff = (-Qp[t] + pQp) / Q[t][t];
+            p[t] += diff;
+            pQp = (pQp + diff * (diff * Q[t][t] + 2 * Qp[t])) / (1 + diff) / (1 + diff);
+            for (int j = 0; j < k; ++j) {
+                Qp[j] = (Qp[j] + diff * Q[t][j]) / (1 + diff);
+                p[j] /= (1 + diff);
+            }
+        }
+    }
+    if (iter >= max_it) printf("Exceeds max_iter in multiclass_prob\n");
+}
+
+// probA / probB of every class pair from out-of-fold decision values.  Five folds cut class by class from the
+// grouped order (the last fold takes the remainder); every fold trains a plain C-SVC model with the same
+// parameters, as the reference does also when the model being trained is a NuSVC.
+void SVC::probability_train(const DataSet &grouped) {
+    SvmParam param_no_prob = param;
+    param_no_prob.probability = 0;
+    const int n_fold = 5;
+    std::vector<float_type> dec_all(grouped.n_instances() * (size_t) n_binary_models);
+    for (int fold = 0; fold < n_fold; ++fold) {
+        DataSet::node2d x_train, x_test;
+        std::vector<float_type> y_train;
+        std::vector<int> test_idx;
+        for (size_t c = 0; c < grouped.n_classes(); ++c) {
+            const std::vector<int> ids = grouped.original_index((int) c);
+            const size_t per_fold = ids.size() / n_fold;
+            const size_t begin = per_fold * fold;
+            const size_t end = fold == n_fold - 1 ? ids.size() : std::min(ids.size(), begin + per_fold);
+            for (size_t l = 0; l < ids.size(); ++l) {
+                if (l >= begin && l < end) {
+                    x_test.push_back(grouped.instances()[ids[l]]);
+                    test_idx.push_back(ids[l]);
+                } else {
+                    x_train.push_back(grouped.instances()[ids[l]]);
+                    y_train.push_back(grouped.y()[ids[l]]);
+                }
+            }
+        }
+        SVC fold_model;
+        fold_model.set_max_iter(max_iter);
+        fold_model.cache_bytes = cache_bytes;
+        fold_model.pair_lanes = pair_lanes;
+        fold_model.train(DataSet(x_train, (int) grouped.n_features(), y_train), param_no_prob);
+        std::vector<float_type> dec;
+        fold_model.predict_dec_values(x_test, dec, 1000);
+        for (size_t t = 0; t < x_test.size(); ++t)
+            std::copy(dec.begin() + t * n_binary_models, dec.begin() + (t + 1) * n_binary_models,
+                      dec_all.begin() + (size_t) test_idx[t] * n_binary_models);
+    }
+    int k = 0;
+    for (int i = 0; i < n_classes; ++i)
+        for (int j = i + 1; j < n_classes; ++j, ++k) {
+            std::vector<int> y;
+            std::vector<float_type> dec_pair;
+            for (int side = 0; side < 2; ++side)
+                for (int id : grouped.original_index(side == 0 ? i : j)) {
+                    y.push_back(side == 0 ? +1 : -1);
+                    dec_pair.push_back(dec_all[(size_t) id * n_binary_models + k]);
+                }
+            sigmoid_train(dec_pair, y, probA[k], probB[k]);
+        }
+}
+
+// Labels from decision values (svc.cpp:265-316): one-vs-one vote, ties to the lowest class index; with
+// probability estimates, the class of highest coupled probability (prob_predict keeps all of them).
+std::vector<float_type> SVC::predict_label(const std::vector<float_type> &dec, int n_instances) {
     std::vector<float_type> out(n_instances);
-    std::vector<int> votes(n_classes);
-    for (int r = 0; r < n_instances; ++r) {
-        std::fill(votes.begin(), votes.end(), 0);
+    if (param.probability == 0) {
+        std::vector<int> votes(n_classes);
+        for (int r = 0; r < n_instances; ++r) {
+            std::fill(votes.begin(), votes.end(), 0);
+            int k = 0;
+            for (int i = 0; i < n_classes; ++i)
+                for (int j = i + 1; j < n_classes; ++j, ++k) votes[dec[(size_t) r * n_binary_models + k] > 0 ? i : j]++;
+            int best = 0;
+            for (int c = 1; c < n_classes; ++c) if (votes[c] > votes[best]) best = c;
+            out[r] = (float) label[best];
+        }
+        return out;
+    }
+    TSVM_LOG << "predict with probability";
+    prob_predict.clear();
+    const float_type min_prob = 1e-7;
+    std::vector<std::vector<float_type>> r(n_classes, std::vector<float_type>(n_classes));
+    std::vector<float_type> p(n_classes);
+    for (int row = 0; row < n_instances; ++row) {
         int k = 0;
         for (int i = 0; i < n_classes; ++i)
-            for (int j = i + 1; j < n_classes; ++j, ++k) votes[dec[(size_t) r * n_binary_models + k] > 0 ? i : j]++;
+            for (int j = i + 1; j < n_classes; ++j, ++k) {
+                r[i][j] = std::min(std::max(sigmoid_predict(dec[(size_t) row * n_binary_models + k], probA[k], probB[k]), min_prob),
+                                   1 - min_prob);
+                r[j][i] = 1 - r[i][j];
+            }
+        multiclass_probability(r, p);
+        prob_predict.insert(prob_predict.end(), p.begin(), p.end());
         int best = 0;
-        for (int c = 1; c < n_classes; ++c) if (votes[c] > votes[best]) best = c;
-        out[r] = (float) label[best];
+        for (int c = 1; c < n_classes; ++c) if (p[c] > p[best]) best = c;
+        out[row] = (float) label[best];
     }
     return out;
 }

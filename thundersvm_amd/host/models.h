@@ -103,7 +103,9 @@ protected:
     virtual void setup_binary(const DataSet &dataset, int i, int j, BinaryProblem &p);   // svc.cpp:147-170
     void finish_binary(BinaryProblem &p, std::vector<float_type> &alpha_out);            // svc.cpp:171-177
     void train_pairs_in_lockstep(const DataSet &grouped, int lanes, std::vector<std::vector<float_type>> &alpha);
-    std::vector<float_type> predict_label(const std::vector<float_type> &dec_values, int n_instances) const;
+    std::vector<float_type> predict_label(const std::vector<float_type> &dec_values, int n_instances);
+    void probability_train(const DataSet &grouped);                                            // svc.cpp:432-491
+    void multiclass_probability(const std::vector<std::vector<float_type>> &r, std::vector<float_type> &p) const;   // svc.cpp:206-263
     std::vector<float_type> c_weight;
 };
 
