@@ -13,7 +13,7 @@ const char *CMDParser::train_usage() {
            "-d degree (default 3)   -g gamma (default 1/num_features)   -r coef0 (default 0)\n"
            "-c cost (default 1)   -n nu (default 0.5)   -p epsilon of epsilon-SVR (default 0.1)\n"
            "-m memory size in MB (default 8192)   -e tolerance of termination criterion (default 0.001)\n"
-           "-b probability_estimates (not supported in this build)   -wi weight: C of class i = weight*C\n"
+           "-b probability_estimates: 0 or 1 (C-SVC, nu-SVC)   -wi weight: C of class i = weight*C\n"
            "-v n: n-fold cross validation   -u n: gpu to use (default 0)   -o n: cpu cores (-1 = all)   -q quiet\n";
 }
 
