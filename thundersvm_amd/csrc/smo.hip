@@ -15,7 +15,11 @@
 // update_f: f[j] -= sum_t alpha_diff[t] * K_t[j]  (smo_kernel.cpp:300-319)
 // Bandwidth-bound stream over the ws x n kernel rows.  The non-zero alpha_diff entries are
 // compacted (in order) into LDS once per workgroup; rows with alpha_diff == 0 are never read.
-// Each thread owns one or two adjacent columns and keeps 16 (or 8 two-column) row loads in flight.
+// Each thread owns one to four adjacent columns and keeps 8 to 32 row loads in flight.  On the vector-load
+// path the columns are dealt evenly to a number of workgroups that is a multiple of 248 (every CU, or every
+// CU left to a stream that leaves one CU per XCD to the local solver, gets the same number of workgroups):
+// with a grid of full 256-thread workgroups some CUs stream 2 and others 1, and the launch lasts as long as
+// the busiest one.
 // ------------------------------------------------------------------------------------------------
 #define UF_T 256
 #define UF_CHUNK 1024
@@ -26,15 +30,16 @@
 template <typename TK, int COLS, int UNROLL>
 __global__ __launch_bounds__(UF_T) void update_f_kernel(double *__restrict__ f, const double *__restrict__ alpha_diff,
                                                         int ws, const TK *__restrict__ k_rows,
-                                                        const int *__restrict__ slots, int64_t ld, int64_t n, int repeat) {
+                                                        const int *__restrict__ slots, int64_t ld, int64_t n, int repeat,
+                                                        int vec_per_wg) {
     typedef TK vec_t __attribute__((ext_vector_type(COLS)));
     __shared__ double s_ad[UF_CHUNK];
     __shared__ int64_t s_off[UF_CHUNK];
     __shared__ int s_wave_cnt[UF_T / 64];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    const int64_t j = ((int64_t) blockIdx.x * UF_T + tid) * COLS;
-    const bool act = j < n;   // a vector may reach past n, but never past the padded row (checked by the launcher)
+    const int64_t j = ((int64_t) blockIdx.x * vec_per_wg + tid) * COLS;
+    const bool act = tid < vec_per_wg && j < n;   // a vector may reach past n, but never past the padded row (checked by the launcher)
     double sum[COLS];
 #pragma unroll
     for (int c = 0; c < COLS; ++c) sum[c] = 0.0;
@@ -589,9 +594,18 @@ __global__ __launch_bounds__(MAX_WS) void sel_final_kernel(SelWorkspace w, SelGe
 template <typename TK, int COLS, int UNROLL>
 static void launch_update_f(double *f, const double *alpha_diff, int ws_size, const void *k_rows, const int *slots,
                             int64_t ld, int64_t n, int repeat, hipStream_t s) {
-    const unsigned grid = (unsigned) (((n + COLS - 1) / COLS + UF_T - 1) / UF_T);
-    hipLaunchKernelGGL((update_f_kernel<TK, COLS, UNROLL>), dim3(grid), dim3(UF_T), 0, s, f, alpha_diff, ws_size,
-                       (const TK *) k_rows, slots, ld, n, repeat);
+    const int64_t vecs = (n + COLS - 1) / COLS;                        // column vectors, one per thread
+    int64_t grid = (vecs + UF_T - 1) / UF_T;
+    int vec_per_wg = UF_T;
+    if (COLS > 1) {
+        // (with one column per thread a workgroup's share has to start on a cache line, or every wavefront's
+        // 256-byte read touches three lines instead of two: measured slower than the uneven grid)
+        const int64_t per_cu = (vecs + 248 * UF_T - 1) / (248 * UF_T);   // workgroups per CU
+        grid = 248 * per_cu;
+        vec_per_wg = (int) ((vecs + grid - 1) / grid);
+    }
+    hipLaunchKernelGGL((update_f_kernel<TK, COLS, UNROLL>), dim3((unsigned) grid), dim3(UF_T), 0, s, f, alpha_diff, ws_size,
+                       (const TK *) k_rows, slots, ld, n, repeat, vec_per_wg);
 }
 
 extern "C" {
