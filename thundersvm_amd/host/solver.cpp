@@ -1,6 +1,8 @@
 #include "solver.h"
 
 #include <chrono>
+#include <map>
+#include <mutex>
 #include <climits>
 #include <cmath>
 #include <algorithm>
@@ -80,6 +82,16 @@ struct PhaseTimer {
     }
 };
 
+// CU-masked streams are kept for the life of the process and handed from one solve to the next: creating one
+// makes a hardware queue, which costs far more than a solve's other set-up (and every few creations the runtime
+// spends tens of milliseconds on queue housekeeping).  Keyed by device, lane and lane count (which fix the masks).
+struct MaskedStreams {
+    hipStream_t chip = nullptr, solver = nullptr;
+    bool in_use = false;
+};
+std::mutex g_masked_mutex;
+std::map<long long, std::vector<MaskedStreams>> g_masked;
+
 }  // namespace
 
 struct SolveTask::Impl {
@@ -123,6 +135,7 @@ struct SolveTask::Impl {
     // Once the cache holds every row there is no get_rows left to run next to the solver; the iteration then
     // stays on `sa` from start to end and saves the two hand-overs between the streams.
     bool on_one_stream = false, alone = true;   // alone: no other task's kernels on the chip
+    long long masked_key = 0;
 
     void *k_rows = nullptr;
     bool caching = false;
@@ -239,9 +252,10 @@ struct SolveTask::Impl {
 
     ~Impl() {
         if (sa) (void) hipStreamSynchronize(sa);   // a selection enqueued ahead may still be running
-        if (ss && ss != sa) { (void) hipStreamSynchronize(ss); (void) hipStreamDestroy(ss); }
+        if (ss && ss != sa) (void) hipStreamSynchronize(ss);
         if (ids && ids != sa) { (void) hipStreamSynchronize(ids); (void) hipStreamDestroy(ids); }
-        if (sa) (void) hipStreamDestroy(sa);
+        if (split) release_split_streams();         // masked streams go back to the pool
+        else if (sa) (void) hipStreamDestroy(sa);
         if (block_done) (void) hipEventDestroy(block_done);
         if (solved) (void) hipEventDestroy(solved);
         if (selected) (void) hipEventDestroy(selected);
@@ -258,6 +272,19 @@ struct SolveTask::Impl {
     // Lane l's solver gets CU l of every XCD; the chip-wide kernels of all lanes get the CUs no lane's solver has.
     bool create_split_streams(int lane, int n_lanes) {
         if (!SolveTask::cu_split_available() || n_lanes < 1 || n_lanes > 4 || lane < 0 || lane >= n_lanes) return false;
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess) return false;
+        masked_key = ((long long) dev * 8 + n_lanes) * 8 + lane;
+        {
+            std::lock_guard<std::mutex> lock(g_masked_mutex);
+            for (MaskedStreams &m : g_masked[masked_key])
+                if (!m.in_use) {
+                    m.in_use = true;
+                    sa = m.chip;
+                    ss = m.solver;
+                    return true;
+                }
+        }
         uint32_t small[8] = {0xffu << (8 * lane), 0, 0, 0, 0, 0, 0, 0};
         uint32_t big[8] = {0, ~0u, ~0u, ~0u, ~0u, ~0u, ~0u, ~0u};
         big[0] = n_lanes == 4 ? 0u : ~0u << (8 * n_lanes);
@@ -268,7 +295,19 @@ struct SolveTask::Impl {
             ss = sa = nullptr;
             return false;
         }
+        std::lock_guard<std::mutex> lock(g_masked_mutex);
+        MaskedStreams m;
+        m.chip = sa;
+        m.solver = ss;
+        m.in_use = true;
+        g_masked[masked_key].push_back(m);
         return true;
+    }
+
+    void release_split_streams() {
+        std::lock_guard<std::mutex> lock(g_masked_mutex);
+        for (MaskedStreams &m : g_masked[masked_key])
+            if (m.chip == sa) m.in_use = false;
     }
 
     // without a cache the slot tables just alternate: the two halves of the working set swap places
