@@ -92,6 +92,18 @@ struct MaskedStreams {
 std::mutex g_masked_mutex;
 std::map<long long, std::vector<MaskedStreams>> g_masked;
 
+// The pooled streams are destroyed by an atexit handler, registered when the first one is made and therefore run
+// before the HIP runtime's own tear-down (which, under a profiler, crashed on queues still alive at that point).
+void destroy_masked_streams() {
+    std::lock_guard<std::mutex> lock(g_masked_mutex);
+    for (auto &kv : g_masked)
+        for (MaskedStreams &m : kv.second) {
+            if (m.solver) (void) hipStreamDestroy(m.solver);
+            if (m.chip) (void) hipStreamDestroy(m.chip);
+        }
+    g_masked.clear();
+}
+
 }  // namespace
 
 struct SolveTask::Impl {
@@ -296,6 +308,11 @@ struct SolveTask::Impl {
             return false;
         }
         std::lock_guard<std::mutex> lock(g_masked_mutex);
+        static bool registered = false;
+        if (!registered) {
+            registered = true;
+            atexit(destroy_masked_streams);
+        }
         MaskedStreams m;
         m.chip = sa;
         m.solver = ss;
