@@ -191,7 +191,7 @@ int tsvm_model_get(void *model, int *label, int *n_sv, double *rho, double *coef
         if (sv_indices && !m.get_sv_ind().empty()) memcpy(sv_indices, m.get_sv_ind().data(), sizeof(int) * m.get_sv_ind().size());
         int64_t e = 0;
         if (sv_ptr) sv_ptr[0] = 0;
-        for (size_t r = 0; r < m.svs().size(); ++r) {
+        for (size_t r = 0; (sv_ptr || sv_col || sv_val) && r < m.svs().size(); ++r) {
             for (const auto &nd : m.svs()[r]) {
                 if (sv_col) sv_col[e] = nd.index;
                 if (sv_val) sv_val[e] = nd.value;

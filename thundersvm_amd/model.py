@@ -161,12 +161,32 @@ class Model:
         self.rho = np.zeros(self.n_binary)
         self.coef = np.zeros((self.n_classes - 1) * self.total_sv if cls else self.total_sv)
         self.sv_indices = np.zeros(self.total_sv, dtype=np.int32)
-        self.sv_ptr = np.zeros(self.total_sv + 1, dtype=np.int64)
-        self.sv_col = np.zeros(nnz.value, dtype=np.int32)
-        self.sv_val = np.zeros(nnz.value)
         _check(L.tsvm_model_get(self.h, _p(self.label, _ip), _p(self.n_sv, _ip), _p(self.rho, _dp), _p(self.coef, _dp),
-                                _p(self.sv_indices, _ip), _p(self.sv_ptr, _i64p), _p(self.sv_col, _ip),
-                                _p(self.sv_val, _dp)))
+                                _p(self.sv_indices, _ip), None, None, None))
+        self._sv_nnz = nnz.value
+        self._sv = None   # the support vectors' CSR copy is made when first asked for (sv_ptr / sv_col / sv_val)
+
+    def _support_vectors(self):
+        if self._sv is None:
+            sv_ptr = np.zeros(self.total_sv + 1, dtype=np.int64)
+            sv_col = np.zeros(self._sv_nnz, dtype=np.int32)
+            sv_val = np.zeros(self._sv_nnz)
+            _check(host_lib().tsvm_model_get(self.h, None, None, None, None, None, _p(sv_ptr, _i64p), _p(sv_col, _ip),
+                                             _p(sv_val, _dp)))
+            self._sv = (sv_ptr, sv_col, sv_val)
+        return self._sv
+
+    @property
+    def sv_ptr(self):
+        return self._support_vectors()[0]
+
+    @property
+    def sv_col(self):
+        return self._support_vectors()[1]
+
+    @property
+    def sv_val(self):
+        return self._support_vectors()[2]
 
     def stats(self, k=0):
         ni, li, obj = C.c_int64(), C.c_int64(), C.c_double()
