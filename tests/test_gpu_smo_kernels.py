@@ -187,3 +187,28 @@ def test_longer_selection_starts_with_the_shorter_one(tie_mode, nu):
     assert np.array_equal(outs[1], O.select_working_set(f, y, alpha, C, C, marked, 768, nu=bool(nu)))
     tail = outs[1][512:]
     assert (tail >= 0).all() and len(set(tail.tolist()) | set(outs[0].tolist()) | set(marked.tolist())) == 768 + n_marked
+
+
+def test_empty_inputs_are_no_ops():
+    """Zero rows, zero columns, an empty working set, nothing to select: every entry point returns success and
+    leaves its outputs untouched."""
+    x = torch.zeros((4, 8), dtype=torch.float64, device="cuda")
+    sd = torch.zeros(4, dtype=torch.float64, device="cuda")
+    out = torch.full((4, 8), 7.0, dtype=torch.float64, device="cuda")
+    for n, m in ((0, 4), (4, 0)):
+        capi.call("tsvm_get_rows_dense", G.ptr(x), 8, None, n, 3, G.ptr(sd), G.ptr(x), 8, None, m, G.ptr(sd), 2, 0.5, 0.0, 3,
+                  G.ptr(out), capi.ROW_F64, None, 8, G.stream())
+    f = torch.full((5,), 3.0, dtype=torch.float64, device="cuda")
+    ad = torch.ones(4, dtype=torch.float64, device="cuda")
+    capi.call("tsvm_update_f", G.ptr(f), G.ptr(ad), 0, G.ptr(out), capi.ROW_F64, None, 8, 5, 1, G.stream())
+    capi.call("tsvm_update_f", G.ptr(f), G.ptr(ad), 4, G.ptr(out), capi.ROW_F64, None, 8, 0, 1, G.stream())
+    ids = torch.full((4,), -7, dtype=torch.int32, device="cuda")
+    y = torch.ones(5, dtype=torch.int32, device="cuda")
+    wsp = torch.empty(capi.kernel_lib().tsvm_select_workspace(5), dtype=torch.uint8, device="cuda")
+    capi.call("tsvm_select_working_set", G.ptr(f), G.ptr(y), G.ptr(f), 5, 1.0, 1.0, None, 0, G.ptr(ids), 0, 0, G.ptr(wsp),
+              G.stream())
+    assert (G.host(out) == 7.0).all() and (G.host(f) == 3.0).all() and (G.host(ids) == -7).all()
+    # an all-zero alpha_diff reads no row at all and leaves f as it is
+    capi.call("tsvm_update_f", G.ptr(f), G.ptr(torch.zeros(4, dtype=torch.float64, device="cuda")), 4, G.ptr(out), capi.ROW_F64,
+              None, 8, 5, 1, G.stream())
+    assert (G.host(f) == 3.0).all()
