@@ -94,6 +94,39 @@ def test_random_dense(name, kt, prm, n, d, m, density):
         assert got32.dtype == torch.float32 and np.array_equal(G.host(got32).astype(np.float64), G.host(got))
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_ragged_shapes_sweep(seed):
+    """Seeded sweep over ragged shapes: feature counts around the 8/16-column K tiles, row and column counts around
+    the 64/128-row tiles, with column subsets (x_idx), working-row subsets (a_idx) and scattered output slots at
+    the same time; RBF, both row element types, bit for bit against the oracle."""
+    rng = np.random.default_rng(1000 + seed)
+    n = int(rng.choice([1, 2, 63, 64, 65, 127, 129, 255, 300, 641]))
+    d = int(rng.choice([1, 3, 7, 8, 9, 15, 16, 17, 31, 33, 47, 48, 100, 129, 130, 257]))
+    m = int(rng.choice([1, 31, 33, 64, 65, 127, 128, 130]))
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    x[rng.random((n, d)) > 0.6] = 0
+    x[:, -1] = rng.standard_normal(n).astype(np.float32)     # the last feature is used: n_features == d
+    data = from_dense(x)
+    kt, prm = O.RBF, dict(gamma=0.25)
+    okm = O.KernelMatrix(data.ptr, data.col, data.val, O.make_param(kernel_type=kt, expf_mode=1, **prm))
+    x_d, nf, ld, sd, _ = _device_km(data, kt, prm)
+    cols = rng.permutation(n)[:max(1, n - int(rng.integers(0, 3)))].astype(np.int32)     # x_idx: a subset, permuted
+    rows = rng.integers(0, n, size=m).astype(np.int32)
+    slots = rng.permutation(m + 3)[:m].astype(np.int32)
+    want = okm.get_rows(rows)[:, cols]
+    cols_d, rows_d, slots_d = G.dev(cols), G.dev(rows), G.dev(slots)
+    for row_type, dt in ((capi.ROW_F64, torch.float64), (capi.ROW_F32, torch.float32)):
+        out = torch.full((m + 3, len(cols) + 5), -3.0, dtype=dt, device="cuda")
+        capi.call("tsvm_get_rows_dense", G.ptr(x_d), ld, G.ptr(cols_d), len(cols), nf, G.ptr(sd), G.ptr(x_d), ld,
+                  G.ptr(rows_d), m, G.ptr(sd), kt, prm["gamma"], 0.0, 3, G.ptr(out), row_type, G.ptr(slots_d),
+                  len(cols) + 5, G.stream())
+        got = G.host(out).astype(np.float64)
+        assert np.array_equal(got[slots][:, :len(cols)], want), (n, d, m)
+        assert (got[:, len(cols):] == -3.0).all()                 # nothing is written beyond the n columns
+        untouched = np.setdiff1d(np.arange(m + 3), slots)
+        assert (got[untouched] == -3.0).all()                     # nor into slots that were not named
+
+
 def test_float_rows_rejected_for_linear_kernel():
     x_d = torch.zeros((8, 8), dtype=torch.float64, device="cuda")
     out = torch.zeros((8, 8), dtype=torch.float32, device="cuda")
