@@ -209,6 +209,6 @@ def test_empty_inputs_are_no_ops():
               G.stream())
     assert (G.host(out) == 7.0).all() and (G.host(f) == 3.0).all() and (G.host(ids) == -7).all()
     # an all-zero alpha_diff reads no row at all and leaves f as it is
-    capi.call("tsvm_update_f", G.ptr(f), G.ptr(torch.zeros(4, dtype=torch.float64, device="cuda")), 4, G.ptr(out), capi.ROW_F64,
-              None, 8, 5, 1, G.stream())
+    zeros = torch.zeros(4, dtype=torch.float64, device="cuda")
+    capi.call("tsvm_update_f", G.ptr(f), G.ptr(zeros), 4, G.ptr(out), capi.ROW_F64, None, 8, 5, 1, G.stream())
     assert (G.host(f) == 3.0).all()
