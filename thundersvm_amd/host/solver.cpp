@@ -147,6 +147,11 @@ struct SolveTask::Impl {
     // Once the cache holds every row there is no get_rows left to run next to the solver; the iteration then
     // stays on `sa` from start to end and saves the two hand-overs between the streams.
     bool on_one_stream = false, alone = true;   // alone: no other task's kernels on the chip
+    // When the previous iteration computed many rows this one probably will too, and its get_rows will outlast the
+    // solver by far.  The block is then computed on the solver's few CUs (several times slower, still well inside
+    // the time get_rows takes), so that get_rows need not wait for it on the chip-wide stream.
+    int last_rows_computed = 0;
+    bool block_on_solver_cus = false;
     long long masked_key = 0;
 
     void *k_rows = nullptr;
@@ -401,6 +406,7 @@ struct SolveTask::Impl {
             std::copy(miss_ids.begin(), miss_ids.end(), h_miss_ids);
             std::copy(miss_slots.begin(), miss_slots.end(), h_miss_slots);
             const int n_miss = (int) miss_ids.size();
+            last_rows_computed = n_miss;
             TSVM_HIP_CHECK(hipMemcpyAsync(d_slots_a.data(), h_slots, sizeof(int) * ws_size, hipMemcpyHostToDevice, sa));
             if (n_miss) {
                 TSVM_HIP_CHECK(hipMemcpyAsync(d_miss_ids.data(), h_miss_ids, sizeof(int) * n_miss, hipMemcpyHostToDevice, sa));
@@ -426,6 +432,7 @@ struct SolveTask::Impl {
             const bool on_a = ((iter - rotation_base) % 2) == 0;
             slots = on_a ? d_slots_a.data() : d_slots_b.data();
             // new rows go to the slots the dropped rows occupied
+            last_rows_computed = n_new;
             k_mat.get_rows(ws_u + first_new, n_new, k_rows, ld, slots + first_new, sa);
         }
         timer.end(stats.ms_get_rows);
@@ -433,19 +440,24 @@ struct SolveTask::Impl {
 
     void enqueue_block() {
         timer.begin();
-        if (block_first)
-            k_mat.get_block(ws_u, ws_size, d_kws.data(), ldk, sa);
-        else
-            abi_check(tsvm_smo_gather_block(k_rows, row_type, slots, ld, ws_u, ws_size, d_kws.data(), sa));
-        timer.end(stats.ms_local);
         on_one_stream = !split || (alone && caching && cache.used == n_u);
-        if (!on_one_stream) TSVM_HIP_CHECK(hipEventRecord(block_done, sa));
+        block_on_solver_cus = !on_one_stream && alone && block_first && last_rows_computed >= ws_size / 4;
+        if (block_on_solver_cus) {
+            TSVM_HIP_CHECK(hipStreamWaitEvent(ss, selected, 0));
+            k_mat.get_block(ws_u, ws_size, d_kws.data(), ldk, ss);
+        } else if (block_first) {
+            k_mat.get_block(ws_u, ws_size, d_kws.data(), ldk, sa);
+        } else {
+            abi_check(tsvm_smo_gather_block(k_rows, row_type, slots, ld, ws_u, ws_size, d_kws.data(), sa));
+        }
+        timer.end(stats.ms_local);
+        if (!on_one_stream && !block_on_solver_cus) TSVM_HIP_CHECK(hipEventRecord(block_done, sa));
     }
 
     void enqueue_solver() {
         timer.begin();
         hipStream_t st = on_one_stream ? sa : ss;
-        if (!on_one_stream) TSVM_HIP_CHECK(hipStreamWaitEvent(ss, block_done, 0));
+        if (!on_one_stream && !block_on_solver_cus) TSVM_HIP_CHECK(hipStreamWaitEvent(ss, block_done, 0));
         if (nu) {
             abi_check(tsvm_nu_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), d_ws.data(), ws_size,
                                               Cp, d_kws.data(), k_mat.diag(), eps, d_diff.data(), max_iter, st));
