@@ -441,7 +441,8 @@ struct SolveTask::Impl {
     void enqueue_block() {
         timer.begin();
         on_one_stream = !split || (alone && caching && cache.used == n_u);
-        block_on_solver_cus = !on_one_stream && alone && block_first && last_rows_computed >= ws_size / 4;
+        // (dense rows only: the CSR block takes too long on eight CUs)
+        block_on_solver_cus = !on_one_stream && alone && block_first && k_mat.dense_layout() && last_rows_computed >= ws_size / 4;
         if (block_on_solver_cus) {
             TSVM_HIP_CHECK(hipStreamWaitEvent(ss, selected, 0));
             k_mat.get_block(ws_u, ws_size, d_kws.data(), ldk, ss);
