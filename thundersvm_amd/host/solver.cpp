@@ -441,8 +441,15 @@ struct SolveTask::Impl {
     void enqueue_block() {
         timer.begin();
         on_one_stream = !split || (alone && caching && cache.used == n_u);
-        // (dense rows only: the CSR block takes too long on eight CUs)
-        block_on_solver_cus = !on_one_stream && alone && block_first && k_mat.dense_layout() && last_rows_computed >= ws_size / 4;
+        // (Dense rows only: the CSR block takes too long on eight CUs.  Both launches are matrix-core work with the
+        // same cost per value; the block plus the solver's ~0.4 ms has to fit into the time of the rows.)
+        block_on_solver_cus = false;
+        if (!on_one_stream && alone && block_first && k_mat.dense_layout()) {
+            const double per_value = 2.0 * ((k_mat.n_features() + 15) / 16 * 16) / 6.6e13;   // seconds on the whole chip
+            const double t_block = per_value * 32.0 * ws_size * (double) ws_size;           // on 8 of 256 CUs
+            const double t_rows = per_value * (double) last_rows_computed * n_u;
+            block_on_solver_cus = t_block + 0.4e-3 <= t_rows;
+        }
         if (block_on_solver_cus) {
             TSVM_HIP_CHECK(hipStreamWaitEvent(ss, selected, 0));
             k_mat.get_block(ws_u, ws_size, d_kws.data(), ldk, ss);
