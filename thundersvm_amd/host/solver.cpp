@@ -127,7 +127,9 @@ struct SolveTask::Impl {
     SolverStats stats;
     std::chrono::steady_clock::time_point wall0;
 
-    DeviceBuffer<int> d_y, d_ws, d_slots_a, d_slots_b, d_miss_ids, d_miss_slots, d_ws_folded;
+    // d_slots_a holds three tables of ws entries back to back: the slot of every working-set row, then the ids and
+    // the slots of the rows to compute; the host fills the same layout in h_slots and sends it with one copy.
+    DeviceBuffer<int> d_y, d_ws, d_slots_a, d_slots_b, d_ws_folded;
     DeviceBuffer<float_type> d_alpha, d_f, d_alpha_diff, d_diff;
     DeviceBuffer<unsigned char> d_sel_ws;
     DeviceBuffer<kernel_type> d_kws;
@@ -180,8 +182,7 @@ struct SolveTask::Impl {
           row_type(k_mat.row_type()), row_esz(k_mat.row_elem_size()), q(ws_size / 2), ld(((int64_t) n_u + 7) / 8 * 8),
           nu(solver.is_nu()), ldk(tsvm_smo_solve_block_ld(ws_size)), timer(solver.profile) {
         wall0 = std::chrono::steady_clock::now();
-        d_y.resize(n); d_ws.resize(ws_size); d_slots_a.resize(ws_size); d_slots_b.resize(ws_size);
-        d_miss_ids.resize(ws_size); d_miss_slots.resize(ws_size);
+        d_y.resize(n); d_ws.resize(ws_size); d_slots_a.resize(3 * (size_t) ws_size); d_slots_b.resize(ws_size);
         if (rep > 1) d_ws_folded.resize(ws_size);
         ws_u = rep > 1 ? d_ws_folded.data() : d_ws.data();
         d_alpha.resize(n); d_f.resize(n); d_alpha_diff.resize(ws_size); d_diff.resize(2);
@@ -407,11 +408,10 @@ struct SolveTask::Impl {
             std::copy(miss_slots.begin(), miss_slots.end(), h_miss_slots);
             const int n_miss = (int) miss_ids.size();
             last_rows_computed = n_miss;
-            TSVM_HIP_CHECK(hipMemcpyAsync(d_slots_a.data(), h_slots, sizeof(int) * ws_size, hipMemcpyHostToDevice, sa));
+            TSVM_HIP_CHECK(hipMemcpyAsync(d_slots_a.data(), h_slots, sizeof(int) * (n_miss ? 3 * (size_t) ws_size : (size_t) ws_size),
+                                          hipMemcpyHostToDevice, sa));
             if (n_miss) {
-                TSVM_HIP_CHECK(hipMemcpyAsync(d_miss_ids.data(), h_miss_ids, sizeof(int) * n_miss, hipMemcpyHostToDevice, sa));
-                TSVM_HIP_CHECK(hipMemcpyAsync(d_miss_slots.data(), h_miss_slots, sizeof(int) * n_miss, hipMemcpyHostToDevice, sa));
-                k_mat.get_rows(d_miss_ids.data(), n_miss, k_rows, ld, d_miss_slots.data(), sa);
+                k_mat.get_rows(d_slots_a.data() + ws_size, n_miss, k_rows, ld, d_slots_a.data() + 2 * ws_size, sa);
             }
             slots = d_slots_a.data();
             // A cache that has started evicting and still does not hit only costs the id read-back:
