@@ -135,8 +135,8 @@ struct SolveTask::Impl {
     DeviceBuffer<kernel_type> d_kws;
     const int *ws_u = nullptr;   // working set as folded ids
 
-    // Everything of a task is enqueued on stream `sa`; `ids` only carries the read-back of the newly
-    // selected ids for the host-side cache bookkeeping, so that it does not wait behind the solver.
+    // The chip-wide work of a task is enqueued on stream `sa` (`ids` is the stream the newly selected ids are read
+    // back on for the host-side cache bookkeeping: the same one).
     hipStream_t sa = nullptr, ids = nullptr;
     hipEvent_t selected = nullptr, ids_ready = nullptr, diff_ready = nullptr;
     // A task that runs alone splits the chip: the local solver (one workgroup, a chain of dependent steps) gets a
@@ -200,11 +200,9 @@ struct SolveTask::Impl {
             TSVM_HIP_CHECK(hipStreamCreateWithFlags(&sa, hipStreamNonBlocking));
             ss = sa;
         }
-        // A task that runs alone enqueues its solver before the host looks at the new ids, so their
-        // read-back gets a stream of its own; tasks in lockstep read them back on their one stream (the
-        // device has few hardware queues, and streams that share one wait for each other).
-        if (pool) ids = sa;
-        else TSVM_HIP_CHECK(hipStreamCreateWithFlags(&ids, hipStreamNonBlocking));
+        // The read-back of the newly selected ids follows the selection on the same stream: it is enqueued before
+        // anything else of the iteration, so it waits for nothing but the selection.
+        ids = sa;
         TSVM_HIP_CHECK(hipEventCreateWithFlags(&selected, hipEventDisableTiming));
         TSVM_HIP_CHECK(hipEventCreateWithFlags(&ids_ready, hipEventDisableTiming));
         TSVM_HIP_CHECK(hipEventCreateWithFlags(&diff_ready, hipEventDisableTiming));
