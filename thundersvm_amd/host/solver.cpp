@@ -133,7 +133,14 @@ struct SolveTask::Impl {
     DeviceBuffer<float_type> d_alpha, d_f, d_alpha_diff, d_diff;
     DeviceBuffer<unsigned char> d_sel_ws;
     DeviceBuffer<kernel_type> d_kws;
-    const int *ws_u = nullptr;   // working set as folded ids
+    // The working set of iteration t is the window d_ws[ws_off .. ws_off + ws_size): the ids kept from the previous
+    // set (its second half) are the first half of the next window, so the window just moves on by q per iteration
+    // and nothing is copied (csmosolver.cpp:65-71 copies q ids per iteration); at the end of the buffer the last
+    // half is moved back to the start.
+    static constexpr int WS_HALVES = 64;
+    int ws_off = 0, sel_off = 0;   // window of the current iteration / of the latest selection launched
+    const int *ws_ids() const { return d_ws.data() + ws_off; }
+    const int *ws_u() const { return rep > 1 ? d_ws_folded.data() : d_ws.data() + ws_off; }   // working set as folded ids
 
     // The chip-wide work of a task is enqueued on stream `sa` (`ids` is the stream the newly selected ids are read
     // back on for the host-side cache bookkeeping: the same one).
@@ -182,9 +189,8 @@ struct SolveTask::Impl {
           row_type(k_mat.row_type()), row_esz(k_mat.row_elem_size()), q(ws_size / 2), ld(((int64_t) n_u + 7) / 8 * 8),
           nu(solver.is_nu()), ldk(tsvm_smo_solve_block_ld(ws_size)), timer(solver.profile) {
         wall0 = std::chrono::steady_clock::now();
-        d_y.resize(n); d_ws.resize(ws_size); d_slots_a.resize(3 * (size_t) ws_size); d_slots_b.resize(ws_size);
+        d_y.resize(n); d_ws.resize((size_t) WS_HALVES * q + ws_size); d_slots_a.resize(3 * (size_t) ws_size); d_slots_b.resize(ws_size);
         if (rep > 1) d_ws_folded.resize(ws_size);
-        ws_u = rep > 1 ? d_ws_folded.data() : d_ws.data();
         d_alpha.resize(n); d_f.resize(n); d_alpha_diff.resize(ws_size); d_diff.resize(2);
         d_sel_ws.resize(tsvm_select_workspace(n));
         d_kws.resize((size_t) ws_size * ldk);
@@ -345,14 +351,20 @@ struct SolveTask::Impl {
     // half of the previous set and pick q new ids (csmosolver.cpp:63-77).
     void launch_select(int it) {
         if (it == 0) {
+            sel_off = 0;
             abi_check(tsvm_select_working_set(d_f.data(), d_y.data(), d_alpha.data(), n, Cp, Cn, nullptr, 0, d_ws.data(),
                                               ws_size, nu, d_sel_ws.data(), sa));
         } else {
-            TSVM_HIP_CHECK(hipMemcpyAsync(d_ws.data(), d_ws.data() + q, sizeof(int) * q, hipMemcpyDeviceToDevice, sa));
-            abi_check(tsvm_select_working_set(d_f.data(), d_y.data(), d_alpha.data(), n, Cp, Cn, d_ws.data(), q,
-                                              d_ws.data() + q, q, nu, d_sel_ws.data(), sa));
+            int next = sel_off + q;
+            if (next + ws_size > (int) d_ws.size()) {
+                TSVM_HIP_CHECK(hipMemcpyAsync(d_ws.data(), d_ws.data() + next, sizeof(int) * q, hipMemcpyDeviceToDevice, sa));
+                next = 0;
+            }
+            sel_off = next;
+            abi_check(tsvm_select_working_set(d_f.data(), d_y.data(), d_alpha.data(), n, Cp, Cn, d_ws.data() + sel_off, q,
+                                              d_ws.data() + sel_off + q, q, nu, d_sel_ws.data(), sa));
         }
-        if (rep > 1) abi_check(tsvm_fold_ids(d_ws.data(), ws_size, n_u, d_ws_folded.data(), sa));
+        if (rep > 1) abi_check(tsvm_fold_ids(d_ws.data() + sel_off, ws_size, n_u, d_ws_folded.data(), sa));
     }
 
     void enqueue_select() {
@@ -361,12 +373,13 @@ struct SolveTask::Impl {
         timer.begin();
         if (!select_enqueued) launch_select(iter);
         select_enqueued = false;
+        ws_off = sel_off;
         timer.end(stats.ms_select);
         TSVM_HIP_CHECK(hipEventRecord(selected, sa));
         if (caching) {
             // the new ids travel to the host, on their own stream if there is one
             if (ids != sa) TSVM_HIP_CHECK(hipStreamWaitEvent(ids, selected, 0));
-            TSVM_HIP_CHECK(hipMemcpyAsync(h_ids, d_ws.data() + first_new, sizeof(int) * n_new, hipMemcpyDeviceToHost, ids));
+            TSVM_HIP_CHECK(hipMemcpyAsync(h_ids, ws_ids() + first_new, sizeof(int) * n_new, hipMemcpyDeviceToHost, ids));
             TSVM_HIP_CHECK(hipEventRecord(ids_ready, ids));
         }
     }
@@ -431,7 +444,7 @@ struct SolveTask::Impl {
             slots = on_a ? d_slots_a.data() : d_slots_b.data();
             // new rows go to the slots the dropped rows occupied
             last_rows_computed = n_new;
-            k_mat.get_rows(ws_u + first_new, n_new, k_rows, ld, slots + first_new, sa);
+            k_mat.get_rows(ws_u() + first_new, n_new, k_rows, ld, slots + first_new, sa);
         }
         timer.end(stats.ms_get_rows);
     }
@@ -450,11 +463,11 @@ struct SolveTask::Impl {
         }
         if (block_on_solver_cus) {
             TSVM_HIP_CHECK(hipStreamWaitEvent(ss, selected, 0));
-            k_mat.get_block(ws_u, ws_size, d_kws.data(), ldk, ss);
+            k_mat.get_block(ws_u(), ws_size, d_kws.data(), ldk, ss);
         } else if (block_first) {
-            k_mat.get_block(ws_u, ws_size, d_kws.data(), ldk, sa);
+            k_mat.get_block(ws_u(), ws_size, d_kws.data(), ldk, sa);
         } else {
-            abi_check(tsvm_smo_gather_block(k_rows, row_type, slots, ld, ws_u, ws_size, d_kws.data(), sa));
+            abi_check(tsvm_smo_gather_block(k_rows, row_type, slots, ld, ws_u(), ws_size, d_kws.data(), sa));
         }
         timer.end(stats.ms_local);
         if (!on_one_stream && !block_on_solver_cus) TSVM_HIP_CHECK(hipEventRecord(block_done, sa));
@@ -465,10 +478,10 @@ struct SolveTask::Impl {
         hipStream_t st = on_one_stream ? sa : ss;
         if (!on_one_stream && !block_on_solver_cus) TSVM_HIP_CHECK(hipStreamWaitEvent(ss, block_done, 0));
         if (nu) {
-            abi_check(tsvm_nu_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), d_ws.data(), ws_size,
+            abi_check(tsvm_nu_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), ws_ids(), ws_size,
                                               Cp, d_kws.data(), k_mat.diag(), eps, d_diff.data(), max_iter, st));
         } else {
-            abi_check(tsvm_c_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), d_ws.data(), ws_size,
+            abi_check(tsvm_c_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), ws_ids(), ws_size,
                                              Cp, Cn, d_kws.data(), k_mat.diag(), eps, d_diff.data(), max_iter, st));
         }
         timer.end(stats.ms_local);
@@ -497,7 +510,7 @@ struct SolveTask::Impl {
             trace->diff.push_back(diff0);
             trace->diff.push_back(diff1);
             std::vector<int> w = d_ws.to_host();
-            trace->ws.insert(trace->ws.end(), w.begin(), w.end());
+            trace->ws.insert(trace->ws.end(), w.begin() + ws_off, w.begin() + ws_off + ws_size);
         }
         // stall guards and stopping rule (csmosolver.cpp:86-111)
         if (fabs(diff0 - previous_local_diff) < eps * 0.001) {
