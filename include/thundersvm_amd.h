@@ -81,6 +81,14 @@ int tsvm_get_rows_dense(const double *x, int64_t ldx, const int *x_idx, int64_t 
                         double coef0, int degree, void *out, int row_type, const int *out_slots, int64_t ldo,
                         tsvm_stream stream);
 
+/* tsvm_get_rows_dense when the number of working rows is only known on the device: the grid is sized for m_max
+ * rows, *m_dev (read by the kernel, 0 <= *m_dev <= m_max) says how many of them exist; entries of a_idx and
+ * out_slots from *m_dev on are not read. */
+int tsvm_get_rows_dense_counted(const double *x, int64_t ldx, const int *x_idx, int64_t n, int d, const double *sd_x,
+                                const double *a, int64_t lda, const int *a_idx, int m_max, const int *m_dev,
+                                const double *sd_a, int kernel_type, double gamma, double coef0, int degree, void *out,
+                                int row_type, const int *out_slots, int64_t ldo, tsvm_stream stream);
+
 /* Transposed dense staging of selected CSR rows: w[c*m + i] = value of feature c in row idx[i]
  * (idx == NULL: row i of the given CSR), w is [n_features][m] and is zero-filled first.
  * The sparse-path counterpart of get_working_set_ins (kernelmatrix_kernel.cpp:9-25). */
@@ -147,6 +155,22 @@ int tsvm_smo_solve_block_ld(int ws_size);
 int tsvm_smo_gather_block(const void *k_rows, int row_type, const int *slots, int64_t ld, const int *cols, int ws_size,
                           double *kws, tsvm_stream stream);
 
+/* The block when slot_of_id[i] names the slot that holds instance i's row (a row cache that holds every row):
+ * kws[r*ldk + t] = element ids[t] of the row in slot slot_of_id[ids[r]]; slots_out[r] receives that slot (the
+ * table tsvm_update_f takes).  Nothing has to come from the host between the selection and this call. */
+int tsvm_smo_gather_block_by_id(const void *k_rows, int row_type, const int *slot_of_id, int64_t ld, const int *ids,
+                                int ws_size, double *kws, int *slots_out, tsvm_stream stream);
+
+/* Slots for the new rows of a working set, decided on the device, for a row store with a slot for every
+ * instance (the reference recomputes the rows of every working set, csmosolver.cpp:65-77; rows kept here are the
+ * rows get_rows would recompute).  ids_new[0..n_new) are distinct instances; those without a slot yet
+ * (slot_of_id[i] < 0) take the slots state[0], state[0]+1, ... in list order.  Outputs: slot_of_id and state[0]
+ * (slots in use) updated; state[1] = number of such instances, listed in miss_ids / miss_slots (the a_idx /
+ * out_slots / m_dev of tsvm_get_rows_dense_counted); slots_ws[t] = slot of ids_ws[t], t < ws_size; info[0..1] =
+ * state[1], state[0] (for the host: info may be pinned host memory).  Start from slot_of_id = -1, state = 0. */
+int tsvm_row_slots_assign(const int *ids_new, int n_new, int *slot_of_id, int *state, int *miss_ids, int *miss_slots,
+                          const int *ids_ws, int ws_size, int *slots_ws, int *info, tsvm_stream stream);
+
 /* c_smo_solve / nu_smo_solve on a precomputed block kws[r*ldk + t] = K(x_ws[r], x_ws[t]) (ldk from
  * tsvm_smo_solve_block_ld, columns t >= ws zero or arbitrary finite values): the solver touches nothing
  * else of the kernel matrix, so it can run while the full rows are still being computed on another
@@ -175,6 +199,14 @@ size_t tsvm_select_workspace(int64_t n);
 int tsvm_select_working_set(const double *f, const int *y, const double *alpha, int64_t n, double Cp, double Cn,
                             const int *marked, int n_marked, int *out, int n_select, int nu, void *workspace,
                             tsvm_stream stream);
+
+/* The same selection for a workspace whose last use was a call of either function with the same n and nu,
+ * complete on this stream or ordered before it: that call has left the workspace's counters cleared, and
+ * this one skips the launch that clears them (CSMOSolver::solve, csmosolver.cpp:63-77, selects once per
+ * outer iteration on the same problem).  On any other workspace content the result is undefined. */
+int tsvm_select_working_set_again(const double *f, const int *y, const double *alpha, int64_t n, double Cp, double Cn,
+                                  const int *marked, int n_marked, int *out, int n_select, int nu, void *workspace,
+                                  tsvm_stream stream);
 
 /* ---------------------------------------------------------------------------------------------
  * predict (kernelmatrix_kernel.cpp:110-147)

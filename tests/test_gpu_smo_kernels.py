@@ -189,6 +189,34 @@ def test_longer_selection_starts_with_the_shorter_one(tie_mode, nu):
     assert (tail >= 0).all() and len(set(tail.tolist()) | set(outs[0].tolist()) | set(marked.tolist())) == 768 + n_marked
 
 
+@pytest.mark.parametrize("nu", [0, 1])
+@pytest.mark.parametrize("n", [700, 3200, 100000, 300001])
+def test_selections_in_a_row_on_one_workspace(n, nu):
+    """The solver's pattern (csmosolver.cpp:63-77): one full selection, then one per outer iteration that keeps
+    half of the previous set, all on one workspace that each call leaves ready for the next.  The f values change
+    from call to call between distinct values, massive ties (the remaining digits are then resolved by the final
+    kernel's workgroup) and few distinct values."""
+    ws = min(1024, 1 << (n.bit_length() - 1))
+    q = ws // 2
+    wsp = torch.empty(capi.kernel_lib().tsvm_select_workspace(n), dtype=torch.uint8, device="cuda")
+    wsp.random_(0, 256)   # whatever an earlier user of the memory left there
+    prev = None
+    for it, tie_mode in enumerate([0, 1, 0, 2, 1, 1, 0]):
+        f, y, alpha, C, _ = _select_case(n, q, 0, 7 * n + it, tie_mode, nu)
+        marked = np.zeros(0, dtype=np.int32) if it == 0 else np.ascontiguousarray(prev[q:])
+        n_select = ws if it == 0 else q
+        want = O.select_working_set(f, y, alpha, C, C, marked, n_select, nu=bool(nu))
+        f_d, y_d, a_d, m_d = G.dev(f), G.dev(y), G.dev(alpha), G.dev(marked if it else np.zeros(1, dtype=np.int32))
+        out_d = torch.full((n_select,), -7, dtype=torch.int32, device="cuda")
+        capi.call("tsvm_select_working_set" if it == 0 else "tsvm_select_working_set_again", G.ptr(f_d), G.ptr(y_d),
+                  G.ptr(a_d), n, C, C, G.ptr(m_d) if it else None, len(marked), G.ptr(out_d), n_select, nu, G.ptr(wsp),
+                  G.stream())
+        got = G.host(out_d)
+        assert np.array_equal(got, want), "call %d: first mismatch at %s" % (it, np.flatnonzero(got != want)[:5])
+        prev = got if it == 0 else np.concatenate([prev[q:], got])
+        assert (prev >= 0).all()
+
+
 def test_empty_inputs_are_no_ops():
     """Zero rows, zero columns, an empty working set, nothing to select: every entry point returns success and
     leaves its outputs untouched."""

@@ -27,6 +27,7 @@ SIGNATURES = {
     "tsvm_kernel_diag": (_int, [_p, _i64, _int, _dbl, _dbl, _int, _p, _p]),
     "tsvm_csr_to_dense": (_int, [_p, _p, _p, _i64, _p, _i64, _p]),
     "tsvm_get_rows_dense": (_int, [_p, _i64, _p, _i64, _int, _p, _p, _i64, _p, _int, _p, _int, _dbl, _dbl, _int, _p, _int, _p, _i64, _p]),
+    "tsvm_get_rows_dense_counted": (_int, [_p, _i64, _p, _i64, _int, _p, _p, _i64, _p, _int, _p, _p, _int, _dbl, _dbl, _int, _p, _int, _p, _i64, _p]),
     "tsvm_csr_stage_rows": (_int, [_p, _p, _p, _p, _int, _int, _p, _p]),
     "tsvm_get_rows_csr": (_int, [_p, _p, _p, _p, _i64, _p, _p, _int, _p, _int, _dbl, _dbl, _int, _p, _int, _p, _i64, _p]),
     "tsvm_fold_ids": (_int, [_p, _int, _int, _p, _p]),
@@ -39,10 +40,13 @@ SIGNATURES = {
     "tsvm_nu_smo_solve": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _p, _int, _p, _i64, _p, _dbl, _p, _int, _p, _p]),
     "tsvm_smo_solve_block_ld": (_int, [_int]),
     "tsvm_smo_gather_block": (_int, [_p, _int, _p, _i64, _p, _int, _p, _p]),
+    "tsvm_row_slots_assign": (_int, [_p, _int, _p, _p, _p, _p, _p, _int, _p, _p, _p]),
+    "tsvm_smo_gather_block_by_id": (_int, [_p, _int, _p, _i64, _p, _int, _p, _p, _p]),
     "tsvm_c_smo_solve_block": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _dbl, _p, _p, _dbl, _p, _int, _p]),
     "tsvm_nu_smo_solve_block": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _p, _p, _dbl, _p, _int, _p]),
     "tsvm_select_workspace": (C.c_size_t, [_i64]),
     "tsvm_select_working_set": (_int, [_p, _p, _p, _i64, _dbl, _dbl, _p, _int, _p, _int, _int, _p, _p]),
+    "tsvm_select_working_set_again": (_int, [_p, _p, _p, _i64, _dbl, _dbl, _p, _int, _p, _int, _int, _p, _p]),
     "tsvm_sum_kernel_values": (_int, [_p, _int, _p, _p, _p, _p, _int, _i64, _p, _int, _i64, _p]),
 }
 

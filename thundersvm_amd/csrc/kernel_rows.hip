@@ -44,7 +44,7 @@ __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
     const double *__restrict__ x, int64_t ldx, const int *__restrict__ x_idx, int64_t n, int d,
     const double *__restrict__ sd_x, const double *__restrict__ a, int64_t lda, const int *__restrict__ a_idx, int m,
     const double *__restrict__ sd_a, KernelParam kp_in, TO *__restrict__ out, const int *__restrict__ out_slots,
-    int64_t ldo, unsigned m_blocks) {
+    int64_t ldo, unsigned m_blocks, const int *__restrict__ m_dev) {
     constexpr int BM = 32 * TI;
     constexpr int KTILE = TI == 2 ? 16 : 8;
     constexpr int LS = TI == 2 ? 129 : 130;
@@ -67,6 +67,11 @@ __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
     const unsigned logical = xcd_remap(blockIdx.x, gridDim.x);
     const int j0 = (int) (logical / m_blocks) * GR_BN;   // n fits 31 bits (checked by the host)
     const int i0 = (int) (logical % m_blocks) * BM;
+    if (m_dev) {
+        // the number of working rows is only known on the device (m sized the grid): workgroups beyond it leave
+        m = *m_dev;
+        if (i0 >= m) return;
+    }
     const int n_last = (int) n - 1, m_last = m - 1;
 
     // Staging assignment.  Rows beyond the tile's valid range are clamped to the last valid row: what they
@@ -488,10 +493,10 @@ static bool row_type_ok(int row_type, int kernel_type) {
     return row_type == TSVM_ROW_F64 || (row_type == TSVM_ROW_F32 && kernel_type != TSVM_LINEAR);
 }
 
-int tsvm_get_rows_dense(const double *x, int64_t ldx, const int *x_idx, int64_t n, int d, const double *sd_x, const double *a,
-                        int64_t lda, const int *a_idx, int m, const double *sd_a, int kernel_type, double gamma,
-                        double coef0, int degree, void *out, int row_type, const int *out_slots, int64_t ldo,
-                        tsvm_stream stream) {
+static int get_rows_dense(const double *x, int64_t ldx, const int *x_idx, int64_t n, int d, const double *sd_x, const double *a,
+                          int64_t lda, const int *a_idx, int m, const int *m_dev, const double *sd_a, int kernel_type, double gamma,
+                          double coef0, int degree, void *out, int row_type, const int *out_slots, int64_t ldo,
+                          tsvm_stream stream) {
     TSVM_REQUIRE(x && a && out, "tsvm_get_rows_dense: null pointer");
     TSVM_REQUIRE(n >= 0 && m >= 0 && d >= 0, "tsvm_get_rows_dense: negative size");
     TSVM_REQUIRE(n <= 0x7fff0000 && ldx <= 0x7fffffff && lda <= 0x7fffffff && ldo <= 0x7fffffff,
@@ -521,10 +526,10 @@ int tsvm_get_rows_dense(const double *x, int64_t ldx, const int *x_idx, int64_t 
     do {                                                                                                              \
         if (ti == 2)                                                                                                  \
             hipLaunchKernelGGL((get_rows_dense_kernel<KTYPE, 2, TO>), grid, block, 0, tsvm_s(stream), x, ldx, x_idx, n, d, sd_x, \
-                               a, lda, a_idx, m, sd_a, kp, (TO *) out, out_slots, ldo, m_blocks);                     \
+                               a, lda, a_idx, m, sd_a, kp, (TO *) out, out_slots, ldo, m_blocks, m_dev);              \
         else                                                                                                          \
             hipLaunchKernelGGL((get_rows_dense_kernel<KTYPE, 4, TO>), grid, block, 0, tsvm_s(stream), x, ldx, x_idx, n, d, sd_x, \
-                               a, lda, a_idx, m, sd_a, kp, (TO *) out, out_slots, ldo, m_blocks);                     \
+                               a, lda, a_idx, m, sd_a, kp, (TO *) out, out_slots, ldo, m_blocks, m_dev);              \
     } while (0)
 #define GR_LAUNCH(KTYPE)                                        \
     do {                                                        \
@@ -541,6 +546,23 @@ int tsvm_get_rows_dense(const double *x, int64_t ldx, const int *x_idx, int64_t 
 #undef GR_LAUNCH_T
     TSVM_LAUNCH_CHECK();
     return 0;
+}
+
+int tsvm_get_rows_dense(const double *x, int64_t ldx, const int *x_idx, int64_t n, int d, const double *sd_x, const double *a,
+                        int64_t lda, const int *a_idx, int m, const double *sd_a, int kernel_type, double gamma,
+                        double coef0, int degree, void *out, int row_type, const int *out_slots, int64_t ldo,
+                        tsvm_stream stream) {
+    return get_rows_dense(x, ldx, x_idx, n, d, sd_x, a, lda, a_idx, m, nullptr, sd_a, kernel_type, gamma, coef0, degree, out,
+                          row_type, out_slots, ldo, stream);
+}
+
+int tsvm_get_rows_dense_counted(const double *x, int64_t ldx, const int *x_idx, int64_t n, int d, const double *sd_x,
+                                const double *a, int64_t lda, const int *a_idx, int m_max, const int *m_dev,
+                                const double *sd_a, int kernel_type, double gamma, double coef0, int degree, void *out,
+                                int row_type, const int *out_slots, int64_t ldo, tsvm_stream stream) {
+    TSVM_REQUIRE(m_dev, "tsvm_get_rows_dense_counted: null pointer");
+    return get_rows_dense(x, ldx, x_idx, n, d, sd_x, a, lda, a_idx, m_max, m_dev, sd_a, kernel_type, gamma, coef0, degree, out,
+                          row_type, out_slots, ldo, stream);
 }
 
 int tsvm_csr_stage_rows(const double *val, const int *col, const int64_t *row_ptr, const int *idx, int m,

@@ -143,7 +143,6 @@ struct SelState {
 struct SelWorkspace {   // device-side layout, carved from the caller's workspace
     uint64_t *keys;     // [n] order-preserving transform of f
     uint8_t *flags;     // [n] side membership bits
-    uint8_t *ind;       // [n] ws_indicator
     uint32_t *hist;     // [SEL_MAX_PASS][SEL_MAX_SIDES][SEL_BINS]
     SelState *state;    // [SEL_MAX_PASS + 1][SEL_MAX_SIDES]
     uint32_t *count;    // [SEL_MAX_SIDES]
@@ -159,14 +158,13 @@ static size_t sel_carve(void *base, int64_t n, SelWorkspace *w) {
     auto take = [&](size_t bytes) { size_t o = off; off += sel_align(bytes); return b ? b + o : nullptr; };
     void *keys = take(sizeof(uint64_t) * (size_t) n);
     void *flags = take((size_t) n);
-    void *ind = take((size_t) n);
     void *hist = take(sizeof(uint32_t) * SEL_MAX_PASS * SEL_MAX_SIDES * SEL_BINS);
     void *state = take(sizeof(SelState) * (SEL_MAX_PASS + 1) * SEL_MAX_SIDES);
     void *count = take(sizeof(uint32_t) * SEL_MAX_SIDES);
     void *lk = take(sizeof(uint64_t) * SEL_MAX_SIDES * MAX_WS);
     void *li = take(sizeof(uint32_t) * SEL_MAX_SIDES * MAX_WS);
     if (w) {
-        w->keys = (uint64_t *) keys; w->flags = (uint8_t *) flags; w->ind = (uint8_t *) ind;
+        w->keys = (uint64_t *) keys; w->flags = (uint8_t *) flags;
         w->hist = (uint32_t *) hist; w->state = (SelState *) state; w->count = (uint32_t *) count;
         w->list_key = (uint64_t *) lk; w->list_idx = (uint32_t *) li;
     }
@@ -228,22 +226,17 @@ __device__ __forceinline__ uint64_t f_to_key(double f) {
 
 __device__ __forceinline__ bool sel_side_descending(int side, int n_sides) { return n_sides == 2 ? side == 1 : side >= 2; }
 
-__global__ void sel_init_kernel(SelWorkspace w, int64_t n, SelGeom g) {
-    const int64_t gid = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
-    const int64_t stride = (int64_t) gridDim.x * blockDim.x;
-    for (int64_t j = gid; j < n; j += stride) w.ind[j] = 0;
-    for (int64_t e = gid; e < (int64_t) SEL_MAX_PASS * SEL_MAX_SIDES * SEL_BINS; e += stride) w.hist[e] = 0;
-    if (gid < SEL_MAX_SIDES) {
-        w.count[gid] = 0;
-        SelState st;
-        st.pk = 0; st.pi = 0; st.k_rem = g.k; st.done = 0; st.pad = 0;
-        w.state[gid] = st;  // state before pass 0
-    }
+// What a call needs to find in the workspace: zeroed histograms for the digits that are counted with atomics
+// by the whole grid and zeroed list lengths.  Written by sel_init_kernel, and again
+// by sel_final_kernel once it has read what it needs, so that the next call on the same workspace (same n,
+// same sides) can start counting straight away.
+__device__ __forceinline__ void sel_arm(const SelWorkspace &w, const SelGeom &g, int p_full, int64_t gid, int64_t stride) {
+    for (int64_t e = gid; e < (int64_t) p_full * SEL_MAX_SIDES * SEL_BINS; e += stride) w.hist[e] = 0;
+    if (gid < SEL_MAX_SIDES) w.count[gid] = 0;
 }
 
-__global__ void sel_mark_kernel(uint8_t *ind, const int *__restrict__ marked, int n_marked) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n_marked) ind[marked[i]] = 1;
+__global__ void sel_init_kernel(SelWorkspace w, SelGeom g, int p_full) {
+    sel_arm(w, g, p_full, (int64_t) blockIdx.x * blockDim.x + threadIdx.x, (int64_t) gridDim.x * blockDim.x);
 }
 
 // Computes, in LDS, the state after pass p-1's histogram has been consumed (st_out), from the
@@ -329,16 +322,26 @@ __device__ __forceinline__ void sel_count(const SelGeom &g, const SelState *st, 
     }
 }
 
-// Pass p: (p == 0: also builds keys/flags) histogram digit p of the not-yet-decided candidates.
+// Pass p: histogram of digit p of the not-yet-decided candidates.  Pass 0 also builds keys and flags; there a
+// workgroup walks one contiguous chunk of the instances and keeps the chunk's marked instances (the half of the
+// previous working set that stays, csmosolver.cpp:65-71: never candidates) as a bit field in LDS.
+#define SEL_CHUNK_MAX 65536
 __global__ __launch_bounds__(SEL_T) void sel_pass_kernel(SelWorkspace w, const double *__restrict__ f,
                                                          const int *__restrict__ y, const double *__restrict__ alpha,
-                                                         int64_t n, double Cp, double Cn, SelGeom g, int p) {
+                                                         int64_t n, double Cp, double Cn, SelGeom g, int p,
+                                                         const int *__restrict__ marked, int n_marked) {
     __shared__ uint32_t lhist[SEL_MAX_SIDES][SEL_BINS];
     __shared__ SelState st[SEL_MAX_SIDES];
     __shared__ uint32_t scratch[SEL_T + 16];
+    __shared__ uint32_t mark_bits[SEL_CHUNK_MAX / 32];
     const int tid = threadIdx.x;
     if (p == 0) {
-        if (tid < g.n_sides) st[tid] = w.state[tid];
+        if (tid < g.n_sides) {
+            SelState s0;
+            s0.pk = 0; s0.pi = 0; s0.k_rem = g.k; s0.done = 0; s0.pad = 0;
+            st[tid] = s0;
+            if (blockIdx.x == 0) w.state[tid] = s0;   // the state before digit 0, for the next pass
+        }
         __syncthreads();
     } else {
         sel_advance_state(w, g, p, st, scratch);
@@ -348,20 +351,26 @@ __global__ __launch_bounds__(SEL_T) void sel_pass_kernel(SelWorkspace w, const d
     for (int s = 0; s < g.n_sides; ++s) any |= !st[s].done;
     if (!any) return;
     for (int e = tid; e < SEL_MAX_SIDES * SEL_BINS; e += SEL_T) (&lhist[0][0])[e] = 0;
-    __syncthreads();
     bool is_key; int shift, width;
     sel_digit_geom(p, g.idx_bits, is_key, shift, width);
     const uint32_t dmask = (1u << width) - 1;
-    const int64_t stride = (int64_t) gridDim.x * SEL_T;
-    for (int64_t j = (int64_t) blockIdx.x * SEL_T + tid; j < n; j += stride) {
-        uint64_t key;
-        uint32_t fl;
-        if (p == 0) {
+    if (p == 0) {
+        const int64_t chunk = (n + gridDim.x - 1) / gridDim.x;   // <= SEL_CHUNK_MAX (the host sizes the grid)
+        const int64_t lo = (int64_t) blockIdx.x * chunk;
+        const int64_t hi = lo + chunk < n ? lo + chunk : n;
+        for (int e = tid; e < (int) ((chunk + 31) >> 5); e += SEL_T) mark_bits[e] = 0;
+        __syncthreads();
+        for (int i = tid; i < n_marked; i += SEL_T) {
+            const int64_t id = marked[i];
+            if (id >= lo && id < hi) atomicOr(&mark_bits[(id - lo) >> 5], 1u << ((id - lo) & 31));
+        }
+        __syncthreads();
+        for (int64_t j = lo + tid; j < hi; j += SEL_T) {
             const double a = alpha[j];
             const double yy = (double) y[j];
-            key = f_to_key(f[j]);
-            fl = 0;
-            if (!w.ind[j]) {
+            const uint64_t key = f_to_key(f[j]);
+            uint32_t fl = 0;
+            if (!((mark_bits[(j - lo) >> 5] >> ((j - lo) & 31)) & 1u)) {
                 const bool up = is_I_up(a, yy, Cp, Cn), low = is_I_low(a, yy, Cp, Cn);
                 if (g.n_sides == 2) {
                     fl = (up ? 1u : 0u) | (low ? 2u : 0u);
@@ -372,12 +381,16 @@ __global__ __launch_bounds__(SEL_T) void sel_pass_kernel(SelWorkspace w, const d
             }
             w.keys[j] = key;
             w.flags[j] = (uint8_t) fl;
-        } else {
-            fl = w.flags[j];
-            if (!fl) continue;
-            key = w.keys[j];
+            sel_count(g, st, lhist, p, is_key, shift, dmask, key, fl, j);
         }
-        sel_count(g, st, lhist, p, is_key, shift, dmask, key, fl, j);
+    } else {
+        __syncthreads();
+        const int64_t stride = (int64_t) gridDim.x * SEL_T;
+        for (int64_t j = (int64_t) blockIdx.x * SEL_T + tid; j < n; j += stride) {
+            const uint32_t fl = w.flags[j];
+            if (!fl) continue;
+            sel_count(g, st, lhist, p, is_key, shift, dmask, w.keys[j], fl, j);
+        }
     }
     __syncthreads();
     uint32_t *gh = w.hist + (size_t) p * SEL_MAX_SIDES * SEL_BINS;
@@ -387,52 +400,11 @@ __global__ __launch_bounds__(SEL_T) void sel_pass_kernel(SelWorkspace w, const d
     }
 }
 
-// Passes p_first .. n_pass-1 in one workgroup.  After the grid-wide passes every side is normally decided
-// and this kernel only carries the state forward; when a boundary bucket is still too large (many equal f
-// values, e.g. the first iteration of a training run, where the instance index has to break the ties), the
-// one workgroup walks the candidates once per remaining digit.  That is slow but rare, and it replaces one
-// kernel launch per digit in every call.
-#define SEL_TAIL_T 1024
-__global__ __launch_bounds__(SEL_TAIL_T) void sel_tail_kernel(SelWorkspace w, int64_t n, SelGeom g, int p_first) {
-    __shared__ uint32_t lhist[SEL_MAX_SIDES][SEL_BINS];
-    __shared__ SelState st[SEL_MAX_SIDES];
-    __shared__ uint32_t scratch[SEL_T + 16];
-    const int tid = threadIdx.x;
-    for (int p = p_first; p < g.n_pass; ++p) {
-        sel_advance_state(w, g, p, st, scratch);
-        if (tid < g.n_sides) w.state[p * SEL_MAX_SIDES + tid] = st[tid];
-        bool any = false;
-        for (int s = 0; s < g.n_sides; ++s) any |= !st[s].done;
-        if (!any) {
-            // decided: later states are copies (sel_compact_kernel reads the last one)
-            for (int q = p + 1; q < g.n_pass; ++q)
-                if (tid < g.n_sides) w.state[q * SEL_MAX_SIDES + tid] = st[tid];
-            return;
-        }
-        for (int e = tid; e < SEL_MAX_SIDES * SEL_BINS; e += SEL_TAIL_T) (&lhist[0][0])[e] = 0;
-        __syncthreads();
-        bool is_key; int shift, width;
-        sel_digit_geom(p, g.idx_bits, is_key, shift, width);
-        const uint32_t dmask = (1u << width) - 1;
-        for (int64_t j = tid; j < n; j += SEL_TAIL_T) {
-            const uint32_t fl = w.flags[j];
-            if (fl) sel_count(g, st, lhist, p, is_key, shift, dmask, w.keys[j], fl, j);
-        }
-        __syncthreads();
-        uint32_t *gh = w.hist + (size_t) p * SEL_MAX_SIDES * SEL_BINS;   // zeroed by sel_init_kernel
-        for (int e = tid; e < g.n_sides * SEL_BINS; e += SEL_TAIL_T) gh[e] = (&lhist[0][0])[e];
-        __syncthreads();   // the next digit's sel_advance_state reads state[p] and hist[p] back from memory
-    }
-}
-
-// After the last pass: finalise the state and append every selected candidate to its side's list.
-__global__ __launch_bounds__(SEL_T) void sel_compact_kernel(SelWorkspace w, int64_t n, SelGeom g) {
-    __shared__ SelState st[SEL_MAX_SIDES];
-    __shared__ uint32_t scratch[SEL_T + 16];
-    const int tid = threadIdx.x;
-    sel_advance_state(w, g, g.n_pass, st, scratch);
-    const int64_t stride = (int64_t) gridDim.x * SEL_T;
-    for (int64_t j = (int64_t) blockIdx.x * SEL_T + tid; j < n; j += stride) {
+// Appends the selected candidates among instances first, first + stride, ... to their sides' lists; st is the
+// final state of every side.
+__device__ __forceinline__ void sel_collect(const SelWorkspace &w, int64_t n, const SelGeom &g, const SelState *st,
+                                            int64_t first, int64_t stride) {
+    for (int64_t j = first; j < n; j += stride) {
         const uint32_t fl = w.flags[j];
         if (!fl) continue;
         const uint64_t key = w.keys[j];
@@ -441,12 +413,11 @@ __global__ __launch_bounds__(SEL_T) void sel_compact_kernel(SelWorkspace w, int6
             const bool desc = sel_side_descending(s, g.n_sides);
             const uint64_t k2 = desc ? ~key : key;
             const uint32_t i2 = desc ? g.idx_mask - (uint32_t) j : (uint32_t) j;
-            // all digits count as resolved once the side is done: compare on the digits it consumed
             int cmp;
             if (st[s].k_rem == 0 && st[s].done) {
                 cmp = 1;  // nothing to take on this side
             } else {
-                // number of passes whose digit is part of the prefix = passes consumed by this side
+                // compare on the digits this side consumed before it was decided
                 cmp = sel_cmp_prefix(k2, i2, st[s], (int) st[s].pad, g.idx_bits);
             }
             if (cmp <= 0) {
@@ -460,20 +431,71 @@ __global__ __launch_bounds__(SEL_T) void sel_compact_kernel(SelWorkspace w, int6
     }
 }
 
+__device__ __forceinline__ bool sel_undecided(const SelGeom &g, const SelState *st) {
+    bool any = false;
+    for (int s = 0; s < g.n_sides; ++s) any |= !st[s].done;
+    return any;
+}
+
+// After the grid-wide passes every side is normally decided: then this kernel appends every selected candidate
+// to its side's list.  If a boundary bucket is still too large it does nothing, and sel_final_kernel goes on.
+__global__ __launch_bounds__(SEL_T) void sel_compact_kernel(SelWorkspace w, int64_t n, SelGeom g, int p_full) {
+    __shared__ SelState st[SEL_MAX_SIDES];
+    __shared__ uint32_t scratch[SEL_T + 16];
+    sel_advance_state(w, g, p_full, st, scratch);
+    if (sel_undecided(g, st)) return;
+    sel_collect(w, n, g, st, (int64_t) blockIdx.x * SEL_T + threadIdx.x, (int64_t) gridDim.x * SEL_T);
+}
+
+// Digits p_full .. n_pass-1 and the lists, by one workgroup: only when the grid-wide digits left a boundary
+// bucket too large to take whole (many equal f values, e.g. the first iteration of a training run, where the
+// instance index has to break the ties).  The workgroup walks the candidates once per remaining digit: slow but
+// rare, and it keeps a launch per digit out of every call.  st holds the state before digit p_full.
+__device__ void sel_tail(const SelWorkspace &w, int64_t n, const SelGeom &g, int p_full, SelState *st,
+                         uint32_t (*lhist)[SEL_BINS], uint32_t *scratch) {
+    const int tid = threadIdx.x, nt = blockDim.x;
+    for (int p = p_full; p < g.n_pass && sel_undecided(g, st); ++p) {
+        if (tid < g.n_sides) w.state[p * SEL_MAX_SIDES + tid] = st[tid];
+        for (int e = tid; e < SEL_MAX_SIDES * SEL_BINS; e += nt) (&lhist[0][0])[e] = 0;
+        __syncthreads();
+        bool is_key; int shift, width;
+        sel_digit_geom(p, g.idx_bits, is_key, shift, width);
+        const uint32_t dmask = (1u << width) - 1;
+        for (int64_t j = tid; j < n; j += nt) {
+            const uint32_t fl = w.flags[j];
+            if (fl) sel_count(g, st, lhist, p, is_key, shift, dmask, w.keys[j], fl, j);
+        }
+        __syncthreads();
+        uint32_t *gh = w.hist + (size_t) p * SEL_MAX_SIDES * SEL_BINS;
+        for (int e = tid; e < g.n_sides * SEL_BINS; e += nt) gh[e] = (&lhist[0][0])[e];
+        __syncthreads();   // sel_advance_state reads state[p] and hist[p] back from memory
+        sel_advance_state(w, g, p + 1, st, scratch);
+    }
+    sel_collect(w, n, g, st, tid, nt);
+    __syncthreads();
+}
+
 // Final step: sort each side's list, replay the alternating scan, write the selection.
 __device__ __forceinline__ bool comp_less(uint64_t ka, uint32_t ia, uint64_t kb, uint32_t ib) {
     return ka < kb || (ka == kb && ia < ib);
 }
 
-__global__ __launch_bounds__(MAX_WS) void sel_final_kernel(SelWorkspace w, SelGeom g, int *__restrict__ out) {
+__global__ __launch_bounds__(MAX_WS) void sel_final_kernel(SelWorkspace w, int64_t n, SelGeom g, int p_full,
+                                                           int *__restrict__ out) {
     __shared__ uint64_t sk[SEL_MAX_SIDES][MAX_WS];
     __shared__ uint32_t si[SEL_MAX_SIDES][MAX_WS];
     __shared__ int pos_other[SEL_MAX_SIDES][MAX_WS];  // position of the same instance in the paired side's list, or -1
     __shared__ int cnt[SEL_MAX_SIDES];
     __shared__ int conflict;
+    __shared__ SelState st[SEL_MAX_SIDES];
+    __shared__ uint32_t scratch[SEL_T + 16];
     const int tid = threadIdx.x;
+    // the test sel_compact_kernel made: if it left the lists empty, the remaining digits and the lists are made here
+    sel_advance_state(w, g, p_full, st, scratch);
+    if (sel_undecided(g, st)) sel_tail(w, n, g, p_full, st, (uint32_t (*)[SEL_BINS]) &sk[0][0], scratch);
     if (tid < SEL_MAX_SIDES) {
-        int c = tid < g.n_sides ? (int) w.count[tid] : 0;
+        // (an atomic read: the lengths were counted with atomics, by this workgroup itself on the slow path)
+        int c = tid < g.n_sides ? (int) __hip_atomic_load(&w.count[tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0;
         cnt[tid] = c > MAX_WS ? MAX_WS : c;
     }
     if (tid == 0) conflict = 0;
@@ -488,6 +510,7 @@ __global__ __launch_bounds__(MAX_WS) void sel_final_kernel(SelWorkspace w, SelGe
         }
     }
     __syncthreads();
+    sel_arm(w, g, p_full, tid, MAX_WS);   // everything this call needed from the workspace is in LDS now
     // Bitonic sort, ascending composite, all sides at once.  Thread t owns compare-exchange pair t & 511 of
     // side t >> 9 (and of side 2 + (t >> 9) when there are four), so every thread works in every stage.  With
     // strides up to 64 a wavefront's 64 pairs cover one closed block of 128 entries, stage after stage: such
@@ -608,6 +631,48 @@ static void launch_update_f(double *f, const double *alpha_diff, int ws_size, co
                        (const TK *) k_rows, slots, ld, n, repeat, vec_per_wg);
 }
 
+static int select_working_set(const double *f, const int *y, const double *alpha, int64_t n, double Cp, double Cn,
+                              const int *marked, int n_marked, int *out, int n_select, int nu, void *workspace,
+                              bool armed, tsvm_stream stream) {
+    TSVM_REQUIRE(f && y && alpha && out && workspace, "tsvm_select_working_set: null pointer");
+    TSVM_REQUIRE(n >= 1 && n <= 0x7fffffffLL, "tsvm_select_working_set: n %lld outside [1, 2^31)", (long long) n);
+    TSVM_REQUIRE(n_select >= 0 && n_select <= MAX_WS, "tsvm_select_working_set: n_select %d outside [0, %d]", n_select,
+                 MAX_WS);
+    TSVM_REQUIRE(n_marked >= 0 && (n_marked == 0 || marked), "tsvm_select_working_set: bad marked list");
+    if (n_select == 0) return 0;
+    hipStream_t s = tsvm_s(stream);
+    SelWorkspace w;
+    void *base = (void *) (((uintptr_t) workspace + 255) & ~(uintptr_t) 255);
+    sel_carve(base, n, &w);
+    SelGeom g;
+    g.n_sides = nu ? 4 : 2;
+    int bits = 1;
+    while (((int64_t) 1 << bits) < n) ++bits;
+    g.idx_bits = bits;
+    g.idx_mask = (uint32_t) (((uint64_t) 1 << bits) - 1);
+    g.n_pass = 6 + (bits + SEL_DIGIT - 1) / SEL_DIGIT;
+    g.k = (uint32_t) n_select;
+    // The first three digits (33 bits of f) are counted by the whole chip, the rest (rarely needed) by one
+    // workgroup.  Near convergence the free support vectors crowd within epsilon of the threshold, so the third
+    // digit is usually the one that separates them.
+    const int p_full = n > ((int64_t) 1 << 26) ? 4 : 3;   // < n_pass, which is at least 7
+    unsigned grid = (unsigned) std::min<int64_t>((n + SEL_T - 1) / SEL_T, 1024);
+    if ((n + grid - 1) / grid > SEL_CHUNK_MAX) grid = (unsigned) ((n + SEL_CHUNK_MAX - 1) / SEL_CHUNK_MAX);
+    if (!armed) {
+        hipLaunchKernelGGL(sel_init_kernel, dim3(p_full * SEL_MAX_SIDES * SEL_BINS / 1024), dim3(256), 0, s, w, g, p_full);
+        TSVM_LAUNCH_CHECK();
+    }
+    for (int p = 0; p < p_full; ++p) {
+        hipLaunchKernelGGL(sel_pass_kernel, dim3(grid), dim3(SEL_T), 0, s, w, f, y, alpha, n, Cp, Cn, g, p, marked, n_marked);
+        TSVM_LAUNCH_CHECK();
+    }
+    hipLaunchKernelGGL(sel_compact_kernel, dim3(grid), dim3(SEL_T), 0, s, w, n, g, p_full);
+    TSVM_LAUNCH_CHECK();
+    hipLaunchKernelGGL(sel_final_kernel, dim3(1), dim3(MAX_WS), 0, s, w, n, g, p_full, out);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
 extern "C" {
 
 int tsvm_update_f(double *f, const double *alpha_diff, int ws_size, const void *k_rows, int row_type, const int *slots,
@@ -642,48 +707,13 @@ size_t tsvm_select_workspace(int64_t n) {
 int tsvm_select_working_set(const double *f, const int *y, const double *alpha, int64_t n, double Cp, double Cn,
                             const int *marked, int n_marked, int *out, int n_select, int nu, void *workspace,
                             tsvm_stream stream) {
-    TSVM_REQUIRE(f && y && alpha && out && workspace, "tsvm_select_working_set: null pointer");
-    TSVM_REQUIRE(n >= 1 && n <= 0x7fffffffLL, "tsvm_select_working_set: n %lld outside [1, 2^31)", (long long) n);
-    TSVM_REQUIRE(n_select >= 0 && n_select <= MAX_WS, "tsvm_select_working_set: n_select %d outside [0, %d]", n_select,
-                 MAX_WS);
-    TSVM_REQUIRE(n_marked >= 0 && (n_marked == 0 || marked), "tsvm_select_working_set: bad marked list");
-    if (n_select == 0) return 0;
-    hipStream_t s = tsvm_s(stream);
-    SelWorkspace w;
-    void *base = (void *) (((uintptr_t) workspace + 255) & ~(uintptr_t) 255);
-    sel_carve(base, n, &w);
-    SelGeom g;
-    g.n_sides = nu ? 4 : 2;
-    int bits = 1;
-    while (((int64_t) 1 << bits) < n) ++bits;
-    g.idx_bits = bits;
-    g.idx_mask = (uint32_t) (((uint64_t) 1 << bits) - 1);
-    g.n_pass = 6 + (bits + SEL_DIGIT - 1) / SEL_DIGIT;
-    g.k = (uint32_t) n_select;
-    const unsigned grid = (unsigned) std::min<int64_t>((n + SEL_T - 1) / SEL_T, 1024);
-    hipLaunchKernelGGL(sel_init_kernel, dim3(grid), dim3(SEL_T), 0, s, w, n, g);
-    TSVM_LAUNCH_CHECK();
-    if (n_marked > 0) {
-        hipLaunchKernelGGL(sel_mark_kernel, dim3((n_marked + 255) / 256), dim3(256), 0, s, w.ind, marked, n_marked);
-        TSVM_LAUNCH_CHECK();
-    }
-    // The first three digits (33 bits of f) are counted by the whole chip, the rest (rarely needed) by one
-    // workgroup.  Near convergence the free support vectors crowd within epsilon of the threshold, so the third
-    // digit is usually the one that separates them.
-    const int p_full = std::min(g.n_pass, n > ((int64_t) 1 << 26) ? 4 : 3);
-    for (int p = 0; p < p_full; ++p) {
-        hipLaunchKernelGGL(sel_pass_kernel, dim3(grid), dim3(SEL_T), 0, s, w, f, y, alpha, n, Cp, Cn, g, p);
-        TSVM_LAUNCH_CHECK();
-    }
-    if (p_full < g.n_pass) {
-        hipLaunchKernelGGL(sel_tail_kernel, dim3(1), dim3(SEL_TAIL_T), 0, s, w, n, g, p_full);
-        TSVM_LAUNCH_CHECK();
-    }
-    hipLaunchKernelGGL(sel_compact_kernel, dim3(grid), dim3(SEL_T), 0, s, w, n, g);
-    TSVM_LAUNCH_CHECK();
-    hipLaunchKernelGGL(sel_final_kernel, dim3(1), dim3(MAX_WS), 0, s, w, g, out);
-    TSVM_LAUNCH_CHECK();
-    return 0;
+    return select_working_set(f, y, alpha, n, Cp, Cn, marked, n_marked, out, n_select, nu, workspace, false, stream);
+}
+
+int tsvm_select_working_set_again(const double *f, const int *y, const double *alpha, int64_t n, double Cp, double Cn,
+                                  const int *marked, int n_marked, int *out, int n_select, int nu, void *workspace,
+                                  tsvm_stream stream) {
+    return select_working_set(f, y, alpha, n, Cp, Cn, marked, n_marked, out, n_select, nu, workspace, true, stream);
 }
 
 }  // extern "C"

@@ -43,6 +43,64 @@ __global__ void gather_ws_block_kernel(const TK *__restrict__ k_rows, const int 
     for (int t = threadIdx.x; t < ldk; t += blockDim.x) kws[(int64_t) r * ldk + t] = t < ws ? (double) row[working_set[t]] : 0.0;
 }
 
+// The same block when a table names the slot of every instance's row (a row cache that holds them all): row r
+// is the one of instance ids[r]; its slot is also written to slots_out[r], for update_f.
+template <typename TK>
+__global__ void gather_ws_block_by_id_kernel(const TK *__restrict__ k_rows, const int *__restrict__ slot_of_id, int64_t ld,
+                                             const int *__restrict__ ids, int ws, int ldk, double *__restrict__ kws,
+                                             int *__restrict__ slots_out) {
+    const int r = blockIdx.x;
+    const int slot = slot_of_id[ids[r]];
+    if (threadIdx.x == 0) slots_out[r] = slot;
+    const TK *row = k_rows + (int64_t) slot * ld;
+    for (int t = threadIdx.x; t < ldk; t += blockDim.x) kws[(int64_t) r * ldk + t] = t < ws ? (double) row[ids[t]] : 0.0;
+}
+
+// Slots for a working set's new rows when the row store has a slot for every instance (nothing is ever
+// evicted, so the bookkeeping needs no host): instances seen for the first time take the next free slots in the
+// order of the list.  One workgroup; ids_new are distinct.
+//   slot_of_id[i]  slot of instance i's row, -1 while it has none           (updated)
+//   state[0]       slots in use                                              (updated)
+//   state[1]       number of rows to compute for this working set            (written)
+//   miss_ids / miss_slots [0 .. state[1])  the instances to compute and where their rows go
+//   slots_ws[t]    slot of ids_ws[t], t < ws
+//   info[0..1]     state[1], state[0] for the host (pinned host memory or device memory)
+#define RA_T 1024
+__global__ __launch_bounds__(RA_T) void row_slots_assign_kernel(const int *__restrict__ ids_new, int n_new,
+                                                                int *__restrict__ slot_of_id, int *__restrict__ state,
+                                                                int *__restrict__ miss_ids, int *__restrict__ miss_slots,
+                                                                const int *__restrict__ ids_ws, int ws, int *__restrict__ slots_ws,
+                                                                int *__restrict__ info) {
+    __shared__ int wave_total[RA_T / 64];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int id = tid < n_new ? ids_new[tid] : 0;
+    const bool miss = tid < n_new && slot_of_id[id] < 0;
+    const unsigned long long b = __ballot(miss);
+    const int before = __popcll(b & ((1ull << lane) - 1ull));
+    if (lane == 0) wave_total[wave] = __popcll(b);
+    __syncthreads();
+    int rank = before, total = 0;
+    for (int w = 0; w < RA_T / 64; ++w) {
+        const int c = wave_total[w];
+        if (w < wave) rank += c;
+        total += c;
+    }
+    const int base = state[0];
+    if (miss) {
+        slot_of_id[id] = base + rank;
+        miss_ids[rank] = id;
+        miss_slots[rank] = base + rank;
+    }
+    __syncthreads();   // the table's new entries are read back below by other threads of this workgroup
+    if (tid == 0) {
+        state[0] = base + total;
+        state[1] = total;
+        info[0] = total;
+        info[1] = base + total;
+    }
+    if (tid < ws) slots_ws[tid] = slot_of_id[ids_ws[tid]];
+}
+
 // Cross-wavefront combination of the per-wavefront (value, index) minima held in LDS.
 __device__ __forceinline__ void block_argmin(const double *s_v, const int *s_i, double &v, int &i, int none) {
     double m = s_v[0];
@@ -516,6 +574,33 @@ int tsvm_smo_gather_block(const void *k_rows, int row_type, const int *slots, in
     TSVM_REQUIRE(k_rows && cols && kws, "tsvm_smo_gather_block: null pointer");
     TSVM_REQUIRE(ws_size >= 1 && ws_size <= MAX_WS, "tsvm_smo_gather_block: ws_size %d outside [1, %d]", ws_size, MAX_WS);
     return launch_gather(k_rows, row_type, slots, ld, cols, ws_size, kws, tsvm_s(stream));
+}
+
+int tsvm_smo_gather_block_by_id(const void *k_rows, int row_type, const int *slot_of_id, int64_t ld, const int *ids,
+                                int ws_size, double *kws, int *slots_out, tsvm_stream stream) {
+    TSVM_REQUIRE(k_rows && slot_of_id && ids && kws && slots_out, "tsvm_smo_gather_block_by_id: null pointer");
+    TSVM_REQUIRE(ws_size >= 1 && ws_size <= MAX_WS, "tsvm_smo_gather_block_by_id: ws_size %d outside [1, %d]", ws_size, MAX_WS);
+    TSVM_REQUIRE(row_type == TSVM_ROW_F64 || row_type == TSVM_ROW_F32, "tsvm_smo_gather_block_by_id: unknown row type %d", row_type);
+    if (row_type == TSVM_ROW_F32)
+        hipLaunchKernelGGL(gather_ws_block_by_id_kernel<float>, dim3(ws_size), dim3(256), 0, tsvm_s(stream), (const float *) k_rows,
+                           slot_of_id, ld, ids, ws_size, solver_ldk(ws_size), kws, slots_out);
+    else
+        hipLaunchKernelGGL(gather_ws_block_by_id_kernel<double>, dim3(ws_size), dim3(256), 0, tsvm_s(stream), (const double *) k_rows,
+                           slot_of_id, ld, ids, ws_size, solver_ldk(ws_size), kws, slots_out);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+int tsvm_row_slots_assign(const int *ids_new, int n_new, int *slot_of_id, int *state, int *miss_ids, int *miss_slots,
+                          const int *ids_ws, int ws_size, int *slots_ws, int *info, tsvm_stream stream) {
+    TSVM_REQUIRE(ids_new && slot_of_id && state && miss_ids && miss_slots && ids_ws && slots_ws && info,
+                 "tsvm_row_slots_assign: null pointer");
+    TSVM_REQUIRE(n_new >= 0 && n_new <= MAX_WS && ws_size >= 0 && ws_size <= MAX_WS, "tsvm_row_slots_assign: sizes %d, %d outside [0, %d]",
+                 n_new, ws_size, MAX_WS);
+    hipLaunchKernelGGL(row_slots_assign_kernel, dim3(1), dim3(RA_T), 0, tsvm_s(stream), ids_new, n_new, slot_of_id, state, miss_ids,
+                       miss_slots, ids_ws, ws_size, slots_ws, info);
+    TSVM_LAUNCH_CHECK();
+    return 0;
 }
 
 int tsvm_c_smo_solve_block(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,

@@ -1,4 +1,5 @@
 #include "kernelmatrix.h"
+#include <stdexcept>
 
 #include <algorithm>
 #include <cstdio>
@@ -202,6 +203,15 @@ void KernelMatrix::get_rows(const int *d_idx, int m, void *d_out, int64_t ld, co
     abi_check(tsvm_get_rows_csr(R.val.data(), R.col.data(), R.row_ptr.data(), nullptr, n, R.self_dot.data(), stage_.data(),
                                 m, stage_sd_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree, d_out,
                                 row_type(), d_out_slots, ld, stream));
+}
+
+void KernelMatrix::get_rows_counted(const int *d_idx, int m_max, const int *d_m, void *d_out, int64_t ld,
+                                    const int *d_out_slots, hipStream_t stream) const {
+    const DeviceRows &R = *rows_;
+    if (!R.dense) throw std::logic_error("KernelMatrix::get_rows_counted: dense layout only");
+    abi_check(tsvm_get_rows_dense_counted(R.x.data(), R.ld, nullptr, (int) n_unique_, (int) R.n_features, R.self_dot.data(),
+                                          R.x.data(), R.ld, d_idx, m_max, d_m, R.self_dot.data(), (int) param.kernel_type,
+                                          param.gamma, param.coef0, param.degree, d_out, row_type(), d_out_slots, ld, stream));
 }
 
 // K(x_idx[r], x_idx[t]) for r, t < m: the same kernels with the column set restricted to the m rows,

@@ -130,7 +130,7 @@ struct SolveTask::Impl {
     // d_slots_a holds three tables of ws entries back to back: the slot of every working-set row, then the ids and
     // the slots of the rows to compute; the host fills the same layout in h_slots and sends it with one copy.
     DeviceBuffer<int> d_y, d_ws, d_slots_a, d_slots_b, d_ws_folded;
-    DeviceBuffer<float_type> d_alpha, d_f, d_alpha_diff, d_diff;
+    DeviceBuffer<float_type> d_alpha, d_f, d_alpha_diff;
     DeviceBuffer<unsigned char> d_sel_ws;
     DeviceBuffer<kernel_type> d_kws;
     // The working set of iteration t is the window d_ws[ws_off .. ws_off + ws_size): the ids kept from the previous
@@ -167,8 +167,21 @@ struct SolveTask::Impl {
     bool caching = false;
     RowCache cache;
     std::vector<int> cur_slots, cur_ids, miss_ids, miss_slots;
+    // Once the cache holds every row the host's bookkeeping has nothing left to decide: the device gets the
+    // table id -> slot, and from then on an iteration takes its slots from it (no ids to the host, no slot
+    // table back) and gathers the solver's block from the stored rows.
+    bool all_cached = false;
+    DeviceBuffer<int> d_slot_of;
+    // A store with a slot for every instance never evicts, so which slot a new row gets can be decided on the
+    // device (next free one, tsvm_row_slots_assign) and the host hears of it afterwards, with the diff: no ids to
+    // the host and no slot table back between the selection and get_rows.  (Dense rows, unfolded problems.)
+    bool device_cache = false;
+    DeviceBuffer<int> d_cache_state;                  // slots in use, rows to compute
+    int *h_cache_info = nullptr, *d_cache_info = nullptr;   // the same two numbers in pinned host memory
     int *h_ids = nullptr, *h_slots = nullptr;
-    double *h_diff = nullptr;
+    // diff (the solver's 16 bytes for the host, smo_kernel.cpp:87,120) lives in pinned host memory that the device
+    // writes directly: no copy in the stream between update_f and the next selection
+    double *h_diff = nullptr, *d_diff = nullptr;
     int rotation_base = 0;   // iteration at which d_slots_a was valid
     long long window_lookups = 0, window_hits = 0;
     const int *slots = nullptr;
@@ -191,13 +204,12 @@ struct SolveTask::Impl {
         wall0 = std::chrono::steady_clock::now();
         d_y.resize(n); d_ws.resize((size_t) WS_HALVES * q + ws_size); d_slots_a.resize(3 * (size_t) ws_size); d_slots_b.resize(ws_size);
         if (rep > 1) d_ws_folded.resize(ws_size);
-        d_alpha.resize(n); d_f.resize(n); d_alpha_diff.resize(ws_size); d_diff.resize(2);
+        d_alpha.resize(n); d_f.resize(n); d_alpha_diff.resize(ws_size);
         d_sel_ws.resize(tsvm_select_workspace(n));
         d_kws.resize((size_t) ws_size * ldk);
         d_y.upload(y.data(), n);
         d_alpha.upload(alpha.data(), n);
         d_f.upload(f_val.data(), n);
-        d_diff.zero();
         d_alpha_diff.zero();
         d_kws.zero();
         alone = n_lanes == 1;
@@ -237,10 +249,21 @@ struct SolveTask::Impl {
         if (caching) {
             cache.init(n_u, (int) pool_rows);
             stats.cache_rows = pool_rows;
+            if ((size_t) n_u <= pool_rows) d_slot_of.resize(n_u);
+            device_cache = d_slot_of.size() == (size_t) n_u && rep == 1 && k_mat.dense_layout();
+        }
+        if (device_cache) {
+            TSVM_HIP_CHECK(hipMemset(d_slot_of.data(), 0xff, sizeof(int) * (size_t) n_u));
+            d_cache_state.resize(2);
+            d_cache_state.zero();
+            TSVM_HIP_CHECK(hipHostMalloc((void **) &h_cache_info, 2 * sizeof(int), hipHostMallocMapped | hipHostMallocCoherent));
+            TSVM_HIP_CHECK(hipHostGetDevicePointer((void **) &d_cache_info, h_cache_info, 0));
+            h_cache_info[0] = h_cache_info[1] = 0;
         }
         cur_slots.resize(ws_size);
         cur_ids.resize(ws_size);
-        TSVM_HIP_CHECK(hipHostMalloc((void **) &h_diff, 2 * sizeof(double)));
+        TSVM_HIP_CHECK(hipHostMalloc((void **) &h_diff, 2 * sizeof(double), hipHostMallocMapped | hipHostMallocCoherent));
+        TSVM_HIP_CHECK(hipHostGetDevicePointer((void **) &d_diff, h_diff, 0));
         TSVM_HIP_CHECK(hipHostMalloc((void **) &h_ids, ws_size * sizeof(int)));
         TSVM_HIP_CHECK(hipHostMalloc((void **) &h_slots, 3 * ws_size * sizeof(int)));
         h_diff[0] = h_diff[1] = 0;
@@ -284,6 +307,7 @@ struct SolveTask::Impl {
         if (ids_ready) (void) hipEventDestroy(ids_ready);
         if (diff_ready) (void) hipEventDestroy(diff_ready);
         if (h_diff) (void) hipHostFree(h_diff);
+        if (h_cache_info) (void) hipHostFree(h_cache_info);
         if (h_ids) (void) hipHostFree(h_ids);
         if (h_slots) (void) hipHostFree(h_slots);
     }
@@ -361,8 +385,8 @@ struct SolveTask::Impl {
                 next = 0;
             }
             sel_off = next;
-            abi_check(tsvm_select_working_set(d_f.data(), d_y.data(), d_alpha.data(), n, Cp, Cn, d_ws.data() + sel_off, q,
-                                              d_ws.data() + sel_off + q, q, nu, d_sel_ws.data(), sa));
+            abi_check(tsvm_select_working_set_again(d_f.data(), d_y.data(), d_alpha.data(), n, Cp, Cn, d_ws.data() + sel_off, q,
+                                                    d_ws.data() + sel_off + q, q, nu, d_sel_ws.data(), sa));
         }
         if (rep > 1) abi_check(tsvm_fold_ids(d_ws.data() + sel_off, ws_size, n_u, d_ws_folded.data(), sa));
     }
@@ -376,7 +400,7 @@ struct SolveTask::Impl {
         ws_off = sel_off;
         timer.end(stats.ms_select);
         TSVM_HIP_CHECK(hipEventRecord(selected, sa));
-        if (caching) {
+        if (caching && !all_cached && !device_cache) {
             // the new ids travel to the host, on their own stream if there is one
             if (ids != sa) TSVM_HIP_CHECK(hipStreamWaitEvent(ids, selected, 0));
             TSVM_HIP_CHECK(hipMemcpyAsync(h_ids, ws_ids() + first_new, sizeof(int) * n_new, hipMemcpyDeviceToHost, ids));
@@ -387,8 +411,20 @@ struct SolveTask::Impl {
     void enqueue_rows() {
         const int n_new = iter == 0 ? ws_size : q;
         const int first_new = iter == 0 ? 0 : q;
+        if (caching && all_cached) {
+            stats.cache_lookups += n_new;
+            stats.cache_hits += n_new;
+            last_rows_computed = 0;
+            return;
+        }
         timer.begin();
-        if (caching) {
+        if (device_cache) {
+            int *miss_ids = d_slots_a.data() + ws_size, *miss_slots = d_slots_a.data() + 2 * ws_size;
+            abi_check(tsvm_row_slots_assign(ws_u() + first_new, n_new, d_slot_of.data(), d_cache_state.data(), miss_ids, miss_slots,
+                                            ws_u(), ws_size, d_slots_a.data(), d_cache_info, sa));
+            k_mat.get_rows_counted(miss_ids, n_new, d_cache_state.data() + 1, k_rows, ld, miss_slots, sa);
+            slots = d_slots_a.data();
+        } else if (caching) {
             // look the new ids up and compute only the rows that are not cached
             TSVM_HIP_CHECK(hipEventSynchronize(ids_ready));
             if (iter > 0) {
@@ -425,6 +461,11 @@ struct SolveTask::Impl {
                 k_mat.get_rows(d_slots_a.data() + ws_size, n_miss, k_rows, ld, d_slots_a.data() + 2 * ws_size, sa);
             }
             slots = d_slots_a.data();
+            if (cache.used == n_u && d_slot_of.size() == (size_t) n_u) {
+                TSVM_HIP_CHECK(hipMemcpyAsync(d_slot_of.data(), cache.slot_of.data(), sizeof(int) * (size_t) n_u,
+                                              hipMemcpyHostToDevice, sa));
+                all_cached = true;
+            }
             // A cache that has started evicting and still does not hit only costs the id read-back:
             // every 64 iterations, if fewer than 5 % of the window's lookups hit, fall back to rotation.
             // (A cache that can hold every row is never switched off: its misses are first touches.)
@@ -451,17 +492,21 @@ struct SolveTask::Impl {
 
     void enqueue_block() {
         timer.begin();
-        on_one_stream = !split || (alone && caching && cache.used == n_u);
+        on_one_stream = !split || (alone && all_cached);
         // (Dense rows only: the CSR block takes too long on eight CUs.  Both launches are matrix-core work with the
         // same cost per value; the block plus the solver's ~0.4 ms has to fit into the time of the rows.)
         block_on_solver_cus = false;
-        if (!on_one_stream && alone && block_first && k_mat.dense_layout()) {
+        if (!on_one_stream && alone && block_first && k_mat.dense_layout() && !all_cached) {
             const double per_value = 2.0 * ((k_mat.n_features() + 15) / 16 * 16) / 6.6e13;   // seconds on the whole chip
             const double t_block = per_value * 32.0 * ws_size * (double) ws_size;           // on 8 of 256 CUs
             const double t_rows = per_value * (double) last_rows_computed * n_u;
             block_on_solver_cus = t_block + 0.4e-3 <= t_rows;
         }
-        if (block_on_solver_cus) {
+        if (caching && all_cached) {
+            abi_check(tsvm_smo_gather_block_by_id(k_rows, row_type, d_slot_of.data(), ld, ws_u(), ws_size, d_kws.data(),
+                                                  d_slots_a.data(), sa));
+            slots = d_slots_a.data();
+        } else if (block_on_solver_cus) {
             TSVM_HIP_CHECK(hipStreamWaitEvent(ss, selected, 0));
             k_mat.get_block(ws_u(), ws_size, d_kws.data(), ldk, ss);
         } else if (block_first) {
@@ -479,10 +524,10 @@ struct SolveTask::Impl {
         if (!on_one_stream && !block_on_solver_cus) TSVM_HIP_CHECK(hipStreamWaitEvent(ss, block_done, 0));
         if (nu) {
             abi_check(tsvm_nu_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), ws_ids(), ws_size,
-                                              Cp, d_kws.data(), k_mat.diag(), eps, d_diff.data(), max_iter, st));
+                                              Cp, d_kws.data(), k_mat.diag(), eps, d_diff, max_iter, st));
         } else {
             abi_check(tsvm_c_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), ws_ids(), ws_size,
-                                             Cp, Cn, d_kws.data(), k_mat.diag(), eps, d_diff.data(), max_iter, st));
+                                             Cp, Cn, d_kws.data(), k_mat.diag(), eps, d_diff, max_iter, st));
         }
         timer.end(stats.ms_local);
         if (!on_one_stream) TSVM_HIP_CHECK(hipEventRecord(solved, ss));
@@ -493,7 +538,6 @@ struct SolveTask::Impl {
         timer.begin();
         abi_check(tsvm_update_f(d_f.data(), d_alpha_diff.data(), ws_size, k_rows, row_type, slots, ld, n_u, rep, sa));
         timer.end(stats.ms_update_f);
-        TSVM_HIP_CHECK(hipMemcpyAsync(h_diff, d_diff.data(), 2 * sizeof(double), hipMemcpyDeviceToHost, sa));
         TSVM_HIP_CHECK(hipEventRecord(diff_ready, sa));
         if (select_ahead) {
             launch_select(iter + 1);
@@ -505,6 +549,13 @@ struct SolveTask::Impl {
         TSVM_HIP_CHECK(hipEventSynchronize(diff_ready));
         const double diff0 = h_diff[0], diff1 = h_diff[1];
         local_iter += (long long) diff1;
+        if (device_cache && !all_cached) {
+            const int n_new = iter == 0 ? ws_size : q, n_miss = h_cache_info[0];
+            stats.cache_lookups += n_new;
+            stats.cache_hits += n_new - n_miss;
+            last_rows_computed = n_miss;
+            all_cached = h_cache_info[1] == n_u;
+        }
         SolverTrace *trace = solver.trace;
         if (trace && iter < trace->cap_iters) {
             trace->diff.push_back(diff0);
