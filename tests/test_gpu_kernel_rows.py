@@ -298,3 +298,61 @@ def test_dense_rbf_many_columns_few_features(n, d, m):
     got32 = G.host(G.get_rows_dense(x_d, ld, n, nf, sd, x_d, ld, idx_d, m, sd, O.RBF, row_type=capi.ROW_F32,
                                     out_slots=G.dev(slots), out_rows=m + 9, **prm))
     assert np.array_equal(got32[slots].astype(np.float64), want)
+
+
+@pytest.mark.parametrize("n,d,ws", [(300, 20, 64), (5000, 54, 1024), (2600, 200, 1024)])
+def test_row_store_managed_on_the_device(n, d, ws):
+    """A row store with a slot for every instance, run the way the solver runs it: tsvm_row_slots_assign decides the
+    slots of a working set's new rows, tsvm_get_rows_dense_counted computes exactly those rows into their slots
+    (the count stays on the device), tsvm_smo_gather_block_by_id reads the solver's block out of the store.
+    Checked against a host-side replay of the bookkeeping, rows from tsvm_get_rows_dense, and the block gathered
+    from those rows."""
+    rng = np.random.default_rng(n + d)
+    data = from_dense(rng.standard_normal((n, d)).astype(np.float32).astype(np.float64))
+    kt, prm = O.RBF, dict(gamma=0.5)
+    x_d, nf, ld, sd, _ = _device_km(data, kt, prm)
+    ldo = G.round_up(n, 8)
+    all_rows = G.host(G.get_rows_dense(x_d, ld, n, nf, sd, x_d, ld, None, n, sd, kt, row_type=capi.ROW_F32, **prm))
+    store = torch.full((n, ldo), -5.0, dtype=torch.float32, device="cuda")
+    slot_of = torch.full((n,), -1, dtype=torch.int32, device="cuda")
+    state = torch.zeros(2, dtype=torch.int32, device="cuda")
+    info = torch.zeros(2, dtype=torch.int32, device="cuda")
+    miss_ids = torch.full((ws,), -9, dtype=torch.int32, device="cuda")      # stale entries must never be read
+    miss_slots = torch.full((ws,), -9, dtype=torch.int32, device="cuda")
+    slots_ws = torch.zeros(ws, dtype=torch.int32, device="cuda")
+    ldk = capi.kernel_lib().tsvm_smo_solve_block_ld(ws)
+    q = ws // 2
+    h_slot_of, used = np.full(n, -1), 0
+    ws_ids = rng.permutation(n)[:ws].astype(np.int32)
+    for it in range(4 * n // q + 3):
+        if it > 0:   # keep the second half, add q ids that are not in the set: half of them new to the store while any are
+            rest = rng.permutation(np.setdiff1d(np.arange(n), ws_ids[q:]))
+            unseen = rest[h_slot_of[rest] < 0][:q // 2]
+            add = np.concatenate([unseen, np.setdiff1d(rest, unseen, assume_unique=True)[:q - len(unseen)]])
+            ws_ids = np.concatenate([ws_ids[q:], rng.permutation(add)]).astype(np.int32)
+        first_new, n_new = (0, ws) if it == 0 else (q, q)
+        new = ws_ids[first_new:]
+        want_miss = [int(i) for i in new if h_slot_of[i] < 0]
+        for i in want_miss:
+            h_slot_of[i] = used
+            used += 1
+        ids_d = G.dev(ws_ids)
+        capi.call("tsvm_row_slots_assign", G.ptr(ids_d) + 4 * first_new, n_new, G.ptr(slot_of), G.ptr(state), G.ptr(miss_ids),
+                  G.ptr(miss_slots), G.ptr(ids_d), ws, G.ptr(slots_ws), G.ptr(info), G.stream())
+        capi.call("tsvm_get_rows_dense_counted", G.ptr(x_d), ld, None, n, nf, G.ptr(sd), G.ptr(x_d), ld, G.ptr(miss_ids), n_new,
+                  G.ptr(state) + 4, G.ptr(sd), kt, prm["gamma"], 0.0, 3, G.ptr(store), capi.ROW_F32, G.ptr(miss_slots), ldo,
+                  G.stream())
+        assert G.host(state).tolist() == [used, len(want_miss)] and G.host(info).tolist() == [len(want_miss), used]
+        assert G.host(miss_ids)[:len(want_miss)].tolist() == want_miss
+        assert np.array_equal(G.host(slot_of), h_slot_of)
+        assert np.array_equal(G.host(slots_ws), h_slot_of[ws_ids])
+        kws = torch.full((ws, ldk), 3.0, dtype=torch.float64, device="cuda")
+        out_slots = torch.zeros(ws, dtype=torch.int32, device="cuda")
+        capi.call("tsvm_smo_gather_block_by_id", G.ptr(store), capi.ROW_F32, G.ptr(slot_of), ldo, G.ptr(ids_d), ws, G.ptr(kws),
+                  G.ptr(out_slots), G.stream())
+        got = G.host(kws)
+        assert np.array_equal(got[:, :ws], all_rows[np.ix_(ws_ids, ws_ids)].astype(np.float64)) and (got[:, ws:] == 0).all()
+        assert np.array_equal(G.host(out_slots), h_slot_of[ws_ids])
+    assert used == n                                       # every instance has been seen: the store is complete
+    st = G.host(store)
+    assert np.array_equal(st[h_slot_of][:, :n], all_rows)  # each row computed into its slot, nothing else touched
