@@ -99,4 +99,29 @@ private:
     size_t count_ = 0;
 };
 
+// Page-locked host staging memory that only grows (hipHostMalloc; copies from it are asynchronous and run at
+// the link's rate).
+template <typename T>
+class PinnedBuffer {
+public:
+    PinnedBuffer() = default;
+    PinnedBuffer(const PinnedBuffer &) = delete;
+    PinnedBuffer &operator=(const PinnedBuffer &) = delete;
+    ~PinnedBuffer() { if (ptr_) (void) hipHostFree(ptr_); }
+    void reserve(size_t count) {
+        if (count <= count_) return;
+        if (ptr_) (void) hipHostFree(ptr_);
+        ptr_ = nullptr;
+        count_ = 0;
+        TSVM_HIP_CHECK(hipHostMalloc((void **) &ptr_, count * sizeof(T)));
+        count_ = count;
+    }
+    T *data() { return ptr_; }
+    size_t size() const { return count_; }
+
+private:
+    T *ptr_ = nullptr;
+    size_t count_ = 0;
+};
+
 }  // namespace tsvm

@@ -237,24 +237,36 @@ void KernelMatrix::get_block(const int *d_idx, int m, kernel_type *d_out, int64_
 // External batch (kernelmatrix.cpp:281-312, 385-406): features with id >= R.n_features are left out of
 // the dot product but stay in the batch row's self dot.
 void KernelMatrix::get_rows(const DataSet::node2d &instances, void *d_out, int64_t ld) const {
+    get_rows(instances.data(), instances.size(), d_out, ld);
+}
+
+void KernelMatrix::get_rows(const std::vector<DataSet::node> *instances, size_t n_rows, void *d_out, int64_t ld) const {
     const DeviceRows &R = *rows_;
-    const int m = (int) instances.size();
+    const int m = (int) n_rows;
     if (m == 0) return;
-    std::vector<int64_t> ptr(m + 1, 0);
-    size_t total = 0;
-    for (const auto &row : instances) total += row.size();
-    std::vector<kernel_type> val(total);
-    std::vector<int> col(total);
-    size_t e = 0;
+    // The batch goes to the device as CSR: flattened by all cores into pinned memory, copied asynchronously.
+    TSVM_HIP_CHECK(hipStreamSynchronize(nullptr));   // a previous batch's copies have left the staging memory
+    h_ptr_.reserve((size_t) m + 1);
+    int64_t *ptr = h_ptr_.data();
+    ptr[0] = 0;
+    for (int r = 0; r < m; ++r) ptr[r + 1] = ptr[r] + (int64_t) instances[r].size();
+    const size_t total = (size_t) ptr[m];
+    h_val_.reserve(total);
+    h_col_.reserve(total);
+    kernel_type *val = h_val_.data();
+    int *col = h_col_.data();
+#pragma omp parallel for schedule(static)
     for (int r = 0; r < m; ++r) {
+        size_t e = (size_t) ptr[r];
         for (const auto &nd : instances[r]) { val[e] = nd.value; col[e] = nd.index; ++e; }
-        ptr[r + 1] = (int64_t) e;
     }
     if (b_val_.size() < total) { b_val_.resize(total); b_col_.resize(total); }
     if (b_ptr_.size() < (size_t) m + 1) b_ptr_.resize(m + 1);
-    b_val_.upload(val.data(), total);
-    b_col_.upload(col.data(), total);
-    b_ptr_.upload(ptr.data(), m + 1);
+    if (total) {
+        TSVM_HIP_CHECK(hipMemcpyAsync(b_val_.data(), val, total * sizeof(kernel_type), hipMemcpyHostToDevice, nullptr));
+        TSVM_HIP_CHECK(hipMemcpyAsync(b_col_.data(), col, total * sizeof(int), hipMemcpyHostToDevice, nullptr));
+    }
+    TSVM_HIP_CHECK(hipMemcpyAsync(b_ptr_.data(), ptr, ((size_t) m + 1) * sizeof(int64_t), hipMemcpyHostToDevice, nullptr));
     if (stage_sd_.size() < (size_t) m) stage_sd_.resize(m);
     abi_check(tsvm_csr_self_dot(b_val_.data(), b_ptr_.data(), m, stage_sd_.data(), nullptr));
     const int n = (int) n_unique_;

@@ -62,6 +62,7 @@ public:
     void get_block(const int *d_idx, int m, kernel_type *d_out, int64_t ld, hipStream_t stream = nullptr) const;
     // kernel rows of an external batch -> element i*ld + j of d_out (row_type() elements)
     void get_rows(const DataSet::node2d &instances, void *d_out, int64_t ld) const;
+    void get_rows(const std::vector<DataSet::node> *instances, size_t m, void *d_out, int64_t ld) const;   // the same for a slice
 
     const kernel_type *diag() const { return diag_.data(); }          // device, n_instances() entries
     const kernel_type *self_dot() const { return rows_->self_dot.data(); }  // device, n_columns() entries
@@ -92,4 +93,7 @@ private:
     mutable tsvm::DeviceBuffer<kernel_type> b_val_;
     mutable tsvm::DeviceBuffer<int> b_col_;
     mutable tsvm::DeviceBuffer<int64_t> b_ptr_;
+    mutable tsvm::PinnedBuffer<kernel_type> h_val_;   // host side of the batch staging
+    mutable tsvm::PinnedBuffer<int> h_col_;
+    mutable tsvm::PinnedBuffer<int64_t> h_ptr_;
 };

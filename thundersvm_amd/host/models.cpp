@@ -113,8 +113,7 @@ void SvmModel::predict_dec_values(const DataSet::node2d &instances, std::vector<
     DeviceBuffer<float_type> d_dec(bmax * n_binary_models);
     for (size_t b0 = 0; b0 < instances.size(); b0 += batch_size) {
         const size_t bm = std::min((size_t) batch_size, instances.size() - b0);
-        DataSet::node2d batch(instances.begin() + b0, instances.begin() + b0 + bm);
-        k_mat.get_rows(batch, d_k, (int64_t) T);
+        k_mat.get_rows(instances.data() + b0, bm, d_k, (int64_t) T);
         abi_check(tsvm_sum_kernel_values(d_coef.data(), (int) T, d_start.data(), d_count.data(), d_rho.data(), d_k,
                                          k_mat.row_type(), (int64_t) T, d_dec.data(), n_classes, (int64_t) bm, nullptr));
         d_dec.download(dec.data() + b0 * n_binary_models, bm * n_binary_models);
