@@ -182,6 +182,31 @@ struct SolveTask::Impl {
     // diff (the solver's 16 bytes for the host, smo_kernel.cpp:87,120) lives in pinned host memory that the device
     // writes directly: no copy in the stream between update_f and the next selection
     double *h_diff = nullptr, *d_diff = nullptr;
+    // The host does not wait for an event behind update_f (a marker in the stream costs the device about 6 us
+    // before the next kernel starts): it marks the word the solver writes last as pending before it enqueues the
+    // solver (diff[1] for c_smo_solve; nu_smo_solve writes diff[0] only, smo_kernel.cpp:283), and waits for that
+    // word to change.  Everything the host enqueues meanwhile is ordered by the streams.
+    static constexpr uint64_t DIFF_PENDING = 0x7ff8dead00000001ull;   // a NaN no computation produces
+    bool wait_by_event = false;
+    hipStream_t solver_stream = nullptr;
+    volatile uint64_t *diff_word() const { return reinterpret_cast<volatile uint64_t *>(h_diff + (nu ? 0 : 1)); }
+    void wait_for_diff() {
+        volatile uint64_t *w = diff_word();
+        // (asking the runtime about the stream puts a marker into it: only done when the wait is suspiciously long)
+        auto next_check = std::chrono::steady_clock::now() + std::chrono::milliseconds(200);
+        for (unsigned long long spins = 1; *w == DIFF_PENDING; ++spins) {
+            if (spins % 4096 == 0 && std::chrono::steady_clock::now() > next_check) {
+                next_check = std::chrono::steady_clock::now() + std::chrono::milliseconds(200);
+                const hipError_t e = hipStreamQuery(solver_stream);
+                if (e == hipSuccess) {   // the solver has run: its write is on its way or it never made one
+                    if (*w == DIFF_PENDING) throw std::runtime_error("SolveTask: the local solver finished without reporting");
+                } else if (e != hipErrorNotReady) {
+                    TSVM_HIP_CHECK(e);
+                }
+            }
+        }
+        __atomic_thread_fence(__ATOMIC_ACQUIRE);
+    }
     int rotation_base = 0;   // iteration at which d_slots_a was valid
     long long window_lookups = 0, window_hits = 0;
     const int *slots = nullptr;
@@ -276,6 +301,7 @@ struct SolveTask::Impl {
 
         max_iter = std::max(100000, ws_size > INT_MAX / 100 ? INT_MAX : 100 * ws_size);
         timer.stream = sa;
+        wait_by_event = timer.on;   // phase timing reads its own events after every phase anyway
         if (solver.trace) {
             solver.trace->ws_size = ws_size;
             solver.trace->diff.clear();
@@ -399,7 +425,6 @@ struct SolveTask::Impl {
         select_enqueued = false;
         ws_off = sel_off;
         timer.end(stats.ms_select);
-        TSVM_HIP_CHECK(hipEventRecord(selected, sa));
         if (caching && !all_cached && !device_cache) {
             // the new ids travel to the host, on their own stream if there is one
             if (ids != sa) TSVM_HIP_CHECK(hipStreamWaitEvent(ids, selected, 0));
@@ -507,6 +532,7 @@ struct SolveTask::Impl {
                                                   d_slots_a.data(), sa));
             slots = d_slots_a.data();
         } else if (block_on_solver_cus) {
+            TSVM_HIP_CHECK(hipEventRecord(selected, sa));   // the selection is the last thing enqueued on sa
             TSVM_HIP_CHECK(hipStreamWaitEvent(ss, selected, 0));
             k_mat.get_block(ws_u(), ws_size, d_kws.data(), ldk, ss);
         } else if (block_first) {
@@ -521,6 +547,11 @@ struct SolveTask::Impl {
     void enqueue_solver() {
         timer.begin();
         hipStream_t st = on_one_stream ? sa : ss;
+        solver_stream = st;
+        if (!wait_by_event) {
+            *diff_word() = DIFF_PENDING;
+            __atomic_thread_fence(__ATOMIC_RELEASE);
+        }
         if (!on_one_stream && !block_on_solver_cus) TSVM_HIP_CHECK(hipStreamWaitEvent(ss, block_done, 0));
         if (nu) {
             abi_check(tsvm_nu_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), ws_ids(), ws_size,
@@ -538,7 +569,7 @@ struct SolveTask::Impl {
         timer.begin();
         abi_check(tsvm_update_f(d_f.data(), d_alpha_diff.data(), ws_size, k_rows, row_type, slots, ld, n_u, rep, sa));
         timer.end(stats.ms_update_f);
-        TSVM_HIP_CHECK(hipEventRecord(diff_ready, sa));
+        if (wait_by_event) TSVM_HIP_CHECK(hipEventRecord(diff_ready, sa));
         if (select_ahead) {
             launch_select(iter + 1);
             select_enqueued = true;
@@ -546,14 +577,15 @@ struct SolveTask::Impl {
     }
 
     bool finish_iteration() {
-        TSVM_HIP_CHECK(hipEventSynchronize(diff_ready));
+        if (wait_by_event) TSVM_HIP_CHECK(hipEventSynchronize(diff_ready));
+        else wait_for_diff();
         const double diff0 = h_diff[0], diff1 = h_diff[1];
         local_iter += (long long) diff1;
         if (device_cache && !all_cached) {
-            const int n_new = iter == 0 ? ws_size : q, n_miss = h_cache_info[0];
-            stats.cache_lookups += n_new;
-            stats.cache_hits += n_new - n_miss;
-            last_rows_computed = n_miss;
+            // (the two numbers may still be the previous iteration's: the slots are assigned after the solver was
+            // enqueued; they only steer the schedule, and the hit count is made exact at the end)
+            stats.cache_lookups += iter == 0 ? ws_size : q;
+            last_rows_computed = h_cache_info[0];
             all_cached = h_cache_info[1] == n_u;
         }
         SolverTrace *trace = solver.trace;
@@ -579,6 +611,7 @@ struct SolveTask::Impl {
         const bool stalled = (same_local_diff_cnt >= 10 || swap_local_diff_cnt >= 10) && fabs(diff0 - 2.0) > eps;
         if (stalled || diff0 < eps || (out_max_iter != -1 && iter == out_max_iter)) {
             TSVM_HIP_CHECK(hipStreamSynchronize(sa));   // a selection enqueued ahead may still be running
+            if (device_cache) stats.cache_hits = stats.cache_lookups - h_cache_info[1];   // every slot in use was one miss
             d_alpha.download(alpha.data(), n);
             d_f.download(f_val.data(), n);
             rho = solver.calculate_rho(f_val, y, alpha, Cp, Cn);
