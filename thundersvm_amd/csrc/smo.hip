@@ -656,7 +656,9 @@ static int select_working_set(const double *f, const int *y, const double *alpha
     // workgroup.  Near convergence the free support vectors crowd within epsilon of the threshold, so the third
     // digit is usually the one that separates them.
     const int p_full = n > ((int64_t) 1 << 26) ? 4 : 3;   // < n_pass, which is at least 7
-    unsigned grid = (unsigned) std::min<int64_t>((n + SEL_T - 1) / SEL_T, 1024);
+    // two workgroups per CU: every workgroup adds its histogram to the global one with atomics, and with more
+    // workgroups those take longer than the counting they spread (n = 800k: 92 us per call with 1024, 80 with 496)
+    unsigned grid = (unsigned) std::min<int64_t>((n + SEL_T - 1) / SEL_T, 496);
     if ((n + grid - 1) / grid > SEL_CHUNK_MAX) grid = (unsigned) ((n + SEL_CHUNK_MAX - 1) / SEL_CHUNK_MAX);
     if (!armed) {
         hipLaunchKernelGGL(sel_init_kernel, dim3(p_full * SEL_MAX_SIDES * SEL_BINS / 1024), dim3(256), 0, s, w, g, p_full);
