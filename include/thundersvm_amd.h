@@ -95,6 +95,12 @@ int tsvm_get_rows_dense_counted(const double *x, int64_t ldx, const int *x_idx, 
 int tsvm_csr_stage_rows(const double *val, const int *col, const int64_t *row_ptr, const int *idx, int m,
                         int n_features, double *w, tsvm_stream stream);
 
+/* The scatter of tsvm_csr_stage_rows without the zero fill, for a staging matrix that is kept all-zero between
+ * uses: clear == 0 writes the rows' values, clear != 0 writes 0.0 to the same places (after the matrix has been
+ * used).  Touches nnz entries instead of n_features x m. */
+int tsvm_csr_scatter_rows(const double *val, const int *col, const int64_t *row_ptr, const int *idx, int m,
+                          int n_features, double *w, int clear, tsvm_stream stream);
+
 /* CSR get_rows: out[s_i*ldo + j] = kappa(w_i, x_j) (s_i as above) with x in CSR (n rows) and the m working rows
  * staged by tsvm_csr_stage_rows.  Accumulates over the stored order of row j's non-zeros
  * (dns_csr_mul, kernelmatrix_kernel.cpp:149-160) and applies the epilogue.  sd_w[i] are the

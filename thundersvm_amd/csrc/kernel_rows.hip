@@ -227,9 +227,9 @@ __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
 // One workgroup = 256 working rows i (one per thread) x 16 consecutive rows j; the 16 dot products
 // live in registers and each thread stores its 16 results as one 128-byte run of output row i.
 // ------------------------------------------------------------------------------------------------
-#define CS_JB 16
-
-template <typename TO>
+// (JB = 16 stored rows per workgroup; 4 when there are only a few thousand of them, as for the solver's ws x ws
+// block, so that the grid still covers the chip and a workgroup's chain of dependent loads is a quarter as long)
+template <typename TO, int CS_JB>
 __global__ __launch_bounds__(256) void get_rows_csr_kernel(
     const double *__restrict__ val, const int *__restrict__ col, const int64_t *__restrict__ row_ptr,
     const int *__restrict__ x_idx, int64_t n, const double *__restrict__ sd_x, const double *__restrict__ w, int m,
@@ -306,17 +306,18 @@ __global__ void fill_f64_kernel(double *p, int64_t count, double v) {
         p[e] = v;
 }
 
-// w[c*m + i] = value of feature c in CSR row idx[i]; one wavefront per staged row.
+// w[c*m + i] = value of feature c in CSR row idx[i] (clear: 0.0 instead, which takes the rows out of a staging
+// matrix again); one wavefront per staged row.
 __global__ void csr_stage_rows_kernel(const double *__restrict__ val, const int *__restrict__ col,
                                       const int64_t *__restrict__ row_ptr, const int *__restrict__ idx, int m,
-                                      int n_features, double *__restrict__ w) {
+                                      int n_features, double *__restrict__ w, int clear) {
     const int i = (int) ((blockIdx.x * (int64_t) blockDim.x + threadIdx.x) >> 6);
     const int lane = threadIdx.x & 63;
     if (i >= m) return;
     const int64_t r = idx ? (int64_t) idx[i] : (int64_t) i;
     for (int64_t e = row_ptr[r] + lane; e < row_ptr[r + 1]; e += 64) {
         const int c = col[e];
-        if (c < n_features) w[(int64_t) c * m + i] = val[e];
+        if (c < n_features) w[(int64_t) c * m + i] = clear ? 0.0 : val[e];
     }
 }
 
@@ -572,7 +573,17 @@ int tsvm_csr_stage_rows(const double *val, const int *col, const int64_t *row_pt
     hipLaunchKernelGGL(fill_f64_kernel, dim3(2048), dim3(256), 0, tsvm_s(stream), w, (int64_t) m * n_features, 0.0);
     TSVM_LAUNCH_CHECK();
     hipLaunchKernelGGL(csr_stage_rows_kernel, dim3(grid_for((int64_t) m * 64, 256)), dim3(256), 0, tsvm_s(stream), val, col,
-                       row_ptr, idx, m, n_features, w);
+                       row_ptr, idx, m, n_features, w, 0);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+int tsvm_csr_scatter_rows(const double *val, const int *col, const int64_t *row_ptr, const int *idx, int m,
+                          int n_features, double *w, int clear, tsvm_stream stream) {
+    TSVM_REQUIRE(row_ptr && w && m >= 0 && n_features >= 0, "tsvm_csr_scatter_rows: bad argument");
+    if (m == 0 || n_features == 0) return 0;
+    hipLaunchKernelGGL(csr_stage_rows_kernel, dim3(grid_for((int64_t) m * 64, 256)), dim3(256), 0, tsvm_s(stream), val, col,
+                       row_ptr, idx, m, n_features, w, clear);
     TSVM_LAUNCH_CHECK();
     return 0;
 }
@@ -590,14 +601,19 @@ int tsvm_get_rows_csr(const double *val, const int *col, const int64_t *row_ptr,
     if (n == 0 || m == 0) return 0;
     KernelParam kp{kernel_type, degree, gamma, coef0};
     const unsigned i_blocks = (unsigned) ((m + 255) / 256);
-    const int64_t j_blocks = (n + CS_JB - 1) / CS_JB;
+    const int jb = n <= 4096 ? 4 : 16;
+    const int64_t j_blocks = (n + jb - 1) / jb;
     TSVM_REQUIRE(j_blocks * i_blocks < (int64_t) 0x7fffffff, "tsvm_get_rows_csr: grid too large");
-    if (row_type == TSVM_ROW_F32)
-        hipLaunchKernelGGL(get_rows_csr_kernel<float>, dim3((unsigned) (j_blocks * i_blocks)), dim3(256), 0, tsvm_s(stream), val,
-                           col, row_ptr, x_idx, n, sd_x, w, m, sd_w, kp, (float *) out, out_slots, ldo, i_blocks);
-    else
-        hipLaunchKernelGGL(get_rows_csr_kernel<double>, dim3((unsigned) (j_blocks * i_blocks)), dim3(256), 0, tsvm_s(stream), val,
-                           col, row_ptr, x_idx, n, sd_x, w, m, sd_w, kp, (double *) out, out_slots, ldo, i_blocks);
+    const dim3 grid((unsigned) (j_blocks * i_blocks));
+#define CSR_LAUNCH(TO, JB)                                                                                                   \
+    hipLaunchKernelGGL((get_rows_csr_kernel<TO, JB>), grid, dim3(256), 0, tsvm_s(stream), val, col, row_ptr, x_idx, n, sd_x, w, m, \
+                       sd_w, kp, (TO *) out, out_slots, ldo, i_blocks)
+    if (row_type == TSVM_ROW_F32) {
+        if (jb == 4) CSR_LAUNCH(float, 4); else CSR_LAUNCH(float, 16);
+    } else {
+        if (jb == 4) CSR_LAUNCH(double, 4); else CSR_LAUNCH(double, 16);
+    }
+#undef CSR_LAUNCH
     TSVM_LAUNCH_CHECK();
     return 0;
 }

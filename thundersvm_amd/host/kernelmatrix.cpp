@@ -185,6 +185,13 @@ void KernelMatrix::finish(int repeat) {
     TSVM_HIP_CHECK(hipDeviceSynchronize());
 }
 
+// A staging buffer that is all-zero whenever it is not in use: grown (and cleared) only when a call needs more.
+static void grow_zeroed(tsvm::DeviceBuffer<kernel_type> &b, size_t count, hipStream_t stream) {
+    if (b.size() >= count) return;
+    b.resize(count);
+    TSVM_HIP_CHECK(hipMemsetAsync(b.data(), 0, count * sizeof(kernel_type), stream));
+}
+
 void KernelMatrix::get_rows(const int *d_idx, int m, void *d_out, int64_t ld, const int *d_out_slots,
                             hipStream_t stream) const {
     const DeviceRows &R = *rows_;
@@ -195,14 +202,18 @@ void KernelMatrix::get_rows(const int *d_idx, int m, void *d_out, int64_t ld, co
                                       d_out, row_type(), d_out_slots, ld, stream));
         return;
     }
-    if (stage_.size() < (size_t) m * R.n_features) stage_.resize((size_t) m * R.n_features);
+    // The staging matrix [n_features][m] is kept all-zero between uses: the working rows' non-zeros are written
+    // into it and taken out again afterwards (nnz entries each way instead of a fill of n_features x m).
+    grow_zeroed(stage_w_, (size_t) m * R.n_features, stream);
     if (stage_sd_.size() < (size_t) m) stage_sd_.resize(m);
-    abi_check(tsvm_csr_stage_rows(R.val.data(), R.col.data(), R.row_ptr.data(), d_idx, m, (int) R.n_features,
-                                  stage_.data(), stream));
+    abi_check(tsvm_csr_scatter_rows(R.val.data(), R.col.data(), R.row_ptr.data(), d_idx, m, (int) R.n_features,
+                                    stage_w_.data(), 0, stream));
     abi_check(tsvm_gather_f64(R.self_dot.data(), d_idx, m, stage_sd_.data(), stream));
-    abi_check(tsvm_get_rows_csr(R.val.data(), R.col.data(), R.row_ptr.data(), nullptr, n, R.self_dot.data(), stage_.data(),
+    abi_check(tsvm_get_rows_csr(R.val.data(), R.col.data(), R.row_ptr.data(), nullptr, n, R.self_dot.data(), stage_w_.data(),
                                 m, stage_sd_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree, d_out,
                                 row_type(), d_out_slots, ld, stream));
+    abi_check(tsvm_csr_scatter_rows(R.val.data(), R.col.data(), R.row_ptr.data(), d_idx, m, (int) R.n_features,
+                                    stage_w_.data(), 1, stream));
 }
 
 void KernelMatrix::get_rows_counted(const int *d_idx, int m_max, const int *d_m, void *d_out, int64_t ld,
@@ -224,14 +235,16 @@ void KernelMatrix::get_block(const int *d_idx, int m, kernel_type *d_out, int64_
                                       d_out, TSVM_ROW_F64, nullptr, ld, stream));
         return;
     }
-    if (stage_blk_.size() < (size_t) m * R.n_features) stage_blk_.resize((size_t) m * R.n_features);
+    grow_zeroed(stage_blk_, (size_t) m * R.n_features, stream);   // kept all-zero between uses, as in get_rows
     if (stage_blk_sd_.size() < (size_t) m) stage_blk_sd_.resize(m);
-    abi_check(tsvm_csr_stage_rows(R.val.data(), R.col.data(), R.row_ptr.data(), d_idx, m, (int) R.n_features,
-                                  stage_blk_.data(), stream));
+    abi_check(tsvm_csr_scatter_rows(R.val.data(), R.col.data(), R.row_ptr.data(), d_idx, m, (int) R.n_features,
+                                    stage_blk_.data(), 0, stream));
     abi_check(tsvm_gather_f64(R.self_dot.data(), d_idx, m, stage_blk_sd_.data(), stream));
     abi_check(tsvm_get_rows_csr(R.val.data(), R.col.data(), R.row_ptr.data(), d_idx, m, R.self_dot.data(), stage_blk_.data(),
                                 m, stage_blk_sd_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
                                 d_out, TSVM_ROW_F64, nullptr, ld, stream));
+    abi_check(tsvm_csr_scatter_rows(R.val.data(), R.col.data(), R.row_ptr.data(), d_idx, m, (int) R.n_features,
+                                    stage_blk_.data(), 1, stream));
 }
 
 // External batch (kernelmatrix.cpp:281-312, 385-406): features with id >= R.n_features are left out of

@@ -88,6 +88,7 @@ private:
     tsvm::DeviceBuffer<kernel_type> diag_;
     // reusable staging for the sparse path and for external batches
     mutable tsvm::DeviceBuffer<kernel_type> stage_;
+    mutable tsvm::DeviceBuffer<kernel_type> stage_w_;   // transposed staging of CSR working rows, all-zero between uses
     mutable tsvm::DeviceBuffer<kernel_type> stage_blk_, stage_blk_sd_;   // staging of get_block (its own stream)
     mutable tsvm::DeviceBuffer<kernel_type> stage_sd_;
     mutable tsvm::DeviceBuffer<kernel_type> b_val_;
