@@ -97,9 +97,18 @@ int tsvm_csr_stage_rows(const double *val, const int *col, const int64_t *row_pt
 
 /* The scatter of tsvm_csr_stage_rows without the zero fill, for a staging matrix that is kept all-zero between
  * uses: clear == 0 writes the rows' values, clear != 0 writes 0.0 to the same places (after the matrix has been
- * used).  Touches nnz entries instead of n_features x m. */
+ * used).  Touches nnz entries instead of n_features x m.  w holds w_type elements (TSVM_ROW_F64 / TSVM_ROW_F32). */
 int tsvm_csr_scatter_rows(const double *val, const int *col, const int64_t *row_ptr, const int *idx, int m,
-                          int n_features, double *w, int clear, tsvm_stream stream);
+                          int n_features, void *w, int w_type, int clear, tsvm_stream stream);
+
+/* tsvm_get_rows_csr with the staged working rows held as w_type elements (TSVM_ROW_F64 or TSVM_ROW_F32).  Float
+ * staging is exact when every value of the working rows is a float (values read from a LibSVM file or handed over
+ * as float arrays are): products and sums are formed in double either way, and the kernel's time goes into
+ * reading the staged rows, m elements per stored non-zero. */
+int tsvm_get_rows_csr_staged(const double *val, const int *col, const int64_t *row_ptr, const int *x_idx, int64_t n,
+                             const double *sd_x, const void *w, int w_type, int m, const double *sd_w, int kernel_type,
+                             double gamma, double coef0, int degree, void *out, int row_type, const int *out_slots, int64_t ldo,
+                             tsvm_stream stream);
 
 /* CSR get_rows: out[s_i*ldo + j] = kappa(w_i, x_j) (s_i as above) with x in CSR (n rows) and the m working rows
  * staged by tsvm_csr_stage_rows.  Accumulates over the stored order of row j's non-zeros

@@ -229,10 +229,13 @@ __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
 // ------------------------------------------------------------------------------------------------
 // (JB = 16 stored rows per workgroup; 4 when there are only a few thousand of them, as for the solver's ws x ws
 // block, so that the grid still covers the chip and a workgroup's chain of dependent loads is a quarter as long)
-template <typename TO, int CS_JB>
+// TW: element type of the staged working rows.  Values that are float-exact (everything a LibSVM file or the
+// reference's float interfaces can deliver) are staged as float: the products are formed in double either way,
+// and these reads, m x 8 bytes per stored non-zero, are what the kernel's time goes into.
+template <typename TO, int CS_JB, typename TW>
 __global__ __launch_bounds__(256) void get_rows_csr_kernel(
     const double *__restrict__ val, const int *__restrict__ col, const int64_t *__restrict__ row_ptr,
-    const int *__restrict__ x_idx, int64_t n, const double *__restrict__ sd_x, const double *__restrict__ w, int m,
+    const int *__restrict__ x_idx, int64_t n, const double *__restrict__ sd_x, const TW *__restrict__ w, int m,
     const double *__restrict__ sd_w, KernelParam kp, TO *__restrict__ out, const int *__restrict__ out_slots,
     int64_t ldo, unsigned i_blocks) {
     __shared__ uint64_t exp_tab[32];
@@ -253,11 +256,21 @@ __global__ __launch_bounds__(256) void get_rows_csr_kernel(
             const int64_t rj = x_idx ? (int64_t) x_idx[j] : j;
             const int64_t e0 = row_ptr[rj], e1 = row_ptr[rj + 1];
             double s = 0.0;
-            for (int64_t e = e0; e < e1; ++e) {
-                const double v = val[e];
-                const int c = col[e];
-                s = __builtin_fma(v, w[(int64_t) c * m + ic], s);
+            // eight non-zeros at a time: their loads are all issued before the first product is needed; the
+            // products are still added in stored order
+            int64_t e = e0;
+            for (; e + 8 <= e1; e += 8) {
+                double v[8];
+                TW x[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    v[u] = val[e + u];
+                    x[u] = w[(int64_t) col[e + u] * m + ic];
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) s = __builtin_fma(v[u], (double) x[u], s);
             }
+            for (; e < e1; ++e) s = __builtin_fma(val[e], (double) w[(int64_t) col[e] * m + ic], s);
             acc[jj] = s;
         }
     }
@@ -308,16 +321,17 @@ __global__ void fill_f64_kernel(double *p, int64_t count, double v) {
 
 // w[c*m + i] = value of feature c in CSR row idx[i] (clear: 0.0 instead, which takes the rows out of a staging
 // matrix again); one wavefront per staged row.
+template <typename TW>
 __global__ void csr_stage_rows_kernel(const double *__restrict__ val, const int *__restrict__ col,
                                       const int64_t *__restrict__ row_ptr, const int *__restrict__ idx, int m,
-                                      int n_features, double *__restrict__ w, int clear) {
+                                      int n_features, TW *__restrict__ w, int clear) {
     const int i = (int) ((blockIdx.x * (int64_t) blockDim.x + threadIdx.x) >> 6);
     const int lane = threadIdx.x & 63;
     if (i >= m) return;
     const int64_t r = idx ? (int64_t) idx[i] : (int64_t) i;
     for (int64_t e = row_ptr[r] + lane; e < row_ptr[r + 1]; e += 64) {
         const int c = col[e];
-        if (c < n_features) w[(int64_t) c * m + i] = clear ? 0.0 : val[e];
+        if (c < n_features) w[(int64_t) c * m + i] = clear ? (TW) 0 : (TW) val[e];
     }
 }
 
@@ -572,26 +586,32 @@ int tsvm_csr_stage_rows(const double *val, const int *col, const int64_t *row_pt
     if (m == 0 || n_features == 0) return 0;
     hipLaunchKernelGGL(fill_f64_kernel, dim3(2048), dim3(256), 0, tsvm_s(stream), w, (int64_t) m * n_features, 0.0);
     TSVM_LAUNCH_CHECK();
-    hipLaunchKernelGGL(csr_stage_rows_kernel, dim3(grid_for((int64_t) m * 64, 256)), dim3(256), 0, tsvm_s(stream), val, col,
+    hipLaunchKernelGGL(csr_stage_rows_kernel<double>, dim3(grid_for((int64_t) m * 64, 256)), dim3(256), 0, tsvm_s(stream), val, col,
                        row_ptr, idx, m, n_features, w, 0);
     TSVM_LAUNCH_CHECK();
     return 0;
 }
 
 int tsvm_csr_scatter_rows(const double *val, const int *col, const int64_t *row_ptr, const int *idx, int m,
-                          int n_features, double *w, int clear, tsvm_stream stream) {
+                          int n_features, void *w, int w_type, int clear, tsvm_stream stream) {
     TSVM_REQUIRE(row_ptr && w && m >= 0 && n_features >= 0, "tsvm_csr_scatter_rows: bad argument");
+    TSVM_REQUIRE(w_type == TSVM_ROW_F64 || w_type == TSVM_ROW_F32, "tsvm_csr_scatter_rows: unknown element type %d", w_type);
     if (m == 0 || n_features == 0) return 0;
-    hipLaunchKernelGGL(csr_stage_rows_kernel, dim3(grid_for((int64_t) m * 64, 256)), dim3(256), 0, tsvm_s(stream), val, col,
-                       row_ptr, idx, m, n_features, w, clear);
+    if (w_type == TSVM_ROW_F32)
+        hipLaunchKernelGGL(csr_stage_rows_kernel<float>, dim3(grid_for((int64_t) m * 64, 256)), dim3(256), 0, tsvm_s(stream), val,
+                           col, row_ptr, idx, m, n_features, (float *) w, clear);
+    else
+        hipLaunchKernelGGL(csr_stage_rows_kernel<double>, dim3(grid_for((int64_t) m * 64, 256)), dim3(256), 0, tsvm_s(stream), val,
+                           col, row_ptr, idx, m, n_features, (double *) w, clear);
     TSVM_LAUNCH_CHECK();
     return 0;
 }
 
-int tsvm_get_rows_csr(const double *val, const int *col, const int64_t *row_ptr, const int *x_idx, int64_t n, const double *sd_x,
-                      const double *w, int m, const double *sd_w, int kernel_type, double gamma, double coef0,
-                      int degree, void *out, int row_type, const int *out_slots, int64_t ldo, tsvm_stream stream) {
+static int get_rows_csr(const double *val, const int *col, const int64_t *row_ptr, const int *x_idx, int64_t n, const double *sd_x,
+                        const void *w, int w_type, int m, const double *sd_w, int kernel_type, double gamma, double coef0,
+                        int degree, void *out, int row_type, const int *out_slots, int64_t ldo, tsvm_stream stream) {
     TSVM_REQUIRE(row_ptr && w && out, "tsvm_get_rows_csr: null pointer");
+    TSVM_REQUIRE(w_type == TSVM_ROW_F64 || w_type == TSVM_ROW_F32, "tsvm_get_rows_csr: unknown staging type %d", w_type);
     TSVM_REQUIRE(n >= 0 && m >= 0 && ldo >= n, "tsvm_get_rows_csr: bad size");
     TSVM_REQUIRE(kernel_type >= 0 && kernel_type <= 4, "tsvm_get_rows_csr: unknown kernel type %d", kernel_type);
     TSVM_REQUIRE(row_type_ok(row_type, kernel_type), "tsvm_get_rows_csr: row type %d not valid for kernel type %d", row_type,
@@ -605,17 +625,38 @@ int tsvm_get_rows_csr(const double *val, const int *col, const int64_t *row_ptr,
     const int64_t j_blocks = (n + jb - 1) / jb;
     TSVM_REQUIRE(j_blocks * i_blocks < (int64_t) 0x7fffffff, "tsvm_get_rows_csr: grid too large");
     const dim3 grid((unsigned) (j_blocks * i_blocks));
-#define CSR_LAUNCH(TO, JB)                                                                                                   \
-    hipLaunchKernelGGL((get_rows_csr_kernel<TO, JB>), grid, dim3(256), 0, tsvm_s(stream), val, col, row_ptr, x_idx, n, sd_x, w, m, \
-                       sd_w, kp, (TO *) out, out_slots, ldo, i_blocks)
+#define CSR_LAUNCH_W(TO, JB, TW)                                                                                             \
+    hipLaunchKernelGGL((get_rows_csr_kernel<TO, JB, TW>), grid, dim3(256), 0, tsvm_s(stream), val, col, row_ptr, x_idx, n, sd_x, \
+                       (const TW *) w, m, sd_w, kp, (TO *) out, out_slots, ldo, i_blocks)
+#define CSR_LAUNCH(TO, JB)                                                   \
+    do {                                                                     \
+        if (w_type == TSVM_ROW_F32) CSR_LAUNCH_W(TO, JB, float);             \
+        else CSR_LAUNCH_W(TO, JB, double);                                   \
+    } while (0)
     if (row_type == TSVM_ROW_F32) {
         if (jb == 4) CSR_LAUNCH(float, 4); else CSR_LAUNCH(float, 16);
     } else {
         if (jb == 4) CSR_LAUNCH(double, 4); else CSR_LAUNCH(double, 16);
     }
 #undef CSR_LAUNCH
+#undef CSR_LAUNCH_W
     TSVM_LAUNCH_CHECK();
     return 0;
+}
+
+int tsvm_get_rows_csr(const double *val, const int *col, const int64_t *row_ptr, const int *x_idx, int64_t n, const double *sd_x,
+                      const double *w, int m, const double *sd_w, int kernel_type, double gamma, double coef0,
+                      int degree, void *out, int row_type, const int *out_slots, int64_t ldo, tsvm_stream stream) {
+    return get_rows_csr(val, col, row_ptr, x_idx, n, sd_x, w, TSVM_ROW_F64, m, sd_w, kernel_type, gamma, coef0, degree, out, row_type,
+                        out_slots, ldo, stream);
+}
+
+int tsvm_get_rows_csr_staged(const double *val, const int *col, const int64_t *row_ptr, const int *x_idx, int64_t n,
+                             const double *sd_x, const void *w, int w_type, int m, const double *sd_w, int kernel_type,
+                             double gamma, double coef0, int degree, void *out, int row_type, const int *out_slots, int64_t ldo,
+                             tsvm_stream stream) {
+    return get_rows_csr(val, col, row_ptr, x_idx, n, sd_x, w, w_type, m, sd_w, kernel_type, gamma, coef0, degree, out, row_type,
+                        out_slots, ldo, stream);
 }
 
 int tsvm_gather_rows_f64(const double *x, int64_t ld, const int *idx, int64_t m, double *out, tsvm_stream stream) {

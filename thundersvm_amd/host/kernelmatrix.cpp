@@ -90,12 +90,19 @@ std::shared_ptr<DeviceRows> DeviceRows::from_host(const DataSet::node2d &all, co
     r.n_features = (size_t) max_index + 1;
     std::vector<kernel_type> val(r.nnz);
     std::vector<int> col(r.nnz);
-#pragma omp parallel for schedule(static)
+    int all_float = 1;
+#pragma omp parallel for schedule(static) reduction(min : all_float)
     for (size_t i = 0; i < n_rows; ++i) {
         const auto &row = all[rows ? rows[i] : i];
         size_t e = (size_t) ptr[i];
-        for (const auto &nd : row) { val[e] = nd.value; col[e] = nd.index; ++e; }
+        for (const auto &nd : row) {
+            val[e] = nd.value;
+            col[e] = nd.index;
+            if ((double) (float) nd.value != (double) nd.value) all_float = 0;
+            ++e;
+        }
     }
+    r.values_fit_float = all_float != 0;
     r.val.upload(val);
     r.col.upload(col);
     r.row_ptr.upload(ptr);
@@ -122,6 +129,7 @@ std::shared_ptr<DeviceRows> DeviceRows::subset(const DeviceRows &base, const int
     r.n = n_rows;
     r.n_features = base.n_features;
     r.dense = base.dense;
+    r.values_fit_float = base.values_fit_float;
     r.ld = base.ld;
     tsvm::DeviceBuffer<int> d_rows(n_rows);
     d_rows.upload(rows, n_rows);
@@ -186,10 +194,10 @@ void KernelMatrix::finish(int repeat) {
 }
 
 // A staging buffer that is all-zero whenever it is not in use: grown (and cleared) only when a call needs more.
-static void grow_zeroed(tsvm::DeviceBuffer<kernel_type> &b, size_t count, hipStream_t stream) {
-    if (b.size() >= count) return;
-    b.resize(count);
-    TSVM_HIP_CHECK(hipMemsetAsync(b.data(), 0, count * sizeof(kernel_type), stream));
+static void grow_zeroed(tsvm::DeviceBuffer<unsigned char> &b, size_t bytes, hipStream_t stream) {
+    if (b.size() >= bytes) return;
+    b.resize(bytes);
+    TSVM_HIP_CHECK(hipMemsetAsync(b.data(), 0, bytes, stream));
 }
 
 void KernelMatrix::get_rows(const int *d_idx, int m, void *d_out, int64_t ld, const int *d_out_slots,
@@ -204,16 +212,17 @@ void KernelMatrix::get_rows(const int *d_idx, int m, void *d_out, int64_t ld, co
     }
     // The staging matrix [n_features][m] is kept all-zero between uses: the working rows' non-zeros are written
     // into it and taken out again afterwards (nnz entries each way instead of a fill of n_features x m).
-    grow_zeroed(stage_w_, (size_t) m * R.n_features, stream);
+    const int wt = R.values_fit_float ? TSVM_ROW_F32 : TSVM_ROW_F64;
+    grow_zeroed(stage_w_, (size_t) m * R.n_features * (R.values_fit_float ? sizeof(float) : sizeof(double)), stream);
     if (stage_sd_.size() < (size_t) m) stage_sd_.resize(m);
     abi_check(tsvm_csr_scatter_rows(R.val.data(), R.col.data(), R.row_ptr.data(), d_idx, m, (int) R.n_features,
-                                    stage_w_.data(), 0, stream));
+                                    stage_w_.data(), wt, 0, stream));
     abi_check(tsvm_gather_f64(R.self_dot.data(), d_idx, m, stage_sd_.data(), stream));
-    abi_check(tsvm_get_rows_csr(R.val.data(), R.col.data(), R.row_ptr.data(), nullptr, n, R.self_dot.data(), stage_w_.data(),
-                                m, stage_sd_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree, d_out,
-                                row_type(), d_out_slots, ld, stream));
+    abi_check(tsvm_get_rows_csr_staged(R.val.data(), R.col.data(), R.row_ptr.data(), nullptr, n, R.self_dot.data(),
+                                       stage_w_.data(), wt, m, stage_sd_.data(), (int) param.kernel_type, param.gamma,
+                                       param.coef0, param.degree, d_out, row_type(), d_out_slots, ld, stream));
     abi_check(tsvm_csr_scatter_rows(R.val.data(), R.col.data(), R.row_ptr.data(), d_idx, m, (int) R.n_features,
-                                    stage_w_.data(), 1, stream));
+                                    stage_w_.data(), wt, 1, stream));
 }
 
 void KernelMatrix::get_rows_counted(const int *d_idx, int m_max, const int *d_m, void *d_out, int64_t ld,
@@ -235,16 +244,18 @@ void KernelMatrix::get_block(const int *d_idx, int m, kernel_type *d_out, int64_
                                       d_out, TSVM_ROW_F64, nullptr, ld, stream));
         return;
     }
-    grow_zeroed(stage_blk_, (size_t) m * R.n_features, stream);   // kept all-zero between uses, as in get_rows
+    const int wt = R.values_fit_float ? TSVM_ROW_F32 : TSVM_ROW_F64;
+    // kept all-zero between uses, as in get_rows
+    grow_zeroed(stage_blk_, (size_t) m * R.n_features * (R.values_fit_float ? sizeof(float) : sizeof(double)), stream);
     if (stage_blk_sd_.size() < (size_t) m) stage_blk_sd_.resize(m);
     abi_check(tsvm_csr_scatter_rows(R.val.data(), R.col.data(), R.row_ptr.data(), d_idx, m, (int) R.n_features,
-                                    stage_blk_.data(), 0, stream));
+                                    stage_blk_.data(), wt, 0, stream));
     abi_check(tsvm_gather_f64(R.self_dot.data(), d_idx, m, stage_blk_sd_.data(), stream));
-    abi_check(tsvm_get_rows_csr(R.val.data(), R.col.data(), R.row_ptr.data(), d_idx, m, R.self_dot.data(), stage_blk_.data(),
-                                m, stage_blk_sd_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
-                                d_out, TSVM_ROW_F64, nullptr, ld, stream));
+    abi_check(tsvm_get_rows_csr_staged(R.val.data(), R.col.data(), R.row_ptr.data(), d_idx, m, R.self_dot.data(),
+                                       stage_blk_.data(), wt, m, stage_blk_sd_.data(), (int) param.kernel_type, param.gamma,
+                                       param.coef0, param.degree, d_out, TSVM_ROW_F64, nullptr, ld, stream));
     abi_check(tsvm_csr_scatter_rows(R.val.data(), R.col.data(), R.row_ptr.data(), d_idx, m, (int) R.n_features,
-                                    stage_blk_.data(), 1, stream));
+                                    stage_blk_.data(), wt, 1, stream));
 }
 
 // External batch (kernelmatrix.cpp:281-312, 385-406): features with id >= R.n_features are left out of

@@ -25,6 +25,7 @@
 struct DeviceRows {
     size_t n = 0, n_features = 0, nnz = 0;
     bool dense = false;
+    bool values_fit_float = false;               // every stored value is exactly a float (CSR layout: staging type)
     int64_t ld = 0;                              // dense row stride (n_features rounded up to 8)
     tsvm::DeviceBuffer<kernel_type> x;           // dense layout [n][ld]
     tsvm::DeviceBuffer<kernel_type> val;         // CSR layout
@@ -88,8 +89,10 @@ private:
     tsvm::DeviceBuffer<kernel_type> diag_;
     // reusable staging for the sparse path and for external batches
     mutable tsvm::DeviceBuffer<kernel_type> stage_;
-    mutable tsvm::DeviceBuffer<kernel_type> stage_w_;   // transposed staging of CSR working rows, all-zero between uses
-    mutable tsvm::DeviceBuffer<kernel_type> stage_blk_, stage_blk_sd_;   // staging of get_block (its own stream)
+    // transposed staging of CSR working rows (get_rows / get_block), all-zero between uses; float elements when
+    // the rows' values are floats
+    mutable tsvm::DeviceBuffer<unsigned char> stage_w_, stage_blk_;
+    mutable tsvm::DeviceBuffer<kernel_type> stage_blk_sd_;
     mutable tsvm::DeviceBuffer<kernel_type> stage_sd_;
     mutable tsvm::DeviceBuffer<kernel_type> b_val_;
     mutable tsvm::DeviceBuffer<int> b_col_;
