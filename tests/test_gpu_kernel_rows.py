@@ -135,10 +135,11 @@ def test_float_rows_rejected_for_linear_kernel():
                   G.ptr(out), capi.ROW_F32, None, 8, G.stream())
 
 
+@pytest.mark.parametrize("n", [700, 5000])   # four / sixteen stored rows per workgroup
 @pytest.mark.parametrize("name,kt,prm", KERNELS)
-def test_csr_path(name, kt, prm):
+def test_csr_path(name, kt, prm, n):
     rng = np.random.default_rng(7)
-    n, d, m = 700, 3000, 70
+    d, m = 3000, 70
     ptr = [0]
     col, val = [], []
     for i in range(n):
@@ -172,6 +173,19 @@ def test_csr_path(name, kt, prm):
                   kt, prm.get("gamma", 0.0), prm.get("coef0", 0.0), prm.get("degree", 3), G.ptr(out32), capi.ROW_F32, None,
                   n, G.stream())
         assert np.array_equal(G.host(out32).astype(np.float64), G.host(out))
+    # a staging matrix kept all-zero between uses, with float elements (the values are floats): rows scattered in,
+    # the same bits out of the kernel, rows scattered out again
+    for wt, dt in ((capi.ROW_F32, torch.float32), (capi.ROW_F64, torch.float64)):
+        wz = torch.zeros((nf, m), dtype=dt, device="cuda")
+        capi.call("tsvm_csr_scatter_rows", G.ptr(val_d), G.ptr(col_d), G.ptr(ptr_d), G.ptr(idx_d), m, nf, G.ptr(wz), wt, 0, G.stream())
+        assert np.array_equal(G.host(wz).astype(np.float64), G.host(w))
+        out_s = torch.empty((m, n), dtype=torch.float64, device="cuda")
+        capi.call("tsvm_get_rows_csr_staged", G.ptr(val_d), G.ptr(col_d), G.ptr(ptr_d), None, n, G.ptr(sd), G.ptr(wz), wt, m,
+                  G.ptr(sdw), kt, prm.get("gamma", 0.0), prm.get("coef0", 0.0), prm.get("degree", 3), G.ptr(out_s), capi.ROW_F64,
+                  None, n, G.stream())
+        assert np.array_equal(G.host(out_s), G.host(out))
+        capi.call("tsvm_csr_scatter_rows", G.ptr(val_d), G.ptr(col_d), G.ptr(ptr_d), G.ptr(idx_d), m, nf, G.ptr(wz), wt, 1, G.stream())
+        assert not G.host(wz).any()
     # the dense path on the same data gives the same bits (both sum in ascending feature order)
     xh, nf2, ld = G.dense_padded(data)
     x_d = G.dev(xh)
