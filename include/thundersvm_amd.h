@@ -223,6 +223,14 @@ int tsvm_select_working_set_again(const double *f, const int *y, const double *a
                                   const int *marked, int n_marked, int *out, int n_select, int nu, void *workspace,
                                   tsvm_stream stream);
 
+/* Either selection (again == 0: any workspace content; again != 0: as tsvm_select_working_set_again) that also
+ * writes the ids modulo fold_n to out_folded[0..n_select): the stored row of each selected instance when the n
+ * instances are stacked copies of fold_n rows (the 2n-variable problem of SVR, svr.cpp:14-28).  Saves the separate
+ * tsvm_fold_ids launch of every outer iteration. */
+int tsvm_select_working_set_folded(const double *f, const int *y, const double *alpha, int64_t n, double Cp, double Cn,
+                                   const int *marked, int n_marked, int *out, int n_select, int nu, void *workspace,
+                                   int again, int fold_n, int *out_folded, tsvm_stream stream);
+
 /* ---------------------------------------------------------------------------------------------
  * predict (kernelmatrix_kernel.cpp:110-147)
  * ------------------------------------------------------------------------------------------- */

@@ -217,6 +217,32 @@ def test_selections_in_a_row_on_one_workspace(n, nu):
         assert (prev >= 0).all()
 
 
+@pytest.mark.parametrize("nu", [0, 1])
+@pytest.mark.parametrize("n,tie_mode", [(150, 0), (5000, 2), (200000, 0), (200000, 1)])
+def test_selection_with_folded_ids(n, tie_mode, nu):
+    """The 2n-variable problem of SVR (svr.cpp:14-28): the selection also delivers each id modulo n / 2, the stored row
+    behind the variable; same ids as the plain selection, on a fresh and on a re-used workspace."""
+    half = n // 2
+    ws = min(1024, 1 << (n.bit_length() - 1))
+    q = ws // 2
+    wsp = torch.empty(capi.kernel_lib().tsvm_select_workspace(n), dtype=torch.uint8, device="cuda")
+    prev = None
+    for it in range(3):
+        f, y, alpha, C, _ = _select_case(n, q, 0, 5 * n + it, tie_mode, nu)
+        marked = np.zeros(0, dtype=np.int32) if it == 0 else np.ascontiguousarray(prev[q:])
+        n_select = ws if it == 0 else q
+        want = O.select_working_set(f, y, alpha, C, C, marked, n_select, nu=bool(nu))
+        f_d, y_d, a_d, m_d = G.dev(f), G.dev(y), G.dev(alpha), G.dev(marked if it else np.zeros(1, dtype=np.int32))
+        out_d = torch.full((n_select,), -7, dtype=torch.int32, device="cuda")
+        fold_d = torch.full((n_select,), -7, dtype=torch.int32, device="cuda")
+        capi.call("tsvm_select_working_set_folded", G.ptr(f_d), G.ptr(y_d), G.ptr(a_d), n, C, C, G.ptr(m_d) if it else None,
+                  len(marked), G.ptr(out_d), n_select, nu, G.ptr(wsp), int(it > 0), half, G.ptr(fold_d), G.stream())
+        got = G.host(out_d)
+        assert np.array_equal(got, want)
+        assert np.array_equal(G.host(fold_d), np.where(want >= 0, want % half, -1))
+        prev = got if it == 0 else np.concatenate([prev[q:], got])
+
+
 def test_empty_inputs_are_no_ops():
     """Zero rows, zero columns, an empty working set, nothing to select: every entry point returns success and
     leaves its outputs untouched."""

@@ -49,6 +49,7 @@ SIGNATURES = {
     "tsvm_select_workspace": (C.c_size_t, [_i64]),
     "tsvm_select_working_set": (_int, [_p, _p, _p, _i64, _dbl, _dbl, _p, _int, _p, _int, _int, _p, _p]),
     "tsvm_select_working_set_again": (_int, [_p, _p, _p, _i64, _dbl, _dbl, _p, _int, _p, _int, _int, _p, _p]),
+    "tsvm_select_working_set_folded": (_int, [_p, _p, _p, _i64, _dbl, _dbl, _p, _int, _p, _int, _int, _p, _int, _int, _p, _p]),
     "tsvm_sum_kernel_values": (_int, [_p, _int, _p, _p, _p, _p, _int, _i64, _p, _int, _i64, _p]),
 }
 

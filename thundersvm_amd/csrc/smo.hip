@@ -480,8 +480,10 @@ __device__ __forceinline__ bool comp_less(uint64_t ka, uint32_t ia, uint64_t kb,
     return ka < kb || (ka == kb && ia < ib);
 }
 
+// (fold_n > 0: the ids are also written modulo fold_n to out_folded, for problems whose instances are stacked
+// copies of fold_n stored rows)
 __global__ __launch_bounds__(MAX_WS) void sel_final_kernel(SelWorkspace w, int64_t n, SelGeom g, int p_full,
-                                                           int *__restrict__ out) {
+                                                           int *__restrict__ out, int fold_n, int *__restrict__ out_folded) {
     __shared__ uint64_t sk[SEL_MAX_SIDES][MAX_WS];
     __shared__ uint32_t si[SEL_MAX_SIDES][MAX_WS];
     __shared__ int pos_other[SEL_MAX_SIDES][MAX_WS];  // position of the same instance in the paired side's list, or -1
@@ -587,7 +589,11 @@ __global__ __launch_bounds__(MAX_WS) void sel_final_kernel(SelWorkspace w, int64
     __syncthreads();
     if (ok && !conflict) {
         if (tid < per)
-            for (int s = 0; s < g.n_sides; ++s) out[tid * g.n_sides + s] = (int) si[s][tid];
+            for (int s = 0; s < g.n_sides; ++s) {
+                const int id = (int) si[s][tid];
+                out[tid * g.n_sides + s] = id;
+                if (fold_n > 0) out_folded[tid * g.n_sides + s] = id % fold_n;
+            }
         return;
     }
     // general path: replay the scan serially (small problems, or sides that run dry)
@@ -600,6 +606,7 @@ __global__ __launch_bounds__(MAX_WS) void sel_final_kernel(SelWorkspace w, int64
                 const int o = s < half ? s + half : s - half;
                 while (ptr[s] < cnt[s] && pos_other[s][ptr[s]] >= 0 && pos_other[s][ptr[s]] < ptr[o]) ++ptr[s];
                 if (ptr[s] < cnt[s] && n_sel < k) {
+                    if (fold_n > 0) out_folded[n_sel] = (int) si[s][ptr[s]] % fold_n;
                     out[n_sel++] = (int) si[s][ptr[s]];
                     ++ptr[s];
                     progressed = true;
@@ -607,7 +614,10 @@ __global__ __launch_bounds__(MAX_WS) void sel_final_kernel(SelWorkspace w, int64
             }
             if (!progressed) break;
         }
-        for (; n_sel < k; ++n_sel) out[n_sel] = -1;
+        for (; n_sel < k; ++n_sel) {
+            out[n_sel] = -1;
+            if (fold_n > 0) out_folded[n_sel] = -1;
+        }
     }
 }
 
@@ -633,12 +643,13 @@ static void launch_update_f(double *f, const double *alpha_diff, int ws_size, co
 
 static int select_working_set(const double *f, const int *y, const double *alpha, int64_t n, double Cp, double Cn,
                               const int *marked, int n_marked, int *out, int n_select, int nu, void *workspace,
-                              bool armed, tsvm_stream stream) {
+                              bool armed, int fold_n, int *out_folded, tsvm_stream stream) {
     TSVM_REQUIRE(f && y && alpha && out && workspace, "tsvm_select_working_set: null pointer");
     TSVM_REQUIRE(n >= 1 && n <= 0x7fffffffLL, "tsvm_select_working_set: n %lld outside [1, 2^31)", (long long) n);
     TSVM_REQUIRE(n_select >= 0 && n_select <= MAX_WS, "tsvm_select_working_set: n_select %d outside [0, %d]", n_select,
                  MAX_WS);
     TSVM_REQUIRE(n_marked >= 0 && (n_marked == 0 || marked), "tsvm_select_working_set: bad marked list");
+    TSVM_REQUIRE(fold_n >= 0 && (fold_n == 0 || out_folded), "tsvm_select_working_set: bad fold arguments");
     if (n_select == 0) return 0;
     hipStream_t s = tsvm_s(stream);
     SelWorkspace w;
@@ -670,7 +681,7 @@ static int select_working_set(const double *f, const int *y, const double *alpha
     }
     hipLaunchKernelGGL(sel_compact_kernel, dim3(grid), dim3(SEL_T), 0, s, w, n, g, p_full);
     TSVM_LAUNCH_CHECK();
-    hipLaunchKernelGGL(sel_final_kernel, dim3(1), dim3(MAX_WS), 0, s, w, n, g, p_full, out);
+    hipLaunchKernelGGL(sel_final_kernel, dim3(1), dim3(MAX_WS), 0, s, w, n, g, p_full, out, fold_n, out_folded);
     TSVM_LAUNCH_CHECK();
     return 0;
 }
@@ -709,13 +720,21 @@ size_t tsvm_select_workspace(int64_t n) {
 int tsvm_select_working_set(const double *f, const int *y, const double *alpha, int64_t n, double Cp, double Cn,
                             const int *marked, int n_marked, int *out, int n_select, int nu, void *workspace,
                             tsvm_stream stream) {
-    return select_working_set(f, y, alpha, n, Cp, Cn, marked, n_marked, out, n_select, nu, workspace, false, stream);
+    return select_working_set(f, y, alpha, n, Cp, Cn, marked, n_marked, out, n_select, nu, workspace, false, 0, nullptr, stream);
 }
 
 int tsvm_select_working_set_again(const double *f, const int *y, const double *alpha, int64_t n, double Cp, double Cn,
                                   const int *marked, int n_marked, int *out, int n_select, int nu, void *workspace,
                                   tsvm_stream stream) {
-    return select_working_set(f, y, alpha, n, Cp, Cn, marked, n_marked, out, n_select, nu, workspace, true, stream);
+    return select_working_set(f, y, alpha, n, Cp, Cn, marked, n_marked, out, n_select, nu, workspace, true, 0, nullptr, stream);
+}
+
+int tsvm_select_working_set_folded(const double *f, const int *y, const double *alpha, int64_t n, double Cp, double Cn,
+                                   const int *marked, int n_marked, int *out, int n_select, int nu, void *workspace,
+                                   int again, int fold_n, int *out_folded, tsvm_stream stream) {
+    TSVM_REQUIRE(fold_n >= 1, "tsvm_select_working_set_folded: fold_n %d < 1", fold_n);
+    return select_working_set(f, y, alpha, n, Cp, Cn, marked, n_marked, out, n_select, nu, workspace, again != 0, fold_n, out_folded,
+                              stream);
 }
 
 }  // extern "C"

@@ -140,7 +140,8 @@ struct SolveTask::Impl {
     static constexpr int WS_HALVES = 64;
     int ws_off = 0, sel_off = 0;   // window of the current iteration / of the latest selection launched
     const int *ws_ids() const { return d_ws.data() + ws_off; }
-    const int *ws_u() const { return rep > 1 ? d_ws_folded.data() : d_ws.data() + ws_off; }   // working set as folded ids
+    // working set as folded ids: a second window, at the same offsets, that the selection fills along with the first
+    const int *ws_u() const { return rep > 1 ? d_ws_folded.data() + ws_off : d_ws.data() + ws_off; }
 
     // The chip-wide work of a task is enqueued on stream `sa` (`ids` is the stream the newly selected ids are read
     // back on for the host-side cache bookkeeping: the same one).
@@ -228,7 +229,7 @@ struct SolveTask::Impl {
           nu(solver.is_nu()), ldk(tsvm_smo_solve_block_ld(ws_size)), timer(solver.profile) {
         wall0 = std::chrono::steady_clock::now();
         d_y.resize(n); d_ws.resize((size_t) WS_HALVES * q + ws_size); d_slots_a.resize(3 * (size_t) ws_size); d_slots_b.resize(ws_size);
-        if (rep > 1) d_ws_folded.resize(ws_size);
+        if (rep > 1) d_ws_folded.resize(d_ws.size());
         d_alpha.resize(n); d_f.resize(n); d_alpha_diff.resize(ws_size);
         d_sel_ws.resize(tsvm_select_workspace(n));
         d_kws.resize((size_t) ws_size * ldk);
@@ -400,21 +401,33 @@ struct SolveTask::Impl {
     // Working-set selection of iteration `it`: the first one picks ws_size ids, later ones keep the last
     // half of the previous set and pick q new ids (csmosolver.cpp:63-77).
     void launch_select(int it) {
+        const int n_sel = it == 0 ? ws_size : q;
         if (it == 0) {
             sel_off = 0;
-            abi_check(tsvm_select_working_set(d_f.data(), d_y.data(), d_alpha.data(), n, Cp, Cn, nullptr, 0, d_ws.data(),
-                                              ws_size, nu, d_sel_ws.data(), sa));
         } else {
             int next = sel_off + q;
             if (next + ws_size > (int) d_ws.size()) {
                 TSVM_HIP_CHECK(hipMemcpyAsync(d_ws.data(), d_ws.data() + next, sizeof(int) * q, hipMemcpyDeviceToDevice, sa));
+                if (rep > 1)
+                    TSVM_HIP_CHECK(hipMemcpyAsync(d_ws_folded.data(), d_ws_folded.data() + next, sizeof(int) * q,
+                                                  hipMemcpyDeviceToDevice, sa));
                 next = 0;
             }
             sel_off = next;
-            abi_check(tsvm_select_working_set_again(d_f.data(), d_y.data(), d_alpha.data(), n, Cp, Cn, d_ws.data() + sel_off, q,
-                                                    d_ws.data() + sel_off + q, q, nu, d_sel_ws.data(), sa));
         }
-        if (rep > 1) abi_check(tsvm_fold_ids(d_ws.data() + sel_off, ws_size, n_u, d_ws_folded.data(), sa));
+        const int *kept = it == 0 ? nullptr : d_ws.data() + sel_off;            // the half that stays: no candidates
+        int *out = d_ws.data() + sel_off + (it == 0 ? 0 : q);
+        if (rep > 1) {
+            abi_check(tsvm_select_working_set_folded(d_f.data(), d_y.data(), d_alpha.data(), n, Cp, Cn, kept, it == 0 ? 0 : q, out,
+                                                     n_sel, nu, d_sel_ws.data(), it > 0, n_u,
+                                                     d_ws_folded.data() + sel_off + (it == 0 ? 0 : q), sa));
+        } else if (it == 0) {
+            abi_check(tsvm_select_working_set(d_f.data(), d_y.data(), d_alpha.data(), n, Cp, Cn, kept, 0, out, n_sel, nu,
+                                              d_sel_ws.data(), sa));
+        } else {
+            abi_check(tsvm_select_working_set_again(d_f.data(), d_y.data(), d_alpha.data(), n, Cp, Cn, kept, q, out, n_sel, nu,
+                                                    d_sel_ws.data(), sa));
+        }
     }
 
     void enqueue_select() {
