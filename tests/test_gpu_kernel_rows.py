@@ -370,3 +370,26 @@ def test_row_store_managed_on_the_device(n, d, ws):
     assert used == n                                       # every instance has been seen: the store is complete
     st = G.host(store)
     assert np.array_equal(st[h_slot_of][:, :n], all_rows)  # each row computed into its slot, nothing else touched
+
+
+@pytest.mark.parametrize("name,kt,prm", KERNELS)
+@pytest.mark.parametrize("n,d,ws", [(300, 20, 64), (3000, 54, 1000), (2600, 200, 1024), (1500, 784, 200)])
+def test_working_set_block(name, kt, prm, n, d, ws):
+    """The solver's ws x ws block (x_idx = a_idx = the working set): the same bits as the corresponding entries of the
+    full kernel rows, although only the tiles on and above the diagonal are computed and the rest is mirrored."""
+    rng = np.random.default_rng(n + ws)
+    data = from_dense(rng.standard_normal((n, d)).astype(np.float32).astype(np.float64))
+    x_d, nf, ld, sd, _ = _device_km(data, kt, prm)
+    ids = rng.permutation(n)[:ws].astype(np.int32)
+    if ws >= 8: ids[5] = ids[2]                     # the same row twice (a folded problem can select both copies)
+    ids_d = G.dev(ids)
+    rows = G.host(G.get_rows_dense(x_d, ld, n, nf, sd, x_d, ld, ids_d, ws, sd, kt, **prm))       # [ws, n]
+    ldk = G.round_up(ws, 256)
+    blk = torch.full((ws, ldk), 9.0, dtype=torch.float64, device="cuda")
+    capi.call("tsvm_get_rows_dense", G.ptr(x_d), ld, G.ptr(ids_d), ws, nf, G.ptr(sd), G.ptr(x_d), ld, G.ptr(ids_d), ws, G.ptr(sd),
+              kt, prm.get("gamma", 0.0), prm.get("coef0", 0.0), prm.get("degree", 3), G.ptr(blk), capi.ROW_F64, None, ldk,
+              G.stream())
+    got = G.host(blk)
+    assert np.array_equal(got[:, :ws], rows[:, ids])
+    assert np.array_equal(got[:, :ws], got[:, :ws].T)
+    assert (got[:, ws:] == 9.0).all()

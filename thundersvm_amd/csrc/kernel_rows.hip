@@ -39,21 +39,30 @@ typedef double v4d __attribute__((ext_vector_type(4)));
 // TO: element type of the output rows.  The RBF / polynomial / sigmoid values are float-rounded by
 // definition (kernelmatrix_kernel.cpp:77-108 calls expf / powf / tanhf), so storing them as float
 // loses nothing and halves the bytes written here and read back by update_f.
-template <int KT, int TI, typename TO>
-__global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
+template <int TI> struct GrShape {
+    static constexpr int BM = 32 * TI;
+    static constexpr int KTILE = TI == 2 ? 16 : 8;
+    static constexpr int LS = TI == 2 ? 129 : 130;
+    static constexpr int LDS_DOUBLES = KTILE * LS;   // per operand
+};
+
+// One (32*TI) x 128 output tile at rows i0.., columns j0..; As / Bs hold GrShape<TI>::LDS_DOUBLES doubles each.
+// SYM: the output is a symmetric matrix (same rows on both sides, out[i][j] at i*ldo + j): every value is also
+// written to its mirror position, so that tiles below the diagonal need no workgroup.  kappa(a, b) and kappa(b, a)
+// are the same bits: the products of the dot product commute, their order does not change, and the self dot
+// products enter as a commutative sum.
+template <int KT, int TI, typename TO, bool SYM = false>
+__device__ __forceinline__ void get_rows_tile(
     const double *__restrict__ x, int64_t ldx, const int *__restrict__ x_idx, int64_t n, int d,
     const double *__restrict__ sd_x, const double *__restrict__ a, int64_t lda, const int *__restrict__ a_idx, int m,
     const double *__restrict__ sd_a, KernelParam kp_in, TO *__restrict__ out, const int *__restrict__ out_slots,
-    int64_t ldo, unsigned m_blocks, const int *__restrict__ m_dev) {
-    constexpr int BM = 32 * TI;
-    constexpr int KTILE = TI == 2 ? 16 : 8;
-    constexpr int LS = TI == 2 ? 129 : 130;
+    int64_t ldo, int i0, int j0, double *__restrict__ As, double *__restrict__ Bs, const uint64_t *__restrict__ exp_tab) {
+    constexpr int BM = GrShape<TI>::BM;
+    constexpr int KTILE = GrShape<TI>::KTILE;
+    constexpr int LS = GrShape<TI>::LS;
     constexpr int A_TPR = 256 / BM;           // threads per A row
     constexpr int A_VEC = KTILE / 4 / A_TPR;  // 4-double vectors per thread for the A tile
     constexpr int B_VEC = KTILE / 8;          // 4-double vectors per thread for the B tile (2 threads per row)
-    __shared__ double As[KTILE * LS];
-    __shared__ double Bs[KTILE * LS];
-    __shared__ uint64_t exp_tab[32];
     KernelParam kp = kp_in;
     kp.kernel_type = KT;
 
@@ -61,17 +70,6 @@ __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int wi = wave >> 1, wj = wave & 1;
-    if (tid < 32) exp_tab[tid] = TSVM_EXP2F_TAB[tid];
-    __syncthreads();
-
-    const unsigned logical = xcd_remap(blockIdx.x, gridDim.x);
-    const int j0 = (int) (logical / m_blocks) * GR_BN;   // n fits 31 bits (checked by the host)
-    const int i0 = (int) (logical % m_blocks) * BM;
-    if (m_dev) {
-        // the number of working rows is only known on the device (m sized the grid): workgroups beyond it leave
-        m = *m_dev;
-        if (i0 >= m) return;
-    }
     const int n_last = (int) n - 1, m_last = m - 1;
 
     // Staging assignment.  Rows beyond the tile's valid range are clamped to the last valid row: what they
@@ -202,8 +200,11 @@ __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
             for (int v = 0; v < 4; ++v) {
                 TO *orow = out + orow_off[ti * 4 + v] + jb;
 #pragma unroll
-                for (int tj = 0; tj < 4; ++tj)
-                    orow[tj * 16] = tsvm_epilogue_as<TO>(acc[ti][tj][v], sdi[ti * 4 + v], sdj[tj], kp, exp_tab);
+                for (int tj = 0; tj < 4; ++tj) {
+                    const TO val = tsvm_epilogue_as<TO>(acc[ti][tj][v], sdi[ti * 4 + v], sdj[tj], kp, exp_tab);
+                    orow[tj * 16] = val;
+                    if (SYM) out[(int64_t) (jb + tj * 16) * ldo + (i0 + wi * (16 * TI) + ti * 16 + 4 * v + lk)] = val;
+                }
             }
         }
     } else {
@@ -216,10 +217,59 @@ __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
                 TO *orow = out + orow_off[ti * 4 + v] + jb;
 #pragma unroll
                 for (int tj = 0; tj < 4; ++tj)
-                    if (jb + tj * 16 < n) orow[tj * 16] = tsvm_epilogue_as<TO>(acc[ti][tj][v], sdi[ti * 4 + v], sdj[tj], kp, exp_tab);
+                    if (jb + tj * 16 < n) {
+                        const TO val = tsvm_epilogue_as<TO>(acc[ti][tj][v], sdi[ti * 4 + v], sdj[tj], kp, exp_tab);
+                        orow[tj * 16] = val;
+                        if (SYM) out[(int64_t) (jb + tj * 16) * ldo + i] = val;
+                    }
             }
         }
     }
+}
+
+template <int KT, int TI, typename TO>
+__global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
+    const double *__restrict__ x, int64_t ldx, const int *__restrict__ x_idx, int64_t n, int d,
+    const double *__restrict__ sd_x, const double *__restrict__ a, int64_t lda, const int *__restrict__ a_idx, int m,
+    const double *__restrict__ sd_a, KernelParam kp, TO *__restrict__ out, const int *__restrict__ out_slots,
+    int64_t ldo, unsigned m_blocks, const int *__restrict__ m_dev) {
+    __shared__ double As[GrShape<TI>::LDS_DOUBLES];
+    __shared__ double Bs[GrShape<TI>::LDS_DOUBLES];
+    __shared__ uint64_t exp_tab[32];
+    if (threadIdx.x < 32) exp_tab[threadIdx.x] = TSVM_EXP2F_TAB[threadIdx.x];
+    __syncthreads();
+    const unsigned logical = xcd_remap(blockIdx.x, gridDim.x);
+    const int j0 = (int) (logical / m_blocks) * GR_BN;   // n fits 31 bits (checked by the host)
+    const int i0 = (int) (logical % m_blocks) * GrShape<TI>::BM;
+    if (m_dev) {
+        // the number of working rows is only known on the device (m sized the grid): workgroups beyond it leave
+        m = *m_dev;
+        if (i0 >= m) return;
+    }
+    get_rows_tile<KT, TI, TO>(x, ldx, x_idx, n, d, sd_x, a, lda, a_idx, m, sd_a, kp, out, out_slots, ldo, i0, j0, As, Bs, exp_tab);
+}
+
+// The m x m block K(x_idx[r], x_idx[t]) (a == x, a_idx == x_idx, rows written in place): tiles that lie below the
+// diagonal are filled by the mirror writes of the others and get no workgroup.  Column tile j (128 wide) needs the
+// 64-row tiles 0 .. 2j+1, so workgroup c works on column tile j = the largest j with j(j+1) <= c, row tile
+// c - j(j+1); dealt out in this order, every XCD gets the same share of the work.
+template <int KT>
+__global__ __launch_bounds__(256, 3) void get_rows_dense_sym_kernel(
+    const double *__restrict__ x, int64_t ldx, const int *__restrict__ idx, int m, int d, const double *__restrict__ sd_x,
+    KernelParam kp, double *__restrict__ out, int64_t ldo, unsigned m_blocks) {
+    __shared__ double As[GrShape<2>::LDS_DOUBLES];
+    __shared__ double Bs[GrShape<2>::LDS_DOUBLES];
+    __shared__ uint64_t exp_tab[32];
+    const int c = (int) blockIdx.x;
+    int jt = (int) ((sqrtf(4.0f * (float) c + 1.0f) - 1.0f) * 0.5f);
+    while (jt > 0 && jt * (jt + 1) > c) --jt;
+    while ((jt + 1) * (jt + 2) <= c) ++jt;
+    const int j0 = jt * GR_BN;
+    const int i0 = (c - jt * (jt + 1)) * GrShape<2>::BM;
+    if (i0 >= m) return;               // (the last column tile has fewer row tiles when m is not a multiple of 128)
+    if (threadIdx.x < 32) exp_tab[threadIdx.x] = TSVM_EXP2F_TAB[threadIdx.x];
+    __syncthreads();
+    get_rows_tile<KT, 2, double, true>(x, ldx, idx, m, d, sd_x, x, ldx, idx, m, sd_x, kp, out, nullptr, ldo, i0, j0, As, Bs, exp_tab);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -536,7 +586,33 @@ static int get_rows_dense(const double *x, int64_t ldx, const int *x_idx, int64_
     const unsigned m_blocks = (unsigned) ((m + 32 * ti - 1) / (32 * ti));
     const int64_t n_blocks = (n + GR_BN - 1) / GR_BN;
     TSVM_REQUIRE(n_blocks * m_blocks < (int64_t) 0x7fffffff, "tsvm_get_rows_dense: grid too large");
-    const dim3 grid((unsigned) (n_blocks * m_blocks)), block(256);
+    dim3 grid((unsigned) (n_blocks * m_blocks)), block(256);
+    // the solver's ws x ws block: symmetric, computed from the tiles on and above the diagonal
+    const bool sym = x == a && ldx == lda && x_idx && x_idx == a_idx && n == m && sd_x == sd_a && !out_slots && !m_dev &&
+                     row_type == TSVM_ROW_F64 && ti == 2 && ldo >= n;
+    if (sym) {
+        grid = dim3((unsigned) (n_blocks * (n_blocks + 1)));   // column tile j: row tiles 0 .. 2j+1
+        switch (kernel_type) {
+            case TSVM_LINEAR:
+                hipLaunchKernelGGL(get_rows_dense_sym_kernel<TSVM_LINEAR>, grid, block, 0, tsvm_s(stream), x, ldx, x_idx, m, d, sd_x,
+                                   kp, (double *) out, ldo, m_blocks);
+                break;
+            case TSVM_POLY:
+                hipLaunchKernelGGL(get_rows_dense_sym_kernel<TSVM_POLY>, grid, block, 0, tsvm_s(stream), x, ldx, x_idx, m, d, sd_x, kp,
+                                   (double *) out, ldo, m_blocks);
+                break;
+            case TSVM_SIGMOID:
+                hipLaunchKernelGGL(get_rows_dense_sym_kernel<TSVM_SIGMOID>, grid, block, 0, tsvm_s(stream), x, ldx, x_idx, m, d, sd_x,
+                                   kp, (double *) out, ldo, m_blocks);
+                break;
+            default:
+                hipLaunchKernelGGL(get_rows_dense_sym_kernel<TSVM_RBF>, grid, block, 0, tsvm_s(stream), x, ldx, x_idx, m, d, sd_x, kp,
+                                   (double *) out, ldo, m_blocks);
+                break;
+        }
+        TSVM_LAUNCH_CHECK();
+        return 0;
+    }
 #define GR_LAUNCH_T(KTYPE, TO)                                                                                        \
     do {                                                                                                              \
         if (ti == 2)                                                                                                  \

@@ -536,7 +536,7 @@ struct SolveTask::Impl {
         block_on_solver_cus = false;
         if (!on_one_stream && alone && block_first && k_mat.dense_layout() && !all_cached) {
             const double per_value = 2.0 * ((k_mat.n_features() + 15) / 16 * 16) / 6.6e13;   // seconds on the whole chip
-            const double t_block = per_value * 32.0 * ws_size * (double) ws_size;           // on 8 of 256 CUs
+            const double t_block = per_value * 32.0 * 0.56 * ws_size * (double) ws_size;   // on 8 of 256 CUs; 72 of its 128 tiles
             const double t_rows = per_value * (double) last_rows_computed * n_u;
             block_on_solver_cus = t_block + 0.4e-3 <= t_rows;
         }
