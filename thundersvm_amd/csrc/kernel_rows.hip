@@ -469,7 +469,27 @@ __global__ __launch_bounds__(SK_T) void sum_kernel_values_kernel(
             double part[SK_R];
 #pragma unroll
             for (int rr = 0; rr < SK_R; ++rr) part[rr] = 0.0;
-            for (int l = tid; l < cnt; l += SK_T) {
+            // four support vectors per thread at a time: their loads go out together, the sums keep their order
+            int l = tid;
+            for (; l + 3 * SK_T < cnt; l += 4 * SK_T) {
+                double cv[4];
+                TK kv[4][SK_R];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    cv[u] = cf[l + u * SK_T];
+#pragma unroll
+                    for (int rr = 0; rr < SK_R; ++rr) {
+                        const int64_t r = r0 + rr < n_instances ? r0 + rr : n_instances - 1;   // a valid row; not added below
+                        kv[u][rr] = k_mat[r * ldk + st + l + u * SK_T];
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+#pragma unroll
+                    for (int rr = 0; rr < SK_R; ++rr)
+                        if (r0 + rr < n_instances) part[rr] = __builtin_fma(cv[u], (double) kv[u][rr], part[rr]);
+            }
+            for (; l < cnt; l += SK_T) {
                 const double cv = cf[l];
 #pragma unroll
                 for (int rr = 0; rr < SK_R; ++rr) {
