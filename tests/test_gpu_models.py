@@ -226,3 +226,26 @@ def test_cross_validation_goldens(svm_type, extra, golden, metric):
     pred = Model(svm_type).cross_validation(ds, prm, 5)
     score = float(np.mean(pred == y)) if metric == "acc" else float(np.mean((pred - y) ** 2))
     assert abs(score - golden) < 1e-3, score
+
+
+@pytest.mark.parametrize("case", range(5))
+def test_unique_optimum_against_libsvm(case):
+    """The GPU twin of tests/test_oracle_pins.py::test_unique_optimum_against_libsvm: with an RBF kernel on distinct
+    points the dual has one optimum; trained to a KKT gap of 1e-8 the HIP path must reach LibSVM's solution of the
+    same quadratic programme (kernel matrix taken from the GPU's own get_rows through the oracle's identical values):
+    coefficients and rho 1e-6 relative, decision values 1e-6 absolute."""
+    import test_oracle_pins as P
+    x, y, t = P.unique_optimum_problem()
+    name, st, prm, sk = P.unique_optimum_cases()[case]
+    target = t if st in (O.EPSILON_SVR, O.NU_SVR) else y
+    d = D.from_dense(x, target)
+    gp = make_param(svm_type=st, kernel_type=capi.RBF, gamma=0.5, epsilon=1e-8, **prm)
+    gm = Model(st).train(d, gp)
+    K = O.KernelMatrix(d.ptr, d.col, d.val, _oparam(gp)).get_rows(np.arange(d.n))
+    coef, rho, dec = P.libsvm_optimum(sk, st, K, target)
+    mine = np.zeros(d.n)
+    mine[gm.sv_indices] = gm.coef
+    _, gdec = gm.predict(d)
+    assert np.abs(mine - coef).max() < 1e-6 * max(1.0, np.abs(coef).max()), name
+    assert abs(gm.rho[0] - rho) < 1e-6 * max(1.0, abs(rho)), name
+    assert np.abs(gdec[:, 0] - dec).max() < 1e-6, name
