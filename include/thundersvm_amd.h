@@ -161,6 +161,16 @@ int tsvm_c_smo_solve(const int *y, const double *f_val, double *alpha, double *a
                      const double *k_diag, double eps, double *diff, int max_iter, void *workspace,
                      tsvm_stream stream);
 
+/* tsvm_c_smo_solve without a workspace argument, for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * The ws x ws block goes into a static device array of 1024 x 1024 doubles (8 MiB per device, held until the
+ * process ends); ws_size > 1024 is rejected with TSVM_EINVAL.  The call allocates and frees nothing.  Every call on
+ * a device shares that device's array: calls that overlap on one device (different streams or threads) race, the
+ * caller has to order them.  Results are those of tsvm_c_smo_solve. */
+int tsvm_c_smo_solve_static(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
+                            int ws_size, double Cp, double Cn, const void *k_rows, int row_type, const int *slots,
+                            int64_t ld, const double *k_diag, double eps, double *diff, int max_iter, tsvm_stream stream);
+
 /* Row stride (in doubles) of the ws x ws block the solver kernels read: ws rounded up to 256, 512 or 1024. */
 int tsvm_smo_solve_block_ld(int ws_size);
 

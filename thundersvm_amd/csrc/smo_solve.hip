@@ -26,6 +26,8 @@
 #include "tsvm_device.h"
 #include "tsvm_internal.h"
 
+#include <mutex>
+
 #define TSVM_INF __builtin_inf()
 #define MAX_WS 1024
 #define SV_T 256           // threads of the solver workgroup
@@ -561,6 +563,52 @@ int tsvm_c_smo_solve(const int *y, const double *f_val, double *alpha, double *a
     int rc = launch_gather(k_rows, row_type, slots, ld, working_set, ws_size, workspace, s);
     if (rc) return rc;
     const double *kws = (const double *) workspace;
+    TSVM_DISPATCH_E(c_smo_solve_kernel, y, f_val, alpha, alpha_diff, working_set, ws_size, Cp, Cn, kws, k_diag, eps, diff,
+                    max_iter);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+// c_smo_solve for callers that cannot allocate: the ws x ws block that tsvm_c_smo_solve gathers into the caller's
+// workspace goes into a file-scope device array instead (8 MiB, held by every device the library runs on until the
+// process ends).  Its device address is looked up once per device; host code never uses the array's name otherwise.
+static __device__ __align__(256) double g_solver_block[(size_t) MAX_WS * MAX_WS];
+#define TSVM_MAX_DEVICES 64
+static double *g_solver_block_ptr[TSVM_MAX_DEVICES];
+static std::mutex g_solver_block_mutex;
+
+static int solver_block_address(double **out) {
+    int dev = 0;
+    TSVM_HIP(hipGetDevice(&dev));
+    TSVM_REQUIRE(dev >= 0 && dev < TSVM_MAX_DEVICES, "tsvm_c_smo_solve_static: device ordinal %d outside [0, %d)", dev,
+                 TSVM_MAX_DEVICES);
+    std::lock_guard<std::mutex> lock(g_solver_block_mutex);
+    if (!g_solver_block_ptr[dev]) {
+        double *p = nullptr;
+        TSVM_HIP(hipGetSymbolAddress((void **) &p, HIP_SYMBOL(g_solver_block)));
+        TSVM_REQUIRE(p != nullptr, "tsvm_c_smo_solve_static: no device address for the static block");
+        g_solver_block_ptr[dev] = p;
+    }
+    *out = g_solver_block_ptr[dev];
+    return 0;
+}
+
+int tsvm_c_smo_solve_static(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
+                            int ws_size, double Cp, double Cn, const void *k_rows, int row_type, const int *slots, int64_t ld,
+                            const double *k_diag, double eps, double *diff, int max_iter, tsvm_stream stream) {
+    TSVM_REQUIRE(y && f_val && alpha && alpha_diff && working_set && k_rows && k_diag && diff,
+                 "tsvm_c_smo_solve_static: null pointer");
+    TSVM_REQUIRE(ws_size >= 1 && ws_size <= MAX_WS, "tsvm_c_smo_solve_static: ws_size %d outside [1, %d] (the static block holds %d x %d values)",
+                 ws_size, MAX_WS, MAX_WS, MAX_WS);
+    double *block = nullptr;
+    int rc = solver_block_address(&block);
+    if (rc) return rc;
+    hipStream_t s = tsvm_s(stream);
+    // the gather writes every element of the ws x ldk block the solver reads (columns beyond ws as zeros), so
+    // nothing of the previous call's content is read
+    rc = launch_gather(k_rows, row_type, slots, ld, working_set, ws_size, block, s);
+    if (rc) return rc;
+    const double *kws = block;
     TSVM_DISPATCH_E(c_smo_solve_kernel, y, f_val, alpha, alpha_diff, working_set, ws_size, Cp, Cn, kws, k_diag, eps, diff,
                     max_iter);
     TSVM_LAUNCH_CHECK();
