@@ -66,6 +66,13 @@ int tsvm_kernel_diag(const double *self_dot, int64_t n, int kernel_type, double 
 int tsvm_csr_to_dense(const double *val, const int *col, const int64_t *row_ptr, int64_t n, double *x, int64_t ld,
                       tsvm_stream stream);
 
+/* Column statistics of the data rows (dense row-major [n][ld], columns 0..d-1; or the nnz stored entries of a CSR
+ * matrix with column ids below d): counts[c] = entries of column c (dense: non-zero values; CSR: stored entries),
+ * counts[d + c] = how many values of the column are neither 0 nor 1.  counts holds 2*d ints and is cleared by the call.  The per-column entry counts are what the reference's
+ * KernelMatrix constructor splits the matrix by (CSR_DenseCSR, kernelmatrix.cpp:16-74). */
+int tsvm_column_stats_dense(const double *x, int64_t ld, int64_t n, int d, int *counts, tsvm_stream stream);
+int tsvm_column_stats_csr(const double *val, const int *col, int64_t nnz, int d, int *counts, tsvm_stream stream);
+
 /* Dense get_rows: out[s_i*ldo + j] = kappa(a_i, x_j), i < m, j < n, where a_i is row a_idx[i] of `a`
  * (a_idx == NULL: row i) and s_i = out_slots[i] (out_slots == NULL: i) is the output row, so new kernel
  * rows can be written straight into the slots of a row cache.  x_idx != NULL restricts the columns to

@@ -85,9 +85,10 @@ int tsvm_model_get(void *model, int *label, int *n_sv, double *rho, double *coef
                    int *sv_col, double *sv_val);
 
 /* Solver diagnostics of binary sub-problem k: outer iterations, inner iterations, objective and
- * phase[10]: device milliseconds of select, get_rows, local solve, update_f (zeros unless profiled),
+ * phase[11]: device milliseconds of select, get_rows, local solve, update_f (zeros unless profiled),
  * then kernel-row cache lookups, hits, capacity in rows, 1 if the cache was switched off, and the host
- * wall-clock milliseconds of the whole solve and of its set-up (allocations, uploads, init_f). */
+ * wall-clock milliseconds of the whole solve and of its set-up (allocations, uploads, init_f), and the
+ * working-set size the problem was solved with. */
 int tsvm_model_stats(void *model, int k, int64_t *n_iter, int64_t *local_iter, double *obj, double *phase_ms);
 
 int64_t tsvm_model_binary_size(void *model, int k);
@@ -110,6 +111,17 @@ int tsvm_cmdparser_train(int argc, char **argv, tsvm_param *param, int *gamma_se
 /* Frees the device allocation that holds kernel rows between solves (it is otherwise kept until the
  * process ends, because releasing it costs up to seconds). */
 int tsvm_release_device_cache(void);
+
+/* Self-test of the host's bounded wait for the local solver's report (no device needed): waits on a word that
+ * nobody writes, with a stream that reports "still running", and returns 0 when the wait gave up with its
+ * time-out error after timeout_ms (within a second of it), -1 otherwise.  never_written != 0 makes the stream
+ * report "drained" instead: the wait must then fail with its "finished without reporting" error at once. */
+int tsvm_selftest_solver_wait(int timeout_ms, int never_written);
+
+/* Self-test of the device buffer type that stands in for the reference's SyncArray (needs a device): byte
+ * accounting on allocation, resize, move and destruction, and an upload / download round trip; the cases of
+ * src/test/test_syncmem.cpp and test_syncarray.cpp that apply.  0 on success, -1 with a message otherwise. */
+int tsvm_selftest_device_buffer(void);
 
 int tsvm_model_save(void *model, const char *path);
 int tsvm_model_load(void *model, const char *path);

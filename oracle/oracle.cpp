@@ -763,6 +763,7 @@ struct OrcModel {
     vector<double> sv_val;
     // per binary problem diagnostics
     vector<long long> n_iter, local_iter;
+    vector<int> ws_size;        // working-set size of every binary problem
     vector<double> obj;
     vector<vector<double>> alpha_bin;  // signed alpha of every binary problem (alpha*y), training order
     vector<vector<double>> f_bin;
@@ -784,21 +785,59 @@ struct Csr {
     }
 };
 
-// Bytes the reference's SyncMem counter holds when get_working_set_size runs in a CPU build:
-// the KernelMatrix arrays (val, col_ind, row_ptr, self_dot, diag; kernelmatrix.cpp:211-226) plus y,
-// alpha and f.  The dense/sparse column partition buffers (kernelmatrix.cpp:16-181) are not
-// restated; with the default 8192 MiB budget they cannot change the result for n + n_features
-// below ~5e5 and every caller here passes the resulting size explicitly when it matters.
-static long long tally_bytes(long long nnz, long long n) {
-    return nnz * 12 + (n + 1) * 4 + n * 8 * 2 + n * (4 + 8 + 8);
+// Bytes the reference's SyncMem counter (syncmem.cpp:58-108: every array counts once, when its host side is first
+// touched) holds when get_working_set_size runs in train_binary of a CPU build (svc.cpp:147-166):
+//   * the KernelMatrix arrays val_, col_ind_, row_ptr_, self_dot_, diag_ (kernelmatrix.cpp:211-226);
+//   * the two parts CSR_DenseCSR splits the columns into (kernelmatrix.cpp:16-181): columns are ordered by entry
+//     count (ties by index) and moved to the sparse part one by one until the part would be more than 5 % full,
+//     the column more than 50 % full, or four times the part's entries exceed the cells left to the dense part;
+//     the dense part is an m x densecol array, the sparse part a CSR (built only if some value lies outside the
+//     dense part);
+//   * y (int), alpha and f (double) of the problem;
+//   * `held`: what the model keeps from earlier problems (the alpha arrays of earlier class pairs, svc.cpp:50-61).
+// Small model members (rho, n_sv, label) are left out.
+static long long partition_bytes(long long m, long long n_features, const long long *ptr, const int *col, const double *val) {
+    vector<long long> col_num((size_t) n_features, 0);
+    for (long long e = 0; e < ptr[m]; ++e) col_num[col[e]]++;
+    vector<int> col_indices((size_t) n_features);
+    for (long long i = 0; i < n_features; ++i) col_indices[i] = (int) i;
+    std::sort(col_indices.begin(), col_indices.end(), [&](int a, int b) {
+        return col_num[a] != col_num[b] ? col_num[a] < col_num[b] : a < b;
+    });
+    vector<char> densefg((size_t) n_features, 1);
+    long long densecolnum = n_features, total_csr = 0, total_dense = m * n_features, row_sum_num = 0;
+    for (long long i = 0; i < n_features; ++i) {
+        total_csr += col_num[col_indices[i]];
+        total_dense -= m;
+        row_sum_num += m;
+        long double ratio = 1.0l * total_csr / row_sum_num;
+        if (ratio > 0.05 || 1.0l * col_num[col_indices[i]] / m > 0.5 || total_csr * 4 > total_dense) break;
+        densecolnum--;
+        densefg[col_indices[i]] = 0;
+    }
+    long long bytes = 0, dense_data_count = 0, sparse_entries = 0;
+    for (long long e = 0; e < ptr[m]; ++e) {
+        if (densefg[col[e]]) dense_data_count += val[e] != 0;
+        else sparse_entries++;
+    }
+    if (densecolnum > 0) bytes += m * densecolnum * 8;
+    if (densecolnum < n_features && dense_data_count != ptr[m]) bytes += sparse_entries * 12 + (m + 1) * 4;
+    return bytes;
+}
+
+static long long tally_bytes(const Csr &ins, long long n_features, long long held) {
+    const long long n = ins.rows(), nnz = (long long) ins.col.size();
+    return nnz * 12 + (n + 1) * 4 + n * 8 * 2 + partition_bytes(n, n_features, ins.ptr.data(), ins.col.data(), ins.val.data()) +
+           n * (4 + 8 + 8) + held;
 }
 
 static void train_binary_generic(OrcModel &m, const Csr &ins, vector<int> &y, vector<double> &alpha,
                                  vector<double> &f, double Cp, double Cn, bool nu, bool for_svr, double *rho,
-                                 int ws_override, bool want_trace) {
+                                 int ws_override, bool want_trace, long long held = 0) {
     OrcKernelMatrix *k = km_build(ins.rows(), ins.ptr.data(), ins.col.data(), ins.val.data(), m.param);
     int ws = ws_override > 0 ? ws_override
-                             : working_set_size(k->n, k->n_features, m.param.max_mem_size, tally_bytes(k->nnz, k->n));
+                             : working_set_size(k->n, k->n_features, m.param.max_mem_size, tally_bytes(ins, k->n_features, held));
+    m.ws_size.push_back(ws);
     OrcTrace tr;
     if (want_trace) {
         tr.cap_iters = 4096;
@@ -955,6 +994,7 @@ void *orc_train(int n, const long long *ptr, const int *col, const double *val, 
         vector<vector<double>> alpha(m->n_binary_models);
         vector<char> is_sv(n, 0);
         int k = 0;
+        long long held = 0;
         for (int i = 0; i < nc; ++i) {
             for (int j = i + 1; j < nc; ++j) {
                 Csr ins;
@@ -970,7 +1010,7 @@ void *orc_train(int n, const long long *ptr, const int *col, const double *val, 
                     for (int l = 0; l < count[i]; ++l) { y[l] = +1; f[l] = -1; }
                     for (int l = 0; l < count[j]; ++l) { y[count[i] + l] = -1; f[count[i] + l] = +1; }
                     train_binary_generic(*m, ins, y, alpha[k], f, param.C * c_weight[i], param.C * c_weight[j], false,
-                                         false, &m->rho[k], ws_override, want_trace && k == 0);
+                                         false, &m->rho[k], ws_override, want_trace && k == 0, held);
                 } else {
                     // NuSVC::train_binary (nusvc.cpp:7-45)
                     double sum_pos = param.nu * nn / 2;
@@ -978,8 +1018,9 @@ void *orc_train(int n, const long long *ptr, const int *col, const double *val, 
                     for (int l = 0; l < count[i]; ++l) { y[l] = +1; alpha[k][l] = std::min(1., sum_pos); sum_pos -= alpha[k][l]; }
                     for (int l = 0; l < count[j]; ++l) { y[count[i] + l] = -1; alpha[k][count[i] + l] = std::min(1., sum_neg); sum_neg -= alpha[k][count[i] + l]; }
                     train_binary_generic(*m, ins, y, alpha[k], f, 1, 1, true, false, &m->rho[k], ws_override,
-                                         want_trace && k == 0);
+                                         want_trace && k == 0, held);
                 }
+                held += 8LL * nn;   // alpha[k] stays allocated until the coefficients are assembled (svc.cpp:50-61)
                 for (int l = 0; l < nn; ++l) alpha[k][l] *= y[l];
                 for (int l = 0; l < nn; ++l) is_sv[original_index[l]] = is_sv[original_index[l]] || (alpha[k][l] != 0);
                 m->alpha_bin.push_back(alpha[k]);
@@ -1097,6 +1138,13 @@ void orc_model_binary_get(void *mp, int k, double *alpha_signed, double *f) {
     OrcModel *m = (OrcModel *) mp;
     if (alpha_signed) memcpy(alpha_signed, m->alpha_bin[k].data(), sizeof(double) * m->alpha_bin[k].size());
     if (f) memcpy(f, m->f_bin[k].data(), sizeof(double) * m->f_bin[k].size());
+}
+int orc_model_ws_size(void *mp, int k) { return ((OrcModel *) mp)->ws_size.at(k); }
+// the restated SyncMem counter for one problem given as CSR (n rows, feature ids < n_features)
+long long orc_reference_bytes(int n, const long long *ptr, const int *col, const double *val, int n_features, long long held) {
+    Csr ins;
+    for (int r = 0; r < n; ++r) ins.push_row(ptr, col, val, r);
+    return tally_bytes(ins, n_features, held);
 }
 int orc_model_trace(void *mp, int *ws_size, const double **diff, const int **ws) {
     OrcModel *m = (OrcModel *) mp;

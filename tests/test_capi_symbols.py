@@ -73,3 +73,13 @@ def test_no_cpu_fallback():
     w = D.workload_c1(0.05)
     with pytest.raises((capi.TsvmError, MemoryError)):
         model.Model(0).train(w["train"], model.make_param(**w["params"]))
+
+
+def test_bounded_wait_for_the_local_solver():
+    """The host's wait for the solver's report gives up with an error instead of spinning for ever (host only:
+    the word is never written, no kernel is involved)."""
+    lib = model.host_lib()
+    assert lib.tsvm_selftest_solver_wait(300, 0) == 0, lib.tsvm_model_last_error()
+    assert b"TSVM_SOLVER_TIMEOUT_MS" in lib.tsvm_model_last_error()
+    assert lib.tsvm_selftest_solver_wait(60000, 1) == 0, lib.tsvm_model_last_error()
+    assert b"without reporting" in lib.tsvm_model_last_error()

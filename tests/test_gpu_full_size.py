@@ -114,3 +114,116 @@ def test_c5_full_size_epsilon_svr():
     ref = _oracle_decision(gm, prm, ts)
     assert np.abs(dec_t[:, 0] - ref).max() < 1e-6
     assert np.abs(val_t - ref).max() < 1e-6
+
+
+def _check_binary_problem(a, f, ysub, Cp, Cn, eps, rho):
+    """Dual constraints, the stopping rule on the returned f and rho of one C-SVC sub-problem (alpha*y and f in the
+    sub-problem's own order)."""
+    alpha = a * ysub
+    cmax = np.where(ysub > 0, Cp, Cn)
+    assert alpha.min() >= 0 and np.all(alpha <= cmax)
+    assert abs(a.sum()) < 1e-9 * max(Cp, Cn) * max(1.0, np.count_nonzero(a) ** 0.5)
+    up = ((ysub > 0) & (alpha < cmax)) | ((ysub < 0) & (alpha > 0))
+    low = ((ysub > 0) & (alpha > 0)) | ((ysub < 0) & (alpha < cmax))
+    assert f[low].max() - f[up].min() < eps
+    free = (alpha > 0) & (alpha < cmax)
+    if free.any():
+        assert abs(rho - f[free].mean()) < 1e-9
+    else:
+        assert abs(rho + (f[up].min() + f[low].max()) / 2) < 1e-9
+    return alpha, free
+
+
+@pytest.mark.parametrize("kernel", ["rbf", "linear"])
+def test_c3_full_size_sparse_csvc(kernel):
+    """72,000 x 20,958 CSR rows through the sparse get_rows kernel, both kernels of the benchmark configuration."""
+    w = D.workload_c3(kernel=kernel)
+    tr, p = w["train"], w["params"]
+    prm = make_param(**p)
+    eps, C_ = prm.epsilon, p["C"]
+    gm = Model(0).train(tr, prm, keep_binary=True)
+    a, f = gm.binary(0)
+    n = tr.n
+    lab0, lab1 = gm.label
+    perm = np.concatenate([np.flatnonzero(tr.y == lab0), np.flatnonzero(tr.y == lab1)])
+    ysub = np.concatenate([np.ones((tr.y == lab0).sum()), -np.ones((tr.y == lab1).sum())])
+    alpha, free = _check_binary_problem(a, f, ysub, C_, C_, eps, gm.rho[0])
+    assert free.any() and gm.total_sv == int((alpha > 0).sum())
+    # f from scratch on a sample of instances, by the oracle's kernel rows
+    rng = np.random.default_rng(7)
+    pick = rng.choice(n, 48, replace=False)
+    km = O.KernelMatrix(tr.ptr, tr.col, tr.val, _oparam(prm))
+    a_orig = np.zeros(n)
+    a_orig[perm] = a
+    f_ref = km.get_rows(perm[pick]) @ a_orig - ysub[pick]
+    np.testing.assert_allclose(f[pick], f_ref, rtol=0, atol=1e-8)
+    # Karush-Kuhn-Tucker conditions of every training instance, from the model's own predictions
+    lab, dec = gm.predict(tr)
+    margin = ysub * dec[perm, 0]
+    tol = eps + 1e-6
+    assert np.all(margin[alpha == 0] >= 1 - tol)
+    assert np.all(np.abs(margin[free] - 1) <= tol)
+    assert np.all(margin[alpha == C_] <= 1 + tol)
+    # decision values of sampled rows against the oracle's kernel sum over the model's support vectors
+    ts = tr.rows(rng.choice(n, 96, replace=False))
+    lab_t, dec_t = gm.predict(ts)
+    ref = _oracle_decision(gm, prm, ts)
+    assert np.abs(dec_t[:, 0] - ref).max() < 1e-6
+    assert np.array_equal(lab_t, np.where(ref > 0, lab0, lab1))
+
+
+def test_c4_full_size_seven_class_csvc():
+    """500,000 x 54, 21 class pairs solved two at a time with slices of the row arena: the six largest pairs run with a
+    partial row cache, the others with every row stored."""
+    w = D.workload_c4(n_test=4000)
+    tr, te, p = w["train"], w["test"], w["params"]
+    prm = make_param(**p)
+    eps, C_ = prm.epsilon, p["C"]
+    gm = Model(0).train(tr, prm, keep_binary=True)
+    k = len(gm.label)
+    assert k == 7 and gm.n_binary == 21
+    groups = [np.flatnonzero(tr.y == c) for c in gm.label]      # grouped order: classes by first appearance
+    rng = np.random.default_rng(8)
+    is_sv = np.zeros(tr.n, dtype=bool)
+    b = 0
+    partial = 0
+    for i in range(k):
+        for j in range(i + 1, k):
+            a, f = gm.binary(b)
+            ids = np.concatenate([groups[i], groups[j]])
+            ysub = np.concatenate([np.ones(len(groups[i])), -np.ones(len(groups[j]))])
+            assert len(a) == len(ids)
+            alpha, free = _check_binary_problem(a, f, ysub, C_, C_, eps, gm.rho[b])
+            is_sv[ids[alpha > 0]] = True
+            st = gm.stats(b)
+            assert st["ws_size"] == 1024 and st["n_iter"] >= 1
+            partial += 0 < st["cache_rows"] < len(ids)
+            # f from scratch on a few instances of the pair, by the oracle's kernel rows over the pair's rows
+            sub = tr.rows(ids)
+            km = O.KernelMatrix(sub.ptr, sub.col, sub.val, _oparam(prm))
+            pick = rng.choice(len(ids), 6, replace=False)
+            f_ref = km.get_rows(pick) @ a - ysub[pick]
+            np.testing.assert_allclose(f[pick], f_ref, rtol=0, atol=1e-8)
+            b += 1
+    assert partial >= 1                                          # the large pairs did run with a partial cache
+    assert gm.total_sv == int(is_sv.sum())
+    assert np.array_equal(gm.sv_indices, np.concatenate([g[is_sv[g]] for g in groups]))
+    # decision values of test rows against the oracle's kernel sum, and the one-vs-one vote (svc.cpp:265-288)
+    ts = te.rows(rng.choice(te.n, 128, replace=False))
+    lab, dec = gm.predict(ts)
+    km = O.KernelMatrix(gm.sv_ptr, gm.sv_col, gm.sv_val, _oparam(prm))
+    kv = km.get_rows_instances(ts.ptr, ts.col, ts.val)
+    start = np.concatenate([[0], np.cumsum(gm.n_sv)[:-1]]).astype(np.int32)
+    ref = O.sum_kernel_values(gm.coef.reshape(k - 1, gm.total_sv), gm.total_sv, start, gm.n_sv, gm.rho, kv, k, ts.n)
+    assert np.abs(dec - ref).max() < 1e-6
+    votes = np.zeros((ts.n, k), dtype=int)
+    b = 0
+    for i in range(k):
+        for j in range(i + 1, k):
+            votes[:, i] += ref[:, b] > 0
+            votes[:, j] += ~(ref[:, b] > 0)
+            b += 1
+    clear = np.abs(ref).min(axis=1) > 1e-6                       # rows without a decision value on the margin
+    assert np.array_equal(lab[clear], np.asarray(gm.label)[votes.argmax(axis=1)][clear])
+    lab_all, _ = gm.predict(te)
+    assert (lab_all == te.y).mean() > 0.8

@@ -216,10 +216,10 @@ def test_out_of_range_test_features():
     assert np.array_equal(G.host(got), want)
 
 
-@pytest.mark.parametrize("n_classes,rows", [(2, 5), (3, 150), (7, 333)])
+@pytest.mark.parametrize("n_classes,rows", [(2, 5), (3, 150), (7, 333), (33, 9), (100, 6)])
 def test_sum_kernel_values(n_classes, rows):
     rng = np.random.default_rng(n_classes)
-    cnt = rng.integers(1, 300, size=n_classes).astype(np.int32)
+    cnt = rng.integers(1, 300 if n_classes <= 32 else 40, size=n_classes).astype(np.int32)
     if n_classes == 7:
         cnt[3] = 0
     start = np.concatenate([[0], np.cumsum(cnt)[:-1]]).astype(np.int32)

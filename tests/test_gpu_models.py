@@ -24,7 +24,7 @@ FIXTURE = os.path.join(os.path.dirname(__file__), "golden", "test_dataset.txt")
 def _oparam(prm):
     return O.make_param(svm_type=prm.svm_type, kernel_type=prm.kernel_type, degree=prm.degree, gamma=prm.gamma,
                         coef0=prm.coef0, C_=prm.C, nu=prm.nu, p=prm.p, epsilon=prm.epsilon, max_iter=prm.max_iter,
-                        expf_mode=1)
+                        max_mem_size=prm.max_mem_size, expf_mode=1)
 
 
 def _compare(train, test, prm, ws=0, trace=8):
@@ -249,3 +249,100 @@ def test_unique_optimum_against_libsvm(case):
     assert np.abs(mine - coef).max() < 1e-6 * max(1.0, np.abs(coef).max()), name
     assert abs(gm.rho[0] - rho) < 1e-6 * max(1.0, abs(rho)), name
     assert np.abs(gdec[:, 0] - dec).max() < 1e-6, name
+
+
+def test_more_than_32_classes():
+    """The reference's sum_kernel_values has no class limit (kernelmatrix_kernel.cpp:110-147): a 34-class model
+    (561 class pairs) trains and predicts like the oracle's."""
+    rng = np.random.default_rng(34)
+    k, per, d = 34, 10, 6
+    centres = 3.0 * rng.standard_normal((k, d))
+    cls = rng.permutation(np.repeat(np.arange(k), per))
+    x = (centres[cls] + 0.6 * rng.standard_normal((k * per, d))).astype(np.float32)
+    tr = D.from_dense(x, (cls + 1).astype(np.float64))
+    prm = make_param(svm_type=0, kernel_type=2, gamma=0.2, C=5.0)
+    gm = Model(0).train(tr, prm)
+    om = O.Model(tr.ptr, tr.col, tr.val, tr.y, _oparam(prm))
+    assert gm.n_binary == 561 and gm.total_sv == om.total_sv
+    np.testing.assert_allclose(gm.rho, om.rho, rtol=1e-6, atol=1e-12)
+    np.testing.assert_allclose(gm.coef, om.coef, rtol=1e-6, atol=1e-12)
+    glab, gdec = gm.predict(tr, 100)
+    olab, odec = om.predict(tr.ptr, tr.col, tr.val, 100)
+    assert np.abs(gdec - odec).max() < 1e-6 and np.array_equal(glab, olab)
+    assert (glab == tr.y).mean() > 0.9
+
+
+@pytest.mark.parametrize("svm_type,extra", [(3, dict(p=0.1)), (3, dict(p=0.0)), (4, dict(nu=0.4))])
+def test_cache_switched_off_mid_run_on_a_stacked_problem(svm_type, extra):
+    """A row cache that has filled up and does not hit is switched off in mid-run (rotation between two slot
+    tables from then on).  On the 2n-variable problems of SVR two working-set positions may share one stored row;
+    after the switch every position must own a slot.  Same trajectory and model as without a cache, bit for bit."""
+    w = D.workload_c5(scale=0.01)
+    tr = w["train"]
+    p = dict(w["params"], svm_type=svm_type)
+    p.update(extra)
+    res = []
+    for cache_bytes in (0, 5 << 20):
+        m = Model(svm_type).train(tr, make_param(cache_bytes=cache_bytes, **p), ws_override=64, keep_binary=True)
+        st = m.stats(0)
+        assert st["cache_disabled"] == (cache_bytes != 0) and st["n_iter"] > 64
+        res.append((m.coef.copy(), m.rho.copy(), m.sv_indices.copy(), st["n_iter"], st["local_iter"]) + m.binary(0))
+    for a, b in zip(*res):
+        assert np.array_equal(a, b)
+
+
+def _ws_sizes(model, n_binary):
+    return [model.stats(b)["ws_size"] for b in range(n_binary)]
+
+
+@pytest.mark.parametrize("kind", ["mixed_3class", "svr", "csr_text"])
+def test_working_set_size_follows_the_reference_memory_budget(kind):
+    """SvmModel::get_working_set_size (svmmodel.cpp:437-451) subtracts what the reference's SyncMem counter holds from
+    the -m budget.  With the budget set just around the point where floor(free / 8 / (n + n_features)) crosses 1024,
+    the host layer's restated counter must flip the working-set size at the same byte as the oracle's."""
+    rng = np.random.default_rng(77)
+    if kind == "mixed_3class":
+        w = D.workload_c4(scale=0.012)
+        keep = np.flatnonzero(w["train"].y <= 3)
+        tr, p = w["train"].rows(keep), dict(w["params"])
+    elif kind == "svr":
+        w = D.workload_c5(scale=0.006)
+        tr, p = w["train"], dict(w["params"])
+    else:
+        w = D.workload_c3(scale=0.035)
+        tr, p = w["train"], dict(w["params"])
+    p["max_iter"] = 2                                   # the size is decided before the first iteration
+    base = O.Model(tr.ptr, tr.col, tr.val, tr.y, _oparam(make_param(**p)))
+    nb = base.n_binary
+    L = O.lib()
+    default = [L.orc_model_ws_size(base.h, b) for b in range(nb)]
+    assert max(default) == 1024
+    # bisect the budget at which the oracle's first problem drops from 1024 to 512
+    lo, hi = 1 << 20, 8192 << 20
+    while hi - lo > 1:
+        mid = (lo + hi) // 2
+        try:
+            om = O.Model(tr.ptr, tr.col, tr.val, tr.y, _oparam(make_param(max_mem_size=mid, **p)))
+            ok = L.orc_model_ws_size(om.h, 0) == 1024
+        except Exception:
+            ok = False
+        lo, hi = (lo, mid) if ok else (mid, hi)
+    flips = 0
+    for budget in (hi - 4096, hi - 8, hi - 1, hi, hi + 1, hi + 4096, hi + (64 << 10), hi + (1 << 20)):
+        prm = make_param(max_mem_size=budget, **p)
+        om = O.Model(tr.ptr, tr.col, tr.val, tr.y, _oparam(prm))
+        gm = Model(prm.svm_type).train(tr, prm)
+        want = [L.orc_model_ws_size(om.h, b) for b in range(nb)]
+        assert _ws_sizes(gm, nb) == want, (budget - hi, _ws_sizes(gm, nb), want)
+        flips += want[0] == 1024
+    assert 0 < flips < 8
+
+
+def test_device_buffer_accounting_and_round_trip():
+    """DeviceBuffer<T>, the device-only stand-in for SyncArray<T>: the checks of the reference's
+    src/test/test_syncmem.cpp:7-50 and test_syncarray.cpp:7-60 that apply to a buffer without a host mirror
+    (allocation counted once, released on destruction and on resize, moves transfer ownership without
+    counting twice, upload -> download round trip), run inside the host library."""
+    from thundersvm_amd.model import host_lib
+    lib = host_lib()
+    assert lib.tsvm_selftest_device_buffer() == 0, lib.tsvm_model_last_error()

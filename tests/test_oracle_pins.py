@@ -167,3 +167,67 @@ def test_unique_optimum_against_libsvm(case):
     assert np.abs(mine - coef).max() < 1e-6 * max(1.0, np.abs(coef).max()), name
     assert abs(m.rho[0] - rho) < 1e-6 * max(1.0, abs(rho)), name
     assert np.abs(odec[:, 0] - dec).max() < 1e-6, name
+
+
+# ---------------------------------------------------------------------------------------------
+# The reference's SyncMem counter at get_working_set_size (svmmodel.cpp:437-451), restated in the oracle
+# ---------------------------------------------------------------------------------------------
+def _reference_bytes_brute(x, held=0):
+    """x: dense [m, nf] array whose non-zeros are the stored entries.  The column split of
+    kernelmatrix.cpp:16-74 written with running sums over the sorted column counts."""
+    m, nf = x.shape
+    cnt = (x != 0).sum(axis=0)
+    order = sorted(range(nf), key=lambda c: (cnt[c], c))
+    sparse_cols = []
+    total = 0
+    for rank, c in enumerate(order, start=1):
+        total += cnt[c]
+        cells_taken = m * rank
+        if total / cells_taken > 0.05 or cnt[c] / m > 0.5 or 4 * total > m * nf - cells_taken:
+            break
+        sparse_cols.append(c)
+    nnz = int(cnt.sum())
+    dense_cols = nf - len(sparse_cols)
+    nnz_sparse = int(cnt[sparse_cols].sum()) if sparse_cols else 0
+    b = 12 * nnz + 4 * (m + 1) + 16 * m            # val, col_ind, row_ptr, self_dot, diag
+    if dense_cols > 0:
+        b += 8 * m * dense_cols                    # dense part, m x dense_cols doubles
+    if dense_cols < nf and nnz_sparse > 0:
+        b += 12 * nnz_sparse + 4 * (m + 1)         # sparse part as CSR
+    return b + 20 * m + held                       # y, alpha, f
+
+
+def _oracle_reference_bytes(x, held=0):
+    import ctypes as Ct
+    d = from_dense(x[:, 1:])                        # column c of x = feature id c (column 0 is never used)
+    L = O.lib()
+    L.orc_reference_bytes.restype = Ct.c_longlong
+    ptr, col, val = O.csr_arrays(d.ptr, d.col, d.val)
+    return L.orc_reference_bytes(Ct.c_int(d.n), O._ptr(ptr, Ct.c_longlong), O._ptr(col, Ct.c_int), O._ptr(val, Ct.c_double),
+                                 Ct.c_int(x.shape[1]), Ct.c_longlong(held))
+
+
+def test_reference_memory_counter():
+    rng = np.random.default_rng(8)
+    m = 400
+    # hand-computed: 3 full columns + the unused column 0 -> column 0 alone goes to the sparse part (0 entries), the
+    # dense part is m x 3, no sparse CSR is built
+    x = np.zeros((m, 4), dtype=np.float32)
+    x[:, 1:] = 1 + rng.random((m, 3))
+    want = 12 * 3 * m + 4 * (m + 1) + 16 * m + 8 * m * 3 + 20 * m
+    assert _reference_bytes_brute(x) == want == _oracle_reference_bytes(x)
+    # continuous columns plus one-hot groups (the 500k x 54 benchmark's shape): the rare indicator columns go sparse
+    x = np.zeros((m, 55), dtype=np.float32)
+    x[:, 1:11] = rng.standard_normal((m, 10))
+    x[np.arange(m), 11 + rng.integers(0, 4, m)] = 1
+    x[np.arange(m), 15 + rng.integers(0, 40, m)] = 1
+    assert _reference_bytes_brute(x, 1000) == _oracle_reference_bytes(x, 1000)
+    # text-like: everything sparse but a few head columns
+    x = np.zeros((m, 300), dtype=np.float32)
+    p = 1.0 / np.arange(1, 300) ** 1.1
+    x[:, 1:] = (rng.random((m, 299)) < 6 * p) * rng.random((m, 299))
+    assert _reference_bytes_brute(x) == _oracle_reference_bytes(x)
+    # pixel-like, 20 % filled: no column qualifies for the sparse part except the unused one
+    x = np.zeros((m, 65), dtype=np.float32)
+    x[:, 1:] = (rng.random((m, 64)) < 0.2) * rng.random((m, 64))
+    assert _reference_bytes_brute(x) == _oracle_reference_bytes(x)

@@ -431,6 +431,42 @@ __global__ void kernel_diag_kernel(const double *__restrict__ self_dot, int64_t 
     diag[i] = v;
 }
 
+// Column statistics of the data rows: counts[c] = number of entries in column c (dense layout: non-zero values; CSR:
+// stored entries), counts[d + c] = how many values are neither 0 nor 1 (none: an indicator column).  The reference's
+// KernelMatrix constructor counts the stored entries per column to split the matrix into a dense and a sparse
+// part (CSR_DenseCSR, kernelmatrix.cpp:16-74).
+__global__ __launch_bounds__(256) void column_stats_dense_kernel(const double *__restrict__ x, int64_t ld, int64_t n, int d,
+                                                                 int *__restrict__ counts) {
+    const int64_t rows_per = (n + gridDim.x - 1) / gridDim.x;
+    const int64_t r0 = (int64_t) blockIdx.x * rows_per, r1 = r0 + rows_per < n ? r0 + rows_per : n;
+    for (int c = threadIdx.x; c < d; c += blockDim.x) {
+        int nz = 0, nu = 0;
+        for (int64_t r = r0; r < r1; ++r) {
+            const double v = x[r * ld + c];
+            nz += v != 0.0;
+            nu += v != 0.0 && v != 1.0;
+        }
+        if (nz) atomicAdd(&counts[c], nz);
+        if (nu) atomicAdd(&counts[d + c], nu);
+    }
+}
+
+__global__ __launch_bounds__(256) void column_stats_csr_kernel(const double *__restrict__ val, const int *__restrict__ col,
+                                                               int64_t nnz, int d, int *__restrict__ counts) {
+    for (int64_t e = (int64_t) blockIdx.x * blockDim.x + threadIdx.x; e < nnz; e += (int64_t) gridDim.x * blockDim.x) {
+        const double v = val[e];
+        const int c = col[e];
+        if (c < 0 || c >= d) continue;
+        atomicAdd(&counts[c], 1);   // stored entries, as the reference counts them (a stored 0.0 included)
+        if (v != 1.0 && v != 0.0) atomicAdd(&counts[d + c], 1);
+    }
+}
+
+__global__ void fill_i32_kernel(int *p, int64_t count, int v) {
+    for (int64_t e = (int64_t) blockIdx.x * blockDim.x + threadIdx.x; e < count; e += (int64_t) gridDim.x * blockDim.x)
+        p[e] = v;
+}
+
 __global__ void gather_f64_kernel(const double *__restrict__ in, const int *__restrict__ idx, int m,
                                   double *__restrict__ out) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -441,7 +477,10 @@ __global__ void gather_f64_kernel(const double *__restrict__ in, const int *__re
 // sum_kernel_values (kernelmatrix_kernel.cpp:110-147).
 // One workgroup handles SK_R test rows.  For coefficient row c (0..k-2) and SV class s the segment
 // sum S[c][s] = sum_{l in SV_s} coef[c*T + l] * K[r][l] is accumulated by 256 threads striding over
-// the segment and tree-reduced through LDS; dec(i,j) = S[j-1][i] + S[i][j] - rho.  The summation
+// the segment and tree-reduced through LDS; dec(i,j) = S[j-1][i] + S[i][j] - rho.  Every (c, s) belongs to
+// exactly one pair, and with s as the outer loop a pair's first term S[j-1][i] (s = i) is always ready before
+// its second S[i][j] (s = j): the first is parked in dec itself and the thread that parked it completes the
+// value when the second arrives, so no table grows with the number of classes.  The summation
 // order differs from the reference's serial loop (results agree to ~1e-13 relative, inside the
 // 1e-6 absolute tolerance on decision values).
 // ------------------------------------------------------------------------------------------------
@@ -453,18 +492,17 @@ __global__ __launch_bounds__(SK_T) void sum_kernel_values_kernel(
     const double *__restrict__ coef, int total_sv, const int *__restrict__ sv_start, const int *__restrict__ sv_count,
     const double *__restrict__ rho, const TK *__restrict__ k_mat, int64_t ldk, double *__restrict__ dec,
     int n_classes, int64_t n_instances) {
-    extern __shared__ double sm[];  // [SK_R][(k-1)*k] segment sums, then reduction scratch [SK_T/64][SK_R]
+    __shared__ double red[(SK_T / 64) * SK_R];   // per-wavefront partial sums
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int64_t r0 = (int64_t) blockIdx.x * SK_R;
     const int km1 = n_classes - 1;
-    double *S = sm;
-    double *red = sm + SK_R * km1 * n_classes;
-    const int P = n_classes * km1 / 2;
+    const int64_t P = (int64_t) n_classes * km1 / 2;
     for (int s = 0; s < n_classes; ++s) {
         const int st = sv_start[s], cnt = sv_count[s];
         for (int c = 0; c < km1; ++c) {
-            // every (c, s) is used by exactly one pair: (i=s, j=c+1) when c >= s, (i=c, j=s) when c < s
+            // every (c, s) is used by exactly one pair: (i=s, j=c+1) when c >= s (its first term), (i=c, j=s) when
+            // c < s (its second term)
             const double *cf = coef + (int64_t) c * total_sv + st;
             double part[SK_R];
 #pragma unroll
@@ -505,25 +543,17 @@ __global__ __launch_bounds__(SK_T) void sum_kernel_values_kernel(
                 if (lane == 0) red[wave * SK_R + rr] = v;
             }
             __syncthreads();
-            if (tid < SK_R) {
+            if (tid < SK_R && r0 + tid < n_instances) {
                 double t = 0.0;
                 for (int wv = 0; wv < SK_T / 64; ++wv) t += red[wv * SK_R + tid];
-                S[(tid * km1 + c) * n_classes + s] = t;
+                const bool first = c >= s;
+                const int i = first ? s : c, j = first ? c + 1 : s;
+                const int64_t p = (int64_t) i * (2 * n_classes - i - 1) / 2 + (j - i - 1);
+                double *out = dec + (r0 + tid) * P + p;
+                *out = first ? t : (*out + t) - rho[p];
             }
             __syncthreads();
         }
-    }
-    __syncthreads();
-    for (int e = tid; e < SK_R * P; e += SK_T) {
-        const int rr = e / P, p = e % P;
-        const int64_t r = r0 + rr;
-        if (r >= n_instances) continue;
-        // decode pair index p -> (i, j)
-        int i = 0, rem = p;
-        while (rem >= n_classes - 1 - i) { rem -= n_classes - 1 - i; ++i; }
-        const int j = i + 1 + rem;
-        const double sum = S[(rr * km1 + (j - 1)) * n_classes + i] + S[(rr * km1 + i) * n_classes + j];
-        dec[r * P + p] = sum - rho[p];
     }
 }
 
@@ -784,6 +814,30 @@ int tsvm_fold_ids(const int *ids, int count, int period, int *out, tsvm_stream s
     return 0;
 }
 
+int tsvm_column_stats_dense(const double *x, int64_t ld, int64_t n, int d, int *counts, tsvm_stream stream) {
+    TSVM_REQUIRE(x && counts && n >= 0 && d >= 0 && d <= ld, "tsvm_column_stats_dense: bad argument");
+    if (d == 0) return 0;
+    hipLaunchKernelGGL(fill_i32_kernel, dim3(grid_for(2 * (int64_t) d, 256)), dim3(256), 0, tsvm_s(stream), counts, 2 * (int64_t) d, 0);
+    TSVM_LAUNCH_CHECK();
+    if (n == 0) return 0;
+    const unsigned grid = (unsigned) std::min<int64_t>((n + 63) / 64, 2048);
+    hipLaunchKernelGGL(column_stats_dense_kernel, dim3(grid), dim3(256), 0, tsvm_s(stream), x, ld, n, d, counts);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+int tsvm_column_stats_csr(const double *val, const int *col, int64_t nnz, int d, int *counts, tsvm_stream stream) {
+    TSVM_REQUIRE(counts && nnz >= 0 && d >= 0 && (nnz == 0 || (val && col)), "tsvm_column_stats_csr: bad argument");
+    if (d == 0) return 0;
+    hipLaunchKernelGGL(fill_i32_kernel, dim3(grid_for(2 * (int64_t) d, 256)), dim3(256), 0, tsvm_s(stream), counts, 2 * (int64_t) d, 0);
+    TSVM_LAUNCH_CHECK();
+    if (nnz == 0) return 0;
+    const unsigned grid = (unsigned) std::min<int64_t>((nnz + 255) / 256, 4096);
+    hipLaunchKernelGGL(column_stats_csr_kernel, dim3(grid), dim3(256), 0, tsvm_s(stream), val, col, nnz, d, counts);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
 int tsvm_gather_f64(const double *in, const int *idx, int m, double *out, tsvm_stream stream) {
     TSVM_REQUIRE(in && idx && out && m >= 0, "tsvm_gather_f64: bad argument");
     if (m == 0) return 0;
@@ -796,11 +850,11 @@ int tsvm_sum_kernel_values(const double *coef, int total_sv, const int *sv_start
                            const double *rho, const void *k_mat, int row_type, int64_t ldk, double *dec_values,
                            int n_classes, int64_t n_instances, tsvm_stream stream) {
     TSVM_REQUIRE(sv_start && sv_count && rho && dec_values, "tsvm_sum_kernel_values: null pointer");
-    TSVM_REQUIRE(n_classes >= 2 && n_classes <= 32, "tsvm_sum_kernel_values: n_classes %d outside [2, 32]", n_classes);
+    TSVM_REQUIRE(n_classes >= 2 && n_classes <= 32768, "tsvm_sum_kernel_values: n_classes %d outside [2, 32768]", n_classes);
     TSVM_REQUIRE(total_sv >= 0 && ldk >= total_sv && n_instances >= 0, "tsvm_sum_kernel_values: bad size");
     TSVM_REQUIRE(row_type == TSVM_ROW_F64 || row_type == TSVM_ROW_F32, "tsvm_sum_kernel_values: unknown row type %d", row_type);
     if (n_instances == 0) return 0;
-    const size_t shm = sizeof(double) * ((size_t) SK_R * (n_classes - 1) * n_classes + (SK_T / 64) * SK_R);
+    const size_t shm = 0;
     if (row_type == TSVM_ROW_F32)
         hipLaunchKernelGGL(sum_kernel_values_kernel<float>, dim3(grid_for(n_instances, SK_R)), dim3(SK_T), shm, tsvm_s(stream),
                            coef, total_sv, sv_start, sv_count, rho, (const float *) k_mat, ldk, dec_values, n_classes,

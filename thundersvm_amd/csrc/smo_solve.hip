@@ -311,7 +311,12 @@ __global__ __launch_bounds__(SV_T) void c_smo_solve_kernel(
             alpha[working_set[t]] = a;
         }
     }
-    if (tid == 0) diff[1] = (double) numOfIter;
+    // diff may be host memory that a waiting host thread polls: diff[1] is the kernel's last word, and everything
+    // written before it (diff[0] in particular) has to be visible system-wide first
+    if (tid == 0) {
+        __threadfence_system();
+        diff[1] = (double) numOfIter;
+    }
     if (touched == 0x7ff00001u && numOfIter < 0) diff[0] = 0.0;   // keeps the row-touching loads alive; never true
 }
 
@@ -360,7 +365,7 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
     double pend_ai = a_old[0], pend_aj = a_old[0];
     // initial gap -> local stopping threshold (smo_kernel.cpp:176-183); inside the loop the stopping
     // test is evaluated per element, as in the C variant
-    double local_eps;
+    double local_eps, first_diff;
     {
         double mnp = TSVM_INF, mnn = TSVM_INF, mxp = -TSVM_INF, mxn = -TSVM_INF;
 #pragma unroll
@@ -384,7 +389,7 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
         const double local_diff = dp > dn ? dp : dn;
         const double t = 0.1 * local_diff;
         local_eps = eps > t ? eps : t;
-        if (tid == 0) diff[0] = local_diff;
+        first_diff = local_diff;
         __syncthreads();
     }
     int numOfIter = 0;
@@ -493,6 +498,12 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
             alpha_diff[t] = -(a - a_old[e]) * (double) s_y[t];
             alpha[working_set[t]] = a;
         }
+    }
+    // diff[0] is the only word this variant reports (smo_kernel.cpp:283 leaves diff[1] alone).  It is written last,
+    // behind a system-wide fence, so that a host thread polling it in host memory sees the kernel's end.
+    if (tid == 0) {
+        __threadfence_system();
+        diff[0] = first_diff;
     }
     if (touched == 0x7ff00001u && numOfIter < 0) diff[0] = 0.0;   // keeps the row-touching loads alive; never true
 }

@@ -146,20 +146,27 @@ def workload_c3(scale=1.0, kernel="rbf"):
     pz = ranks ** -1.1
     pz /= pz.sum()
     nnz_row = np.maximum(rng.poisson(50, size=n), 1)
-    ptr = np.zeros(n + 1, dtype=np.int64)
-    cols, vals = [], []
     wcols = rng.choice(d, size=400, replace=False, p=pz)
     w = np.zeros(d + 1)
     w[wcols + 1] = rng.standard_normal(400)
-    for i in range(n):
-        c = np.unique(rng.choice(d, size=nnz_row[i], replace=True, p=pz)) + 1
-        v = rng.lognormal(0.0, 1.0, size=len(c))
-        v = (v / np.sqrt((v * v).sum())).astype(np.float32).astype(np.float64)
-        cols.append(c)
-        vals.append(v)
-        ptr[i + 1] = ptr[i] + len(c)
-    col = np.concatenate(cols).astype(np.int32)
-    val = np.concatenate(vals)
+    # every row's draws at once: each row draws until it holds nnz_row distinct columns (more draws than needed are
+    # made up front and the first nnz_row distinct ones kept, in draw order), columns ascending per row
+    n_draw = 2 * nnz_row + 16
+    row_of = np.repeat(np.arange(n, dtype=np.int64), n_draw)
+    drawn = rng.choice(d, size=int(n_draw.sum()), replace=True, p=pz).astype(np.int64) + 1
+    _, first = np.unique(row_of * (d + 2) + drawn, return_index=True)   # first occurrence of every (row, column)
+    first.sort()
+    r = row_of[first]
+    start = np.zeros(n + 1, dtype=np.int64)
+    np.cumsum(np.bincount(r, minlength=n), out=start[1:])
+    keep = first[np.arange(len(first)) - start[r] < nnz_row[r]]
+    key = np.sort(row_of[keep] * (d + 2) + drawn[keep])
+    row_of, col = key // (d + 2), (key % (d + 2)).astype(np.int32)
+    ptr = np.zeros(n + 1, dtype=np.int64)
+    np.cumsum(np.bincount(row_of, minlength=n), out=ptr[1:])
+    v = rng.lognormal(0.0, 1.0, size=len(col))
+    norm = np.sqrt(np.add.reduceat(v * v, ptr[:-1]))
+    val = (v / norm[row_of]).astype(np.float32).astype(np.float64)
     score = np.add.reduceat(val * w[col], ptr[:-1])
     y = np.where(score > np.median(score), 1.0, -1.0)
     flip = rng.random(n) < 0.03

@@ -154,6 +154,16 @@ std::shared_ptr<DeviceRows> DeviceRows::subset(const DeviceRows &base, const int
     return out;
 }
 
+const std::vector<int> &DeviceRows::column_stats() const {
+    if (column_stats_.size() != 2 * n_features) {
+        tsvm::DeviceBuffer<int> d_counts(2 * n_features);
+        if (dense) abi_check(tsvm_column_stats_dense(x.data(), ld, (int64_t) n, (int) n_features, d_counts.data(), nullptr));
+        else abi_check(tsvm_column_stats_csr(val.data(), col.data(), (int64_t) nnz, (int) n_features, d_counts.data(), nullptr));
+        column_stats_ = d_counts.to_host();
+    }
+    return column_stats_;
+}
+
 std::shared_ptr<DeviceRows> DeviceRows::of(const DataSet &dataset) {
     std::shared_ptr<void> &slot = dataset.device_cache();
     if (!slot) slot = from_host(dataset.instances(), nullptr, dataset.instances().size());
@@ -191,6 +201,40 @@ void KernelMatrix::finish(int repeat) {
         TSVM_HIP_CHECK(hipMemcpyAsync(diag_.data() + rep * n_unique_, diag_.data(), n_unique_ * sizeof(kernel_type),
                                       hipMemcpyDeviceToDevice, nullptr));
     TSVM_HIP_CHECK(hipDeviceSynchronize());
+}
+
+size_t KernelMatrix::reference_syncmem_bytes() const {
+    const DeviceRows &R = *rows_;
+    const std::vector<int> &stats = R.column_stats();
+    const long long nf = (long long) R.n_features, m = (long long) n_instances();
+    std::vector<long long> cnt(nf);
+    long long entries = 0;
+    for (long long c = 0; c < nf; ++c) {
+        cnt[c] = (long long) stats[c] * repeat_;
+        entries += cnt[c];
+    }
+    // columns by entry count ascending, ties by index (kernelmatrix.cpp:32-41); leading columns go to the sparse part
+    // while the part stays under 5 % full, the column under 50 % full, and four times its entries do not exceed
+    // the cells left to the dense part (kernelmatrix.cpp:58-74)
+    std::vector<int> order(nf);
+    for (long long c = 0; c < nf; ++c) order[c] = (int) c;
+    std::sort(order.begin(), order.end(), [&](int a, int b) { return cnt[a] != cnt[b] ? cnt[a] < cnt[b] : a < b; });
+    long long total_csr = 0, total_dense = m * nf, row_sum = 0, dense_cols = nf, nnz_sparse = 0;
+    for (long long i = 0; i < nf; ++i) {
+        const long long c = cnt[order[i]];
+        total_csr += c;
+        total_dense -= m;
+        row_sum += m;
+        if ((long double) total_csr / row_sum > 0.05 || (long double) c / m > 0.5 || total_csr * 4 > total_dense) break;
+        --dense_cols;
+        nnz_sparse += c;
+    }
+    size_t bytes = (size_t) entries * (sizeof(kernel_type) + sizeof(int)) + (size_t) (m + 1) * sizeof(int) +
+                   2 * (size_t) m * sizeof(kernel_type);
+    if (dense_cols > 0) bytes += (size_t) m * dense_cols * sizeof(kernel_type);                      // dense.val, kernelmatrix.cpp:79-83
+    if (dense_cols < nf && nnz_sparse != 0)   // some entry lies outside the dense part (kernelmatrix.cpp:151-176)
+        bytes += (size_t) nnz_sparse * (sizeof(kernel_type) + sizeof(int)) + (size_t) (m + 1) * sizeof(int);
+    return bytes;
 }
 
 // A staging buffer that is all-zero whenever it is not in use: grown (and cleared) only when a call needs more.

@@ -33,6 +33,10 @@ struct DeviceRows {
     tsvm::DeviceBuffer<int64_t> row_ptr;
     std::vector<int64_t> host_row_ptr;           // CSR layout only: needed to lay out a subset
     tsvm::DeviceBuffer<kernel_type> self_dot;    // [n]
+    // per column c < n_features: [c] = entries (dense: non-zero values; CSR: stored entries), [n_features + c] = values
+    // that are neither 0 nor 1; counted on the device on first use
+    const std::vector<int> &column_stats() const;
+    mutable std::vector<int> column_stats_;
 
     // rows[0..n_rows) of `all` (rows == nullptr: the first n_rows), assembled on the host and uploaded
     static std::shared_ptr<DeviceRows> from_host(const DataSet::node2d &all, const int *rows, size_t n_rows);
@@ -78,6 +82,13 @@ public:
     const SvmParam &get_param() const { return param; }
 
     static bool choose_dense(size_t n, size_t n_features, size_t nnz);
+
+    // Bytes the reference's SyncMem counter (syncmem.cpp:58-108) holds for its KernelMatrix of the same rows in a
+    // USE_DOUBLE build: val_, col_ind_, row_ptr_, self_dot_, diag_ (kernelmatrix.cpp:211-226) and the dense and
+    // sparse parts its constructor splits the columns into (CSR_DenseCSR, kernelmatrix.cpp:16-181).  This is
+    // what SvmModel::get_working_set_size subtracts from the memory budget (svmmodel.cpp:437-451).  An entry
+    // stored with the value 0 counts as absent in the dense layout and as a non-zero entry in the CSR layout.
+    size_t reference_syncmem_bytes() const;
 
 private:
     void finish(int repeat);

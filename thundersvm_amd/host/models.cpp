@@ -40,19 +40,30 @@ void SvmModel::model_setup(const DataSet &, SvmParam &p) {   // svmmodel.cpp:22-
     binary_alpha.clear();
     binary_f.clear();
     param = p;
+    // The class weights are the caller's arrays and need not outlive this call: SVC::model_setup folds them into
+    // c_weight while they are alive, and the model's own copy of the parameters drops the pointers.
+    param.nr_weight = 0;
+    param.weight_label = nullptr;
+    param.weight = nullptr;
 }
 
 static int max2power(double n) { return (int) pow(2, floor(log2f(float(n)))); }   // util/common.h:20-23
 
-// svmmodel.cpp:437-451.  The reference subtracts the bytes its SyncMem counter holds; the device
-// allocations of this build play that role.
-int SvmModel::get_working_set_size(int n_instances, int n_features) {
+// svmmodel.cpp:437-451.  The reference subtracts the bytes its SyncMem counter holds at this point of
+// train_binary (svc.cpp:147-166; svr.cpp:9-35 and the other models alike): its KernelMatrix of the problem, the
+// problem's y (int), alpha and f (float_type), and `held_bytes`, what the model has kept from earlier problems
+// (the alpha arrays of the class pairs already trained, svc.cpp:50-61).  The counter is restated from the
+// problem's shape, not read from this build's own device allocations, so the working-set size -- and with it the
+// trajectory -- is the reference's wherever its memory budget starts to bind (n + n_features above ~10^6 with the
+// default 8192 MiB).  Small model members (rho, n_sv, label) are left out.
+int SvmModel::get_working_set_size(const KernelMatrix &k_mat, size_t held_bytes) {
     if (ws_override > 0) return ws_override;
-    const size_t used = tsvm::device_bytes_in_use();
+    const size_t n_instances = k_mat.n_instances(), n_features = k_mat.n_features();
+    const size_t used = k_mat.reference_syncmem_bytes() + n_instances * (sizeof(int) + 2 * sizeof(float_type)) + held_bytes;
     if (param.max_mem_size < used) throw std::bad_alloc();
     const size_t free_mem = param.max_mem_size - used;
-    const size_t by_mem = (size_t) max2power((double) (free_mem / sizeof(kernel_type) / ((size_t) n_instances + n_features)));
-    const int ws = std::min(max2power(n_instances), (int) std::min(by_mem, (size_t) 1024));
+    const size_t by_mem = (size_t) max2power((double) (free_mem / sizeof(kernel_type) / (n_instances + n_features)));
+    const int ws = std::min(max2power((double) n_instances), (int) std::min(by_mem, (size_t) 1024));
     TSVM_LOG << "working set size = " << ws;
     return ws;
 }
@@ -68,8 +79,8 @@ void SvmModel::copy_support_vectors(const DataSet::node2d &instances) {
 
 void SvmModel::run_solver(CSMOSolver &solver, const KernelMatrix &k_mat, const std::vector<int> &y,
                           std::vector<float_type> &alpha, float_type &rho_out, std::vector<float_type> &f_val,
-                          float_type Cp, float_type Cn) {
-    const int ws = get_working_set_size((int) k_mat.n_instances(), (int) k_mat.n_features());
+                          float_type Cp, float_type Cn, size_t held_bytes) {
+    const int ws = get_working_set_size(k_mat, held_bytes);
     solver.profile = profile;
     solver.cache_bytes = cache_bytes;
     solver.trace = solver_stats.empty() ? trace_first : nullptr;
@@ -331,12 +342,14 @@ void SVC::train(const DataSet &dataset, SvmParam p) {   // svc.cpp:41-145
     if (lanes > 1 && !profile && !trace_first) {
         train_pairs_in_lockstep(grouped, lanes, alpha);
     } else {
+        size_t held = 0;   // alpha arrays of the pairs already trained (svc.cpp:50-61 keeps them to the end)
         for (int i = 0; i < n_classes; ++i)
             for (int j = i + 1; j < n_classes; ++j, ++k) {
                 BinaryProblem p;
                 p.k = k;
                 setup_binary(grouped, i, j, p);
-                run_solver(*p.solver, *p.k_mat, p.y, p.alpha, rho[k], p.f_val, p.Cp, p.Cn);
+                run_solver(*p.solver, *p.k_mat, p.y, p.alpha, rho[k], p.f_val, p.Cp, p.Cn, held);
+                held += p.y.size() * sizeof(float_type);
                 finish_binary(p, alpha[k]);
             }
     }
@@ -449,6 +462,12 @@ void SVC::train_pairs_in_lockstep(const DataSet &grouped, int lanes, std::vector
     const size_t slice = std::max(budget / lanes, need_min) / 256 * 256;
     char *const pool = (char *) arena.acquire(slice * lanes, cache_bytes < 0);
 
+    // what the reference still holds of the pairs trained before pair k when it sizes pair k's working set: their
+    // alpha arrays (svc.cpp:50-61), whatever runs beside pair k here
+    std::vector<size_t> alpha_bytes_before(pairs.size() + 1, 0);
+    for (size_t k = 0; k < pairs.size(); ++k)
+        alpha_bytes_before[k + 1] = alpha_bytes_before[k] +
+                                    ((size_t) grouped.count()[pairs[k].i] + grouped.count()[pairs[k].j]) * sizeof(float_type);
     solver_stats.assign(pairs.size(), SolverStats());
     if (keep_binary) binary_f.assign(pairs.size(), std::vector<float_type>());
     std::vector<std::unique_ptr<BinaryProblem>> active;
@@ -462,7 +481,7 @@ void SVC::train_pairs_in_lockstep(const DataSet &grouped, int lanes, std::vector
         ++next;
         p->lane = free_lanes.back();
         free_lanes.pop_back();
-        const int ws = get_working_set_size((int) p->k_mat->n_instances(), (int) p->k_mat->n_features());
+        const int ws = get_working_set_size(*p->k_mat, alpha_bytes_before[p->k]);
         p->solver->cache_bytes = cache_bytes;
         p->task.reset(new SolveTask(*p->solver, *p->k_mat, p->y, p->alpha, rho[p->k], p->f_val, param.epsilon, p->Cp, p->Cn, ws,
                                     max_iter, pool + (size_t) p->lane * slice, slice, p->lane, lanes));

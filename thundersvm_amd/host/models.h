@@ -41,7 +41,7 @@ public:
     const std::vector<float> &get_prob_predict() const { return prob_predict; }
     bool is_prob() const { return param.probability; }
     const SvmParam &get_param() const { return param; }
-    int get_working_set_size(int n_instances, int n_features);
+    int get_working_set_size(const KernelMatrix &k_mat, size_t held_bytes = 0);
 
     // diagnostics of the last train() call, one entry per binary sub-problem
     std::vector<SolverStats> solver_stats;
@@ -58,7 +58,7 @@ protected:
     virtual void model_setup(const DataSet &dataset, SvmParam &param);
     void copy_support_vectors(const DataSet::node2d &instances);
     void run_solver(CSMOSolver &solver, const KernelMatrix &k_mat, const std::vector<int> &y, std::vector<float_type> &alpha,
-                    float_type &rho, std::vector<float_type> &f_val, float_type Cp, float_type Cn);
+                    float_type &rho, std::vector<float_type> &f_val, float_type Cp, float_type Cn, size_t held_bytes = 0);
     void compute_linear_coef_single_model(size_t n_feature, bool zero_based);
 
     SvmParam param;

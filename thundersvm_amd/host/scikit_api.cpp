@@ -3,6 +3,8 @@
 // the classes of models.h.  No exception leaves this file.
 #include <omp.h>
 
+#include <algorithm>
+#include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -83,20 +85,24 @@ void train_on(DataSet &train, int svm_type, int kernel_type, int degree, float g
     if (!ok) succeed[0] = -1;
 }
 
+// A failed prediction must not pass for a result: the caller's buffer is filled with NaN and the status is non-zero
+// (the reference aborts the process in that case, include/thundersvm/util/common.h:38).
 int predict_on(DataSet &data, SvmModel *model, float *predict_label, int verbose) {
     tsvm::Log::enabled() = verbose != 0;
-    guarded("prediction", [&] {
+    const bool ok = guarded("prediction", [&] {
         const std::vector<float_type> y = model->predict(data.instances(), -1);
         for (size_t i = 0; i < y.size(); ++i) predict_label[i] = (float) y[i];
     });
-    return 0;
+    if (!ok) std::fill(predict_label, predict_label + data.n_instances(), std::nanf(""));
+    return ok ? 0 : -1;
 }
 
 void decision_on(DataSet &data, SvmModel *model, int value_size, float *dec_value) {
-    guarded("decision values", [&] {
+    const bool ok = guarded("decision values", [&] {
         model->predict(data.instances(), -1);
         copy_out(model->get_dec_value(), dec_value, (size_t) (value_size > 0 ? value_size : 0));
     });
+    if (!ok) std::fill(dec_value, dec_value + (value_size > 0 ? value_size : 0), std::nanf(""));
 }
 
 }  // namespace

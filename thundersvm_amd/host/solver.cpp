@@ -106,6 +106,40 @@ void destroy_masked_streams() {
 
 }  // namespace
 
+namespace tsvm {
+
+long long solver_timeout_ms() {
+    const char *e = getenv("TSVM_SOLVER_TIMEOUT_MS");
+    const long long v = e ? atoll(e) : 0;
+    return v > 0 ? v : 300000;
+}
+
+void wait_while_pending(const volatile uint64_t *word, uint64_t pending, long long timeout_ms, hipError_t (*stream_state)(void *),
+                        void *stream) {
+    using clock = std::chrono::steady_clock;
+    const auto start = clock::now();
+    // (asking the runtime about the stream puts a marker into it: only done when the wait is suspiciously long)
+    auto next_check = start + std::chrono::milliseconds(200);
+    for (unsigned long long spins = 1; *word == pending; ++spins) {
+        if (spins % 4096 != 0) continue;
+        const auto now = clock::now();
+        if (now < next_check) continue;
+        next_check = now + std::chrono::milliseconds(200);
+        const hipError_t e = stream_state(stream);
+        if (e == hipSuccess) {   // everything enqueued has run: the write is on its way or was never made
+            if (*word == pending) throw std::runtime_error("SolveTask: the local solver finished without reporting");
+        } else if (e != hipErrorNotReady) {
+            TSVM_HIP_CHECK(e);
+        }
+        if (now - start > std::chrono::milliseconds(timeout_ms))
+            throw std::runtime_error("SolveTask: no word from the local solver after " + std::to_string(timeout_ms) +
+                                     " ms (TSVM_SOLVER_TIMEOUT_MS); the device may be hung");
+    }
+    __atomic_thread_fence(__ATOMIC_ACQUIRE);
+}
+
+}  // namespace tsvm
+
 struct SolveTask::Impl {
     const CSMOSolver &solver;
     const KernelMatrix &k_mat;
@@ -185,28 +219,16 @@ struct SolveTask::Impl {
     double *h_diff = nullptr, *d_diff = nullptr;
     // The host does not wait for an event behind update_f (a marker in the stream costs the device about 6 us
     // before the next kernel starts): it marks the word the solver writes last as pending before it enqueues the
-    // solver (diff[1] for c_smo_solve; nu_smo_solve writes diff[0] only, smo_kernel.cpp:283), and waits for that
-    // word to change.  Everything the host enqueues meanwhile is ordered by the streams.
+    // solver (diff[1] for c_smo_solve; nu_smo_solve reports diff[0] only, smo_kernel.cpp:283, and writes it at its
+    // end), and waits for that word to change.  Both kernels put a system-wide fence before that last write.
+    // Everything the host enqueues meanwhile is ordered by the streams.
     static constexpr uint64_t DIFF_PENDING = 0x7ff8dead00000001ull;   // a NaN no computation produces
     bool wait_by_event = false;
     hipStream_t solver_stream = nullptr;
     volatile uint64_t *diff_word() const { return reinterpret_cast<volatile uint64_t *>(h_diff + (nu ? 0 : 1)); }
     void wait_for_diff() {
-        volatile uint64_t *w = diff_word();
-        // (asking the runtime about the stream puts a marker into it: only done when the wait is suspiciously long)
-        auto next_check = std::chrono::steady_clock::now() + std::chrono::milliseconds(200);
-        for (unsigned long long spins = 1; *w == DIFF_PENDING; ++spins) {
-            if (spins % 4096 == 0 && std::chrono::steady_clock::now() > next_check) {
-                next_check = std::chrono::steady_clock::now() + std::chrono::milliseconds(200);
-                const hipError_t e = hipStreamQuery(solver_stream);
-                if (e == hipSuccess) {   // the solver has run: its write is on its way or it never made one
-                    if (*w == DIFF_PENDING) throw std::runtime_error("SolveTask: the local solver finished without reporting");
-                } else if (e != hipErrorNotReady) {
-                    TSVM_HIP_CHECK(e);
-                }
-            }
-        }
-        __atomic_thread_fence(__ATOMIC_ACQUIRE);
+        tsvm::wait_while_pending(diff_word(), DIFF_PENDING, tsvm::solver_timeout_ms(),
+                                 [](void *st) { return hipStreamQuery((hipStream_t) st); }, solver_stream);
     }
     int rotation_base = 0;   // iteration at which d_slots_a was valid
     long long window_lookups = 0, window_hits = 0;
@@ -228,6 +250,7 @@ struct SolveTask::Impl {
           row_type(k_mat.row_type()), row_esz(k_mat.row_elem_size()), q(ws_size / 2), ld(((int64_t) n_u + 7) / 8 * 8),
           nu(solver.is_nu()), ldk(tsvm_smo_solve_block_ld(ws_size)), timer(solver.profile) {
         wall0 = std::chrono::steady_clock::now();
+        stats.ws_size = ws_size;
         d_y.resize(n); d_ws.resize((size_t) WS_HALVES * q + ws_size); d_slots_a.resize(3 * (size_t) ws_size); d_slots_b.resize(ws_size);
         if (rep > 1) d_ws_folded.resize(d_ws.size());
         d_alpha.resize(n); d_f.resize(n); d_alpha_diff.resize(ws_size);
@@ -513,7 +536,18 @@ struct SolveTask::Impl {
                     TSVM_HIP_CHECK(hipStreamSynchronize(sa));
                     caching = false;
                     stats.cache_disabled = true;
-                    upload_rotation(cur_slots);
+                    if (rep > 1) {
+                        // Stacked problems may hold one slot at two positions of the working set (instance i and
+                        // its copy i + n_u share a stored row).  Rotation needs a slot of its own at every position:
+                        // the positions take slots 0 .. ws-1 and all ws rows are computed into them once, as the
+                        // path without a cache does at its first iteration.
+                        for (int t = 0; t < ws_size; ++t) cur_slots[t] = t;
+                        upload_rotation(cur_slots);
+                        k_mat.get_rows(ws_u(), ws_size, k_rows, ld, d_slots_a.data(), sa);
+                        last_rows_computed = ws_size;
+                    } else {
+                        upload_rotation(cur_slots);
+                    }
                     rotation_base = iter;
                 }
             }

@@ -22,9 +22,21 @@ struct SolverStats {
     long long cache_lookups = 0, cache_hits = 0;
     long long cache_rows = 0;     // capacity in rows (0: cache not used)
     bool cache_disabled = false;  // switched off after the warm-up because it was not hitting
+    int ws_size = 0;              // working-set size of the solve
 };
 
 class SolveTask;
+
+namespace tsvm {
+// Spins until *word no longer holds `pending`.  Every 200 ms `stream_state()` is asked for the state of the stream
+// that is to write the word (hipSuccess: everything enqueued has run; hipErrorNotReady: still running; anything else
+// is thrown as that error).  Throws std::runtime_error when the stream has drained without the word changing, or
+// when timeout_ms have passed: a solver kernel that never finishes must not hang its caller for good (the
+// reference's blocking copies surface such failures through CUDA_CHECK, include/thundersvm/util/common.h:33-42).
+void wait_while_pending(const volatile uint64_t *word, uint64_t pending, long long timeout_ms, hipError_t (*stream_state)(void *),
+                        void *stream);
+long long solver_timeout_ms();   // TSVM_SOLVER_TIMEOUT_MS, default 300,000
+}  // namespace tsvm
 
 class CSMOSolver {
 public:
