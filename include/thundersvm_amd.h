@@ -96,6 +96,26 @@ int tsvm_get_rows_dense_counted(const double *x, int64_t ldx, const int *x_idx, 
                                 const double *sd_a, int kernel_type, double gamma, double coef0, int degree, void *out,
                                 int row_type, const int *out_slots, int64_t ldo, tsvm_stream stream);
 
+/* Indicator columns.  When the last columns of the data hold only zeros and ones (one-hot encoded categories; the
+ * reference's KernelMatrix constructor moves such rarely set columns into a separate sparse part and multiplies the
+ * two parts separately, kernelmatrix.cpp:58-74,318-343), the dot product over them is the number of columns both
+ * rows have set.  tsvm_indicator_masks packs columns first_col .. first_col + n_cols - 1 (n_cols <= 64) of every row
+ * into one 64-bit mask (bit b: column first_col + b is non-zero) and writes the largest number of set bits of a row
+ * to *max_ones (device int). */
+int tsvm_indicator_masks(const double *x, int64_t ld, int64_t n, int first_col, int n_cols, uint64_t *masks, int *max_ones,
+                         tsvm_stream stream);
+
+/* tsvm_get_rows_dense / tsvm_get_rows_dense_counted (m_dev != NULL) for data whose columns from d_dense on are
+ * indicator columns, given as the masks of tsvm_indicator_masks (mask_x[j] for row j of x, mask_a[r] for row r of a;
+ * both sides must be 0/1 there).  The matrix cores walk columns 0 .. d_dense-1 only; 1.0 is then added once per
+ * indicator column set in both rows, one addition at a time, which is the serial chain of fused multiply-adds over
+ * those columns bit for bit.  max_ones bounds the set bits of a row.  Results equal tsvm_get_rows_dense on all columns. */
+int tsvm_get_rows_dense_indicator(const double *x, int64_t ldx, const int *x_idx, int64_t n, int d_dense, const double *sd_x,
+                                  const uint64_t *mask_x, const double *a, int64_t lda, const int *a_idx, int m, const int *m_dev,
+                                  const double *sd_a, const uint64_t *mask_a, int max_ones, int kernel_type, double gamma,
+                                  double coef0, int degree, void *out, int row_type, const int *out_slots, int64_t ldo,
+                                  tsvm_stream stream);
+
 /* Transposed dense staging of selected CSR rows: w[c*m + i] = value of feature c in row idx[i]
  * (idx == NULL: row i of the given CSR), w is [n_features][m] and is zero-filled first.
  * The sparse-path counterpart of get_working_set_ins (kernelmatrix_kernel.cpp:9-25). */

@@ -393,3 +393,71 @@ def test_working_set_block(name, kt, prm, n, d, ws):
     assert np.array_equal(got[:, :ws], rows[:, ids])
     assert np.array_equal(got[:, :ws], got[:, :ws].T)
     assert (got[:, ws:] == 9.0).all()
+
+
+def _mixed_rows(rng, n, n_cont, groups):
+    """n_cont continuous columns followed by one-hot groups (and, in the last group, rows with no category set)."""
+    x = np.zeros((n, n_cont + sum(groups)), dtype=np.float32)
+    x[:, :n_cont] = rng.standard_normal((n, n_cont))
+    x[:, :n_cont][rng.random((n, n_cont)) < 0.1] = 0
+    at = n_cont
+    for gi, g in enumerate(groups):
+        cat = rng.integers(0, g, n)
+        x[np.arange(n), at + cat] = 1
+        if gi == len(groups) - 1:
+            x[rng.random(n) < 0.05, at:at + g] = 0
+        at += g
+    return x
+
+
+@pytest.mark.parametrize("n,n_cont,groups,m", [(140001, 10, (4, 40), 512), (70000, 3, (2, 3, 5, 7), 130), (3000, 0, (6, 10), 64),
+                                                (50000, 21, (64,), 200)])
+@pytest.mark.parametrize("name,kt,prm", [("rbf", O.RBF, dict(gamma=1.0)), ("linear", O.LINEAR, dict()),
+                                         ("poly", O.POLY, dict(gamma=0.3, coef0=0.5, degree=3))])
+def test_indicator_columns(n, n_cont, groups, m, name, kt, prm):
+    """Trailing 0/1 columns handled by the epilogue (one addition of 1.0 per column set in both rows) instead of the
+    matrix cores: the same bits as the plain kernel and the oracle, for every kernel, float and double rows, output
+    slots, a device-side row count and a column subset."""
+    rng = np.random.default_rng(n + n_cont)
+    x = _mixed_rows(rng, n, n_cont, groups)
+    data = from_dense(x)
+    p = O.make_param(kernel_type=kt, expf_mode=1, **prm)
+    okm = O.KernelMatrix(data.ptr, data.col, data.val, p)
+    x_d, nf, ld, sd, diag = _device_km(data, kt, prm)
+    first = 1 + n_cont                                    # column 0 is the unused feature id 0
+    n_ind = nf - first
+    masks = torch.zeros(n, dtype=torch.int64, device="cuda")
+    max_ones = torch.full((1,), -7, dtype=torch.int32, device="cuda")
+    capi.call("tsvm_indicator_masks", G.ptr(x_d), ld, n, first, n_ind, G.ptr(masks), G.ptr(max_ones), G.stream())
+    want_mask = (x[:, n_cont:] != 0).astype(np.uint64) @ (np.uint64(1) << np.arange(n_ind, dtype=np.uint64))
+    assert np.array_equal(G.host(masks).view(np.uint64), want_mask)
+    mo = int(G.host(max_ones)[0])
+    assert mo == int((x[:, n_cont:] != 0).sum(axis=1).max()) == len(groups)
+    idx = rng.integers(0, n, size=m).astype(np.int32)
+    idx[-1] = n - 1
+    want = okm.get_rows(idx)
+    idx_d = G.dev(idx)
+    g = prm.get("gamma", 0.0), prm.get("coef0", 0.0), prm.get("degree", 3)
+
+    def run(row_type, out, m_run, m_dev=None, slots=None, x_idx=None, n_cols=n):
+        capi.call("tsvm_get_rows_dense_indicator", G.ptr(x_d), ld, G.ptr(x_idx), n_cols, first, G.ptr(sd), G.ptr(masks), G.ptr(x_d),
+                  ld, G.ptr(idx_d), m_run, G.ptr(m_dev), G.ptr(sd), G.ptr(masks), mo, kt, *g, G.ptr(out), row_type,
+                  G.ptr(slots), out.shape[1], G.stream())
+
+    out = torch.full((m, n), -3.0, dtype=torch.float64, device="cuda")
+    run(capi.ROW_F64, out, m)
+    _check(name, G.host(out), want)
+    if kt != O.LINEAR:
+        # float rows into permuted slots, the row count read on the device (grid sized for more rows)
+        slots = rng.permutation(m + 9)[:m].astype(np.int32)
+        out32 = torch.full((m + 9, n), -3.0, dtype=torch.float32, device="cuda")
+        m_dev = G.dev(np.array([m - 5], dtype=np.int32))
+        run(capi.ROW_F32, out32, m, m_dev=m_dev, slots=G.dev(slots))
+        got = G.host(out32)
+        _check(name, got[slots[:m - 5]].astype(np.float64), want[:m - 5])
+        assert (got[slots[m - 5:]] == -3.0).all()
+    # a column subset (the solver's block shape)
+    cols = rng.permutation(n)[:777].astype(np.int32)
+    outb = torch.empty((m, 777), dtype=torch.float64, device="cuda")
+    run(capi.ROW_F64, outb, m, x_idx=G.dev(cols), n_cols=777)
+    _check(name, G.host(outb), want[:, cols])

@@ -28,6 +28,9 @@ SIGNATURES = {
     "tsvm_csr_to_dense": (_int, [_p, _p, _p, _i64, _p, _i64, _p]),
     "tsvm_column_stats_dense": (_int, [_p, _i64, _i64, _int, _p, _p]),
     "tsvm_column_stats_csr": (_int, [_p, _p, _i64, _int, _p, _p]),
+    "tsvm_indicator_masks": (_int, [_p, _i64, _i64, _int, _int, _p, _p, _p]),
+    "tsvm_get_rows_dense_indicator": (_int, [_p, _i64, _p, _i64, _int, _p, _p, _p, _i64, _p, _int, _p, _p, _p, _int, _int, _dbl, _dbl,
+                                             _int, _p, _int, _p, _i64, _p]),
     "tsvm_get_rows_dense": (_int, [_p, _i64, _p, _i64, _int, _p, _p, _i64, _p, _int, _p, _int, _dbl, _dbl, _int, _p, _int, _p, _i64, _p]),
     "tsvm_get_rows_dense_counted": (_int, [_p, _i64, _p, _i64, _int, _p, _p, _i64, _p, _int, _p, _p, _int, _dbl, _dbl, _int, _p, _int, _p, _i64, _p]),
     "tsvm_csr_stage_rows": (_int, [_p, _p, _p, _p, _int, _int, _p, _p]),

@@ -7,6 +7,7 @@
 #include "tsvm_internal.h"
 
 #include <algorithm>
+#include <cstdlib>
 
 typedef double v4d __attribute__((ext_vector_type(4)));
 
@@ -247,6 +248,259 @@ __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
         if (i0 >= m) return;
     }
     get_rows_tile<KT, TI, TO>(x, ldx, x_idx, n, d, sd_x, a, lda, a_idx, m, sd_a, kp, out, out_slots, ldo, i0, j0, As, Bs, exp_tab);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Dense get_rows for few features (d <= 128), the shape of the multi-class and regression workloads:
+// hundreds of thousands of columns, a K loop of only one to eight 16-column tiles, and an epilogue that
+// costs as much as the matrix work.  A workgroup keeps its 64 working rows and walks a run of consecutive
+// 128-column tiles.  What is fixed per working row (index, slot, self dot product, output offset) is set up
+// once, and the first K tile of the next column tile is requested from memory before the current tile's
+// epilogue starts, so that the load latency is spent under the epilogue's arithmetic instead of in front of
+// the next tile's first MFMA.
+//
+// IND: the last columns of the data are indicator columns (every value 0 or 1).  The matrix cores then only
+// walk the columns before them (d), and the epilogue adds 1.0 once per indicator column that both rows have
+// set, one addition at a time: fma(1, 1, acc) = fl(acc + 1) and a product with a zero adds nothing, so this
+// is the serial chain over the indicator columns, bit for bit (a pre-summed count would round differently).
+// mask_x / mask_a hold one bit per indicator column and row; max_ones bounds the set bits of a row.
+// ------------------------------------------------------------------------------------------------
+template <int KT, typename TO, int IND>
+__global__ __launch_bounds__(256, 3) void get_rows_dense_stream_kernel(
+    const double *__restrict__ x, int64_t ldx, const int *__restrict__ x_idx, int64_t n, int d,
+    const double *__restrict__ sd_x, const double *__restrict__ a, int64_t lda, const int *__restrict__ a_idx, int m,
+    const double *__restrict__ sd_a, KernelParam kp_in, TO *__restrict__ out, const int *__restrict__ out_slots,
+    int64_t ldo, unsigned m_blocks, unsigned j_tiles, unsigned tiles_per_wg, const int *__restrict__ m_dev,
+    const uint64_t *__restrict__ mask_x, const uint64_t *__restrict__ mask_a, int max_ones, int vec_ok) {
+    constexpr int TI = 2;
+    constexpr int BM = GrShape<TI>::BM;
+    constexpr int KTILE = GrShape<TI>::KTILE;
+    constexpr int LS = GrShape<TI>::LS;
+    constexpr int A_TPR = 256 / BM;
+    constexpr int A_VEC = KTILE / 4 / A_TPR;
+    constexpr int B_VEC = KTILE / 8;
+    __shared__ double As[GrShape<TI>::LDS_DOUBLES];
+    __shared__ double Bs[GrShape<TI>::LDS_DOUBLES];
+    __shared__ uint64_t exp_tab[32];
+    // per working row of the tile (fixed for the workgroup) and per column of the current tile (two generations: a
+    // wavefront may stage the next tile's while another still reads this tile's in its epilogue)
+    __shared__ double s_sdi[BM];
+    __shared__ uint64_t s_mi[BM];
+    __shared__ int s_slot[BM];
+    __shared__ double s_sdj[2][GR_BN];
+    __shared__ uint64_t s_mj[2][GR_BN];
+    KernelParam kp = kp_in;
+    kp.kernel_type = KT;
+    const unsigned logical = xcd_remap(blockIdx.x, gridDim.x);
+    const int i0 = (int) (logical % m_blocks) * BM;
+    const unsigned jt0 = (logical / m_blocks) * tiles_per_wg;
+    const unsigned jt1 = jt0 + tiles_per_wg < j_tiles ? jt0 + tiles_per_wg : j_tiles;
+    if (m_dev) {
+        m = *m_dev;
+        if (i0 >= m) return;
+    }
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wi = wave >> 1, wj = wave & 1;
+    const int n_last = (int) n - 1, m_last = m - 1;
+    const int a_row = tid / A_TPR, a_k = (tid % A_TPR) * (4 * A_VEC);
+    const int b_row = tid >> 1, b_k = (tid & 1) * (4 * B_VEC);
+    const int lrow = lane & 15;
+    const int lk = lane >> 4;
+    // Which column of the tile sits in which column slot of the B operand is free to choose.  Slot (tj, l) of a
+    // wavefront's 64 columns holds column 4*l + tj, so the four accumulator tiles of a lane are four consecutive
+    // columns and a lane's results for one working row leave as one 16- or 32-byte store (16 lanes: one run of 256
+    // or 512 bytes of the output row) instead of four stores 64 columns apart.
+    const int b_col = (b_row & 64) + ((b_row & 15) << 2) + ((b_row >> 4) & 3);   // column (in the tile) staged by this thread
+
+    if (tid < 32) exp_tab[tid] = TSVM_EXP2F_TAB[tid];
+    if (tid < BM) {
+        const int r = min(i0 + tid, m_last);
+        const int id = a_idx ? a_idx[r] : r;
+        s_slot[tid] = out_slots ? out_slots[r] : r;
+        s_sdi[tid] = sd_a ? sd_a[id] : 0.0;
+        s_mi[tid] = IND ? mask_a[id] : 0;
+    }
+    int a_r = min(i0 + a_row, m_last);
+    if (a_idx) a_r = a_idx[a_r];
+    const double *a_ptr = a + (uint64_t) (uint32_t) a_r * (uint32_t) lda;
+
+    const int n_kt = (d + KTILE - 1) / KTILE;
+    const int n_ks_last = (d - (n_kt - 1) * KTILE + 3) / 4;   // groups of four columns in the last K tile, 1 .. KTILE / 4
+    v4d ra[A_VEC], rb[B_VEC];
+    double pre_sd = 0.0;      // the next tile's column data for column tid (threads below 128)
+    uint64_t pre_m = 0;
+    const double *x_ptr = x;
+    // requests everything of column tile jt that comes from memory: the first K tile and the columns' self dot
+    // products and masks
+    auto request_tile = [&](unsigned jt) {
+        int x_r = min((int) jt * GR_BN + b_col, n_last);
+        if (x_idx) x_r = x_idx[x_r];
+        x_ptr = x + (uint64_t) (uint32_t) x_r * (uint32_t) ldx;
+        if (tid < GR_BN) {
+            int jc = min((int) jt * GR_BN + tid, n_last);
+            if (x_idx) jc = x_idx[jc];
+            pre_sd = sd_x ? sd_x[jc] : 0.0;
+            pre_m = IND ? mask_x[jc] : 0;
+        }
+    };
+    // Rows are zero-padded up to ldx / lda (multiples of 8); the last 16-column tile may reach past that: vectors
+    // that would start beyond the row re-read its last four columns instead (staged, never multiplied).
+    auto load_tile = [&](int kt, bool last) {
+        const int k0 = kt * KTILE;
+        if (!last) {
+#pragma unroll
+            for (int q = 0; q < A_VEC; ++q) ra[q] = *(const v4d *) (a_ptr + (k0 + a_k + 4 * q));
+#pragma unroll
+            for (int q = 0; q < B_VEC; ++q) rb[q] = *(const v4d *) (x_ptr + (k0 + b_k + 4 * q));
+        } else {
+#pragma unroll
+            for (int q = 0; q < A_VEC; ++q) ra[q] = *(const v4d *) (a_ptr + min(k0 + a_k + 4 * q, (int) lda - 4));
+#pragma unroll
+            for (int q = 0; q < B_VEC; ++q) rb[q] = *(const v4d *) (x_ptr + min(k0 + b_k + 4 * q, (int) ldx - 4));
+        }
+    };
+    // (IND: the columns from d on are live data, not padding, and the last group of four columns may reach into
+    // them: the working rows' values there are staged as zeros, which makes every such product an exact zero)
+    const int k_live = d - (n_kt - 1) * KTILE;   // columns of the last K tile that belong to the product
+    auto stage_tile = [&](bool last) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+#pragma unroll
+            for (int q = 0; q < A_VEC; ++q)
+                As[(a_k + 4 * q + e) * LS + a_row] = (IND && last && a_k + 4 * q + e >= k_live) ? 0.0 : ra[q][e];
+#pragma unroll
+            for (int q = 0; q < B_VEC; ++q) Bs[(b_k + 4 * q + e) * LS + b_row] = rb[q][e];
+        }
+    };
+    if (jt0 < jt1) {
+        request_tile(jt0);
+        if (n_kt > 0) load_tile(0, n_kt == 1);
+    }
+    for (unsigned jt = jt0; jt < jt1; ++jt) {
+        const int gen = (int) (jt & 1u);
+        const int j0 = (int) jt * GR_BN;
+        const int jb = j0 + wj * 64 + lrow * 4;   // first of this lane's four columns
+        const bool full = (i0 + BM <= m) && (j0 + GR_BN <= (int) n);
+        if (tid < GR_BN) {
+            s_sdj[gen][tid] = pre_sd;
+            s_mj[gen][tid] = pre_m;
+        }
+        v4d acc[TI][4];
+#pragma unroll
+        for (int ti = 0; ti < TI; ++ti)
+#pragma unroll
+            for (int tj = 0; tj < 4; ++tj) acc[ti][tj] = (v4d){0.0, 0.0, 0.0, 0.0};
+        auto mma_step = [&](int ks) {
+            double af[TI], bf[4];
+            const int kk = (ks * 4 + lk) * LS;
+#pragma unroll
+            for (int t = 0; t < TI; ++t) af[t] = As[kk + wi * (16 * TI) + t * 16 + lrow];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) bf[t] = Bs[kk + wj * 64 + t * 16 + lrow];
+#pragma unroll
+            for (int ti = 0; ti < TI; ++ti)
+#pragma unroll
+                for (int tj = 0; tj < 4; ++tj)
+                    acc[ti][tj] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[ti], bf[tj], acc[ti][tj], 0, 0, 0);
+        };
+        if (n_kt > 0) {
+            for (int kt = 0; kt + 1 < n_kt; ++kt) {
+                stage_tile(false);
+                __syncthreads();
+                load_tile(kt + 1, kt + 2 == n_kt);
+#pragma unroll
+                for (int ks = 0; ks < KTILE / 4; ++ks) mma_step(ks);
+                __syncthreads();
+            }
+            stage_tile(true);
+        }
+        __syncthreads();   // the staged tile, this tile's column data and (first tile) the row data are in LDS
+        if (jt + 1 < jt1) {   // the next column tile's requests go out now, ahead of this tile's epilogue
+            request_tile(jt + 1);
+            if (n_kt > 0) load_tile(0, n_kt == 1);
+        }
+        if (n_kt > 0) {
+#pragma unroll
+            for (int ks = 0; ks < KTILE / 4; ++ks)
+                if (ks < n_ks_last) mma_step(ks);
+            __syncthreads();   // every wavefront is done with the staged tile before the next one is written
+        }
+        double sdj[4];
+        uint64_t mj[4];
+#pragma unroll
+        for (int tj = 0; tj < 4; ++tj) {
+            sdj[tj] = s_sdj[gen][wj * 64 + lrow * 4 + tj];
+            mj[tj] = IND ? s_mj[gen][wj * 64 + lrow * 4 + tj] : 0;
+        }
+        // one value: the indicator columns' share, then the kernel function.  IND = 1..4: that many additions,
+        // unrolled (the addend is 1.0 or 0.0: no branch); IND = 5: max_ones of them in a loop
+        auto finish = [&](double dot, double sdi, uint64_t mi, int tj) -> TO {
+            if (IND) {
+                const int cnt = __popcll(mi & mj[tj]);
+                if (IND <= 4) {
+#pragma unroll
+                    for (int t = 0; t < IND; ++t) dot += cnt > t ? 1.0 : 0.0;
+                } else {
+                    for (int t = 0; t < max_ones; ++t) dot += cnt > t ? 1.0 : 0.0;
+                }
+            }
+            return tsvm_epilogue_as<TO>(dot, sdi, sdj[tj], kp, exp_tab);
+        };
+        // interior tiles store without a test, four columns at a time; edge tiles (and outputs whose rows are not
+        // 16-byte aligned) test and store every element
+        typedef TO vec4_t __attribute__((ext_vector_type(4)));
+        if (full && vec_ok) {
+#pragma unroll
+            for (int ti = 0; ti < TI; ++ti) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int r = wi * (16 * TI) + ti * 16 + 4 * v + lk;   // row of the tile
+                    const double sdi = s_sdi[r];
+                    const uint64_t mi = IND ? s_mi[r] : 0;
+                    TO *orow = out + (int64_t) ((uint64_t) (uint32_t) s_slot[r] * (uint32_t) ldo) + jb;
+                    vec4_t res;
+#pragma unroll
+                    for (int tj = 0; tj < 4; ++tj) res[tj] = finish(acc[ti][tj][v], sdi, mi, tj);
+                    *(vec4_t *) orow = res;
+                }
+            }
+        } else {
+#pragma unroll
+            for (int ti = 0; ti < TI; ++ti) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int r = wi * (16 * TI) + ti * 16 + 4 * v + lk;
+                    if (i0 + r >= m) continue;
+                    const double sdi = s_sdi[r];
+                    const uint64_t mi = IND ? s_mi[r] : 0;
+                    TO *orow = out + (int64_t) ((uint64_t) (uint32_t) s_slot[r] * (uint32_t) ldo) + jb;
+#pragma unroll
+                    for (int tj = 0; tj < 4; ++tj)
+                        if (jb + tj < n) orow[tj] = finish(acc[ti][tj][v], sdi, mi, tj);
+                }
+            }
+        }
+    }
+}
+
+// mask[r] = bit b set where x[r][first + b] != 0, b < count <= 64; *max_ones = largest number of set bits of a row
+// (raised with atomicMax: the caller clears it)
+__global__ void indicator_masks_kernel(const double *__restrict__ x, int64_t ld, int64_t n, int first, int count,
+                                       uint64_t *__restrict__ mask, int *__restrict__ max_ones) {
+    const int64_t r = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
+    int ones = 0;
+    if (r < n) {
+        uint64_t mk = 0;
+        const double *row = x + r * ld + first;
+        for (int b = 0; b < count; ++b) mk |= (uint64_t) (row[b] != 0.0) << b;
+        mask[r] = mk;
+        ones = __popcll(mk);
+    }
+#pragma unroll
+    for (int msk = 32; msk >= 1; msk >>= 1) ones = max(ones, __shfl_xor(ones, msk, 64));
+    if ((threadIdx.x & 63) == 0 && ones > 0) atomicMax(max_ones, ones);
 }
 
 // The m x m block K(x_idx[r], x_idx[t]) (a == x, a_idx == x_idx, rows written in place): tiles that lie below the
@@ -608,10 +862,21 @@ static bool row_type_ok(int row_type, int kernel_type) {
     return row_type == TSVM_ROW_F64 || (row_type == TSVM_ROW_F32 && kernel_type != TSVM_LINEAR);
 }
 
+// Column tiles a workgroup of the few-feature kernel walks (TSVM_GR_TILES overrides the default of 4).
+static int stream_tiles_per_wg() {
+    static const int v = [] {
+        const char *e = getenv("TSVM_GR_TILES");
+        const int t = e ? atoi(e) : 0;
+        return t >= 1 && t <= 64 ? t : 4;
+    }();
+    return v;
+}
+
 static int get_rows_dense(const double *x, int64_t ldx, const int *x_idx, int64_t n, int d, const double *sd_x, const double *a,
                           int64_t lda, const int *a_idx, int m, const int *m_dev, const double *sd_a, int kernel_type, double gamma,
                           double coef0, int degree, void *out, int row_type, const int *out_slots, int64_t ldo,
-                          tsvm_stream stream) {
+                          tsvm_stream stream, const uint64_t *mask_x = nullptr, const uint64_t *mask_a = nullptr,
+                          int max_ones = 0) {
     TSVM_REQUIRE(x && a && out, "tsvm_get_rows_dense: null pointer");
     TSVM_REQUIRE(n >= 0 && m >= 0 && d >= 0, "tsvm_get_rows_dense: negative size");
     TSVM_REQUIRE(n <= 0x7fff0000 && ldx <= 0x7fffffff && lda <= 0x7fffffff && ldo <= 0x7fffffff,
@@ -632,7 +897,7 @@ static int get_rows_dense(const double *x, int64_t ldx, const int *x_idx, int64_
     // (also when the 128-row tile would leave most of the chip without a workgroup, as for the solver's
     // ws x ws block, whose latency is that of one workgroup walking the whole feature range)
     const int64_t wg4 = ((n + GR_BN - 1) / GR_BN) * ((m + 127) / 128);
-    const int ti = (d <= 128 || wg4 < 512) ? 2 : 4;
+    const int ti = (d <= 128 || wg4 < 512 || mask_x) ? 2 : 4;
     const unsigned m_blocks = (unsigned) ((m + 32 * ti - 1) / (32 * ti));
     const int64_t n_blocks = (n + GR_BN - 1) / GR_BN;
     TSVM_REQUIRE(n_blocks * m_blocks < (int64_t) 0x7fffffff, "tsvm_get_rows_dense: grid too large");
@@ -663,12 +928,30 @@ static int get_rows_dense(const double *x, int64_t ldx, const int *x_idx, int64_
         TSVM_LAUNCH_CHECK();
         return 0;
     }
+    // few features: workgroups walk runs of column tiles (one tile each while the launch is too small to fill the chip
+    // several times over)
+    const int64_t total_tiles = n_blocks * m_blocks;
+    const unsigned tpw = (unsigned) std::max<int64_t>(1, std::min<int64_t>(stream_tiles_per_wg(), total_tiles / 3072));
+    const dim3 sgrid((unsigned) (((n_blocks + tpw - 1) / tpw) * m_blocks));
+    // four results per store need every group of four columns of every output row 16-byte aligned
+    const int vec_ok = ((uintptr_t) out % 16 == 0) && (ldo % 4 == 0);
+    const int ind_mode = !mask_x ? 0 : (max_ones >= 1 && max_ones <= 4) ? max_ones : 5;   // additions unrolled up to four
+#define GR_STREAM(KTYPE, TO, IND)                                                                                     \
+    hipLaunchKernelGGL((get_rows_dense_stream_kernel<KTYPE, TO, IND>), sgrid, block, 0, tsvm_s(stream), x, ldx, x_idx, n, d, sd_x, \
+                       a, lda, a_idx, m, sd_a, kp, (TO *) out, out_slots, ldo, m_blocks, (unsigned) n_blocks, tpw, m_dev, mask_x, \
+                       mask_a, max_ones, vec_ok)
 #define GR_LAUNCH_T(KTYPE, TO)                                                                                        \
     do {                                                                                                              \
-        if (ti == 2)                                                                                                  \
-            hipLaunchKernelGGL((get_rows_dense_kernel<KTYPE, 2, TO>), grid, block, 0, tsvm_s(stream), x, ldx, x_idx, n, d, sd_x, \
-                               a, lda, a_idx, m, sd_a, kp, (TO *) out, out_slots, ldo, m_blocks, m_dev);              \
-        else                                                                                                          \
+        if (ti == 2) {                                                                                                \
+            switch (ind_mode) {                                                                                       \
+                case 0: GR_STREAM(KTYPE, TO, 0); break;                                                               \
+                case 1: GR_STREAM(KTYPE, TO, 1); break;                                                               \
+                case 2: GR_STREAM(KTYPE, TO, 2); break;                                                               \
+                case 3: GR_STREAM(KTYPE, TO, 3); break;                                                               \
+                case 4: GR_STREAM(KTYPE, TO, 4); break;                                                               \
+                default: GR_STREAM(KTYPE, TO, 5); break;                                                              \
+            }                                                                                                         \
+        } else                                                                                                        \
             hipLaunchKernelGGL((get_rows_dense_kernel<KTYPE, 4, TO>), grid, block, 0, tsvm_s(stream), x, ldx, x_idx, n, d, sd_x, \
                                a, lda, a_idx, m, sd_a, kp, (TO *) out, out_slots, ldo, m_blocks, m_dev);              \
     } while (0)
@@ -685,6 +968,7 @@ static int get_rows_dense(const double *x, int64_t ldx, const int *x_idx, int64_
     }
 #undef GR_LAUNCH
 #undef GR_LAUNCH_T
+#undef GR_STREAM
     TSVM_LAUNCH_CHECK();
     return 0;
 }
@@ -704,6 +988,32 @@ int tsvm_get_rows_dense_counted(const double *x, int64_t ldx, const int *x_idx, 
     TSVM_REQUIRE(m_dev, "tsvm_get_rows_dense_counted: null pointer");
     return get_rows_dense(x, ldx, x_idx, n, d, sd_x, a, lda, a_idx, m_max, m_dev, sd_a, kernel_type, gamma, coef0, degree, out,
                           row_type, out_slots, ldo, stream);
+}
+
+int tsvm_indicator_masks(const double *x, int64_t ld, int64_t n, int first_col, int n_cols, uint64_t *masks, int *max_ones,
+                         tsvm_stream stream) {
+    TSVM_REQUIRE(x && masks && max_ones && n >= 0, "tsvm_indicator_masks: bad argument");
+    TSVM_REQUIRE(first_col >= 0 && n_cols >= 1 && n_cols <= 64 && first_col + n_cols <= ld,
+                 "tsvm_indicator_masks: columns %d..%d outside the row (ld %lld) or more than 64", first_col, first_col + n_cols,
+                 (long long) ld);
+    hipLaunchKernelGGL(fill_i32_kernel, dim3(1), dim3(64), 0, tsvm_s(stream), max_ones, (int64_t) 1, 0);
+    TSVM_LAUNCH_CHECK();
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(indicator_masks_kernel, dim3(grid_for(n, 256)), dim3(256), 0, tsvm_s(stream), x, ld, n, first_col, n_cols,
+                       masks, max_ones);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+int tsvm_get_rows_dense_indicator(const double *x, int64_t ldx, const int *x_idx, int64_t n, int d_dense, const double *sd_x,
+                                  const uint64_t *mask_x, const double *a, int64_t lda, const int *a_idx, int m, const int *m_dev,
+                                  const double *sd_a, const uint64_t *mask_a, int max_ones, int kernel_type, double gamma,
+                                  double coef0, int degree, void *out, int row_type, const int *out_slots, int64_t ldo,
+                                  tsvm_stream stream) {
+    TSVM_REQUIRE(mask_x && mask_a, "tsvm_get_rows_dense_indicator: null mask");
+    TSVM_REQUIRE(max_ones >= 0 && max_ones <= 64, "tsvm_get_rows_dense_indicator: max_ones %d outside [0, 64]", max_ones);
+    return get_rows_dense(x, ldx, x_idx, n, d_dense, sd_x, a, lda, a_idx, m, m_dev, sd_a, kernel_type, gamma, coef0, degree, out,
+                          row_type, out_slots, ldo, stream, mask_x, mask_a, max_ones);
 }
 
 int tsvm_csr_stage_rows(const double *val, const int *col, const int64_t *row_ptr, const int *idx, int m,

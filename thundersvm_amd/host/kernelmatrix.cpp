@@ -117,6 +117,7 @@ std::shared_ptr<DeviceRows> DeviceRows::from_host(const DataSet::node2d &all, co
         r.val.release();
         r.col.release();
         r.row_ptr.release();
+        r.find_indicator_columns();
     } else {
         r.host_row_ptr = std::move(ptr);
     }
@@ -139,6 +140,13 @@ std::shared_ptr<DeviceRows> DeviceRows::subset(const DeviceRows &base, const int
         r.x.resize(n_rows * (size_t) r.ld);
         abi_check(tsvm_gather_rows_f64(base.x.data(), base.ld, d_rows.data(), (int64_t) n_rows, r.x.data(), nullptr));
         r.nnz = n_rows ? base.nnz / std::max<size_t>(base.n, 1) * n_rows : 0;   // estimate, informational only
+        if (base.ind_first >= 0) {   // indicator columns of all rows are indicator columns of a subset (masks move as 8-byte words)
+            r.ind_first = base.ind_first;
+            r.ind_max_ones = base.ind_max_ones;
+            r.ind_mask.resize(n_rows);
+            abi_check(tsvm_gather_f64(reinterpret_cast<const double *>(base.ind_mask.data()), d_rows.data(), (int) n_rows,
+                                      reinterpret_cast<double *>(r.ind_mask.data()), nullptr));
+        }
     } else {
         r.host_row_ptr.assign(n_rows + 1, 0);
         for (size_t i = 0; i < n_rows; ++i)
@@ -162,6 +170,27 @@ const std::vector<int> &DeviceRows::column_stats() const {
         column_stats_ = d_counts.to_host();
     }
     return column_stats_;
+}
+
+// The trailing run of columns whose values are all 0 or 1, if leaving it out of the matrix product saves more than
+// the additions it costs in the epilogue: one 4-column step of the matrix cores per value is worth about one
+// epilogue instruction, an indicator column that may match costs about three.
+void DeviceRows::find_indicator_columns() {
+    ind_first = -1;
+    if (!dense || n == 0 || n_features == 0 || getenv("TSVM_NO_INDICATOR")) return;
+    const std::vector<int> &stats = column_stats();
+    int first = (int) n_features;
+    while (first > 0 && (int) n_features - first < 64 && stats[n_features + first - 1] == 0) --first;
+    if (first == (int) n_features) return;
+    tsvm::DeviceBuffer<uint64_t> masks(n);
+    tsvm::DeviceBuffer<int> d_max(1);
+    abi_check(tsvm_indicator_masks(x.data(), ld, (int64_t) n, first, (int) n_features - first, masks.data(), d_max.data(), nullptr));
+    const int max_ones = d_max.to_host()[0];
+    const int steps_saved = (int) ((n_features + 3) / 4) - (first + 3) / 4;
+    if (steps_saved < 2 + 3 * max_ones) return;
+    ind_first = first;
+    ind_max_ones = max_ones;
+    ind_mask = std::move(masks);
 }
 
 std::shared_ptr<DeviceRows> DeviceRows::of(const DataSet &dataset) {
@@ -248,6 +277,13 @@ void KernelMatrix::get_rows(const int *d_idx, int m, void *d_out, int64_t ld, co
                             hipStream_t stream) const {
     const DeviceRows &R = *rows_;
     const int n = (int) n_unique_;
+    if (R.dense && R.ind_first >= 0) {
+        abi_check(tsvm_get_rows_dense_indicator(R.x.data(), R.ld, nullptr, n, R.ind_first, R.self_dot.data(), R.ind_mask.data(),
+                                                R.x.data(), R.ld, d_idx, m, nullptr, R.self_dot.data(), R.ind_mask.data(),
+                                                R.ind_max_ones, (int) param.kernel_type, param.gamma, param.coef0, param.degree,
+                                                d_out, row_type(), d_out_slots, ld, stream));
+        return;
+    }
     if (R.dense) {
         abi_check(tsvm_get_rows_dense(R.x.data(), R.ld, nullptr, n, (int) R.n_features, R.self_dot.data(), R.x.data(), R.ld, d_idx,
                                       m, R.self_dot.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
@@ -273,6 +309,13 @@ void KernelMatrix::get_rows_counted(const int *d_idx, int m_max, const int *d_m,
                                     const int *d_out_slots, hipStream_t stream) const {
     const DeviceRows &R = *rows_;
     if (!R.dense) throw std::logic_error("KernelMatrix::get_rows_counted: dense layout only");
+    if (R.ind_first >= 0) {
+        abi_check(tsvm_get_rows_dense_indicator(R.x.data(), R.ld, nullptr, (int) n_unique_, R.ind_first, R.self_dot.data(),
+                                                R.ind_mask.data(), R.x.data(), R.ld, d_idx, m_max, d_m, R.self_dot.data(),
+                                                R.ind_mask.data(), R.ind_max_ones, (int) param.kernel_type, param.gamma,
+                                                param.coef0, param.degree, d_out, row_type(), d_out_slots, ld, stream));
+        return;
+    }
     abi_check(tsvm_get_rows_dense_counted(R.x.data(), R.ld, nullptr, (int) n_unique_, (int) R.n_features, R.self_dot.data(),
                                           R.x.data(), R.ld, d_idx, m_max, d_m, R.self_dot.data(), (int) param.kernel_type,
                                           param.gamma, param.coef0, param.degree, d_out, row_type(), d_out_slots, ld, stream));

@@ -37,6 +37,12 @@ struct DeviceRows {
     // that are neither 0 nor 1; counted on the device on first use
     const std::vector<int> &column_stats() const;
     mutable std::vector<int> column_stats_;
+    // Dense layout: when the last columns hold only zeros and ones (one-hot encoded categories), columns
+    // ind_first .. n_features-1 (at most 64) are also kept as one bit mask per row, and get_rows leaves them to the
+    // kernel's epilogue instead of the matrix cores.  ind_first < 0: no such part.
+    int ind_first = -1, ind_max_ones = 0;
+    tsvm::DeviceBuffer<uint64_t> ind_mask;       // [n]
+    void find_indicator_columns();
 
     // rows[0..n_rows) of `all` (rows == nullptr: the first n_rows), assembled on the host and uploaded
     static std::shared_ptr<DeviceRows> from_host(const DataSet::node2d &all, const int *rows, size_t n_rows);

@@ -336,9 +336,10 @@ void SVC::train(const DataSet &dataset, SvmParam p) {   // svc.cpp:41-145
     std::vector<std::vector<float_type>> alpha(n_binary_models);
     std::vector<char> is_sv(n, 0);
     int k = 0;
-    // pairs in flight: two when every pair's solver gets CUs of its own (more pairs only add queues), three when
-    // the pairs alternate between a solver phase and a chip-wide phase
-    const int lanes = std::min(pair_lanes > 0 ? pair_lanes : SolveTask::cu_split_available() ? 2 : 3, n_binary_models);
+    // pairs in flight: four when every pair's solver gets CUs of its own and the pairs advance independently (more
+    // gain nothing: the chip-wide kernels of four pairs already keep the chip busy), three when the pairs alternate
+    // between a solver phase and a chip-wide phase
+    const int lanes = std::min(pair_lanes > 0 ? pair_lanes : SolveTask::cu_split_available() ? 4 : 3, n_binary_models);
     if (lanes > 1 && !profile && !trace_first) {
         train_pairs_in_lockstep(grouped, lanes, alpha);
     } else {
@@ -489,16 +490,65 @@ void SVC::train_pairs_in_lockstep(const DataSet &grouped, int lanes, std::vector
         TSVM_HIP_CHECK(hipEventCreateWithFlags(&p->solved, hipEventDisableTiming));
         active.push_back(std::move(p));
     };
+    auto retire = [&](size_t a) {
+        BinaryProblem &p = *active[a];
+        solver_stats[p.k] = p.task->stats();
+        if (keep_binary) binary_f[p.k] = p.f_val;
+        p.task.reset();   // synchronises and releases the pair's stream before its lane is reused
+        (void) hipEventDestroy(p.rows_done);
+        (void) hipEventDestroy(p.solved);
+        finish_binary(p, alpha[p.k]);
+        free_lanes.push_back(p.lane);
+        active.erase(active.begin() + a);
+    };
     while (next < pairs.size() && !free_lanes.empty()) start_next();
+    if (!active.empty() && active.front()->task->split_streams()) {
+        // Every pair's solver has CUs of its own, so the pairs need no common phases: each lane runs at its own
+        // pace.  The host looks at the lanes in turn and serves whichever has something to do: a lane whose
+        // iteration has reported gets its next selection, block and solver enqueued; a lane whose new ids have
+        // arrived (host-side row cache) gets its rows and update_f.  A small pair next to a large one thus makes
+        // several iterations in the time the large one makes one.
+        auto begin_iteration = [](BinaryProblem &p) {
+            p.task->enqueue_select();
+            p.task->enqueue_block();
+            p.task->enqueue_solver();
+            p.rows_pending = true;
+        };
+        for (auto &p : active) begin_iteration(*p);
+        while (!active.empty()) {
+            bool served = false;
+            for (size_t a = 0; a < active.size();) {
+                BinaryProblem &p = *active[a];
+                if (p.rows_pending) {
+                    if (p.task->rows_ready()) {
+                        p.task->enqueue_rows();
+                        p.task->enqueue_update();
+                        p.rows_pending = false;
+                        served = true;
+                    }
+                    ++a;
+                } else if (p.task->iteration_done()) {
+                    served = true;
+                    if (p.task->finish_iteration()) {
+                        retire(a);
+                        const size_t before = active.size();
+                        while (next < pairs.size() && !free_lanes.empty()) start_next();
+                        for (size_t b = before; b < active.size(); ++b) begin_iteration(*active[b]);
+                    } else {
+                        begin_iteration(p);
+                        ++a;
+                    }
+                } else {
+                    ++a;
+                }
+            }
+            if (!served) __builtin_ia32_pause();
+        }
+        return;
+    }
     while (!active.empty()) {
         for (auto &p : active) p->task->enqueue_select();
-        if (active.front()->task->split_streams()) {
-            // Every pair's solver has CUs of its own: the pairs need no phases, their steps are only enqueued in
-            // an order that lets each solver start before the host turns to the cache bookkeeping.
-            for (auto &p : active) { p->task->enqueue_block(); p->task->enqueue_solver(); }
-            for (auto &p : active) p->task->enqueue_rows();
-            for (auto &p : active) p->task->enqueue_update();
-        } else {
+        {
         for (auto &p : active) {
             p->task->enqueue_rows();
             p->task->enqueue_block();
@@ -517,16 +567,8 @@ void SVC::train_pairs_in_lockstep(const DataSet &grouped, int lanes, std::vector
         }
         }
         for (size_t a = 0; a < active.size();) {
-            BinaryProblem &p = *active[a];
-            if (!p.task->finish_iteration()) { ++a; continue; }
-            solver_stats[p.k] = p.task->stats();
-            if (keep_binary) binary_f[p.k] = p.f_val;
-            p.task.reset();   // synchronises and releases the pair's stream before its lane is reused
-            (void) hipEventDestroy(p.rows_done);
-            (void) hipEventDestroy(p.solved);
-            finish_binary(p, alpha[p.k]);
-            free_lanes.push_back(p.lane);
-            active.erase(active.begin() + a);
+            if (!active[a]->task->finish_iteration()) { ++a; continue; }
+            retire(a);
         }
         while (next < pairs.size() && !free_lanes.empty()) start_next();
     }

@@ -99,6 +99,7 @@ protected:
         std::unique_ptr<SolveTask> task;
         hipEvent_t rows_done = nullptr, solved = nullptr;
         int lane = 0;
+        bool rows_pending = false;   // independent lanes: the iteration's rows and update_f are still to be enqueued
     };
     virtual void setup_binary(const DataSet &dataset, int i, int j, BinaryProblem &p);   // svc.cpp:147-170
     void finish_binary(BinaryProblem &p, std::vector<float_type> &alpha_out);            // svc.cpp:171-177

@@ -230,6 +230,39 @@ struct SolveTask::Impl {
         tsvm::wait_while_pending(diff_word(), DIFF_PENDING, tsvm::solver_timeout_ms(),
                                  [](void *st) { return hipStreamQuery((hipStream_t) st); }, solver_stream);
     }
+    // the same wait as a poll (one look per call; the stream is asked, and the time-out checked, every 200 ms)
+    std::chrono::steady_clock::time_point solver_enqueued, next_stream_check;
+    bool diff_arrived() {
+        if (wait_by_event) {
+            const hipError_t e = hipEventQuery(diff_ready);
+            if (e == hipSuccess) return true;
+            if (e != hipErrorNotReady) TSVM_HIP_CHECK(e);
+            return false;
+        }
+        if (*diff_word() != DIFF_PENDING) {
+            __atomic_thread_fence(__ATOMIC_ACQUIRE);
+            return true;
+        }
+        const auto now = std::chrono::steady_clock::now();
+        if (now < next_stream_check) return false;
+        next_stream_check = now + std::chrono::milliseconds(200);
+        const hipError_t e = hipStreamQuery(solver_stream);
+        if (e == hipSuccess) {
+            if (*diff_word() == DIFF_PENDING) throw std::runtime_error("SolveTask: the local solver finished without reporting");
+        } else if (e != hipErrorNotReady) {
+            TSVM_HIP_CHECK(e);
+        }
+        if (now - solver_enqueued > std::chrono::milliseconds(tsvm::solver_timeout_ms()))
+            throw std::runtime_error("SolveTask: no word from the local solver (TSVM_SOLVER_TIMEOUT_MS); the device may be hung");
+        return false;
+    }
+    bool ids_arrived() const {
+        if (!(caching && !all_cached && !device_cache)) return true;
+        const hipError_t e = hipEventQuery(ids_ready);
+        if (e == hipSuccess) return true;
+        if (e != hipErrorNotReady) TSVM_HIP_CHECK(e);
+        return false;
+    }
     int rotation_base = 0;   // iteration at which d_slots_a was valid
     long long window_lookups = 0, window_hits = 0;
     const int *slots = nullptr;
@@ -367,10 +400,10 @@ struct SolveTask::Impl {
     // unexpected (another CU count, the call failing, TSVM_NO_CU_SPLIT set) leaves the task on one plain stream.
     // Lane l's solver gets CU l of every XCD; the chip-wide kernels of all lanes get the CUs no lane's solver has.
     bool create_split_streams(int lane, int n_lanes) {
-        if (!SolveTask::cu_split_available() || n_lanes < 1 || n_lanes > 4 || lane < 0 || lane >= n_lanes) return false;
+        if (!SolveTask::cu_split_available() || n_lanes < 1 || n_lanes > 8 || lane < 0 || lane >= n_lanes) return false;
         int dev = 0;
         if (hipGetDevice(&dev) != hipSuccess) return false;
-        masked_key = ((long long) dev * 8 + n_lanes) * 8 + lane;
+        masked_key = ((long long) dev * 16 + n_lanes) * 16 + lane;
         {
             std::lock_guard<std::mutex> lock(g_masked_mutex);
             for (MaskedStreams &m : g_masked[masked_key])
@@ -381,9 +414,11 @@ struct SolveTask::Impl {
                     return true;
                 }
         }
-        uint32_t small[8] = {0xffu << (8 * lane), 0, 0, 0, 0, 0, 0, 0};
-        uint32_t big[8] = {0, ~0u, ~0u, ~0u, ~0u, ~0u, ~0u, ~0u};
-        big[0] = n_lanes == 4 ? 0u : ~0u << (8 * n_lanes);
+        // lane l's solver: CU l of every XCD = mask bits 8l .. 8l+7; the chip-wide stream: every CU from n_lanes on
+        uint32_t small[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        uint32_t big[8] = {~0u, ~0u, ~0u, ~0u, ~0u, ~0u, ~0u, ~0u};
+        small[lane / 4] = 0xffu << (8 * (lane % 4));
+        for (int l = 0; l < n_lanes; ++l) big[l / 4] &= ~(0xffu << (8 * (l % 4)));
         if (hipExtStreamCreateWithCUMask(&ss, 8, small) != hipSuccess) { (void) hipGetLastError(); ss = nullptr; return false; }
         if (hipExtStreamCreateWithCUMask(&sa, 8, big) != hipSuccess) {
             (void) hipGetLastError();
@@ -425,15 +460,16 @@ struct SolveTask::Impl {
     // half of the previous set and pick q new ids (csmosolver.cpp:63-77).
     void launch_select(int it) {
         const int n_sel = it == 0 ? ws_size : q;
+        hipStream_t sel = sa;
         if (it == 0) {
             sel_off = 0;
         } else {
             int next = sel_off + q;
             if (next + ws_size > (int) d_ws.size()) {
-                TSVM_HIP_CHECK(hipMemcpyAsync(d_ws.data(), d_ws.data() + next, sizeof(int) * q, hipMemcpyDeviceToDevice, sa));
+                TSVM_HIP_CHECK(hipMemcpyAsync(d_ws.data(), d_ws.data() + next, sizeof(int) * q, hipMemcpyDeviceToDevice, sel));
                 if (rep > 1)
                     TSVM_HIP_CHECK(hipMemcpyAsync(d_ws_folded.data(), d_ws_folded.data() + next, sizeof(int) * q,
-                                                  hipMemcpyDeviceToDevice, sa));
+                                                  hipMemcpyDeviceToDevice, sel));
                 next = 0;
             }
             sel_off = next;
@@ -443,13 +479,13 @@ struct SolveTask::Impl {
         if (rep > 1) {
             abi_check(tsvm_select_working_set_folded(d_f.data(), d_y.data(), d_alpha.data(), n, Cp, Cn, kept, it == 0 ? 0 : q, out,
                                                      n_sel, nu, d_sel_ws.data(), it > 0, n_u,
-                                                     d_ws_folded.data() + sel_off + (it == 0 ? 0 : q), sa));
+                                                     d_ws_folded.data() + sel_off + (it == 0 ? 0 : q), sel));
         } else if (it == 0) {
             abi_check(tsvm_select_working_set(d_f.data(), d_y.data(), d_alpha.data(), n, Cp, Cn, kept, 0, out, n_sel, nu,
-                                              d_sel_ws.data(), sa));
+                                              d_sel_ws.data(), sel));
         } else {
             abi_check(tsvm_select_working_set_again(d_f.data(), d_y.data(), d_alpha.data(), n, Cp, Cn, kept, q, out, n_sel, nu,
-                                                    d_sel_ws.data(), sa));
+                                                    d_sel_ws.data(), sel));
         }
     }
 
@@ -599,6 +635,8 @@ struct SolveTask::Impl {
             *diff_word() = DIFF_PENDING;
             __atomic_thread_fence(__ATOMIC_RELEASE);
         }
+        solver_enqueued = std::chrono::steady_clock::now();
+        next_stream_check = solver_enqueued + std::chrono::milliseconds(200);
         if (!on_one_stream && !block_on_solver_cus) TSVM_HIP_CHECK(hipStreamWaitEvent(ss, block_done, 0));
         if (nu) {
             abi_check(tsvm_nu_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), ws_ids(), ws_size,
@@ -686,6 +724,8 @@ void SolveTask::enqueue_block() { impl_->enqueue_block(); }
 void SolveTask::enqueue_solver() { impl_->enqueue_solver(); }
 void SolveTask::enqueue_update() { impl_->enqueue_update(); }
 bool SolveTask::finish_iteration() { return impl_->finish_iteration(); }
+bool SolveTask::rows_ready() const { return impl_->ids_arrived(); }
+bool SolveTask::iteration_done() { return impl_->diff_arrived(); }
 bool SolveTask::block_needs_rows() const { return !impl_->block_first; }
 bool SolveTask::split_streams() const { return impl_->split; }
 bool SolveTask::cu_split_available() {

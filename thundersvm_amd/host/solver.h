@@ -102,6 +102,12 @@ public:
     void enqueue_solver();
     void enqueue_update();
     bool finish_iteration();   // waits for this iteration's diff; true once the solve is complete and its results are written
+    // For a caller that advances several tasks from one thread without blocking on any of them:
+    // rows_ready(): enqueue_rows would not wait (the newly selected ids the host-side row cache needs have arrived, or
+    // are not needed); iteration_done(): finish_iteration would not wait.  iteration_done() throws like the blocking
+    // wait when the solver's stream has drained without a report or nothing has been heard for the time-out.
+    bool rows_ready() const;
+    bool iteration_done();
     bool block_needs_rows() const;
     bool split_streams() const;   // the local solver runs on CUs of its own, next to this task's (and other tasks') chip-wide kernels
     hipStream_t stream() const;
