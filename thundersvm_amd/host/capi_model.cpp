@@ -225,6 +225,8 @@ int tsvm_model_stats(void *model, int k, int64_t *n_iter, int64_t *local_iter, d
             phase_ms[8] = s.ms_wall;
             phase_ms[9] = s.ms_setup;
             phase_ms[10] = (double) s.ws_size;
+            phase_ms[11] = (double) s.rows_computed;
+            phase_ms[12] = (double) s.update_rows;
         }
     })
 }

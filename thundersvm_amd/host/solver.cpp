@@ -552,6 +552,7 @@ struct SolveTask::Impl {
             std::copy(miss_slots.begin(), miss_slots.end(), h_miss_slots);
             const int n_miss = (int) miss_ids.size();
             last_rows_computed = n_miss;
+            stats.rows_computed += n_miss;
             TSVM_HIP_CHECK(hipMemcpyAsync(d_slots_a.data(), h_slots, sizeof(int) * (n_miss ? 3 * (size_t) ws_size : (size_t) ws_size),
                                           hipMemcpyHostToDevice, sa));
             if (n_miss) {
@@ -593,6 +594,7 @@ struct SolveTask::Impl {
             slots = on_a ? d_slots_a.data() : d_slots_b.data();
             // new rows go to the slots the dropped rows occupied
             last_rows_computed = n_new;
+            stats.rows_computed += n_new;
             k_mat.get_rows(ws_u() + first_new, n_new, k_rows, ld, slots + first_new, sa);
         }
         timer.end(stats.ms_get_rows);
@@ -654,6 +656,10 @@ struct SolveTask::Impl {
         timer.begin();
         abi_check(tsvm_update_f(d_f.data(), d_alpha_diff.data(), ws_size, k_rows, row_type, slots, ld, n_u, rep, sa));
         timer.end(stats.ms_update_f);
+        if (timer.on) {   // (profiling runs every step to completion anyway) how many rows did update_f have to read?
+            std::vector<float_type> ad = d_alpha_diff.to_host();
+            for (float_type v : ad) stats.update_rows += v != 0;
+        }
         if (wait_by_event) TSVM_HIP_CHECK(hipEventRecord(diff_ready, sa));
         if (select_ahead) {
             launch_select(iter + 1);
@@ -696,7 +702,10 @@ struct SolveTask::Impl {
         const bool stalled = (same_local_diff_cnt >= 10 || swap_local_diff_cnt >= 10) && fabs(diff0 - 2.0) > eps;
         if (stalled || diff0 < eps || (out_max_iter != -1 && iter == out_max_iter)) {
             TSVM_HIP_CHECK(hipStreamSynchronize(sa));   // a selection enqueued ahead may still be running
-            if (device_cache) stats.cache_hits = stats.cache_lookups - h_cache_info[1];   // every slot in use was one miss
+            if (device_cache) {   // every slot in use was one miss
+                stats.cache_hits = stats.cache_lookups - h_cache_info[1];
+                stats.rows_computed = h_cache_info[1];
+            }
             d_alpha.download(alpha.data(), n);
             d_f.download(f_val.data(), n);
             rho = solver.calculate_rho(f_val, y, alpha, Cp, Cn);

@@ -23,6 +23,8 @@ struct SolverStats {
     long long cache_rows = 0;     // capacity in rows (0: cache not used)
     bool cache_disabled = false;  // switched off after the warm-up because it was not hitting
     int ws_size = 0;              // working-set size of the solve
+    long long rows_computed = 0;  // kernel rows get_rows produced (cache misses), summed over the outer iterations
+    long long update_rows = 0;    // kernel rows update_f read (non-zero alpha_diff entries), counted only when profiling
 };
 
 class SolveTask;
