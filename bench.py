@@ -426,7 +426,7 @@ def main():
     configs = {}
     if args.others and args.scale == 1.0:
         gc.disable()
-        for name in ("c2", "c5", "c3"):
+        for name in ("c1", "c2", "c5", "c3"):
             if name == args.workload:
                 continue
             if name == "c3":
@@ -435,8 +435,8 @@ def main():
                     configs["c3_" + kern_name] = blk
                     del m
             else:
-                blk, m = measure_config(name, gen[name](args.scale), 2, 1)
-                if name == "c2" and args.cpu_seconds > 0:
+                blk, m = measure_config(name, gen[name](args.scale), 2, 1, with_kernels=name != "c1")
+                if name in ("c1", "c2") and args.cpu_seconds > 0:
                     w2 = gen[name](args.scale)
                     blk["cpu_baseline"] = cpu_baseline(w2["train"], w2["params"], m, min(args.cpu_seconds, 12.0))
                 configs[name] = blk
