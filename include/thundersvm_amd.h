@@ -234,6 +234,20 @@ int tsvm_nu_smo_solve_block(const int *y, const double *f_val, double *alpha, do
                             int ws_size, double C, const double *kws, const double *k_diag, double eps, double *diff,
                             int max_iter, tsvm_stream stream);
 
+/* No counterpart in the reference: the two block solvers above, made to run on a chosen accelerator die (XCD, 0..7).
+ * The launch has eight workgroups; under a stream whose CU mask leaves one CU per XCD one of them lands on every XCD,
+ * the one on `xcd` solves, the others leave at once (whatever the placement, exactly one workgroup solves).  The local
+ * solvers of up to eight class pairs can thus share one CU mask of eight CUs and still run on a CU, and behind an L2,
+ * of their own.  gate: three ints of device memory, zero before the first launch, shared by the launches of one
+ * stream only; epoch: 1 for the first launch on a gate, then one more per launch; gate[2] receives the XCD the
+ * solver ran on. */
+int tsvm_c_smo_solve_block_on_xcd(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
+                                  int ws_size, double Cp, double Cn, const double *kws, const double *k_diag, double eps,
+                                  double *diff, int max_iter, int *gate, int epoch, int xcd, tsvm_stream stream);
+int tsvm_nu_smo_solve_block_on_xcd(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
+                                   int ws_size, double C, const double *kws, const double *k_diag, double eps, double *diff,
+                                   int max_iter, int *gate, int epoch, int xcd, tsvm_stream stream);
+
 /* nu_smo_solve (smo_kernel.cpp:127-298), same conventions; diff[1] is left untouched as in the
  * reference's CPU code. */
 int tsvm_nu_smo_solve(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,

@@ -85,11 +85,12 @@ int tsvm_model_get(void *model, int *label, int *n_sv, double *rho, double *coef
                    int *sv_col, double *sv_val);
 
 /* Solver diagnostics of binary sub-problem k: outer iterations, inner iterations, objective and
- * phase[13]: device milliseconds of select, get_rows, local solve, update_f (zeros unless profiled),
+ * phase[16]: device milliseconds of select, get_rows, local solve, update_f (zeros unless profiled),
  * then kernel-row cache lookups, hits, capacity in rows, 1 if the cache was switched off, and the host
  * wall-clock milliseconds of the whole solve and of its set-up (allocations, uploads, init_f), the
  * working-set size the problem was solved with, the kernel rows computed by get_rows over the whole solve, and (when
- * profiled) the kernel rows read by update_f. */
+ * profiled) the kernel rows read by update_f; then, for class pairs solved side by side, the die the pair's local solver ran
+ * on (-1 otherwise), and the host clock at the start and the end of the solve (ms since the process's first solve). */
 int tsvm_model_stats(void *model, int k, int64_t *n_iter, int64_t *local_iter, double *obj, double *phase_ms);
 
 int64_t tsvm_model_binary_size(void *model, int k);

@@ -273,10 +273,13 @@ def test_more_than_32_classes():
 
 
 @pytest.mark.parametrize("svm_type,extra", [(3, dict(p=0.1)), (3, dict(p=0.0)), (4, dict(nu=0.4))])
-def test_cache_switched_off_mid_run_on_a_stacked_problem(svm_type, extra):
+def test_cache_switched_off_mid_run_on_a_stacked_problem(svm_type, extra, monkeypatch):
     """A row cache that has filled up and does not hit is switched off in mid-run (rotation between two slot
     tables from then on).  On the 2n-variable problems of SVR two working-set positions may share one stored row;
-    after the switch every position must own a slot.  Same trajectory and model as without a cache, bit for bit."""
+    after the switch every position must own a slot.  Same trajectory and model as without a cache, bit for bit.
+    (The switch is made to happen at the first check, whatever the hit rate: TSVM_CACHE_OFF_BELOW is the percentage
+    of a window's repeated lookups that must hit for the cache to stay.)"""
+    monkeypatch.setenv("TSVM_CACHE_OFF_BELOW", "101")
     w = D.workload_c5(scale=0.01)
     tr = w["train"]
     p = dict(w["params"], svm_type=svm_type)

@@ -152,13 +152,41 @@ __device__ __forceinline__ unsigned set_member_bits(unsigned m, int tid, int t, 
 #define TSVM_TOUCH_ROW(kws, t, ws, ldk, lane) \
     (((const unsigned *) ((kws) + (int64_t) ((t) < (ws) ? (t) : 0) * (ldk)))[(lane) * 32 < (ldk) * 2 ? (lane) * 32 : 0])
 
+// One solver on a chosen XCD.  A kernel of one workgroup runs on whichever XCD its stream's hardware queue starts
+// dealing at; launched as eight workgroups under a CU mask with one CU per XCD, one workgroup lands on every XCD, and
+// the one that finds itself on target_xcd does the work while the others leave at once.  Exactly one workgroup is
+// elected whatever the dealing: the workgroup on the target claims the launch (gate[0]: the number of the last launch
+// claimed, epoch = that number + 1 for this launch), and the last of the eight to arrive (gate[1] counts arrivals,
+// eight per launch) claims it if nobody has.  gate[2] tells the host where the solver ran.  Launches that share a gate
+// must be ordered (one stream); gate starts as zeros, epoch at 1.
+#define TSVM_SOLVER_GRID_ON_XCD 8
+__device__ __forceinline__ bool solver_elected(int *gate, int epoch, int target_xcd) {
+    __shared__ int s_elected;
+    if (threadIdx.x == 0) {
+        const int xcd = (int) __builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11));   // XCC_ID
+        bool won = false;
+        if (xcd == target_xcd) won = atomicCAS(&gate[0], epoch - 1, epoch) == epoch - 1;
+        __threadfence();
+        const int arrived = atomicAdd(&gate[1], 1);
+        if (!won && (arrived % TSVM_SOLVER_GRID_ON_XCD) == TSVM_SOLVER_GRID_ON_XCD - 1) {
+            __threadfence();
+            won = atomicCAS(&gate[0], epoch - 1, epoch) == epoch - 1;
+        }
+        if (won) gate[2] = xcd;
+        s_elected = won;
+    }
+    __syncthreads();
+    return s_elected != 0;
+}
+
 // Elements beyond ws are given y = 0, which puts them in neither I_up nor I_low.
 template <int E>
 __global__ __launch_bounds__(SV_T) void c_smo_solve_kernel(
     const int *__restrict__ label, const double *__restrict__ f_val, double *__restrict__ alpha,
     double *__restrict__ alpha_diff, const int *__restrict__ working_set, int ws, double Cp, double Cn,
     const double *__restrict__ kws, const double *__restrict__ k_diag, double eps, double *__restrict__ diff,
-    int max_iter) {
+    int max_iter, int *__restrict__ gate, int epoch, int target_xcd) {
+    if (gate && !solver_elected(gate, epoch, target_xcd)) return;
     constexpr int LDK = E * SV_T;
     __shared__ double s_kd[LDK];
     __shared__ float s_y[LDK];
@@ -333,7 +361,8 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
     const int *__restrict__ label, const double *__restrict__ f_val, double *__restrict__ alpha,
     double *__restrict__ alpha_diff, const int *__restrict__ working_set, int ws, double C,
     const double *__restrict__ kws, const double *__restrict__ k_diag, double eps, double *__restrict__ diff,
-    int max_iter) {
+    int max_iter, int *__restrict__ gate, int epoch, int target_xcd) {
+    if (gate && !solver_elected(gate, epoch, target_xcd)) return;
     constexpr int LDK = E * SV_T;
     __shared__ double s_kd[LDK];
     __shared__ float s_y[LDK];
@@ -553,7 +582,7 @@ static int launch_gather(const void *k_rows, int row_type, const int *slots, int
             TSVM_HIP(reserve_cu(KERNEL<EVAL>, fa_.sharedSizeBytes, &dyn_));                          \
             dev_done_ = dev_;                                                                       \
         }                                                                                           \
-        hipLaunchKernelGGL(KERNEL<EVAL>, dim3(1), dim3(SV_T), dyn_, s, __VA_ARGS__);                 \
+        hipLaunchKernelGGL(KERNEL<EVAL>, dim3(solver_grid_), dim3(SV_T), solver_grid_ == 1 ? dyn_ : 0, s, __VA_ARGS__); \
     } while (0)
 
 #define TSVM_DISPATCH_E(KERNEL, ...)                                                            \
@@ -571,11 +600,13 @@ int tsvm_c_smo_solve(const int *y, const double *f_val, double *alpha, double *a
                  "tsvm_c_smo_solve: null pointer");
     TSVM_REQUIRE(ws_size >= 1 && ws_size <= MAX_WS, "tsvm_c_smo_solve: ws_size %d outside [1, %d]", ws_size, MAX_WS);
     hipStream_t s = tsvm_s(stream);
+    int *gate_ = nullptr;
+    const int epoch_ = 0, target_xcd_ = 0, solver_grid_ = 1;
     int rc = launch_gather(k_rows, row_type, slots, ld, working_set, ws_size, workspace, s);
     if (rc) return rc;
     const double *kws = (const double *) workspace;
     TSVM_DISPATCH_E(c_smo_solve_kernel, y, f_val, alpha, alpha_diff, working_set, ws_size, Cp, Cn, kws, k_diag, eps, diff,
-                    max_iter);
+                    max_iter, gate_, epoch_, target_xcd_);
     TSVM_LAUNCH_CHECK();
     return 0;
 }
@@ -615,13 +646,15 @@ int tsvm_c_smo_solve_static(const int *y, const double *f_val, double *alpha, do
     int rc = solver_block_address(&block);
     if (rc) return rc;
     hipStream_t s = tsvm_s(stream);
+    int *gate_ = nullptr;
+    const int epoch_ = 0, target_xcd_ = 0, solver_grid_ = 1;
     // the gather writes every element of the ws x ldk block the solver reads (columns beyond ws as zeros), so
     // nothing of the previous call's content is read
     rc = launch_gather(k_rows, row_type, slots, ld, working_set, ws_size, block, s);
     if (rc) return rc;
     const double *kws = block;
     TSVM_DISPATCH_E(c_smo_solve_kernel, y, f_val, alpha, alpha_diff, working_set, ws_size, Cp, Cn, kws, k_diag, eps, diff,
-                    max_iter);
+                    max_iter, gate_, epoch_, target_xcd_);
     TSVM_LAUNCH_CHECK();
     return 0;
 }
@@ -662,28 +695,56 @@ int tsvm_row_slots_assign(const int *ids_new, int n_new, int *slot_of_id, int *s
     return 0;
 }
 
-int tsvm_c_smo_solve_block(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
-                           int ws_size, double Cp, double Cn, const double *kws, const double *k_diag, double eps,
-                           double *diff, int max_iter, tsvm_stream stream) {
+static int c_block(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set, int ws_size,
+                   double Cp, double Cn, const double *kws, const double *k_diag, double eps, double *diff, int max_iter,
+                   int *gate_, int epoch_, int target_xcd_, tsvm_stream stream) {
     TSVM_REQUIRE(y && f_val && alpha && alpha_diff && working_set && kws && k_diag && diff, "tsvm_c_smo_solve_block: null pointer");
     TSVM_REQUIRE(ws_size >= 1 && ws_size <= MAX_WS, "tsvm_c_smo_solve_block: ws_size %d outside [1, %d]", ws_size, MAX_WS);
     hipStream_t s = tsvm_s(stream);
+    const int solver_grid_ = gate_ ? TSVM_SOLVER_GRID_ON_XCD : 1;
     TSVM_DISPATCH_E(c_smo_solve_kernel, y, f_val, alpha, alpha_diff, working_set, ws_size, Cp, Cn, kws, k_diag, eps, diff,
-                    max_iter);
+                    max_iter, gate_, epoch_, target_xcd_);
     TSVM_LAUNCH_CHECK();
     return 0;
+}
+
+static int nu_block(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set, int ws_size,
+                    double C, const double *kws, const double *k_diag, double eps, double *diff, int max_iter, int *gate_,
+                    int epoch_, int target_xcd_, tsvm_stream stream) {
+    TSVM_REQUIRE(y && f_val && alpha && alpha_diff && working_set && kws && k_diag && diff, "tsvm_nu_smo_solve_block: null pointer");
+    TSVM_REQUIRE(ws_size >= 1 && ws_size <= MAX_WS, "tsvm_nu_smo_solve_block: ws_size %d outside [1, %d]", ws_size, MAX_WS);
+    hipStream_t s = tsvm_s(stream);
+    const int solver_grid_ = gate_ ? TSVM_SOLVER_GRID_ON_XCD : 1;
+    TSVM_DISPATCH_E(nu_smo_solve_kernel, y, f_val, alpha, alpha_diff, working_set, ws_size, C, kws, k_diag, eps, diff,
+                    max_iter, gate_, epoch_, target_xcd_);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+int tsvm_c_smo_solve_block(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
+                           int ws_size, double Cp, double Cn, const double *kws, const double *k_diag, double eps,
+                           double *diff, int max_iter, tsvm_stream stream) {
+    return c_block(y, f_val, alpha, alpha_diff, working_set, ws_size, Cp, Cn, kws, k_diag, eps, diff, max_iter, nullptr, 0, 0, stream);
 }
 
 int tsvm_nu_smo_solve_block(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
                             int ws_size, double C, const double *kws, const double *k_diag, double eps, double *diff,
                             int max_iter, tsvm_stream stream) {
-    TSVM_REQUIRE(y && f_val && alpha && alpha_diff && working_set && kws && k_diag && diff, "tsvm_nu_smo_solve_block: null pointer");
-    TSVM_REQUIRE(ws_size >= 1 && ws_size <= MAX_WS, "tsvm_nu_smo_solve_block: ws_size %d outside [1, %d]", ws_size, MAX_WS);
-    hipStream_t s = tsvm_s(stream);
-    TSVM_DISPATCH_E(nu_smo_solve_kernel, y, f_val, alpha, alpha_diff, working_set, ws_size, C, kws, k_diag, eps, diff,
-                    max_iter);
-    TSVM_LAUNCH_CHECK();
-    return 0;
+    return nu_block(y, f_val, alpha, alpha_diff, working_set, ws_size, C, kws, k_diag, eps, diff, max_iter, nullptr, 0, 0, stream);
+}
+
+int tsvm_c_smo_solve_block_on_xcd(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
+                                  int ws_size, double Cp, double Cn, const double *kws, const double *k_diag, double eps,
+                                  double *diff, int max_iter, int *gate, int epoch, int xcd, tsvm_stream stream) {
+    TSVM_REQUIRE(gate && epoch >= 1 && xcd >= 0 && xcd < TSVM_SOLVER_GRID_ON_XCD, "tsvm_c_smo_solve_block_on_xcd: bad gate, epoch or xcd");
+    return c_block(y, f_val, alpha, alpha_diff, working_set, ws_size, Cp, Cn, kws, k_diag, eps, diff, max_iter, gate, epoch, xcd, stream);
+}
+
+int tsvm_nu_smo_solve_block_on_xcd(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
+                                   int ws_size, double C, const double *kws, const double *k_diag, double eps, double *diff,
+                                   int max_iter, int *gate, int epoch, int xcd, tsvm_stream stream) {
+    TSVM_REQUIRE(gate && epoch >= 1 && xcd >= 0 && xcd < TSVM_SOLVER_GRID_ON_XCD, "tsvm_nu_smo_solve_block_on_xcd: bad gate, epoch or xcd");
+    return nu_block(y, f_val, alpha, alpha_diff, working_set, ws_size, C, kws, k_diag, eps, diff, max_iter, gate, epoch, xcd, stream);
 }
 
 int tsvm_nu_smo_solve(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
@@ -694,11 +755,13 @@ int tsvm_nu_smo_solve(const int *y, const double *f_val, double *alpha, double *
                  "tsvm_nu_smo_solve: null pointer");
     TSVM_REQUIRE(ws_size >= 1 && ws_size <= MAX_WS, "tsvm_nu_smo_solve: ws_size %d outside [1, %d]", ws_size, MAX_WS);
     hipStream_t s = tsvm_s(stream);
+    int *gate_ = nullptr;
+    const int epoch_ = 0, target_xcd_ = 0, solver_grid_ = 1;
     int rc = launch_gather(k_rows, row_type, slots, ld, working_set, ws_size, workspace, s);
     if (rc) return rc;
     const double *kws = (const double *) workspace;
     TSVM_DISPATCH_E(nu_smo_solve_kernel, y, f_val, alpha, alpha_diff, working_set, ws_size, C, kws, k_diag, eps, diff,
-                    max_iter);
+                    max_iter, gate_, epoch_, target_xcd_);
     TSVM_LAUNCH_CHECK();
     return 0;
 }

@@ -227,6 +227,9 @@ int tsvm_model_stats(void *model, int k, int64_t *n_iter, int64_t *local_iter, d
             phase_ms[10] = (double) s.ws_size;
             phase_ms[11] = (double) s.rows_computed;
             phase_ms[12] = (double) s.update_rows;
+            phase_ms[13] = (double) s.solver_xcd;
+            phase_ms[14] = s.ms_start;
+            phase_ms[15] = s.ms_end;
         }
     })
 }

@@ -1,4 +1,6 @@
 #include "models.h"
+#include <deque>
+#include <chrono>
 
 #include <algorithm>
 #include <cmath>
@@ -336,10 +338,10 @@ void SVC::train(const DataSet &dataset, SvmParam p) {   // svc.cpp:41-145
     std::vector<std::vector<float_type>> alpha(n_binary_models);
     std::vector<char> is_sv(n, 0);
     int k = 0;
-    // pairs in flight: four when every pair's solver gets CUs of its own and the pairs advance independently (more
-    // gain nothing: the chip-wide kernels of four pairs already keep the chip busy), three when the pairs alternate
-    // between a solver phase and a chip-wide phase
-    const int lanes = std::min(pair_lanes > 0 ? pair_lanes : SolveTask::cu_split_available() ? 4 : 3, n_binary_models);
+    // pairs in flight: up to eight when every pair's solver gets a CU of its own and the pairs advance independently
+    // (at most three of them large pairs, train_pairs_in_lockstep), three when the pairs alternate between a solver
+    // phase and a chip-wide phase
+    const int lanes = std::min(pair_lanes > 0 ? pair_lanes : SolveTask::cu_split_available() ? 8 : 3, n_binary_models);
     if (lanes > 1 && !profile && !trace_first) {
         train_pairs_in_lockstep(grouped, lanes, alpha);
     } else {
@@ -439,29 +441,81 @@ void SVC::finish_binary(BinaryProblem &p, std::vector<float_type> &alpha_out) { 
 }
 
 // The class pairs are independent problems.  Up to `lanes` of them are in flight, each a SolveTask with its own
-// slice of the kernel-row arena; a pair that finishes hands its lane to the next pair, and the result of a pair
-// does not depend on what runs beside it.  When every lane's local solver has compute units of its own, the
-// steps of the pairs are simply enqueued in turn.  Otherwise the pairs advance one outer iteration at a time in
+// slice of the kernel-row arena; a pair that finishes hands its lane to another pair, and the result of a pair
+// depends neither on what runs beside it nor on when it runs.  When every lane's local solver has a compute unit
+// of its own, the lanes advance independently.  Otherwise the pairs advance one outer iteration at a time in
 // three phases separated by events: (1) selection, kernel rows and the solver's block of every pair, (2) the
 // local solvers of all pairs, single workgroups that run side by side on different CUs, (3) update_f of every
 // pair, so that no chip-wide kernel shares CUs with a local solver (next to one, each solver iteration takes
 // two to three times longer).
+//
+// Which pair runs when, and on how much of the arena.  A large pair keeps the chip busy (rows and update_f of
+// hundreds of thousands of columns); a small one is a chain of short kernels that mostly waits for itself, and what
+// it gains from the arena is a slot for every one of its rows.  So the lanes come in two kinds.  "Small" pairs are
+// those whose whole kernel matrix fits an equal share of the budget: they run on lanes whose slice holds exactly the
+// largest of them, next to the large pairs rather than after them, when nothing else would fill the chip.  The
+// large pairs share the rest of the budget on at most three lanes (more only split the row cache further: three
+// already keep the chip-wide kernels queueing).  Both kinds are taken largest first; a large lane that finds no
+// large pair left takes a small one.
 void SVC::train_pairs_in_lockstep(const DataSet &grouped, int lanes, std::vector<std::vector<float_type>> &alpha) {
     struct PairId { int i, j; };
     std::vector<PairId> pairs;
     for (int i = 0; i < n_classes; ++i)
         for (int j = i + 1; j < n_classes; ++j) pairs.push_back({i, j});
-    // every lane's slice of the arena must hold at least the working-set rows of the largest pair
     const size_t esz = param.kernel_type == SvmParam::LINEAR ? sizeof(double) : sizeof(float);
-    size_t need_min = 0;
-    for (const auto &pr : pairs) {
-        const size_t cols = (size_t) grouped.count()[pr.i] + grouped.count()[pr.j];
-        need_min = std::max(need_min, (size_t) 1024 * ((cols + 7) / 8 * 8) * esz);
-    }
     tsvm::RowArena &arena = tsvm::RowArena::instance();
     const size_t budget = cache_bytes > 0 ? (size_t) cache_bytes : cache_bytes < 0 ? arena.auto_budget() : 0;
-    const size_t slice = std::max(budget / lanes, need_min) / 256 * 256;
-    char *const pool = (char *) arena.acquire(slice * lanes, cache_bytes < 0);
+    // per pair: bytes of its working-set rows (the least a slice must hold) and of its whole kernel matrix
+    std::vector<size_t> ws_bytes(pairs.size()), full_bytes(pairs.size());
+    std::vector<int> by_size(pairs.size());
+    for (size_t k = 0; k < pairs.size(); ++k) {
+        const size_t cols = (size_t) grouped.count()[pairs[k].i] + grouped.count()[pairs[k].j];
+        const size_t ld = (cols + 7) / 8 * 8;
+        ws_bytes[k] = (size_t) 1024 * ld * esz;
+        full_bytes[k] = std::max(cols * ld * esz, ws_bytes[k]);
+        by_size[k] = (int) k;
+    }
+    std::stable_sort(by_size.begin(), by_size.end(), [&](int a, int b) { return full_bytes[a] > full_bytes[b]; });
+    const bool two_kinds = SolveTask::cu_split_available() && !getenv("TSVM_PLAIN_LANES");   // (the lockstep schedule keeps equal lanes and the reference's order)
+    std::deque<int> large_q, small_q;
+    size_t need_min = 0, small_slice = 0;
+    for (int k : by_size) {
+        need_min = std::max(need_min, ws_bytes[k]);
+        if (two_kinds && full_bytes[k] <= budget / lanes) {
+            small_q.push_back(k);
+            small_slice = std::max(small_slice, full_bytes[k]);
+        } else {
+            large_q.push_back(k);
+        }
+    }
+    int n_large_lanes, n_small_lanes;
+    if (!two_kinds) {
+        large_q.assign(by_size.size(), 0);
+        for (size_t k = 0; k < pairs.size(); ++k) large_q[k] = (int) k;
+        n_large_lanes = lanes;
+        n_small_lanes = 0;
+    } else if (small_q.empty()) {
+        n_large_lanes = std::min<int>((int) large_q.size(), std::min(lanes, 4));
+        n_small_lanes = 0;
+    } else if (large_q.empty()) {
+        n_large_lanes = 0;
+        n_small_lanes = std::min<int>((int) small_q.size(), lanes);
+    } else {
+        const int max_large = getenv("TSVM_LARGE_LANES") ? atoi(getenv("TSVM_LARGE_LANES")) : 7;
+        n_large_lanes = std::min<int>((int) large_q.size(), std::max(1, std::min(max_large, lanes)));
+        n_small_lanes = std::min<int>((int) small_q.size(), lanes - n_large_lanes);
+    }
+    lanes = n_large_lanes + n_small_lanes;
+    small_slice = (small_slice + 255) / 256 * 256;
+    size_t large_slice = 0;
+    if (n_large_lanes > 0) {
+        const size_t left = budget > small_slice * n_small_lanes ? budget - small_slice * n_small_lanes : 0;
+        large_slice = std::max(left / n_large_lanes / 256 * 256, (need_min + 255) / 256 * 256);   // never above the budget: the arena would be re-allocated
+    }
+    // lanes 0 .. n_large_lanes-1 are the large ones
+    std::vector<size_t> slice_at(lanes + 1, 0);
+    for (int l = 0; l < lanes; ++l) slice_at[l + 1] = slice_at[l] + (l < n_large_lanes ? large_slice : small_slice);
+    char *const pool = (char *) arena.acquire(slice_at[lanes], cache_bytes < 0);
 
     // what the reference still holds of the pairs trained before pair k when it sizes pair k's working set: their
     // alpha arrays (svc.cpp:50-61), whatever runs beside pair k here
@@ -473,35 +527,60 @@ void SVC::train_pairs_in_lockstep(const DataSet &grouped, int lanes, std::vector
     if (keep_binary) binary_f.assign(pairs.size(), std::vector<float_type>());
     std::vector<std::unique_ptr<BinaryProblem>> active;
     std::vector<int> free_lanes;
-    for (int l = lanes - 1; l >= 0; --l) free_lanes.push_back(l);
-    size_t next = 0;
-    auto start_next = [&]() {
+    for (int l = 0; l < lanes; ++l) free_lanes.push_back(l);
+    // the pair a free lane should run next (-1: none)
+    auto next_for = [&](int lane) {
+        std::deque<int> &mine = lane < n_large_lanes ? large_q : small_q;
+        std::deque<int> &q = !mine.empty() ? mine : lane < n_large_lanes ? small_q : mine;
+        if (q.empty()) return -1;
+        const int k = q.front();
+        q.pop_front();
+        return k;
+    };
+    auto dbg_now = []() { return std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now().time_since_epoch()).count(); };
+    auto start_on = [&](int lane, int k) {
+        const double dbg0 = dbg_now();
         std::unique_ptr<BinaryProblem> p(new BinaryProblem());
-        p->k = (int) next;
-        setup_binary(grouped, pairs[next].i, pairs[next].j, *p);
-        ++next;
-        p->lane = free_lanes.back();
-        free_lanes.pop_back();
+        p->k = k;
+        setup_binary(grouped, pairs[k].i, pairs[k].j, *p);
+        const double dbg1 = dbg_now();
+        p->lane = lane;
         const int ws = get_working_set_size(*p->k_mat, alpha_bytes_before[p->k]);
         p->solver->cache_bytes = cache_bytes;
         p->task.reset(new SolveTask(*p->solver, *p->k_mat, p->y, p->alpha, rho[p->k], p->f_val, param.epsilon, p->Cp, p->Cn, ws,
-                                    max_iter, pool + (size_t) p->lane * slice, slice, p->lane, lanes));
+                                    max_iter, pool + slice_at[lane], slice_at[lane + 1] - slice_at[lane], lane, lanes));
         TSVM_HIP_CHECK(hipEventCreateWithFlags(&p->rows_done, hipEventDisableTiming));
         TSVM_HIP_CHECK(hipEventCreateWithFlags(&p->solved, hipEventDisableTiming));
         active.push_back(std::move(p));
+        if (getenv("TSVM_DEBUG_SCHED")) fprintf(stderr, "start pair %d lane %d: setup_binary %.1f ms, task %.1f ms\n", k, lane, dbg1 - dbg0, dbg_now() - dbg1);
+    };
+    // gives every free lane that can still get a pair one; returns how many were started
+    auto start_more = [&]() {
+        int n_started = 0;
+        for (size_t f = 0; f < free_lanes.size();) {
+            const int k = next_for(free_lanes[f]);
+            if (k < 0) { ++f; continue; }
+            const int lane = free_lanes[f];
+            free_lanes.erase(free_lanes.begin() + f);
+            start_on(lane, k);
+            ++n_started;
+        }
+        return n_started;
     };
     auto retire = [&](size_t a) {
         BinaryProblem &p = *active[a];
+        const double dbg0 = dbg_now();
         solver_stats[p.k] = p.task->stats();
         if (keep_binary) binary_f[p.k] = p.f_val;
         p.task.reset();   // synchronises and releases the pair's stream before its lane is reused
+        if (getenv("TSVM_DEBUG_SCHED")) fprintf(stderr, "retire pair %d: %.1f ms\n", p.k, dbg_now() - dbg0);
         (void) hipEventDestroy(p.rows_done);
         (void) hipEventDestroy(p.solved);
         finish_binary(p, alpha[p.k]);
         free_lanes.push_back(p.lane);
         active.erase(active.begin() + a);
     };
-    while (next < pairs.size() && !free_lanes.empty()) start_next();
+    start_more();
     if (!active.empty() && active.front()->task->split_streams()) {
         // Every pair's solver has CUs of its own, so the pairs need no common phases: each lane runs at its own
         // pace.  The host looks at the lanes in turn and serves whichever has something to do: a lane whose
@@ -532,7 +611,7 @@ void SVC::train_pairs_in_lockstep(const DataSet &grouped, int lanes, std::vector
                     if (p.task->finish_iteration()) {
                         retire(a);
                         const size_t before = active.size();
-                        while (next < pairs.size() && !free_lanes.empty()) start_next();
+                        start_more();
                         for (size_t b = before; b < active.size(); ++b) begin_iteration(*active[b]);
                     } else {
                         begin_iteration(p);
@@ -570,7 +649,7 @@ void SVC::train_pairs_in_lockstep(const DataSet &grouped, int lanes, std::vector
             if (!active[a]->task->finish_iteration()) { ++a; continue; }
             retire(a);
         }
-        while (next < pairs.size() && !free_lanes.empty()) start_next();
+        start_more();
     }
 }
 

@@ -17,19 +17,31 @@ inline bool low_set(float_type a, float_type y, float_type Cp, float_type Cn) { 
 inline bool free_sv(float_type a, float_type y, float_type Cp, float_type Cn) { return a > 0 && (y > 0 ? a < Cp : a < Cn); }
 
 // Kernel-row cache bookkeeping (host side).  Rows of the kernel matrix live in slots of one HBM pool;
-// slot_of maps an instance id to its slot, an intrusive doubly linked list keeps the slots in
-// least-recently-used order.  The device only ever sees slot numbers.  The reference keeps no rows
+// slot_of maps an instance id to its slot, an intrusive doubly linked list keeps the slots that may be evicted in
+// eviction order (tail first).  The device only ever sees slot numbers.  The reference keeps no rows
 // beyond the previous working set's second half (csmosolver.cpp:33-42,65-77); cached rows are the
 // rows get_rows would recompute, so the cache cannot change a result.
+//
+// Which row goes.  A row is pinned (out of the list) while it is in the working set, two outer iterations as a rule.
+// When it leaves, a row that was found in the cache when it entered goes to the front of the list; a row that had to
+// be computed goes to the tail, where the next misses take its slot first (all but every 64th such row, which goes
+// to the front, so that the cache's content can drift).  Plain least-recently-used order loses against SMO's access
+// pattern whenever the rows that keep coming back outnumber the slots: the selection works through them in turn,
+// and every row is evicted shortly before it is wanted again (a 426,315-instance class pair with 35,000 slots: 1 %
+// hits; with this order 26 %, and the best any order could do, knowing the future, is 39 %).
 struct RowCache {
     int cap = 0, used = 0, head = -1, tail = -1;
-    std::vector<int> slot_of, id_of, prev, next;
+    long long released_misses = 0;
+    std::vector<int> slot_of, id_of, prev, next, pins;
+    std::vector<char> was_hit;
     void init(int n, int capacity) {
         cap = capacity;
         slot_of.assign(n, -1);
         id_of.assign(cap, -1);
         prev.assign(cap, -1);
         next.assign(cap, -1);
+        pins.assign(cap, 0);
+        was_hit.assign(cap, 0);
     }
     void unlink(int s) {
         if (prev[s] >= 0) next[prev[s]] = next[s]; else head = next[s];
@@ -42,24 +54,40 @@ struct RowCache {
         head = s;
         if (tail < 0) tail = s;
     }
-    int lookup(int id) {                 // slot of a cached row (marked most recently used) or -1
+    void push_back(int s) {
+        next[s] = -1;
+        prev[s] = tail;
+        if (tail >= 0) next[tail] = s;
+        tail = s;
+        if (head < 0) head = s;
+    }
+    int lookup(int id) {                 // slot of a cached row, pinned from now on, or -1
         const int s = slot_of[id];
-        if (s >= 0) { unlink(s); push_front(s); }
+        if (s >= 0) {
+            if (pins[s]++ == 0) { unlink(s); was_hit[s] = 1; }
+        }
         return s;
     }
-    int insert(int id) {                 // slot for a new row: a free one, else the least recently used
+    int insert(int id) {                 // slot for a new row, pinned: a free one, else the list's tail (-1: every slot is pinned)
         int s;
         if (used < cap) {
             s = used++;
         } else {
             s = tail;
+            if (s < 0) return -1;
             unlink(s);
             slot_of[id_of[s]] = -1;
         }
         id_of[s] = id;
         slot_of[id] = s;
-        push_front(s);
+        pins[s] = 1;
+        was_hit[s] = 0;
         return s;
+    }
+    void release(int s) {                // the row has left the working set
+        if (--pins[s] > 0) return;
+        if (was_hit[s] || (++released_misses & 63) == 0) push_front(s);
+        else push_back(s);
     }
 };
 
@@ -85,23 +113,62 @@ struct PhaseTimer {
 // CU-masked streams are kept for the life of the process and handed from one solve to the next: creating one
 // makes a hardware queue, which costs far more than a solve's other set-up (and every few creations the runtime
 // spends tens of milliseconds on queue housekeeping).  Keyed by device, lane and lane count (which fix the masks).
-struct MaskedStreams {
+struct LaneStreams {
     hipStream_t chip = nullptr, solver = nullptr;
     bool in_use = false;
 };
+// the streams of all lanes of one lane count on one device: made together, because the chip-wide mask leaves out
+// exactly the CUs on which the lanes' solvers land
+struct LaneGroup {
+    std::vector<LaneStreams> lanes;
+};
 std::mutex g_masked_mutex;
-std::map<long long, std::vector<MaskedStreams>> g_masked;
+std::map<long long, std::vector<LaneGroup>> g_masked;   // keyed by device and lane count
+
+// the clock reading of the process's first solve: solves report their start and end relative to it
+std::chrono::steady_clock::time_point process_epoch() {
+    static const std::chrono::steady_clock::time_point t0 = std::chrono::steady_clock::now();
+    return t0;
+}
 
 // The pooled streams are destroyed by an atexit handler, registered when the first one is made and therefore run
 // before the HIP runtime's own tear-down (which, under a profiler, crashed on queues still alive at that point).
 void destroy_masked_streams() {
     std::lock_guard<std::mutex> lock(g_masked_mutex);
     for (auto &kv : g_masked)
-        for (MaskedStreams &m : kv.second) {
+        for (LaneGroup &g : kv.second)
+            for (LaneStreams &m : g.lanes) {
+                if (m.solver) (void) hipStreamDestroy(m.solver);
+                if (m.chip) (void) hipStreamDestroy(m.chip);
+            }
+    g_masked.clear();
+}
+
+// Makes the 2 * n_lanes streams of a group.  Bit i of a CU mask names CU i/8 of XCD i%8 on the 8-XCD, 256-CU part (a
+// mask has to leave every XCD at least one CU: workgroups are dealt to the XCDs in turn).  Every solver stream gets
+// CU 0 of every XCD, every chip-wide stream the other 248 CUs.  With several lanes, lane l's solver is launched so
+// that it runs on XCD l (tsvm_c_smo_solve_block_on_xcd): the lanes share the eight CUs without sharing a CU, each
+// solver behind another L2, and eight lanes cost the chip-wide kernels no more CUs than one.
+bool make_lane_group(int n_lanes, LaneGroup &g) {
+    g.lanes.assign(n_lanes, LaneStreams());
+    uint32_t small[8] = {0xffu, 0, 0, 0, 0, 0, 0, 0};
+    uint32_t big[8] = {~0xffu, ~0u, ~0u, ~0u, ~0u, ~0u, ~0u, ~0u};
+    bool ok = true;
+    for (int l = 0; l < n_lanes && ok; ++l) {
+        ok = hipExtStreamCreateWithCUMask(&g.lanes[l].solver, 8, small) == hipSuccess;
+        if (!ok) { g.lanes[l].solver = nullptr; break; }
+        ok = hipExtStreamCreateWithCUMask(&g.lanes[l].chip, 8, big) == hipSuccess;
+        if (!ok) g.lanes[l].chip = nullptr;
+    }
+    if (!ok) {
+        (void) hipGetLastError();
+        for (LaneStreams &m : g.lanes) {
             if (m.solver) (void) hipStreamDestroy(m.solver);
             if (m.chip) (void) hipStreamDestroy(m.chip);
         }
-    g_masked.clear();
+        g.lanes.clear();
+    }
+    return ok;
 }
 
 }  // namespace
@@ -197,6 +264,9 @@ struct SolveTask::Impl {
     int last_rows_computed = 0;
     bool block_on_solver_cus = false;
     long long masked_key = 0;
+    int masked_lane = 0;
+    int solver_xcd = -1, solver_epoch = 0;   // several lanes: the XCD this lane's solver is launched onto, launches so far
+    tsvm::DeviceBuffer<int> d_gate;
 
     void *k_rows = nullptr;
     bool caching = false;
@@ -264,7 +334,9 @@ struct SolveTask::Impl {
         return false;
     }
     int rotation_base = 0;   // iteration at which d_slots_a was valid
-    long long window_lookups = 0, window_hits = 0;
+    long long window_lookups = 0, window_hits = 0, window_first = 0, first_touches = 0;
+    std::vector<char> seen;        // instances whose row has been asked for at least once
+    int off_below_percent = 5;     // a full cache is switched off when fewer of a window's repeated lookups hit (TSVM_CACHE_OFF_BELOW)
     const int *slots = nullptr;
 
     int max_iter = 0;
@@ -283,6 +355,7 @@ struct SolveTask::Impl {
           row_type(k_mat.row_type()), row_esz(k_mat.row_elem_size()), q(ws_size / 2), ld(((int64_t) n_u + 7) / 8 * 8),
           nu(solver.is_nu()), ldk(tsvm_smo_solve_block_ld(ws_size)), timer(solver.profile) {
         wall0 = std::chrono::steady_clock::now();
+        (void) process_epoch();
         stats.ws_size = ws_size;
         d_y.resize(n); d_ws.resize((size_t) WS_HALVES * q + ws_size); d_slots_a.resize(3 * (size_t) ws_size); d_slots_b.resize(ws_size);
         if (rep > 1) d_ws_folded.resize(d_ws.size());
@@ -296,6 +369,11 @@ struct SolveTask::Impl {
         d_kws.zero();
         alone = n_lanes == 1;
         split = !solver.profile && create_split_streams(lane, n_lanes);
+        if (split && n_lanes > 1) {
+            solver_xcd = lane;
+            d_gate.resize(4);
+            d_gate.zero();
+        }
         if (!split) {
             TSVM_HIP_CHECK(hipStreamCreateWithFlags(&sa, hipStreamNonBlocking));
             ss = sa;
@@ -330,6 +408,8 @@ struct SolveTask::Impl {
         }
         if (caching) {
             cache.init(n_u, (int) pool_rows);
+            seen.assign(n_u, 0);
+            if (const char *e = getenv("TSVM_CACHE_OFF_BELOW")) off_below_percent = atoi(e);
             stats.cache_rows = pool_rows;
             if ((size_t) n_u <= pool_rows) d_slot_of.resize(n_u);
             device_cache = d_slot_of.size() == (size_t) n_u && rep == 1 && k_mat.dense_layout();
@@ -395,55 +475,40 @@ struct SolveTask::Impl {
         if (h_slots) (void) hipHostFree(h_slots);
     }
 
-    // Two streams with disjoint CU masks.  Bit i of a mask names CU i/8 of XCD i%8 on the 8-XCD, 256-CU part
-    // (a mask has to leave every XCD at least one CU: workgroups are dealt to the XCDs in turn).  Anything
-    // unexpected (another CU count, the call failing, TSVM_NO_CU_SPLIT set) leaves the task on one plain stream.
-    // Lane l's solver gets CU l of every XCD; the chip-wide kernels of all lanes get the CUs no lane's solver has.
+    // Two streams with disjoint CU masks from the pool (make_lane_group above).  Anything unexpected (another CU
+    // count, a call failing, TSVM_NO_CU_SPLIT set) leaves the task on one plain stream.
     bool create_split_streams(int lane, int n_lanes) {
         if (!SolveTask::cu_split_available() || n_lanes < 1 || n_lanes > 8 || lane < 0 || lane >= n_lanes) return false;
         int dev = 0;
         if (hipGetDevice(&dev) != hipSuccess) return false;
-        masked_key = ((long long) dev * 16 + n_lanes) * 16 + lane;
-        {
-            std::lock_guard<std::mutex> lock(g_masked_mutex);
-            for (MaskedStreams &m : g_masked[masked_key])
-                if (!m.in_use) {
-                    m.in_use = true;
-                    sa = m.chip;
-                    ss = m.solver;
-                    return true;
-                }
-        }
-        // lane l's solver: CU l of every XCD = mask bits 8l .. 8l+7; the chip-wide stream: every CU from n_lanes on
-        uint32_t small[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-        uint32_t big[8] = {~0u, ~0u, ~0u, ~0u, ~0u, ~0u, ~0u, ~0u};
-        small[lane / 4] = 0xffu << (8 * (lane % 4));
-        for (int l = 0; l < n_lanes; ++l) big[l / 4] &= ~(0xffu << (8 * (l % 4)));
-        if (hipExtStreamCreateWithCUMask(&ss, 8, small) != hipSuccess) { (void) hipGetLastError(); ss = nullptr; return false; }
-        if (hipExtStreamCreateWithCUMask(&sa, 8, big) != hipSuccess) {
-            (void) hipGetLastError();
-            (void) hipStreamDestroy(ss);
-            ss = sa = nullptr;
-            return false;
-        }
+        masked_key = (long long) dev * 16 + n_lanes;
+        masked_lane = lane;
         std::lock_guard<std::mutex> lock(g_masked_mutex);
-        static bool registered = false;
-        if (!registered) {
-            registered = true;
-            atexit(destroy_masked_streams);
+        std::vector<LaneGroup> &groups = g_masked[masked_key];
+        LaneStreams *mine = nullptr;
+        for (LaneGroup &g : groups)
+            if (!g.lanes[lane].in_use) { mine = &g.lanes[lane]; break; }
+        if (!mine) {
+            LaneGroup g;
+            if (!make_lane_group(n_lanes, g)) return false;
+            static bool registered = false;
+            if (!registered) {
+                registered = true;
+                atexit(destroy_masked_streams);
+            }
+            groups.push_back(std::move(g));
+            mine = &groups.back().lanes[lane];
         }
-        MaskedStreams m;
-        m.chip = sa;
-        m.solver = ss;
-        m.in_use = true;
-        g_masked[masked_key].push_back(m);
+        mine->in_use = true;
+        sa = mine->chip;
+        ss = mine->solver;
         return true;
     }
 
     void release_split_streams() {
         std::lock_guard<std::mutex> lock(g_masked_mutex);
-        for (MaskedStreams &m : g_masked[masked_key])
-            if (m.chip == sa) m.in_use = false;
+        for (LaneGroup &g : g_masked[masked_key])
+            if (g.lanes[masked_lane].chip == sa) g.lanes[masked_lane].in_use = false;
     }
 
     // without a cache the slot tables just alternate: the two halves of the working set swap places
@@ -525,9 +590,11 @@ struct SolveTask::Impl {
             // look the new ids up and compute only the rows that are not cached
             TSVM_HIP_CHECK(hipEventSynchronize(ids_ready));
             if (iter > 0) {
-                for (int t = 0; t < q; ++t) {   // rows kept from the previous working set stay most recently used
+                // the first half of the previous working set leaves; the second half moves up and stays pinned
+                for (int t = 0; t < q; ++t) cache.release(cur_slots[t]);
+                for (int t = 0; t < q; ++t) {
                     cur_ids[t] = cur_ids[t + q];
-                    cur_slots[t] = cache.lookup(cur_ids[t]);
+                    cur_slots[t] = cur_slots[t + q];
                 }
             }
             miss_ids.clear();
@@ -536,10 +603,12 @@ struct SolveTask::Impl {
                 const int id = h_ids[t] % n_u;   // a second member with the same folded id hits the slot just assigned
                 int s = cache.lookup(id);
                 stats.cache_lookups++;
+                if (!seen[id]) { seen[id] = 1; ++first_touches; }
                 if (s >= 0) {
                     stats.cache_hits++;
                 } else {
                     s = cache.insert(id);
+                    if (s < 0) throw std::runtime_error("SolveTask: kernel-row cache smaller than a working set");
                     miss_ids.push_back(id);
                     miss_slots.push_back(s);
                 }
@@ -568,8 +637,11 @@ struct SolveTask::Impl {
             // every 64 iterations, if fewer than 5 % of the window's lookups hit, fall back to rotation.
             // (A cache that can hold every row is never switched off: its misses are first touches.)
             if (cache.cap < n_u && cache.used == cache.cap && iter % 64 == 63) {
+                // (lookups of rows never asked for before cannot hit and say nothing about the cache: only the
+                // others count, once they are at least a quarter of the window's lookups)
                 const long long dl = stats.cache_lookups - window_lookups, dh = stats.cache_hits - window_hits;
-                if (dh * 20 < dl) {
+                const long long again = dl - (first_touches - window_first);
+                if (again * 4 >= dl && dh * 100 < again * off_below_percent) {
                     TSVM_HIP_CHECK(hipStreamSynchronize(sa));
                     caching = false;
                     stats.cache_disabled = true;
@@ -588,7 +660,7 @@ struct SolveTask::Impl {
                     rotation_base = iter;
                 }
             }
-            if (iter % 64 == 63) { window_lookups = stats.cache_lookups; window_hits = stats.cache_hits; }
+            if (iter % 64 == 63) { window_lookups = stats.cache_lookups; window_hits = stats.cache_hits; window_first = first_touches; }
         } else {
             const bool on_a = ((iter - rotation_base) % 2) == 0;
             slots = on_a ? d_slots_a.data() : d_slots_b.data();
@@ -640,7 +712,17 @@ struct SolveTask::Impl {
         solver_enqueued = std::chrono::steady_clock::now();
         next_stream_check = solver_enqueued + std::chrono::milliseconds(200);
         if (!on_one_stream && !block_on_solver_cus) TSVM_HIP_CHECK(hipStreamWaitEvent(ss, block_done, 0));
-        if (nu) {
+        if (solver_xcd >= 0 && st == ss) {   // several lanes share the solver CUs: this lane's solver runs on its own XCD
+            ++solver_epoch;
+            if (nu)
+                abi_check(tsvm_nu_smo_solve_block_on_xcd(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), ws_ids(), ws_size, Cp,
+                                                         d_kws.data(), k_mat.diag(), eps, d_diff, max_iter, d_gate.data(), solver_epoch,
+                                                         solver_xcd, st));
+            else
+                abi_check(tsvm_c_smo_solve_block_on_xcd(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), ws_ids(), ws_size, Cp,
+                                                        Cn, d_kws.data(), k_mat.diag(), eps, d_diff, max_iter, d_gate.data(), solver_epoch,
+                                                        solver_xcd, st));
+        } else if (nu) {
             abi_check(tsvm_nu_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), ws_ids(), ws_size,
                                               Cp, d_kws.data(), k_mat.diag(), eps, d_diff, max_iter, st));
         } else {
@@ -714,7 +796,10 @@ struct SolveTask::Impl {
             stats.obj = solver.calculate_obj(f_val, alpha, y);
             TSVM_LOG << "global iter = " << iter << ", total local iter = " << local_iter << ", diff = " << diff0
                      << ", obj = " << stats.obj << ", cache hits " << stats.cache_hits << "/" << stats.cache_lookups;
+            if (solver_xcd >= 0 && solver_epoch > 0) stats.solver_xcd = d_gate.to_host()[2];   // where the last solver launch ran
             stats.ms_wall = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - wall0).count();
+            stats.ms_start = std::chrono::duration<double, std::milli>(wall0 - process_epoch()).count();
+            stats.ms_end = stats.ms_start + stats.ms_wall;
             return true;
         }
         ++iter;

@@ -25,6 +25,8 @@ struct SolverStats {
     int ws_size = 0;              // working-set size of the solve
     long long rows_computed = 0;  // kernel rows get_rows produced (cache misses), summed over the outer iterations
     long long update_rows = 0;    // kernel rows update_f read (non-zero alpha_diff entries), counted only when profiling
+    int solver_xcd = -1;          // several class pairs in flight: the die this pair's local solver ran on (-1: not known)
+    double ms_start = 0, ms_end = 0;   // host clock at the solve's start and end, in ms since the process's first solve
 };
 
 class SolveTask;

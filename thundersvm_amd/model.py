@@ -190,12 +190,13 @@ class Model:
 
     def stats(self, k=0):
         ni, li, obj = C.c_int64(), C.c_int64(), C.c_double()
-        ms = np.zeros(13)
+        ms = np.zeros(16)
         _check(host_lib().tsvm_model_stats(self.h, k, C.byref(ni), C.byref(li), C.byref(obj), _p(ms, _dp)))
         return dict(n_iter=ni.value, local_iter=li.value, obj=obj.value, ms_select=ms[0], ms_get_rows=ms[1],
                     ms_local=ms[2], ms_update_f=ms[3], cache_lookups=int(ms[4]), cache_hits=int(ms[5]), cache_rows=int(ms[6]),
                     cache_disabled=bool(ms[7]), ms_wall=ms[8], ms_setup=ms[9], ws_size=int(ms[10]),
-                    rows_computed=int(ms[11]), update_rows=int(ms[12]))
+                    rows_computed=int(ms[11]), update_rows=int(ms[12]), solver_xcd=int(ms[13]),
+                    ms_start=ms[14], ms_end=ms[15])
 
     def binary(self, k):
         n = host_lib().tsvm_model_binary_size(self.h, k)
