@@ -203,8 +203,12 @@ __device__ __forceinline__ void get_rows_tile(
 #pragma unroll
                 for (int tj = 0; tj < 4; ++tj) {
                     const TO val = tsvm_epilogue_as<TO>(acc[ti][tj][v], sdi[ti * 4 + v], sdj[tj], kp, exp_tab);
-                    orow[tj * 16] = val;
-                    if (SYM) out[(int64_t) (jb + tj * 16) * ldo + (i0 + wi * (16 * TI) + ti * 16 + 4 * v + lk)] = val;
+                    if (SYM) {   // the solver's block: read again at once
+                        orow[tj * 16] = val;
+                        out[(int64_t) (jb + tj * 16) * ldo + (i0 + wi * (16 * TI) + ti * 16 + 4 * v + lk)] = val;
+                    } else {
+                        store_streaming(orow + tj * 16, val);
+                    }
                 }
             }
         }
@@ -220,8 +224,12 @@ __device__ __forceinline__ void get_rows_tile(
                 for (int tj = 0; tj < 4; ++tj)
                     if (jb + tj * 16 < n) {
                         const TO val = tsvm_epilogue_as<TO>(acc[ti][tj][v], sdi[ti * 4 + v], sdj[tj], kp, exp_tab);
-                        orow[tj * 16] = val;
-                        if (SYM) out[(int64_t) (jb + tj * 16) * ldo + i] = val;
+                        if (SYM) {
+                            orow[tj * 16] = val;
+                            out[(int64_t) (jb + tj * 16) * ldo + i] = val;
+                        } else {
+                            store_streaming(orow + tj * 16, val);
+                        }
                     }
             }
         }
@@ -463,7 +471,7 @@ __global__ __launch_bounds__(256, 3) void get_rows_dense_stream_kernel(
                     vec4_t res;
 #pragma unroll
                     for (int tj = 0; tj < 4; ++tj) res[tj] = finish(acc[ti][tj][v], sdi, mi, tj);
-                    *(vec4_t *) orow = res;
+                    store_streaming((vec4_t *) orow, res);
                 }
             }
         } else {
@@ -478,7 +486,7 @@ __global__ __launch_bounds__(256, 3) void get_rows_dense_stream_kernel(
                     TO *orow = out + (int64_t) ((uint64_t) (uint32_t) s_slot[r] * (uint32_t) ldo) + jb;
 #pragma unroll
                     for (int tj = 0; tj < 4; ++tj)
-                        if (jb + tj < n) orow[tj] = finish(acc[ti][tj][v], sdi, mi, tj);
+                        if (jb + tj < n) store_streaming(orow + tj, finish(acc[ti][tj][v], sdi, mi, tj));
                 }
             }
         }
@@ -584,6 +592,8 @@ __global__ __launch_bounds__(256) void get_rows_csr_kernel(
 #pragma unroll
     for (int jj = 0; jj < CS_JB; ++jj) {
         const int64_t j = j0 + jj;
+        // (a plain store: every lane of a wavefront writes into another row, one value at a time, and the L2 has to
+        // gather those into lines: marked non-temporal the launch took 2.3 ms instead of 0.6)
         if (j < n) orow[j] = tsvm_epilogue_as<TO>(acc[jj], sdi, sd_x ? sd_x[x_idx ? (int64_t) x_idx[j] : j] : 0.0, kp, exp_tab);
     }
 }
@@ -772,7 +782,7 @@ __global__ __launch_bounds__(SK_T) void sum_kernel_values_kernel(
 #pragma unroll
                     for (int rr = 0; rr < SK_R; ++rr) {
                         const int64_t r = r0 + rr < n_instances ? r0 + rr : n_instances - 1;   // a valid row; not added below
-                        kv[u][rr] = k_mat[r * ldk + st + l + u * SK_T];
+                        kv[u][rr] = load_streaming(k_mat + r * ldk + st + l + u * SK_T);
                     }
                 }
 #pragma unroll

@@ -83,7 +83,7 @@ __global__ __launch_bounds__(UF_T) void update_f_kernel(double *__restrict__ f, 
             for (; u + UNROLL <= total; u += UNROLL) {
                 vec_t k[UNROLL];
 #pragma unroll
-                for (int e = 0; e < UNROLL; ++e) k[e] = *(const vec_t *) (k_rows + s_off[u + e] + j);
+                for (int e = 0; e < UNROLL; ++e) k[e] = load_streaming((const vec_t *) (k_rows + s_off[u + e] + j));
 #pragma unroll
                 for (int e = 0; e < UNROLL; ++e) {
                     const double ad = s_ad[u + e];
@@ -92,7 +92,7 @@ __global__ __launch_bounds__(UF_T) void update_f_kernel(double *__restrict__ f, 
                 }
             }
             for (; u < total; ++u) {
-                const vec_t k = *(const vec_t *) (k_rows + s_off[u] + j);
+                const vec_t k = load_streaming((const vec_t *) (k_rows + s_off[u] + j));
                 const double ad = s_ad[u];
 #pragma unroll
                 for (int c = 0; c < COLS; ++c) sum[c] = __builtin_fma(ad, (double) k[c], sum[c]);
