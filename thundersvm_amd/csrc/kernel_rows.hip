@@ -537,7 +537,7 @@ __global__ __launch_bounds__(256, 3) void get_rows_dense_sym_kernel(
 // ------------------------------------------------------------------------------------------------
 // CSR get_rows: out[i][j] = epilogue( sum over row j's non-zeros, in stored order, of v * w[col][i] )
 // One workgroup = 256 working rows i (one per thread) x 16 consecutive rows j; the 16 dot products
-// live in registers and each thread stores its 16 results as one 128-byte run of output row i.
+// live in registers and each thread stores its 16 results as one 64- or 128-byte run of output row i.
 // ------------------------------------------------------------------------------------------------
 // (JB = 16 stored rows per workgroup; 4 when there are only a few thousand of them, as for the solver's ws x ws
 // block, so that the grid still covers the chip and a workgroup's chain of dependent loads is a quarter as long)
@@ -549,7 +549,7 @@ __global__ __launch_bounds__(256) void get_rows_csr_kernel(
     const double *__restrict__ val, const int *__restrict__ col, const int64_t *__restrict__ row_ptr,
     const int *__restrict__ x_idx, int64_t n, const double *__restrict__ sd_x, const TW *__restrict__ w, int m,
     const double *__restrict__ sd_w, KernelParam kp, TO *__restrict__ out, const int *__restrict__ out_slots,
-    int64_t ldo, unsigned i_blocks) {
+    int64_t ldo, unsigned i_blocks, int vec_ok) {
     __shared__ uint64_t exp_tab[32];
     const int tid = threadIdx.x;
     if (tid < 32) exp_tab[tid] = TSVM_EXP2F_TAB[tid];
@@ -589,12 +589,30 @@ __global__ __launch_bounds__(256) void get_rows_csr_kernel(
     if (!active) return;
     const double sdi = sd_w ? sd_w[i] : 0.0;
     TO *orow = out + (int64_t) (out_slots ? out_slots[i] : i) * ldo;
+    TO res[CS_JB];
 #pragma unroll
     for (int jj = 0; jj < CS_JB; ++jj) {
-        const int64_t j = j0 + jj;
-        // (a plain store: every lane of a wavefront writes into another row, one value at a time, and the L2 has to
-        // gather those into lines: marked non-temporal the launch took 2.3 ms instead of 0.6)
-        if (j < n) orow[j] = tsvm_epilogue_as<TO>(acc[jj], sdi, sd_x ? sd_x[x_idx ? (int64_t) x_idx[j] : j] : 0.0, kp, exp_tab);
+        const int64_t j = j0 + jj < n ? j0 + jj : n - 1;
+        res[jj] = tsvm_epilogue_as<TO>(acc[jj], sdi, sd_x ? sd_x[x_idx ? (int64_t) x_idx[j] : j] : 0.0, kp, exp_tab);
+    }
+    // The thread's CS_JB results are consecutive elements of output row i: they leave as 16-byte pieces when the
+    // row allows it (every lane of a wavefront writes into another row, so a store instruction touches 64 lines
+    // either way; one value at a time the L2 had four times as many partial writes to gather).  Plain stores:
+    // marked non-temporal, partial lines go to memory as they are, and the launch took 2.3 ms instead of 0.6.
+    constexpr int PER = 16 / (int) sizeof(TO);
+    typedef TO piece_t __attribute__((ext_vector_type(PER)));
+    if (vec_ok && j0 + CS_JB <= n) {
+#pragma unroll
+        for (int jj = 0; jj < CS_JB; jj += PER) {
+            piece_t pc;
+#pragma unroll
+            for (int u = 0; u < PER; ++u) pc[u] = res[jj + u];
+            *(piece_t *) (orow + j0 + jj) = pc;
+        }
+    } else {
+#pragma unroll
+        for (int jj = 0; jj < CS_JB; ++jj)
+            if (j0 + jj < n) orow[j0 + jj] = res[jj];
     }
 }
 
@@ -1067,13 +1085,15 @@ static int get_rows_csr(const double *val, const int *col, const int64_t *row_pt
     if (n == 0 || m == 0) return 0;
     KernelParam kp{kernel_type, degree, gamma, coef0};
     const unsigned i_blocks = (unsigned) ((m + 255) / 256);
-    const int jb = n <= 4096 ? 4 : 16;
+    const int jb = n <= 4096 ? 4 : 16;   // (32, whole 128-byte lines of float rows: 0.78 ms against 0.55 at 72,000 x 20,958)
     const int64_t j_blocks = (n + jb - 1) / jb;
     TSVM_REQUIRE(j_blocks * i_blocks < (int64_t) 0x7fffffff, "tsvm_get_rows_csr: grid too large");
     const dim3 grid((unsigned) (j_blocks * i_blocks));
+    // 16-byte pieces of an output row: every row start and every group of jb columns 16-byte aligned
+    const int vec_ok = (uintptr_t) out % 16 == 0 && (ldo * (row_type == TSVM_ROW_F32 ? 4 : 8)) % 16 == 0;
 #define CSR_LAUNCH_W(TO, JB, TW)                                                                                             \
     hipLaunchKernelGGL((get_rows_csr_kernel<TO, JB, TW>), grid, dim3(256), 0, tsvm_s(stream), val, col, row_ptr, x_idx, n, sd_x, \
-                       (const TW *) w, m, sd_w, kp, (TO *) out, out_slots, ldo, i_blocks)
+                       (const TW *) w, m, sd_w, kp, (TO *) out, out_slots, ldo, i_blocks, vec_ok)
 #define CSR_LAUNCH(TO, JB)                                                   \
     do {                                                                     \
         if (w_type == TSVM_ROW_F32) CSR_LAUNCH_W(TO, JB, float);             \
