@@ -37,7 +37,7 @@ size_t &device_bytes_in_use();   // running total of DeviceBuffer allocations (t
 class RowArena {
 public:
     static RowArena &instance();
-    // bytes a solve may use when the caller gave no explicit budget: half of what is free or already held
+    // bytes a solve may use when the caller gave no explicit budget: three quarters of what is free or already held
     size_t auto_budget();
     void *acquire(size_t bytes, bool auto_sized);
     void release();
