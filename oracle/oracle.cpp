@@ -23,6 +23,8 @@
 //     algorithm glibc >= 2.27 publishes for expf (32-entry 2^(i/32) table,
 //     cubic polynomial, all in double), which the HIP epilogue restates too.
 //     tests/test_oracle_expf.py counts how often the two differ on this host.
+//   * powf() / tanhf() of the polynomial and sigmoid kernels (kernelmatrix_kernel.cpp:94-108): the same two
+//     modes, with orc_powf_det / orc_tanhf_det.
 //
 // Pinning: tests/test_oracle_golden.py (the reference's fixture, row sets and accuracy / MSE / SV-count goldens),
 // tests/test_oracle_expf.py, tests/test_oracle_smo.py, tests/test_oracle_probability.py and tests/test_oracle_pins.py
@@ -32,8 +34,8 @@
 // c_smo_solve / nu_smo_solve + update_f + rho) is pinned at the optimum: run to a gap of 1e-8 on a strictly convex
 // problem it reproduces LibSVM's unique solution for all five SVM types.  What stays "parity unpinned" is only the
 // trajectory at the default gap of 1e-3 against a run of the reference itself (no fixture of the reference holds alpha
-// or rho, and its CPU build cannot be made here: Eigen is absent), and the poly / sigmoid epilogues, which use double
-// pow / tanh rounded once where the reference calls powf / tanhf (one float ulp apart on about 0.1 % of the values).
+// or rho, and its CPU build cannot be made here: Eigen is absent).  The poly / sigmoid epilogues use restatements of
+// libm's powf / tanhf that give libm's bits on every float argument (tests/test_oracle_expf.py samples the sweeps).
 #include <algorithm>
 #include <cmath>
 #include <cstdint>
@@ -60,7 +62,7 @@ struct orc_param {
     int svm_type;
     int kernel_type;
     int degree;
-    int expf_mode;       // 0 = libm expf/powf/tanhf, 1 = orc_expf_det and double pow/tanh rounded to float
+    int expf_mode;       // 0 = libm expf/powf/tanhf, 1 = the restatements orc_expf_det / orc_powf_det / orc_tanhf_det
     double gamma;
     double coef0;
     double C;
@@ -146,6 +148,224 @@ long long orc_expf_count_mismatch(uint32_t lo_bits, uint32_t hi_bits, uint32_t s
 }
 
 // ---------------------------------------------------------------------------
+// powf and tanhf, restated (expf_mode 1) as the HIP epilogues restate them: the published routines of the libm these
+// hosts run (powf: 16-entry log2 table, quartic, y*log2(x) in double, then the expf table and cubic, FMA form;
+// tanhf / expm1f: the fdlibm float versions).  orc_powf_count_mismatch / orc_tanhf_count_mismatch compare them with
+// libm; run over all 2^32 arguments (for powf: for each of fourteen exponents) they found no difference.
+// ---------------------------------------------------------------------------
+static const double ORC_POWF_LOG2_TAB[16][2] = {
+    {0x1.661ec79f8f3bep+0, -0x1.efec65b963019p-2 * 32}, {0x1.571ed4aaf883dp+0, -0x1.b0b6832d4fca4p-2 * 32},
+    {0x1.49539f0f010bp+0, -0x1.7418b0a1fb77bp-2 * 32},  {0x1.3c995b0b80385p+0, -0x1.39de91a6dcf7bp-2 * 32},
+    {0x1.30d190c8864a5p+0, -0x1.01d9bf3f2b631p-2 * 32}, {0x1.25e227b0b8eap+0, -0x1.97c1d1b3b7afp-3 * 32},
+    {0x1.1bb4a4a1a343fp+0, -0x1.2f9e393af3c9fp-3 * 32}, {0x1.12358f08ae5bap+0, -0x1.960cbbf788d5cp-4 * 32},
+    {0x1.0953f419900a7p+0, -0x1.a6f9db6475fcep-5 * 32}, {0x1p+0, 0x0p+0 * 32},
+    {0x1.e608cfd9a47acp-1, 0x1.338ca9f24f53dp-4 * 32},  {0x1.ca4b31f026aap-1, 0x1.476a9543891bap-3 * 32},
+    {0x1.b2036576afce6p-1, 0x1.e840b4ac4e4d2p-3 * 32},  {0x1.9c2d163a1aa2dp-1, 0x1.40645f0c6651cp-2 * 32},
+    {0x1.886e6037841edp-1, 0x1.88e9c2c1b9ff8p-2 * 32},  {0x1.767dcf5534862p-1, 0x1.ce0a44eb17bccp-2 * 32}};
+static inline uint32_t f32_bits(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float bits_f32(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+static inline int powf_checkint(uint32_t iy) {   // 0: not an integer, 1: odd, 2: even
+    int e = iy >> 23 & 0xff;
+    if (e < 0x7f) return 0;
+    if (e > 0x7f + 23) return 2;
+    if (iy & ((1u << (0x7f + 23 - e)) - 1)) return 0;
+    if (iy & (1u << (0x7f + 23 - e))) return 1;
+    return 2;
+}
+static inline bool powf_zeroinfnan(uint32_t ix) { return 2 * ix - 1 >= 2u * 0x7f800000 - 1; }
+
+float orc_powf_det(float x, float y) {
+    const double A0 = 0x1.27616c9496e0bp-2 * 32, A1 = -0x1.71969a075c67ap-2 * 32, A2 = 0x1.ec70a6ca7baddp-2 * 32,
+                 A3 = -0x1.7154748bef6c8p-1 * 32, A4 = 0x1.71547652ab82bp0 * 32;
+    uint32_t sign_bias = 0;
+    uint32_t ix = f32_bits(x), iy = f32_bits(y);
+    if (ix - 0x00800000 >= 0x7f800000 - 0x00800000 || powf_zeroinfnan(iy)) {
+        if (powf_zeroinfnan(iy)) {
+            if (2 * iy == 0) return 2 * (ix ^ 0x00400000) > 2u * 0x7fc00000 ? x + y : 1.0f;   // (a signalling NaN stays a NaN)
+            if (ix == 0x3f800000) return 2 * (iy ^ 0x00400000) > 2u * 0x7fc00000 ? x + y : 1.0f;
+            if (2 * ix > 2u * 0x7f800000 || 2 * iy > 2u * 0x7f800000) return x + y;
+            if (2 * ix == 2 * 0x3f800000) return 1.0f;
+            if ((2 * ix < 2 * 0x3f800000) == !(iy & 0x80000000)) return 0.0f;
+            return y * y;
+        }
+        if (powf_zeroinfnan(ix)) {
+            float x2 = x * x;
+            if ((ix & 0x80000000) && powf_checkint(iy) == 1) x2 = -x2;
+            return (iy & 0x80000000) ? 1 / x2 : x2;
+        }
+        if (ix & 0x80000000) {
+            int yint = powf_checkint(iy);
+            if (yint == 0) return NAN;
+            if (yint == 1) sign_bias = 1u << (5 + 11);
+            ix &= 0x7fffffff;
+        }
+        if (ix < 0x00800000) {
+            ix = f32_bits(x * 0x1p23f);
+            ix &= 0x7fffffff;
+            ix -= 23 << 23;
+        }
+    }
+    uint32_t tmp = ix - 0x3f330000;
+    int i = (tmp >> (23 - 4)) % 16;
+    uint32_t top = tmp & 0xff800000;
+    uint32_t iz = ix - top;
+    int k = (int32_t) top >> (23 - 5);
+    double invc = ORC_POWF_LOG2_TAB[i][0], logc = ORC_POWF_LOG2_TAB[i][1];
+    double z = (double) bits_f32(iz);
+    double r = fma(z, invc, -1.0);
+    double y0 = logc + (double) k;
+    double r2 = r * r;
+    double yy = fma(A0, r, A1);
+    double pp = fma(A2, r, A3);
+    double r4 = r2 * r2;
+    double q = fma(A4, r, y0);
+    q = fma(pp, r2, q);
+    double logx = fma(yy, r4, q);
+    double ylogx = (double) y * logx;
+    if ((double_as_u64(ylogx) >> 47 & 0xffff) >= double_as_u64(126.0 * 32) >> 47) {
+        if (ylogx > 0x1.fffffffd1d571p+6 * 32) return sign_bias ? -INFINITY : INFINITY;
+        if (ylogx <= -150.0 * 32) return sign_bias ? -0.0f : 0.0f;
+    }
+    const double SHIFT = 0x1.8p+52;
+    const double C0 = 0x1.c6af84b912394p-5 / 32 / 32 / 32, C1 = 0x1.ebfce50fac4f3p-3 / 32 / 32, C2 = 0x1.62e42ff0c52d6p-1 / 32;
+    double kd = ylogx + SHIFT;
+    uint64_t ki = double_as_u64(kd);
+    kd -= SHIFT;
+    double rr = ylogx - kd;
+    uint64_t t = ORC_EXP2F_TAB[ki % 32];
+    t += (ki + sign_bias) << (52 - 5);
+    double s = u64_as_double(t);
+    double zz = fma(C0, rr, C1);
+    double rr2 = rr * rr;
+    double e = fma(C2, rr, 1.0);
+    e = fma(zz, rr2, e);
+    return (float) (e * s);
+}
+
+float orc_expm1f_det(float x) {
+    const float one = 1.0f, tiny = 1.0e-30f, huge = 1.0e+30f, o_threshold = 8.8721679688e+01f, ln2_hi = 6.9313812256e-01f,
+                ln2_lo = 9.0580006145e-06f, invln2 = 1.4426950216e+00f, Q1 = -3.3333335072e-02f, Q2 = 1.5873016091e-03f,
+                Q3 = -7.9365076090e-05f, Q4 = 4.0082177293e-06f, Q5 = -2.0109921195e-07f;
+    float y, hi, lo, c = 0, t, e, hxs, hfx, r1;
+    int32_t k;
+    uint32_t hx = f32_bits(x);
+    uint32_t xsb = hx & 0x80000000u;
+    hx &= 0x7fffffff;
+    if (hx >= 0x4195b844) {
+        if (hx >= 0x42b17218) {
+            if (hx > 0x7f800000) return x + x;
+            if (hx == 0x7f800000) return (xsb == 0) ? x : -1.0f;
+            if (x > o_threshold) return huge * huge;
+        }
+        if (xsb != 0) return tiny - one;
+    }
+    if (hx > 0x3eb17218) {
+        if (hx < 0x3F851592) {
+            if (xsb == 0) { hi = x - ln2_hi; lo = ln2_lo; k = 1; }
+            else { hi = x + ln2_hi; lo = -ln2_lo; k = -1; }
+        } else {
+            k = (int32_t) (invln2 * x + ((xsb == 0) ? 0.5f : -0.5f));
+            t = (float) k;
+            hi = x - t * ln2_hi;
+            lo = t * ln2_lo;
+        }
+        x = hi - lo;
+        c = (hi - x) - lo;
+    } else if (hx < 0x33000000) {
+        t = huge + x;
+        return x - (t - (huge + x));
+    } else k = 0;
+    hfx = 0.5f * x;
+    hxs = x * hfx;
+    r1 = one + hxs * (Q1 + hxs * (Q2 + hxs * (Q3 + hxs * (Q4 + hxs * Q5))));
+    t = 3.0f - r1 * hfx;
+    e = hxs * ((r1 - t) / (6.0f - x * t));
+    if (k == 0) return x - (x * e - hxs);
+    e = (x * (e - c) - c);
+    e -= hxs;
+    if (k == -1) return 0.5f * (x - e) - 0.5f;
+    if (k == 1) {
+        if (x < -0.25f) return -2.0f * (e - (x + 0.5f));
+        return one + 2.0f * (x - e);
+    }
+    if (k <= -2 || k > 56) {
+        y = one - (e - x);
+        y = bits_f32(f32_bits(y) + ((uint32_t) k << 23));
+        return y - one;
+    }
+    if (k < 23) {
+        t = bits_f32(0x3f800000 - (0x1000000 >> k));
+        y = t - (e - x);
+        y = bits_f32(f32_bits(y) + ((uint32_t) k << 23));
+    } else {
+        t = bits_f32((uint32_t) (0x7f - k) << 23);
+        y = x - (e + t);
+        y += one;
+        y = bits_f32(f32_bits(y) + ((uint32_t) k << 23));
+    }
+    return y;
+}
+
+float orc_tanhf_det(float x) {
+    const float one = 1.0f, tiny = 1.0e-30f;
+    float t, z;
+    int32_t jx = (int32_t) f32_bits(x), ix = jx & 0x7fffffff;
+    if (ix >= 0x7f800000) { if (jx >= 0) return one / x + one; else return one / x - one; }
+    if (ix < 0x41b00000) {
+        if (ix == 0) return x;
+        if (ix < 0x24000000) return x * (one + x);
+        if (ix >= 0x3f800000) {
+            t = orc_expm1f_det(2.0f * fabsf(x));
+            z = one - 2.0f / (t + 2.0f);
+        } else {
+            t = orc_expm1f_det(-2.0f * fabsf(x));
+            z = -t / (t + 2.0f);
+        }
+    } else z = one - tiny;
+    return (jx >= 0) ? z : -z;
+}
+
+// Arguments with bit patterns lo_bits, lo_bits + stride, ... <= hi_bits on which the restatement and libm differ (two
+// NaNs count as equal).
+long long orc_powf_count_mismatch(uint32_t lo_bits, uint32_t hi_bits, uint32_t stride, float y, uint32_t *first_bad) {
+    long long bad = 0;
+    uint32_t fb = 0;
+    long long nsteps = ((long long) hi_bits - (long long) lo_bits) / stride + 1;
+#pragma omp parallel for reduction(+:bad) schedule(static)
+    for (long long sidx = 0; sidx < nsteps; ++sidx) {
+        uint32_t b = lo_bits + (uint32_t) (sidx * stride);
+        float x = bits_f32(b);
+        float a = orc_powf_det(x, y), c = powf(x, y);
+        if (f32_bits(a) != f32_bits(c) && !(a != a && c != c)) {
+            bad++;
+#pragma omp critical
+            if (fb == 0) fb = b;
+        }
+    }
+    if (first_bad) *first_bad = fb;
+    return bad;
+}
+
+long long orc_tanhf_count_mismatch(uint32_t lo_bits, uint32_t hi_bits, uint32_t stride, uint32_t *first_bad) {
+    long long bad = 0;
+    uint32_t fb = 0;
+    long long nsteps = ((long long) hi_bits - (long long) lo_bits) / stride + 1;
+#pragma omp parallel for reduction(+:bad) schedule(static)
+    for (long long sidx = 0; sidx < nsteps; ++sidx) {
+        uint32_t b = lo_bits + (uint32_t) (sidx * stride);
+        float x = bits_f32(b);
+        float a = orc_tanhf_det(x), c = tanhf(x);
+        if (f32_bits(a) != f32_bits(c) && !(a != a && c != c)) {
+            bad++;
+#pragma omp critical
+            if (fb == 0) fb = b;
+        }
+    }
+    if (first_bad) *first_bad = fb;
+    return bad;
+}
+
+// ---------------------------------------------------------------------------
 // index-set predicates (include/thundersvm/kernel/smo_kernel.h:13-23)
 // ---------------------------------------------------------------------------
 static inline bool is_I_up(double a, double y, double Cp, double Cn) { return (y > 0 && a < Cp) || (y < 0 && a > 0); }
@@ -178,16 +398,16 @@ struct OrcKernelMatrix {
 
 static double epilogue_poly(double dot, const orc_param &p) {
     // kernelmatrix_kernel.cpp:94-100: powf(gamma * dot + coef0, degree), float-rounded argument.
-    // expf_mode 1: double pow rounded once to float (what the HIP epilogue computes).
+    // expf_mode 1: the restated powf (what the HIP epilogue computes).
     float arg = (float) fma(p.gamma, dot, p.coef0);
-    if (p.expf_mode) return (double) (float) pow((double) arg, (double) p.degree);
+    if (p.expf_mode) return (double) orc_powf_det(arg, (float) p.degree);
     return (double) powf(arg, (float) p.degree);
 }
 
 static double epilogue_sigmoid(double dot, const orc_param &p) {
-    // kernelmatrix_kernel.cpp:102-108; expf_mode 1: double tanh rounded once to float.
+    // kernelmatrix_kernel.cpp:102-108; expf_mode 1: the restated tanhf.
     float arg = (float) fma(p.gamma, dot, p.coef0);
-    if (p.expf_mode) return (double) (float) tanh((double) arg);
+    if (p.expf_mode) return (double) orc_tanhf_det(arg);
     return (double) tanhf(arg);
 }
 

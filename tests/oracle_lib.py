@@ -48,6 +48,16 @@ def lib():
         L.orc_expf_libm.argtypes = [C.c_float]
         L.orc_expf_count_mismatch.restype = C.c_longlong
         L.orc_expf_count_mismatch.argtypes = [C.c_uint32, C.c_uint32, C.c_uint32, C.POINTER(C.c_uint32)]
+        L.orc_powf_det.restype = C.c_float
+        L.orc_powf_det.argtypes = [C.c_float, C.c_float]
+        L.orc_tanhf_det.restype = C.c_float
+        L.orc_tanhf_det.argtypes = [C.c_float]
+        L.orc_expm1f_det.restype = C.c_float
+        L.orc_expm1f_det.argtypes = [C.c_float]
+        L.orc_powf_count_mismatch.restype = C.c_longlong
+        L.orc_powf_count_mismatch.argtypes = [C.c_uint32, C.c_uint32, C.c_uint32, C.c_float, C.POINTER(C.c_uint32)]
+        L.orc_tanhf_count_mismatch.restype = C.c_longlong
+        L.orc_tanhf_count_mismatch.argtypes = [C.c_uint32, C.c_uint32, C.c_uint32, C.POINTER(C.c_uint32)]
         L.orc_km_create.restype = C.c_void_p
         L.orc_train.restype = C.c_void_p
         L.orc_calculate_rho.restype = C.c_double

@@ -1,9 +1,9 @@
 """GPU parity: KernelMatrix::get_rows / diag and sum_kernel_values through the C ABI vs the CPU oracle.
 
 Mirrors src/test/test_kernelmatrix.cpp (same fixture, same row sets, all four kernels) and adds
-ragged shapes.  Bars: linear and RBF bit-exact (the oracle runs its restated expf, expf_mode=1);
-poly / sigmoid within 1 float32 ulp and >= 99.9% identical (double pow/tanh rounded to float on both sides,
-but from two different math libraries); decision values 1e-9.
+ragged shapes.  Bars: all four kernels bit-exact (the oracle runs its restated expf / powf / tanhf, expf_mode=1, which
+tests/test_oracle_expf.py pins to libm; test_poly_and_sigmoid_rows_match_libm checks the GPU against libm itself);
+decision values 1e-9.
 """
 import numpy as np
 import pytest
@@ -26,13 +26,36 @@ KERNELS = [
 
 
 def _check(name, got, want):
-    if name in ("rbf", "linear"):
-        bad = np.flatnonzero(got.ravel() != want.ravel())
-        assert bad.size == 0, "%s: %d mismatching entries, first %s got %r want %r" % (
-            name, bad.size, bad[:1], got.ravel()[bad[:1]], want.ravel()[bad[:1]])
-    else:
-        assert G.float_ulp_diff(got, want).max() <= 1
-        assert (got != want).mean() < 1e-3
+    bad = np.flatnonzero(got.ravel() != want.ravel())
+    assert bad.size == 0, "%s: %d mismatching entries, first %s got %r want %r" % (
+        name, bad.size, bad[:1], got.ravel()[bad[:1]], want.ravel()[bad[:1]])
+
+
+@pytest.mark.parametrize("name,kt,prm", [("poly3", O.POLY, dict(gamma=0.5, degree=3, coef0=0.1)),
+                                         ("poly2", O.POLY, dict(gamma=1.5, degree=2, coef0=0.0)),
+                                         ("poly5", O.POLY, dict(gamma=0.05, degree=5, coef0=1.0)),
+                                         ("poly7neg", O.POLY, dict(gamma=-0.3, degree=7, coef0=-0.2)),
+                                         ("poly0", O.POLY, dict(gamma=0.5, degree=0, coef0=0.1)),
+                                         ("sigmoid", O.SIGMOID, dict(gamma=0.5, coef0=0.1)),
+                                         ("sigmoid_small", O.SIGMOID, dict(gamma=1e-3, coef0=0.0)),
+                                         ("sigmoid_large", O.SIGMOID, dict(gamma=9.0, coef0=-2.0))])
+def test_poly_and_sigmoid_rows_match_libm(name, kt, prm):
+    """The polynomial and sigmoid epilogues against the host's libm powf / tanhf themselves (the oracle with
+    expf_mode=0 calls them, as the reference does, kernelmatrix_kernel.cpp:94-108): bit for bit, including negative
+    arguments of odd powers, degree 0 and arguments on both sides of tanhf's ranges."""
+    rng = np.random.default_rng(21)
+    x = rng.standard_normal((300, 12)).astype(np.float32).astype(np.float64)
+    x[::7] *= 40.0            # some large dot products: overflow and saturation
+    x[3::11] *= 1e-3          # and some tiny ones
+    data = from_dense(x, np.ones(300))
+    okm = O.KernelMatrix(data.ptr, data.col, data.val, O.make_param(kernel_type=kt, expf_mode=0, **prm))
+    x_d, nf, ld, sd, diag = _device_km(data, kt, prm)
+    _check(name, G.host(diag), okm.diag())
+    rows = np.arange(0, 300, 3, dtype=np.int32)
+    got = G.get_rows_dense(x_d, ld, data.n, nf, sd, x_d, ld, G.dev(rows), len(rows), sd, kt, **prm)
+    want = okm.get_rows(rows)
+    both_nan = np.isnan(G.host(got)) & np.isnan(want)
+    _check(name, np.where(both_nan, 0.0, G.host(got)), np.where(both_nan, 0.0, want))
 
 
 def _device_km(data, kt, prm):

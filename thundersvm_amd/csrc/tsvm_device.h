@@ -59,6 +59,198 @@ __device__ __forceinline__ float tsvm_expf(float x, const uint64_t *tab) {
     return res;
 }
 
+// powf, the routine glibc (>= 2.28) uses: log2(x) from a 16-entry table and a quartic, in double, times y, then
+// 2^that through the expf table and cubic; every a*b+c is one fma (the form the library's FMA build takes on the
+// hosts this was checked on: all 2^32 arguments x for each of fourteen exponents give libm's bits).  Entries are
+// {1/c, log2(c) * 32}; the polynomial and the product y*log2(x) carry the same factor 32 (the exp table's size).
+__constant__ const double TSVM_POWF_LOG2_TAB[16][2] = {
+    {0x1.661ec79f8f3bep+0, -0x1.efec65b963019p-2 * 32}, {0x1.571ed4aaf883dp+0, -0x1.b0b6832d4fca4p-2 * 32},
+    {0x1.49539f0f010bp+0, -0x1.7418b0a1fb77bp-2 * 32},  {0x1.3c995b0b80385p+0, -0x1.39de91a6dcf7bp-2 * 32},
+    {0x1.30d190c8864a5p+0, -0x1.01d9bf3f2b631p-2 * 32}, {0x1.25e227b0b8eap+0, -0x1.97c1d1b3b7afp-3 * 32},
+    {0x1.1bb4a4a1a343fp+0, -0x1.2f9e393af3c9fp-3 * 32}, {0x1.12358f08ae5bap+0, -0x1.960cbbf788d5cp-4 * 32},
+    {0x1.0953f419900a7p+0, -0x1.a6f9db6475fcep-5 * 32}, {0x1p+0, 0x0p+0 * 32},
+    {0x1.e608cfd9a47acp-1, 0x1.338ca9f24f53dp-4 * 32},  {0x1.ca4b31f026aap-1, 0x1.476a9543891bap-3 * 32},
+    {0x1.b2036576afce6p-1, 0x1.e840b4ac4e4d2p-3 * 32},  {0x1.9c2d163a1aa2dp-1, 0x1.40645f0c6651cp-2 * 32},
+    {0x1.886e6037841edp-1, 0x1.88e9c2c1b9ff8p-2 * 32},  {0x1.767dcf5534862p-1, 0x1.ce0a44eb17bccp-2 * 32}};
+
+// 0: not an integer, 1: odd integer, 2: even integer (the float with bit pattern iy)
+__device__ __forceinline__ int tsvm_powf_checkint(uint32_t iy) {
+    const int e = iy >> 23 & 0xff;
+    if (e < 0x7f) return 0;
+    if (e > 0x7f + 23) return 2;
+    if (iy & ((1u << (0x7f + 23 - e)) - 1)) return 0;
+    if (iy & (1u << (0x7f + 23 - e))) return 1;
+    return 2;
+}
+__device__ __forceinline__ bool tsvm_powf_zeroinfnan(uint32_t ix) { return 2 * ix - 1 >= 2u * 0x7f800000 - 1; }
+
+// `tab`: the 32-entry table of tsvm_expf (LDS or constant).  The reference calls libm powf on float arguments
+// (kernelmatrix_kernel.cpp:94-100).
+__device__ __forceinline__ float tsvm_powf(float x, float y, const uint64_t *tab) {
+    const double A0 = 0x1.27616c9496e0bp-2 * 32, A1 = -0x1.71969a075c67ap-2 * 32, A2 = 0x1.ec70a6ca7baddp-2 * 32,
+                 A3 = -0x1.7154748bef6c8p-1 * 32, A4 = 0x1.71547652ab82bp0 * 32;
+    uint32_t sign_bias = 0;
+    uint32_t ix = __float_as_uint(x);
+    const uint32_t iy = __float_as_uint(y);
+    if (ix - 0x00800000 >= 0x7f800000 - 0x00800000 || tsvm_powf_zeroinfnan(iy)) {
+        // x is subnormal, zero, negative, infinite or NaN, or y is zero, infinite or NaN
+        if (tsvm_powf_zeroinfnan(iy)) {
+            if (2 * iy == 0) return 2 * (ix ^ 0x00400000) > 2u * 0x7fc00000 ? x + y : 1.0f;   // (a signalling NaN stays a NaN)
+            if (ix == 0x3f800000) return 2 * (iy ^ 0x00400000) > 2u * 0x7fc00000 ? x + y : 1.0f;
+            if (2 * ix > 2u * 0x7f800000 || 2 * iy > 2u * 0x7f800000) return x + y;
+            if (2 * ix == 2 * 0x3f800000) return 1.0f;
+            if ((2 * ix < 2 * 0x3f800000) == !(iy & 0x80000000)) return 0.0f;   // |x| < 1 and y = inf, or |x| > 1 and y = -inf
+            return y * y;
+        }
+        if (tsvm_powf_zeroinfnan(ix)) {
+            float x2 = x * x;
+            if ((ix & 0x80000000) && tsvm_powf_checkint(iy) == 1) x2 = -x2;
+            return (iy & 0x80000000) ? 1 / x2 : x2;
+        }
+        if (ix & 0x80000000) {   // finite x < 0
+            const int yint = tsvm_powf_checkint(iy);
+            if (yint == 0) return __uint_as_float(0x7fc00000u);   // a quiet NaN (libm returns one of either sign)
+            if (yint == 1) sign_bias = 1u << (5 + 11);
+            ix &= 0x7fffffff;
+        }
+        if (ix < 0x00800000) {   // subnormal x: normalised
+            ix = __float_as_uint(x * 0x1p23f);
+            ix &= 0x7fffffff;
+            ix -= 23 << 23;
+        }
+    }
+    // x = 2^k z, z in [0x1.66p-1, 0x1.66p0): log2(x) * 32 = k * 32 + log2(c) * 32 + log2(z/c) * 32
+    const uint32_t tmp = ix - 0x3f330000;
+    const int i = (tmp >> (23 - 4)) % 16;
+    const uint32_t top = tmp & 0xff800000;
+    const uint32_t iz = ix - top;
+    const int k = (int32_t) top >> (23 - 5);
+    const double invc = TSVM_POWF_LOG2_TAB[i][0], logc = TSVM_POWF_LOG2_TAB[i][1];
+    const double z = (double) __uint_as_float(iz);
+    const double r = __builtin_fma(z, invc, -1.0);
+    const double y0 = logc + (double) k;
+    const double r2 = r * r;
+    const double yy = __builtin_fma(A0, r, A1);
+    const double pp = __builtin_fma(A2, r, A3);
+    const double r4 = r2 * r2;
+    double q = __builtin_fma(A4, r, y0);
+    q = __builtin_fma(pp, r2, q);
+    const double logx = __builtin_fma(yy, r4, q);
+    const double ylogx = (double) y * logx;
+    if (((uint64_t) __double_as_longlong(ylogx) >> 47 & 0xffff) >= ((uint64_t) __double_as_longlong(126.0 * 32) >> 47)) {
+        if (ylogx > 0x1.fffffffd1d571p+6 * 32) return sign_bias ? -__builtin_inff() : __builtin_inff();
+        if (ylogx <= -150.0 * 32) return sign_bias ? -0.0f : 0.0f;
+    }
+    // 2^(ylogx / 32): as in tsvm_expf, with the sign of the result carried into the table entry's top bit
+    const double SHIFT = 0x1.8p+52;
+    const double C0 = 0x1.c6af84b912394p-5 / 32 / 32 / 32;
+    const double C1 = 0x1.ebfce50fac4f3p-3 / 32 / 32;
+    const double C2 = 0x1.62e42ff0c52d6p-1 / 32;
+    double kd = ylogx + SHIFT;
+    const uint64_t ki = (uint64_t) __double_as_longlong(kd);
+    kd -= SHIFT;
+    const double rr = ylogx - kd;
+    uint64_t t = tab[ki % 32];
+    t += (ki + sign_bias) << (52 - 5);
+    const double s = __longlong_as_double((long long) t);
+    const double zz = __builtin_fma(C0, rr, C1);
+    const double rr2 = rr * rr;
+    double e = __builtin_fma(C2, rr, 1.0);
+    e = __builtin_fma(zz, rr2, e);
+    return (float) (e * s);
+}
+
+// expm1f and tanhf in float arithmetic, statement by statement the routines glibc's libm uses (the fdlibm float
+// versions): all 2^32 arguments give libm's bits.  No operation here may be fused or reassociated (the library is
+// built with -ffp-contract=off; float division is correctly rounded).  The reference calls libm tanhf
+// (kernelmatrix_kernel.cpp:102-108).
+__device__ __forceinline__ float tsvm_expm1f(float x) {
+    const float one = 1.0f, tiny = 1.0e-30f, huge = 1.0e+30f, o_threshold = 8.8721679688e+01f, ln2_hi = 6.9313812256e-01f,
+                ln2_lo = 9.0580006145e-06f, invln2 = 1.4426950216e+00f, Q1 = -3.3333335072e-02f, Q2 = 1.5873016091e-03f,
+                Q3 = -7.9365076090e-05f, Q4 = 4.0082177293e-06f, Q5 = -2.0109921195e-07f;
+    float y, hi, lo, c = 0.0f, t, e;
+    int k;
+    uint32_t hx = __float_as_uint(x);
+    const uint32_t xsb = hx & 0x80000000u;
+    hx &= 0x7fffffffu;
+    if (hx >= 0x4195b844u) {   // |x| >= 27 ln 2
+        if (hx >= 0x42b17218u) {
+            if (hx > 0x7f800000u) return x + x;
+            if (hx == 0x7f800000u) return xsb == 0 ? x : -1.0f;
+            if (x > o_threshold) return huge * huge;
+        }
+        if (xsb != 0) return tiny - one;
+    }
+    if (hx > 0x3eb17218u) {   // |x| > 0.5 ln 2: x = k ln 2 + (hi - lo)
+        if (hx < 0x3F851592u) {
+            if (xsb == 0) { hi = x - ln2_hi; lo = ln2_lo; k = 1; }
+            else { hi = x + ln2_hi; lo = -ln2_lo; k = -1; }
+        } else {
+            k = (int) (invln2 * x + (xsb == 0 ? 0.5f : -0.5f));
+            t = (float) k;
+            hi = x - t * ln2_hi;
+            lo = t * ln2_lo;
+        }
+        x = hi - lo;
+        c = (hi - x) - lo;
+    } else if (hx < 0x33000000u) {   // |x| < 2^-25
+        t = huge + x;
+        return x - (t - (huge + x));
+    } else {
+        k = 0;
+    }
+    const float hfx = 0.5f * x;
+    const float hxs = x * hfx;
+    const float r1 = one + hxs * (Q1 + hxs * (Q2 + hxs * (Q3 + hxs * (Q4 + hxs * Q5))));
+    t = 3.0f - r1 * hfx;
+    e = hxs * ((r1 - t) / (6.0f - x * t));
+    if (k == 0) return x - (x * e - hxs);
+    e = (x * (e - c) - c);
+    e -= hxs;
+    if (k == -1) return 0.5f * (x - e) - 0.5f;
+    if (k == 1) {
+        if (x < -0.25f) return -2.0f * (e - (x + 0.5f));
+        return one + 2.0f * (x - e);
+    }
+    if (k <= -2 || k > 56) {
+        y = one - (e - x);
+        y = __uint_as_float(__float_as_uint(y) + ((uint32_t) k << 23));   // k added to the exponent
+        return y - one;
+    }
+    if (k < 23) {
+        t = __uint_as_float(0x3f800000u - (0x1000000u >> k));   // 1 - 2^-k
+        y = t - (e - x);
+        y = __uint_as_float(__float_as_uint(y) + ((uint32_t) k << 23));
+    } else {
+        t = __uint_as_float((uint32_t) (0x7f - k) << 23);       // 2^-k
+        y = x - (e + t);
+        y += one;
+        y = __uint_as_float(__float_as_uint(y) + ((uint32_t) k << 23));
+    }
+    return y;
+}
+
+__device__ __forceinline__ float tsvm_tanhf(float x) {
+    const float one = 1.0f, tiny = 1.0e-30f;
+    const int jx = (int) __float_as_uint(x), ix = jx & 0x7fffffff;
+    if (ix >= 0x7f800000) return jx >= 0 ? one / x + one : one / x - one;
+    float z;
+    if (ix < 0x41b00000) {   // |x| < 22
+        if (ix == 0) return x;
+        if (ix < 0x24000000) return x * (one + x);   // |x| < 2^-55
+        if (ix >= 0x3f800000) {
+            const float t = tsvm_expm1f(2.0f * __builtin_fabsf(x));
+            z = one - 2.0f / (t + 2.0f);
+        } else {
+            const float t = tsvm_expm1f(-2.0f * __builtin_fabsf(x));
+            z = -t / (t + 2.0f);
+        }
+    } else {
+        z = one - tiny;
+    }
+    return jx >= 0 ? z : -z;
+}
+
 // Kernel epilogues (kernelmatrix_kernel.cpp:61-108).  sd0/sd1 are the two rows' self dot products.
 // The RBF / polynomial / sigmoid values are floats by definition (expf / powf / tanhf); this returns that
 // float, so that a caller storing float rows pays for no round trip through double.
@@ -66,13 +258,12 @@ __device__ __forceinline__ float tsvm_epilogue_f32(double dot, double sd0, doubl
                                                    const uint64_t *tab) {
     switch (p.kernel_type) {
         case TSVM_POLY: {
-            // powf / tanhf of a float-rounded argument: evaluated in double and rounded once to float
             const float arg = (float) __builtin_fma(p.gamma, dot, p.coef0);
-            return (float) pow((double) arg, (double) p.degree);
+            return tsvm_powf(arg, (float) p.degree, tab);
         }
         case TSVM_SIGMOID: {
             const float arg = (float) __builtin_fma(p.gamma, dot, p.coef0);
-            return (float) tanh((double) arg);
+            return tsvm_tanhf(arg);
         }
         default: {
             // -(sd0 + sd1 - 2*dot) * gamma; 2*dot is exact, so the fma rounds exactly where the subtraction would
