@@ -28,7 +28,7 @@ __constant__ const uint64_t TSVM_EXP2F_TAB[32] = {
     0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full, 0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull};
 
 // expf of a float argument, evaluated in double and rounded once to float: the table-driven
-// algorithm glibc (>= 2.27) uses for expf.  `tab` points at the 32-entry table (LDS or constant).
+// algorithm glibc (>= 2.27) uses for expf, in the form its FMA build takes (libm's bits on all 2^32 arguments).  `tab` points at the 32-entry table (LDS or constant).
 // The reference's kernels call libm expf on the host (kernelmatrix_kernel.cpp:71-72,87-89).
 __device__ __forceinline__ float tsvm_expf(float x, const uint64_t *tab) {
     const double InvLn2N = 0x1.71547652b82fep+0 * 32;
@@ -38,12 +38,14 @@ __device__ __forceinline__ float tsvm_expf(float x, const uint64_t *tab) {
     const double C2 = 0x1.62e42ff0c52d6p-1 / 32;
     // The main path runs unconditionally and the out-of-range cases are selected afterwards (no
     // branches in the epilogue); a NaN argument comes out as NaN through the arithmetic itself.
+    // (k and r both come straight from the exact product x * 32/ln2, as in the library's FMA build, where the
+    // compiler fuses the product into the addition of SHIFT and into the subtraction of k: with a rounded product
+    // two of the 2^32 arguments gave a neighbouring float)
     double xd = (double) x;
-    double z = InvLn2N * xd;
-    double kd = z + SHIFT;
+    double kd = __builtin_fma(InvLn2N, xd, SHIFT);
     const uint32_t ki = (uint32_t) __double2loint(kd);
     kd -= SHIFT;
-    double r = z - kd;
+    double r = __builtin_fma(InvLn2N, xd, -kd);
     // s = 2^(k/32): table entry with k/32 added into the exponent field.  The published routine adds
     // ki << 47 to the 64-bit entry; the low word of that term is zero, so only the high word changes.
     const uint64_t t = tab[ki & 31];
