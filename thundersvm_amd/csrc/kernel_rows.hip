@@ -194,6 +194,9 @@ __device__ __forceinline__ void get_rows_tile(
     }
 
     // epilogue + store.  Interior tiles take the unguarded path; edge tiles test every element.
+    // (Sixteen lanes write 64 or 128 consecutive bytes of an output row: streamed past the L2 when those runs are
+    // whole 64-byte pieces of memory, which depends on where the rows start; partial pieces the L2 has to merge.)
+    const bool stream_out = !SYM && ((ldo * (int64_t) sizeof(TO)) % 64 == 0) && ((uintptr_t) out % 64 == 0);
     if (full) {
 #pragma unroll
         for (int ti = 0; ti < TI; ++ti) {
@@ -206,8 +209,10 @@ __device__ __forceinline__ void get_rows_tile(
                     if (SYM) {   // the solver's block: read again at once
                         orow[tj * 16] = val;
                         out[(int64_t) (jb + tj * 16) * ldo + (i0 + wi * (16 * TI) + ti * 16 + 4 * v + lk)] = val;
-                    } else {
+                    } else if (stream_out) {
                         store_streaming(orow + tj * 16, val);
+                    } else {
+                        orow[tj * 16] = val;
                     }
                 }
             }
@@ -228,7 +233,7 @@ __device__ __forceinline__ void get_rows_tile(
                             orow[tj * 16] = val;
                             out[(int64_t) (jb + tj * 16) * ldo + i] = val;
                         } else {
-                            store_streaming(orow + tj * 16, val);
+                            orow[tj * 16] = val;
                         }
                     }
             }
@@ -486,7 +491,7 @@ __global__ __launch_bounds__(256, 3) void get_rows_dense_stream_kernel(
                     TO *orow = out + (int64_t) ((uint64_t) (uint32_t) s_slot[r] * (uint32_t) ldo) + jb;
 #pragma unroll
                     for (int tj = 0; tj < 4; ++tj)
-                        if (jb + tj < n) store_streaming(orow + tj, finish(acc[ti][tj][v], sdi, mi, tj));
+                        if (jb + tj < n) orow[tj] = finish(acc[ti][tj][v], sdi, mi, tj);   // (single values: left to the L2 to merge)
                 }
             }
         }
@@ -800,7 +805,7 @@ __global__ __launch_bounds__(SK_T) void sum_kernel_values_kernel(
 #pragma unroll
                     for (int rr = 0; rr < SK_R; ++rr) {
                         const int64_t r = r0 + rr < n_instances ? r0 + rr : n_instances - 1;   // a valid row; not added below
-                        kv[u][rr] = load_streaming(k_mat + r * ldk + st + l + u * SK_T);
+                        kv[u][rr] = k_mat[r * ldk + st + l + u * SK_T];   // (read once per class: the L2 serves the repeats)
                     }
                 }
 #pragma unroll

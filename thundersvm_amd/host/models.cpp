@@ -121,13 +121,15 @@ void SvmModel::predict_dec_values(const DataSet::node2d &instances, std::vector<
     d_rho.upload(rho);
     const size_t bmax = std::min((size_t) batch_size, instances.size());
     // kernel values of one batch: taken from the persistent row arena (no allocation per call)
-    void *d_k = tsvm::RowArena::instance().acquire(bmax * T * k_mat.row_elem_size(), false);
+    // (rows padded to 16 elements: get_rows then writes whole aligned vectors)
+    const int64_t ldk = ((int64_t) T + 15) / 16 * 16;
+    void *d_k = tsvm::RowArena::instance().acquire(bmax * (size_t) ldk * k_mat.row_elem_size(), false);
     DeviceBuffer<float_type> d_dec(bmax * n_binary_models);
     for (size_t b0 = 0; b0 < instances.size(); b0 += batch_size) {
         const size_t bm = std::min((size_t) batch_size, instances.size() - b0);
-        k_mat.get_rows(instances.data() + b0, bm, d_k, (int64_t) T);
+        k_mat.get_rows(instances.data() + b0, bm, d_k, ldk);
         abi_check(tsvm_sum_kernel_values(d_coef.data(), (int) T, d_start.data(), d_count.data(), d_rho.data(), d_k,
-                                         k_mat.row_type(), (int64_t) T, d_dec.data(), n_classes, (int64_t) bm, nullptr));
+                                         k_mat.row_type(), ldk, d_dec.data(), n_classes, (int64_t) bm, nullptr));
         d_dec.download(dec.data() + b0 * n_binary_models, bm * n_binary_models);
     }
 }
