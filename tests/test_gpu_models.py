@@ -181,10 +181,15 @@ def test_class_pairs_in_lockstep_give_the_same_model():
     w = D.workload_c4(scale=0.01)
     tr = w["train"]
     ref = None
-    for lanes, cache in ((1, -1), (2, -1), (3, 0), (5, 64 << 20)):
+    for lanes, cache in ((1, -1), (2, -1), (3, 0), (5, 64 << 20), (8, -1), (0, -1)):
         m = Model(0).train(tr, make_param(pair_lanes=lanes, cache_bytes=cache, **w["params"]))
         cur = (m.coef.copy(), m.rho.copy(), m.sv_indices.copy(), [m.stats(b)["n_iter"] for b in range(m.n_binary)],
                [m.stats(b)["local_iter"] for b in range(m.n_binary)])
+        xcds = [m.stats(b)["solver_xcd"] for b in range(m.n_binary)]
+        if lanes != 1 and max(xcds) >= 0:   # (-1 everywhere: the lockstep schedule, no CU masks on this device)
+            # every lane's local solver was elected onto an XCD of its own
+            n_lanes = 8 if lanes == 0 else lanes
+            assert all(0 <= x < n_lanes for x in xcds) and len(set(xcds)) >= 2, xcds
         if ref is None:
             ref = cur
             assert m.n_binary == 21

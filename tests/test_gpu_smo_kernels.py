@@ -132,6 +132,50 @@ def test_nu_smo_solve(n, ws):
     assert np.array_equal(G.host(ad_d), ad_want)
 
 
+@pytest.mark.parametrize("nu", [False, True])
+@pytest.mark.parametrize("n,ws", [(300, 16), (2000, 1024), (900, 200)])
+def test_smo_solve_block_on_a_chosen_xcd(n, ws, nu):
+    """The block solvers launched as eight workgroups of which one is elected (tsvm_*_smo_solve_block_on_xcd): the same
+    result as the one-workgroup launch, for every target XCD and launch after launch on one gate.  On an ordinary
+    stream the eight workgroups land wherever there is room, so some targets have a workgroup on them and others
+    do not: both ways of being elected (being on the target, being the last to arrive) are exercised, and exactly one
+    workgroup solves either way (two would apply every step twice)."""
+    Cc, eps = 1.0, 1e-3
+    y, alpha, f, ws_ids, k_rows, diag = _solver_inputs(n, 10, ws, 7 * n + ws, Cc, nu)
+    if nu:
+        a_want, ad_want, diff_want = O.nu_smo_solve(y, f, alpha, ws_ids, Cc, k_rows, diag, n, eps, 100000)
+    else:
+        a_want, ad_want, diff_want = O.c_smo_solve(y, f, alpha, ws_ids, Cc, Cc, k_rows, diag, n, eps, 100000)
+    ldk = capi.kernel_lib().tsvm_smo_solve_block_ld(ws)
+    block = np.zeros((ws, ldk))
+    block[:, :ws] = k_rows[:, ws_ids]
+    y_d, f_d, ws_d, b_d, dg_d = G.dev(y), G.dev(f), G.dev(ws_ids), G.dev(block), G.dev(diag)
+    gate = torch.zeros(4, dtype=torch.int32, device="cuda")
+    seen = set()
+    for epoch, xcd in enumerate([0, 3, 7, 5, 1, 2, 6, 4, 0, 0], start=1):
+        a_d = G.dev(alpha)
+        ad_d = torch.zeros(ws, dtype=torch.float64, device="cuda")
+        diff_d = torch.zeros(2, dtype=torch.float64, device="cuda")
+        if nu:
+            capi.call("tsvm_nu_smo_solve_block_on_xcd", G.ptr(y_d), G.ptr(f_d), G.ptr(a_d), G.ptr(ad_d), G.ptr(ws_d), ws, Cc,
+                      G.ptr(b_d), G.ptr(dg_d), eps, G.ptr(diff_d), 100000, G.ptr(gate), epoch, xcd, G.stream())
+        else:
+            capi.call("tsvm_c_smo_solve_block_on_xcd", G.ptr(y_d), G.ptr(f_d), G.ptr(a_d), G.ptr(ad_d), G.ptr(ws_d), ws, Cc, Cc,
+                      G.ptr(b_d), G.ptr(dg_d), eps, G.ptr(diff_d), 100000, G.ptr(gate), epoch, xcd, G.stream())
+        g = G.host(gate)
+        assert g[0] == epoch and g[1] == 8 * epoch and 0 <= g[2] < 8
+        seen.add(int(g[2]))
+        assert G.host(diff_d)[0] == diff_want[0]
+        assert np.array_equal(G.host(a_d), a_want)
+        assert np.array_equal(G.host(ad_d), ad_want)
+    # bad arguments are refused
+    lib = capi.kernel_lib()
+    assert lib.tsvm_c_smo_solve_block_on_xcd(G.ptr(y_d), G.ptr(f_d), G.ptr(a_d), G.ptr(ad_d), G.ptr(ws_d), ws, Cc, Cc, G.ptr(b_d),
+                                             G.ptr(dg_d), eps, G.ptr(diff_d), 10, G.ptr(gate), 0, 0, G.stream()) != 0
+    assert lib.tsvm_c_smo_solve_block_on_xcd(G.ptr(y_d), G.ptr(f_d), G.ptr(a_d), G.ptr(ad_d), G.ptr(ws_d), ws, Cc, Cc, G.ptr(b_d),
+                                             G.ptr(dg_d), eps, G.ptr(diff_d), 10, G.ptr(gate), 1, 8, G.stream()) != 0
+
+
 def _select_case(n, n_select, n_marked, seed, tie_mode, nu):
     rng = np.random.default_rng(seed)
     y = np.where(rng.random(n) < 0.5, 1, -1).astype(np.int32)
