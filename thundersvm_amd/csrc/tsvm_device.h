@@ -88,7 +88,9 @@ __device__ __forceinline__ bool tsvm_powf_zeroinfnan(uint32_t ix) { return 2 * i
 
 // `tab`: the 32-entry table of tsvm_expf (LDS or constant).  The reference calls libm powf on float arguments
 // (kernelmatrix_kernel.cpp:94-100).
-__device__ __forceinline__ float tsvm_powf(float x, float y, const uint64_t *tab) {
+// (Not inlined, nor tanhf below: the routines are long, their callers' epilogues are instantiated dozens of times, and
+// neither kernel is on a path where a call matters.)
+__device__ __noinline__ float tsvm_powf(float x, float y, const uint64_t *tab) {
     const double A0 = 0x1.27616c9496e0bp-2 * 32, A1 = -0x1.71969a075c67ap-2 * 32, A2 = 0x1.ec70a6ca7baddp-2 * 32,
                  A3 = -0x1.7154748bef6c8p-1 * 32, A4 = 0x1.71547652ab82bp0 * 32;
     uint32_t sign_bias = 0;
@@ -232,7 +234,7 @@ __device__ __forceinline__ float tsvm_expm1f(float x) {
     return y;
 }
 
-__device__ __forceinline__ float tsvm_tanhf(float x) {
+__device__ __noinline__ float tsvm_tanhf(float x) {
     const float one = 1.0f, tiny = 1.0e-30f;
     const int jx = (int) __float_as_uint(x), ix = jx & 0x7fffffff;
     if (ix >= 0x7f800000) return jx >= 0 ? one / x + one : one / x - one;
