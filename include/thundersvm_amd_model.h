@@ -125,6 +125,12 @@ int tsvm_selftest_solver_wait(int timeout_ms, int never_written);
  * src/test/test_syncmem.cpp and test_syncarray.cpp that apply.  0 on success, -1 with a message otherwise. */
 int tsvm_selftest_device_buffer(void);
 
+/* Test hook (no GPU needed): drives the kernel-row cache's bookkeeping as a solve does, with a first working set of ws
+ * ids and ws/2 new ids per iteration, on the cyclic sequence 0, 1, ..., n_ids-1, 0, ..., and checks after every
+ * iteration that each working-set row has a slot of its own, is pinned and off the eviction list.  Returns the
+ * number of hits, or -1 (tsvm_model_last_error says what broke). */
+long long tsvm_selftest_row_cache(int n_ids, int slots, int ws, int iterations);
+
 int tsvm_model_save(void *model, const char *path);
 int tsvm_model_load(void *model, const char *path);
 

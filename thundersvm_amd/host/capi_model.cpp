@@ -336,6 +336,13 @@ int tsvm_selftest_device_buffer(void) {
     })
 }
 
+long long tsvm_selftest_row_cache(int n_ids, int slots, int ws, int iterations) {
+    std::string what;
+    const long long hits = tsvm::row_cache_selftest(n_ids, slots, ws, iterations, what);
+    if (hits < 0) g_error = "row cache: " + what;
+    return hits;
+}
+
 int tsvm_selftest_solver_wait(int timeout_ms, int never_written) {
     static volatile uint64_t word;
     word = 0x7ff8dead00000001ull;

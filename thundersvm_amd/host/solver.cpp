@@ -175,6 +175,55 @@ bool make_lane_group(int n_lanes, LaneGroup &g) {
 
 namespace tsvm {
 
+// Drives RowCache the way a solve does (first working set of ws rows, then q = ws / 2 new rows per iteration while the
+// previous new half stays pinned) on a cyclic sequence of n_ids ids, and checks after every step that each row of the
+// working set has a slot of its own and that the tables agree.  Returns the number of hits, or -1 with `what` set.
+long long row_cache_selftest(int n_ids, int slots, int ws, int iterations, std::string &what) {
+    if (n_ids < ws || slots < 2 * ws || ws < 2 || ws % 2) { what = "bad arguments"; return -1; }
+    RowCache c;
+    c.init(n_ids, slots);
+    const int q = ws / 2;
+    std::vector<int> ids(ws), slot(ws);
+    long long hits = 0;
+    int next_id = 0;
+    for (int it = 0; it < iterations; ++it) {
+        const int n_new = it == 0 ? ws : q, first_new = it == 0 ? 0 : q;
+        if (it > 0) {
+            for (int t = 0; t < q; ++t) c.release(slot[t]);
+            for (int t = 0; t < q; ++t) { ids[t] = ids[t + q]; slot[t] = slot[t + q]; }
+        }
+        for (int t = 0; t < n_new; ++t) {
+            const int id = next_id;
+            next_id = (next_id + 1) % n_ids;
+            int s = c.lookup(id);
+            if (s >= 0) ++hits;
+            else s = c.insert(id);
+            if (s < 0) { what = "no slot left for a working-set row"; return -1; }
+            ids[first_new + t] = id;
+            slot[first_new + t] = s;
+        }
+        std::vector<char> taken(slots, 0);
+        for (int t = 0; t < ws; ++t) {
+            if (slot[t] < 0 || slot[t] >= slots || c.slot_of[ids[t]] != slot[t] || c.id_of[slot[t]] != ids[t]) {
+                what = "a working-set row lost its slot";
+                return -1;
+            }
+            if (taken[slot[t]] && n_ids >= 2 * ws) { what = "two working-set rows share a slot"; return -1; }
+            taken[slot[t]] = 1;
+            if (c.pins[slot[t]] < 1) { what = "a working-set row is not pinned"; return -1; }
+        }
+        int listed = 0;
+        for (int s2 = c.head; s2 >= 0; s2 = c.next[s2]) {
+            if (c.pins[s2] != 0) { what = "a pinned row is on the eviction list"; return -1; }
+            if (++listed > slots) { what = "the eviction list has a cycle"; return -1; }
+        }
+        int pinned = 0;
+        for (int s2 = 0; s2 < c.used; ++s2) pinned += c.pins[s2] > 0;
+        if (listed + pinned != c.used) { what = "rows neither pinned nor listed"; return -1; }
+    }
+    return hits;
+}
+
 long long solver_timeout_ms() {
     const char *e = getenv("TSVM_SOLVER_TIMEOUT_MS");
     const long long v = e ? atoll(e) : 0;

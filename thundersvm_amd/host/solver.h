@@ -2,6 +2,7 @@
 // nusmosolver.cpp) driving the gfx950 kernels.  f, alpha, y, the working set and the ws x n kernel
 // rows stay in HBM for the whole solve; per outer iteration the host reads back 16 bytes (diff).
 #pragma once
+#include <string>
 #include "kernelmatrix.h"
 
 struct SolverTrace {          // optional per-iteration record (parity debugging and tests)
@@ -32,6 +33,8 @@ struct SolverStats {
 class SolveTask;
 
 namespace tsvm {
+// checks the kernel-row cache's bookkeeping on a scripted sequence (see solver.cpp); hits or -1
+long long row_cache_selftest(int n_ids, int slots, int ws, int iterations, std::string &what);
 // Spins until *word no longer holds `pending`.  Every 200 ms `stream_state()` is asked for the state of the stream
 // that is to write the word (hipSuccess: everything enqueued has run; hipErrorNotReady: still running; anything else
 // is thrown as that error).  Throws std::runtime_error when the stream has drained without the word changing, or
