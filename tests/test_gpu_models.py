@@ -118,6 +118,26 @@ def test_workload_c4_small():
     _compare(w["train"], w["test"], make_param(**w["params"]), trace=64)
 
 
+@pytest.mark.parametrize("kernel", ["linear", "rbf"])
+def test_sparse_multiclass(kernel):
+    """Four classes on sparse text-like rows (CSR layout on the device): the class pairs run side by side, each on the
+    CSR kernels, and every pair's trajectory, alpha, f, rho and the assembled coefficients equal the oracle's."""
+    w = D.workload_c3(scale=0.05, kernel=kernel)
+    tr = w["train"]
+    rng = np.random.default_rng(3)
+    proj = rng.standard_normal((4, tr.n_features + 1))
+    scores = np.zeros((tr.n, 4))
+    for r in range(tr.n):
+        cols = tr.col[tr.ptr[r]:tr.ptr[r + 1]]
+        scores[r] = proj[:, cols] @ tr.val[tr.ptr[r]:tr.ptr[r + 1]]
+    y = scores.argmax(axis=1).astype(np.float64) + 1.0
+    y[rng.random(tr.n) < 0.05] = 4.0          # skewed class sizes and some label noise
+    from thundersvm_amd.data import CsrData
+    tr4 = CsrData(tr.ptr, tr.col, tr.val, y)
+    gm, om, _, _ = _compare(tr4, None, make_param(**w["params"]), trace=16)
+    assert gm.n_binary == 6
+
+
 def test_workload_c5_small():
     w = D.workload_c5(scale=0.01)
     _compare(w["train"], w["test"], make_param(**w["params"]), trace=64)
