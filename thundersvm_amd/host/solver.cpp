@@ -146,13 +146,16 @@ void destroy_masked_streams() {
 
 // Makes the 2 * n_lanes streams of a group.  Bit i of a CU mask names CU i/8 of XCD i%8 on the 8-XCD, 256-CU part (a
 // mask has to leave every XCD at least one CU: workgroups are dealt to the XCDs in turn).  Every solver stream gets
-// CU 0 of every XCD, every chip-wide stream the other 248 CUs.  With several lanes, lane l's solver is launched so
-// that it runs on XCD l (tsvm_c_smo_solve_block_on_xcd): the lanes share the eight CUs without sharing a CU, each
-// solver behind another L2, and eight lanes cost the chip-wide kernels no more CUs than one.
+// CU 0 of every XCD, and lane l's solver is launched so that it runs on XCD l (tsvm_c_smo_solve_block_on_xcd: eight
+// workgroups, one per XCD, the one on XCD l solves, the others leave at once).  The lanes thus share the eight CUs
+// without sharing a CU, each solver behind another L2.  The chip-wide streams get every CU but those the solvers
+// really run on, CU 0 of XCDs 0 .. n_lanes-1: 255 CUs for one lane, 248 for eight.  (On the CUs the two masks share,
+// a solver launch's seven idle workgroups wait for room like any workgroup; the solver's result is behind them only in
+// stream order, and they are gone long before it is done.)
 bool make_lane_group(int n_lanes, LaneGroup &g) {
     g.lanes.assign(n_lanes, LaneStreams());
     uint32_t small[8] = {0xffu, 0, 0, 0, 0, 0, 0, 0};
-    uint32_t big[8] = {~0xffu, ~0u, ~0u, ~0u, ~0u, ~0u, ~0u, ~0u};
+    uint32_t big[8] = {~((1u << n_lanes) - 1u), ~0u, ~0u, ~0u, ~0u, ~0u, ~0u, ~0u};   // all but CU 0 of XCDs 0 .. n_lanes-1
     bool ok = true;
     for (int l = 0; l < n_lanes && ok; ++l) {
         ok = hipExtStreamCreateWithCUMask(&g.lanes[l].solver, 8, small) == hipSuccess;
@@ -314,7 +317,7 @@ struct SolveTask::Impl {
     bool block_on_solver_cus = false;
     long long masked_key = 0;
     int masked_lane = 0;
-    int solver_xcd = -1, solver_epoch = 0;   // several lanes: the XCD this lane's solver is launched onto, launches so far
+    int solver_xcd = -1, solver_epoch = 0;   // masked streams: the XCD this lane's solver is launched onto, launches so far
     tsvm::DeviceBuffer<int> d_gate;
 
     void *k_rows = nullptr;
@@ -418,7 +421,7 @@ struct SolveTask::Impl {
         d_kws.zero();
         alone = n_lanes == 1;
         split = !solver.profile && create_split_streams(lane, n_lanes);
-        if (split && n_lanes > 1) {
+        if (split) {
             solver_xcd = lane;
             d_gate.resize(4);
             d_gate.zero();
@@ -761,7 +764,7 @@ struct SolveTask::Impl {
         solver_enqueued = std::chrono::steady_clock::now();
         next_stream_check = solver_enqueued + std::chrono::milliseconds(200);
         if (!on_one_stream && !block_on_solver_cus) TSVM_HIP_CHECK(hipStreamWaitEvent(ss, block_done, 0));
-        if (solver_xcd >= 0 && st == ss) {   // several lanes share the solver CUs: this lane's solver runs on its own XCD
+        if (solver_xcd >= 0 && st == ss) {   // on the masked solver stream: elected onto this lane's XCD
             ++solver_epoch;
             if (nu)
                 abi_check(tsvm_nu_smo_solve_block_on_xcd(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), ws_ids(), ws_size, Cp,
