@@ -282,6 +282,19 @@ int tsvm_select_working_set_folded(const double *f, const int *y, const double *
                                    const int *marked, int n_marked, int *out, int n_select, int nu, void *workspace,
                                    int again, int fold_n, int *out_folded, tsvm_stream stream);
 
+/* tsvm_update_f followed by the selection of the next working set on the updated f, in one call: what
+ * CSMOSolver::solve does at the end of one outer iteration and the start of the next (csmosolver.cpp:63-77,115-117).
+ * The result is that of tsvm_update_f(f, alpha_diff, ws_size, k_rows, row_type, slots, ld, n_cols, repeat) and then
+ * tsvm_select_working_set_again(f, y, alpha, n_cols * repeat, ...) (with out_folded != NULL: of
+ * tsvm_select_working_set_folded with again != 0 and fold_n = n_cols).  The threads that write the new f values
+ * also make the selection's first pass over the instances (keys, candidate flags, the first digit's counts), which
+ * saves one pass over the instances and one launch per outer iteration.  y and alpha hold n_cols * repeat
+ * entries; repeat <= 4; the workspace must be in the state tsvm_select_working_set_again asks for. */
+int tsvm_update_f_select(double *f, const double *alpha_diff, int ws_size, const void *k_rows, int row_type, const int *slots,
+                         int64_t ld, int64_t n_cols, int repeat, const int *y, const double *alpha, double Cp, double Cn,
+                         const int *marked, int n_marked, int *out, int n_select, int nu, void *workspace, int *out_folded,
+                         tsvm_stream stream);
+
 /* ---------------------------------------------------------------------------------------------
  * predict (kernelmatrix_kernel.cpp:110-147)
  * ------------------------------------------------------------------------------------------- */

@@ -287,6 +287,61 @@ def test_selection_with_folded_ids(n, tie_mode, nu):
         prev = got if it == 0 else np.concatenate([prev[q:], got])
 
 
+@pytest.mark.parametrize("nu", [0, 1])
+@pytest.mark.parametrize("row_type", [capi.ROW_F64, capi.ROW_F32])
+@pytest.mark.parametrize("n_cols,repeat,ws,ld_pad,tie_mode", [(1, 1, 1, 0, 0), (700, 1, 512, 3, 0), (4099, 2, 64, 1, 2),
+                                                             (300001, 1, 1024, 7, 0), (270000, 2, 200, 0, 0),
+                                                             (262144, 1, 1024, 0, 1), (150000, 3, 16, 4, 2)])
+def test_update_f_with_the_next_selection(n_cols, repeat, ws, ld_pad, tie_mode, row_type, nu):
+    """One call that updates f and selects the next working set on the new values: f as the oracle's update_f leaves
+    it, the ids as the oracle's selection on that f, with the half of the previous set that stays excluded.  Two such
+    calls in a row on one workspace; with tie_mode 1 and 2 the update changes nothing (all alpha_diff zero), so that
+    the selection meets massive ties and few distinct values."""
+    n = n_cols * repeat
+    rng = np.random.default_rng(n + ws + nu)
+    ld = n_cols + ld_pad
+    k = rng.random((ws, ld))
+    if row_type == capi.ROW_F32:
+        k = k.astype(np.float32)
+    k64 = np.ascontiguousarray(np.concatenate([k.astype(np.float64)[:, :n_cols]] * repeat, axis=1))
+    sel = min(1024, 1 << (n.bit_length() - 1))
+    q = max(sel // 2, 1)
+    f, y, alpha, C, _ = _select_case(n, q, 0, 3 * n + 1, tie_mode, nu)
+    f_d, y_d, a_d, k_d = G.dev(f), G.dev(y), G.dev(alpha), G.dev(k)
+    wsp = torch.empty(capi.kernel_lib().tsvm_select_workspace(n), dtype=torch.uint8, device="cuda")
+    wsp.random_(0, 256)
+    out_d = torch.full((sel,), -7, dtype=torch.int32, device="cuda")
+    capi.call("tsvm_select_working_set", G.ptr(f_d), G.ptr(y_d), G.ptr(a_d), n, C, C, None, 0, G.ptr(out_d), sel, nu, G.ptr(wsp),
+              G.stream())
+    prev = G.host(out_d)
+    assert np.array_equal(prev, O.select_working_set(f, y, alpha, C, C, np.zeros(0, dtype=np.int32), sel, nu=bool(nu)))
+    for call in range(2):
+        marked = np.ascontiguousarray(prev[sel - q:]) if sel > 1 else np.zeros(0, dtype=np.int32)
+        marked = marked[marked >= 0]
+        ad = rng.standard_normal(ws)
+        ad[rng.random(ws) < 0.4] = 0
+        if tie_mode:
+            ad[:] = 0
+        f = O.update_f(f, ad, k64, n)
+        want = O.select_working_set(f, y, alpha, C, C, marked, q, nu=bool(nu))
+        ad_d, m_d = G.dev(ad), G.dev(marked if len(marked) else np.zeros(1, dtype=np.int32))
+        new_d = torch.full((q,), -7, dtype=torch.int32, device="cuda")
+        folded_d = torch.full((q,), -7, dtype=torch.int32, device="cuda")
+        capi.call("tsvm_update_f_select", G.ptr(f_d), G.ptr(ad_d), ws, G.ptr(k_d), row_type, None, ld, n_cols, repeat, G.ptr(y_d),
+                  G.ptr(a_d), C, C, G.ptr(m_d) if len(marked) else None, len(marked), G.ptr(new_d), q, nu, G.ptr(wsp),
+                  G.ptr(folded_d) if repeat > 1 else None, G.stream())
+        assert np.array_equal(G.host(f_d), f)
+        got = G.host(new_d)
+        assert np.array_equal(got, want), "call %d: first mismatch at %s" % (call, np.flatnonzero(got != want)[:5])
+        if repeat > 1:
+            assert np.array_equal(G.host(folded_d), np.where(want >= 0, want % n_cols, -1))
+        prev = np.concatenate([prev[q:], got]) if sel > 1 else got
+        # the instances change their state between the calls, as the local solver would change them
+        alpha = alpha.copy()
+        alpha[rng.integers(0, n, size=min(n, 300))] = rng.choice([0.0, C, 0.5 * C], size=min(n, 300))
+        a_d = G.dev(alpha)
+
+
 def test_empty_inputs_are_no_ops():
     """Zero rows, zero columns, an empty working set, nothing to select: every entry point returns success and
     leaves its outputs untouched."""

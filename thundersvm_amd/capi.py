@@ -58,6 +58,7 @@ SIGNATURES = {
     "tsvm_select_working_set": (_int, [_p, _p, _p, _i64, _dbl, _dbl, _p, _int, _p, _int, _int, _p, _p]),
     "tsvm_select_working_set_again": (_int, [_p, _p, _p, _i64, _dbl, _dbl, _p, _int, _p, _int, _int, _p, _p]),
     "tsvm_select_working_set_folded": (_int, [_p, _p, _p, _i64, _dbl, _dbl, _p, _int, _p, _int, _int, _p, _int, _int, _p, _p]),
+    "tsvm_update_f_select": (_int, [_p, _p, _int, _p, _int, _p, _i64, _i64, _int, _p, _p, _dbl, _dbl, _p, _int, _p, _int, _int, _p, _p, _p]),
     "tsvm_sum_kernel_values": (_int, [_p, _int, _p, _p, _p, _p, _int, _i64, _p, _int, _i64, _p]),
 }
 

@@ -12,104 +12,6 @@
 #define MAX_WS 1024
 
 // ------------------------------------------------------------------------------------------------
-// update_f: f[j] -= sum_t alpha_diff[t] * K_t[j]  (smo_kernel.cpp:300-319)
-// Bandwidth-bound stream over the ws x n kernel rows.  The non-zero alpha_diff entries are
-// compacted (in order) into LDS once per workgroup; rows with alpha_diff == 0 are never read.
-// Each thread owns one to four adjacent columns and keeps 8 to 32 row loads in flight.  On the vector-load
-// path the columns are dealt evenly to a number of workgroups that is a multiple of 248 (every CU, or every
-// CU left to a stream that leaves one CU per XCD to the local solver, gets the same number of workgroups):
-// with a grid of full 256-thread workgroups some CUs stream 2 and others 1, and the launch lasts as long as
-// the busiest one.
-// ------------------------------------------------------------------------------------------------
-#define UF_T 256
-#define UF_CHUNK 1024
-
-// TK: element type of the kernel rows; COLS columns per thread (consecutive, loaded as one vector of
-// COLS elements); UNROLL rows in flight.  Rows are n columns wide and f holds `repeat` stacked copies
-// of the n columns, each of which receives the same sum.
-template <typename TK, int COLS, int UNROLL>
-__global__ __launch_bounds__(UF_T) void update_f_kernel(double *__restrict__ f, const double *__restrict__ alpha_diff,
-                                                        int ws, const TK *__restrict__ k_rows,
-                                                        const int *__restrict__ slots, int64_t ld, int64_t n, int repeat,
-                                                        int vec_per_wg) {
-    typedef TK vec_t __attribute__((ext_vector_type(COLS)));
-    __shared__ double s_ad[UF_CHUNK];
-    __shared__ int64_t s_off[UF_CHUNK];
-    __shared__ int s_wave_cnt[UF_T / 64];
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
-    const int64_t j = ((int64_t) blockIdx.x * vec_per_wg + tid) * COLS;
-    const bool act = tid < vec_per_wg && j < n;   // a vector may reach past n, but never past the padded row (checked by the launcher)
-    double sum[COLS];
-#pragma unroll
-    for (int c = 0; c < COLS; ++c) sum[c] = 0.0;
-    for (int base = 0; base < ws; base += UF_CHUNK) {
-        // ordered compaction of this chunk's non-zero entries: thread t owns entries 4t..4t+3
-        double v[4];
-        int cnt = 0;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int t = base + tid * 4 + e;
-            v[e] = t < ws ? alpha_diff[t] : 0.0;
-            cnt += (v[e] != 0.0);
-        }
-        int incl = cnt;
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-            int o = __shfl_up(incl, d, 64);
-            if (lane >= d) incl += o;
-        }
-        if (lane == 63) s_wave_cnt[wave] = incl;
-        __syncthreads();
-        int wave_base = 0, total = 0;
-#pragma unroll
-        for (int w = 0; w < UF_T / 64; ++w) {
-            if (w < wave) wave_base += s_wave_cnt[w];
-            total += s_wave_cnt[w];
-        }
-        int pos = wave_base + incl - cnt;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            if (v[e] != 0.0) {
-                const int t = base + tid * 4 + e;
-                s_ad[pos] = v[e];
-                s_off[pos] = (int64_t) (slots ? slots[t] : t) * ld;
-                ++pos;
-            }
-        }
-        __syncthreads();
-        if (act) {
-            int u = 0;
-            for (; u + UNROLL <= total; u += UNROLL) {
-                vec_t k[UNROLL];
-#pragma unroll
-                for (int e = 0; e < UNROLL; ++e) k[e] = load_streaming((const vec_t *) (k_rows + s_off[u + e] + j));
-#pragma unroll
-                for (int e = 0; e < UNROLL; ++e) {
-                    const double ad = s_ad[u + e];
-#pragma unroll
-                    for (int c = 0; c < COLS; ++c) sum[c] = __builtin_fma(ad, (double) k[e][c], sum[c]);
-                }
-            }
-            for (; u < total; ++u) {
-                const vec_t k = load_streaming((const vec_t *) (k_rows + s_off[u] + j));
-                const double ad = s_ad[u];
-#pragma unroll
-                for (int c = 0; c < COLS; ++c) sum[c] = __builtin_fma(ad, (double) k[c], sum[c]);
-            }
-        }
-        __syncthreads();
-    }
-    if (act) {
-        for (int r = 0; r < repeat; ++r) {
-#pragma unroll
-            for (int c = 0; c < COLS; ++c)
-                if (j + c < n) f[(int64_t) r * n + j + c] -= sum[c];
-        }
-    }
-}
-
-// ------------------------------------------------------------------------------------------------
 // Fused sort_f + select_working_set.
 //
 // The reference sorts (f, index) pairs ascending (smo_kernel.cpp:321-332) and then walks the
@@ -307,6 +209,21 @@ __device__ void sel_advance_state(const SelWorkspace &w, const SelGeom &g, int p
     __syncthreads();
 }
 
+// One count for `bin` from every lane with `valid` set, added to the LDS histogram h with one atomic per distinct
+// bin of the wavefront instead of one per lane: the first digit of f (sign and exponent) is the same for most
+// instances, and atomics of 64 lanes on one LDS word are carried out one after the other.  May be called in
+// divergent code: only the lanes that call take part.
+__device__ __forceinline__ void sel_hist_add_wave(uint32_t *h, bool valid, uint32_t bin) {
+    uint64_t todo = __ballot(valid);
+    while (todo) {
+        const int leader = __builtin_ctzll(todo);
+        const uint32_t b = (uint32_t) __builtin_amdgcn_readlane((int) bin, leader);
+        const uint64_t same = __ballot(valid && bin == b);
+        if ((int) (threadIdx.x & 63) == leader) atomicAdd(&h[b], (uint32_t) __popcll(same));
+        todo &= ~same;
+    }
+}
+
 // One candidate's contribution to the histograms of digit p: on every undecided side it belongs to, if it
 // matches that side's prefix.
 __device__ __forceinline__ void sel_count(const SelGeom &g, const SelState *st, uint32_t (*lhist)[SEL_BINS], int p,
@@ -319,6 +236,201 @@ __device__ __forceinline__ void sel_count(const SelGeom &g, const SelState *st, 
         if (sel_cmp_prefix(k2, i2, st[s], p, g.idx_bits) != 0) continue;
         const uint32_t dg = is_key ? (uint32_t) (k2 >> shift) & dmask : (i2 >> shift) & dmask;
         atomicAdd(&lhist[s][dg], 1u);
+    }
+}
+
+// Side membership of an unmarked instance (csmosolver.cpp:133-159, nusmosolver.cpp:60-115).
+__device__ __forceinline__ uint32_t sel_flags(double a, double yy, double Cp, double Cn, int n_sides) {
+    const bool up = is_I_up(a, yy, Cp, Cn), low = is_I_low(a, yy, Cp, Cn);
+    if (n_sides == 2) return (up ? 1u : 0u) | (low ? 2u : 0u);
+    return ((up && yy > 0) ? 1u : 0u) | ((up && yy < 0) ? 2u : 0u) | ((low && yy > 0) ? 4u : 0u) | ((low && yy < 0) ? 8u : 0u);
+}
+
+// What the selection's first pass needs besides f when update_f makes it (NS sides; see update_f_kernel).
+struct SelFuse {
+    SelWorkspace w;
+    SelGeom g;
+    const int *y;
+    const double *alpha;
+    double Cp, Cn;
+    const int *marked;
+    int n_marked;
+};
+
+// ------------------------------------------------------------------------------------------------
+// update_f: f[j] -= sum_t alpha_diff[t] * K_t[j]  (smo_kernel.cpp:300-319)
+// Bandwidth-bound stream over the ws x n kernel rows.  The non-zero alpha_diff entries are
+// compacted (in order) into LDS once per workgroup; rows with alpha_diff == 0 are never read.
+// Each thread owns one to four adjacent columns and keeps 8 to 32 row loads in flight.  On the vector-load
+// path the columns are dealt evenly to a number of workgroups that is a multiple of 248 (every CU, or every
+// CU left to a stream that leaves one CU per XCD to the local solver, gets the same number of workgroups):
+// with a grid of full 256-thread workgroups some CUs stream 2 and others 1, and the launch lasts as long as
+// the busiest one.
+// ------------------------------------------------------------------------------------------------
+#define UF_T 256
+#define UF_CHUNK 1024
+
+// TK: element type of the kernel rows; COLS columns per thread (consecutive, loaded as one vector of
+// COLS elements); UNROLL rows in flight.  Rows are n columns wide and f holds `repeat` stacked copies
+// of the n columns, each of which receives the same sum.
+//
+// NS > 0: the kernel also makes the first pass of the working-set selection that follows on the updated f, over
+// the n * repeat stacked instances and NS sides (what sel_pass_kernel does for digit 0: keys, side flags, the
+// first digit's histogram, the state before it), while each new f value is still in a register.  The instances
+// of the kept half of the working set (sf.marked) that fall among a workgroup's columns are a bit field in LDS.
+#define UF_MAX_REPEAT 4
+template <typename TK, int COLS, int UNROLL, int NS>
+__global__ __launch_bounds__(UF_T) void update_f_kernel(double *__restrict__ f, const double *__restrict__ alpha_diff,
+                                                        int ws, const TK *__restrict__ k_rows,
+                                                        const int *__restrict__ slots, int64_t ld, int64_t n, int repeat,
+                                                        int vec_per_wg, SelFuse sf) {
+    typedef TK vec_t __attribute__((ext_vector_type(COLS)));
+    __shared__ uint32_t lhist[NS > 0 ? NS : 1][NS > 0 ? SEL_BINS : 1];
+    __shared__ uint32_t mark_bits[NS > 0 ? UF_MAX_REPEAT : 1][NS > 0 ? UF_T * 4 / 32 : 1];   // a workgroup owns at most UF_T * COLS <= 1024 columns
+    __shared__ double s_ad[UF_CHUNK];
+    __shared__ int64_t s_off[UF_CHUNK];
+    __shared__ int s_wave_cnt[UF_T / 64];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int64_t j = ((int64_t) blockIdx.x * vec_per_wg + tid) * COLS;
+    const bool act = tid < vec_per_wg && j < n;   // a vector may reach past n, but never past the padded row (checked by the launcher)
+    double sum[COLS];
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) sum[c] = 0.0;
+    const int64_t col_lo = (int64_t) blockIdx.x * vec_per_wg * COLS;
+    if (NS > 0) {
+        for (int e = tid; e < NS * SEL_BINS; e += UF_T) (&lhist[0][0])[e] = 0;
+        for (int e = tid; e < UF_MAX_REPEAT * (UF_T * 4 / 32); e += UF_T) (&mark_bits[0][0])[e] = 0;
+        if (blockIdx.x == 0 && tid < NS) {
+            SelState s0;
+            s0.pk = 0; s0.pi = 0; s0.k_rem = sf.g.k; s0.done = 0; s0.pad = 0;
+            sf.w.state[tid] = s0;   // the state before digit 0, for the next pass
+        }
+        __syncthreads();
+        const int64_t col_hi = col_lo + (int64_t) vec_per_wg * COLS;
+        for (int i = tid; i < sf.n_marked; i += UF_T) {
+            const int64_t id = sf.marked[i];
+            for (int r = 0; r < repeat; ++r) {
+                const int64_t c = id - r * n;   // column, if the id lies in copy r
+                if (c >= col_lo && c < col_hi && c < n) atomicOr(&mark_bits[r][(c - col_lo) >> 5], 1u << ((c - col_lo) & 31));
+            }
+        }
+        // (the barriers of the loop below, or the one before the epilogue, order these writes before their readers)
+    }
+    for (int base = 0; base < ws; base += UF_CHUNK) {
+        // ordered compaction of this chunk's non-zero entries: thread t owns entries 4t..4t+3
+        double v[4];
+        int cnt = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int t = base + tid * 4 + e;
+            v[e] = t < ws ? alpha_diff[t] : 0.0;
+            cnt += (v[e] != 0.0);
+        }
+        int incl = cnt;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            int o = __shfl_up(incl, d, 64);
+            if (lane >= d) incl += o;
+        }
+        if (lane == 63) s_wave_cnt[wave] = incl;
+        __syncthreads();
+        int wave_base = 0, total = 0;
+#pragma unroll
+        for (int w = 0; w < UF_T / 64; ++w) {
+            if (w < wave) wave_base += s_wave_cnt[w];
+            total += s_wave_cnt[w];
+        }
+        int pos = wave_base + incl - cnt;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (v[e] != 0.0) {
+                const int t = base + tid * 4 + e;
+                s_ad[pos] = v[e];
+                s_off[pos] = (int64_t) (slots ? slots[t] : t) * ld;
+                ++pos;
+            }
+        }
+        __syncthreads();
+        if (act) {
+            int u = 0;
+            for (; u + UNROLL <= total; u += UNROLL) {
+                vec_t k[UNROLL];
+#pragma unroll
+                for (int e = 0; e < UNROLL; ++e) k[e] = load_streaming((const vec_t *) (k_rows + s_off[u + e] + j));
+#pragma unroll
+                for (int e = 0; e < UNROLL; ++e) {
+                    const double ad = s_ad[u + e];
+#pragma unroll
+                    for (int c = 0; c < COLS; ++c) sum[c] = __builtin_fma(ad, (double) k[e][c], sum[c]);
+                }
+            }
+            for (; u < total; ++u) {
+                const vec_t k = load_streaming((const vec_t *) (k_rows + s_off[u] + j));
+                const double ad = s_ad[u];
+#pragma unroll
+                for (int c = 0; c < COLS; ++c) sum[c] = __builtin_fma(ad, (double) k[c], sum[c]);
+            }
+        }
+        __syncthreads();
+    }
+    if (NS == 0) {
+        if (act) {
+            for (int r = 0; r < repeat; ++r) {
+#pragma unroll
+                for (int c = 0; c < COLS; ++c)
+                    if (j + c < n) f[(int64_t) r * n + j + c] -= sum[c];
+            }
+        }
+        return;
+    }
+    __syncthreads();
+    if (act) {
+        for (int r = 0; r < repeat; ++r) {
+            const int64_t j0 = (int64_t) r * n + j;   // the first of this thread's stacked instances in copy r
+            // every load first, then the arithmetic: one memory latency for the lot
+            double fo[COLS], al[COLS];
+            int yv[COLS];
+#pragma unroll
+            for (int c = 0; c < COLS; ++c) {
+                const bool in = j + c < n;
+                fo[c] = in ? f[j0 + c] : 0.0;
+                al[c] = in ? sf.alpha[j0 + c] : 0.0;
+                yv[c] = in ? sf.y[j0 + c] : 1;
+            }
+            uint32_t fl_all = 0;
+#pragma unroll
+            for (int c = 0; c < COLS; ++c) {
+                const bool in = j + c < n;
+                const double fn = fo[c] - sum[c];
+                const uint64_t key = f_to_key(fn);
+                const int bit = (int) (j + c - col_lo);
+                uint32_t fl = 0;
+                if (in && !((mark_bits[r][bit >> 5] >> (bit & 31)) & 1u)) fl = sel_flags(al[c], (double) yv[c], sf.Cp, sf.Cn, NS);
+                if (in) {
+                    f[j0 + c] = fn;
+                    sf.w.keys[j0 + c] = key;
+                }
+                fl_all |= fl << (8 * c);
+#pragma unroll
+                for (int s = 0; s < NS; ++s) {
+                    const uint64_t k2 = sel_side_descending(s, NS) ? ~key : key;
+                    sel_hist_add_wave(lhist[s], (fl >> s) & 1u, (uint32_t) (k2 >> (64 - SEL_DIGIT)));   // digit 0: the key's top bits
+                }
+            }
+            if (COLS == 4 && (j0 & 3) == 0 && j + COLS <= n) {
+                *(uint32_t *) (sf.w.flags + j0) = fl_all;   // four flag bytes at once
+            } else {
+#pragma unroll
+                for (int c = 0; c < COLS; ++c)
+                    if (j + c < n) sf.w.flags[j0 + c] = (uint8_t) (fl_all >> (8 * c));
+            }
+        }
+    }
+    __syncthreads();
+    for (int e = tid; e < NS * SEL_BINS; e += UF_T) {
+        const uint32_t c = (&lhist[0][0])[e];
+        if (c) atomicAdd(&sf.w.hist[e], c);   // hist[0][s][bin], s < NS
     }
 }
 
@@ -370,15 +482,7 @@ __global__ __launch_bounds__(SEL_T) void sel_pass_kernel(SelWorkspace w, const d
             const double yy = (double) y[j];
             const uint64_t key = f_to_key(f[j]);
             uint32_t fl = 0;
-            if (!((mark_bits[(j - lo) >> 5] >> ((j - lo) & 31)) & 1u)) {
-                const bool up = is_I_up(a, yy, Cp, Cn), low = is_I_low(a, yy, Cp, Cn);
-                if (g.n_sides == 2) {
-                    fl = (up ? 1u : 0u) | (low ? 2u : 0u);
-                } else {
-                    fl = ((up && yy > 0) ? 1u : 0u) | ((up && yy < 0) ? 2u : 0u) | ((low && yy > 0) ? 4u : 0u) |
-                         ((low && yy < 0) ? 8u : 0u);
-                }
-            }
+            if (!((mark_bits[(j - lo) >> 5] >> ((j - lo) & 31)) & 1u)) fl = sel_flags(a, yy, Cp, Cn, g.n_sides);
             w.keys[j] = key;
             w.flags[j] = (uint8_t) fl;
             sel_count(g, st, lhist, p, is_key, shift, dmask, key, fl, j);
@@ -624,9 +728,9 @@ __global__ __launch_bounds__(MAX_WS) void sel_final_kernel(SelWorkspace w, int64
 // ------------------------------------------------------------------------------------------------
 // C ABI
 // ------------------------------------------------------------------------------------------------
-template <typename TK, int COLS, int UNROLL>
+template <typename TK, int COLS, int UNROLL, int NS>
 static void launch_update_f(double *f, const double *alpha_diff, int ws_size, const void *k_rows, const int *slots,
-                            int64_t ld, int64_t n, int repeat, hipStream_t s) {
+                            int64_t ld, int64_t n, int repeat, const SelFuse &sf, hipStream_t s) {
     const int64_t vecs = (n + COLS - 1) / COLS;                        // column vectors, one per thread
     int64_t grid = (vecs + UF_T - 1) / UF_T;
     int vec_per_wg = UF_T;
@@ -637,24 +741,28 @@ static void launch_update_f(double *f, const double *alpha_diff, int ws_size, co
         grid = 248 * per_cu;
         vec_per_wg = (int) ((vecs + grid - 1) / grid);
     }
-    hipLaunchKernelGGL((update_f_kernel<TK, COLS, UNROLL>), dim3((unsigned) grid), dim3(UF_T), 0, s, f, alpha_diff, ws_size,
-                       (const TK *) k_rows, slots, ld, n, repeat, vec_per_wg);
+    hipLaunchKernelGGL((update_f_kernel<TK, COLS, UNROLL, NS>), dim3((unsigned) grid), dim3(UF_T), 0, s, f, alpha_diff, ws_size,
+                       (const TK *) k_rows, slots, ld, n, repeat, vec_per_wg, sf);
 }
 
-static int select_working_set(const double *f, const int *y, const double *alpha, int64_t n, double Cp, double Cn,
-                              const int *marked, int n_marked, int *out, int n_select, int nu, void *workspace,
-                              bool armed, int fold_n, int *out_folded, tsvm_stream stream) {
-    TSVM_REQUIRE(f && y && alpha && out && workspace, "tsvm_select_working_set: null pointer");
-    TSVM_REQUIRE(n >= 1 && n <= 0x7fffffffLL, "tsvm_select_working_set: n %lld outside [1, 2^31)", (long long) n);
-    TSVM_REQUIRE(n_select >= 0 && n_select <= MAX_WS, "tsvm_select_working_set: n_select %d outside [0, %d]", n_select,
-                 MAX_WS);
-    TSVM_REQUIRE(n_marked >= 0 && (n_marked == 0 || marked), "tsvm_select_working_set: bad marked list");
-    TSVM_REQUIRE(fold_n >= 0 && (fold_n == 0 || out_folded), "tsvm_select_working_set: bad fold arguments");
-    if (n_select == 0) return 0;
-    hipStream_t s = tsvm_s(stream);
-    SelWorkspace w;
-    void *base = (void *) (((uintptr_t) workspace + 255) & ~(uintptr_t) 255);
-    sel_carve(base, n, &w);
+// The variant of the kernel for the row type, alignment and size at hand.
+template <int NS>
+static void dispatch_update_f(double *f, const double *alpha_diff, int ws_size, const void *k_rows, int row_type, const int *slots,
+                              int64_t ld, int64_t n, int repeat, const SelFuse &sf, hipStream_t s) {
+    // 16-byte loads need every row start 16-byte aligned and the last vector inside the padded row; with few
+    // columns one column per thread and more rows in flight keeps more of the chip busy
+    const bool big = n >= (int64_t) UF_T * 1024;
+    const bool aligned = (uintptr_t) k_rows % 16 == 0;
+    if (row_type == TSVM_ROW_F32) {
+        if (big && aligned && ld % 4 == 0 && ld >= (n + 3) / 4 * 4) launch_update_f<float, 4, 8, NS>(f, alpha_diff, ws_size, k_rows, slots, ld, n, repeat, sf, s);
+        else launch_update_f<float, 1, 32, NS>(f, alpha_diff, ws_size, k_rows, slots, ld, n, repeat, sf, s);
+    } else {
+        if (big && aligned && ld % 2 == 0 && ld >= (n + 1) / 2 * 2) launch_update_f<double, 2, 8, NS>(f, alpha_diff, ws_size, k_rows, slots, ld, n, repeat, sf, s);
+        else launch_update_f<double, 1, 16, NS>(f, alpha_diff, ws_size, k_rows, slots, ld, n, repeat, sf, s);
+    }
+}
+
+static SelGeom sel_geom(int64_t n, int n_select, int nu) {
     SelGeom g;
     g.n_sides = nu ? 4 : 2;
     int bits = 1;
@@ -663,6 +771,29 @@ static int select_working_set(const double *f, const int *y, const double *alpha
     g.idx_mask = (uint32_t) (((uint64_t) 1 << bits) - 1);
     g.n_pass = 6 + (bits + SEL_DIGIT - 1) / SEL_DIGIT;
     g.k = (uint32_t) n_select;
+    return g;
+}
+
+static SelWorkspace sel_workspace(void *workspace, int64_t n) {
+    SelWorkspace w;
+    sel_carve((void *) (((uintptr_t) workspace + 255) & ~(uintptr_t) 255), n, &w);
+    return w;
+}
+
+// first_pass 1: digit 0 has been counted already, by update_f_kernel, on a workspace left by an earlier selection
+static int select_working_set(const double *f, const int *y, const double *alpha, int64_t n, double Cp, double Cn,
+                              const int *marked, int n_marked, int *out, int n_select, int nu, void *workspace,
+                              bool armed, int fold_n, int *out_folded, int first_pass, tsvm_stream stream) {
+    TSVM_REQUIRE(f && y && alpha && out && workspace, "tsvm_select_working_set: null pointer");
+    TSVM_REQUIRE(n >= 1 && n <= 0x7fffffffLL, "tsvm_select_working_set: n %lld outside [1, 2^31)", (long long) n);
+    TSVM_REQUIRE(n_select >= 0 && n_select <= MAX_WS, "tsvm_select_working_set: n_select %d outside [0, %d]", n_select,
+                 MAX_WS);
+    TSVM_REQUIRE(n_marked >= 0 && (n_marked == 0 || marked), "tsvm_select_working_set: bad marked list");
+    TSVM_REQUIRE(fold_n >= 0 && (fold_n == 0 || out_folded), "tsvm_select_working_set: bad fold arguments");
+    if (n_select == 0) return 0;
+    hipStream_t s = tsvm_s(stream);
+    const SelWorkspace w = sel_workspace(workspace, n);
+    const SelGeom g = sel_geom(n, n_select, nu);
     // The first three digits (33 bits of f) are counted by the whole chip, the rest (rarely needed) by one
     // workgroup.  Near convergence the free support vectors crowd within epsilon of the threshold, so the third
     // digit is usually the one that separates them.
@@ -675,7 +806,7 @@ static int select_working_set(const double *f, const int *y, const double *alpha
         hipLaunchKernelGGL(sel_init_kernel, dim3(p_full * SEL_MAX_SIDES * SEL_BINS / 1024), dim3(256), 0, s, w, g, p_full);
         TSVM_LAUNCH_CHECK();
     }
-    for (int p = 0; p < p_full; ++p) {
+    for (int p = first_pass; p < p_full; ++p) {
         hipLaunchKernelGGL(sel_pass_kernel, dim3(grid), dim3(SEL_T), 0, s, w, f, y, alpha, n, Cp, Cn, g, p, marked, n_marked);
         TSVM_LAUNCH_CHECK();
     }
@@ -695,21 +826,34 @@ int tsvm_update_f(double *f, const double *alpha_diff, int ws_size, const void *
                  ws_size, (long long) n_cols, (long long) ld);
     TSVM_REQUIRE(row_type == TSVM_ROW_F64 || row_type == TSVM_ROW_F32, "tsvm_update_f: unknown row type %d", row_type);
     if (n_cols == 0 || ws_size == 0) return 0;
-    const int64_t n = n_cols;
-    hipStream_t s = tsvm_s(stream);
-    // 16-byte loads need every row start 16-byte aligned and the last vector inside the padded row; with few
-    // columns one column per thread and more rows in flight keeps more of the chip busy
-    const bool big = n >= (int64_t) UF_T * 1024;
-    const bool aligned = (uintptr_t) k_rows % 16 == 0;
-    if (row_type == TSVM_ROW_F32) {
-        if (big && aligned && ld % 4 == 0 && ld >= (n + 3) / 4 * 4) launch_update_f<float, 4, 8>(f, alpha_diff, ws_size, k_rows, slots, ld, n, repeat, s);
-        else launch_update_f<float, 1, 32>(f, alpha_diff, ws_size, k_rows, slots, ld, n, repeat, s);
-    } else {
-        if (big && aligned && ld % 2 == 0 && ld >= (n + 1) / 2 * 2) launch_update_f<double, 2, 8>(f, alpha_diff, ws_size, k_rows, slots, ld, n, repeat, s);
-        else launch_update_f<double, 1, 16>(f, alpha_diff, ws_size, k_rows, slots, ld, n, repeat, s);
-    }
+    dispatch_update_f<0>(f, alpha_diff, ws_size, k_rows, row_type, slots, ld, n_cols, repeat, SelFuse(), tsvm_s(stream));
     TSVM_LAUNCH_CHECK();
     return 0;
+}
+
+int tsvm_update_f_select(double *f, const double *alpha_diff, int ws_size, const void *k_rows, int row_type, const int *slots,
+                         int64_t ld, int64_t n_cols, int repeat, const int *y, const double *alpha, double Cp, double Cn,
+                         const int *marked, int n_marked, int *out, int n_select, int nu, void *workspace, int *out_folded,
+                         tsvm_stream stream) {
+    TSVM_REQUIRE(f && alpha_diff && k_rows, "tsvm_update_f_select: null pointer");
+    TSVM_REQUIRE(ws_size >= 0 && n_cols >= 1 && ld >= n_cols && repeat >= 1 && repeat <= UF_MAX_REPEAT,
+                 "tsvm_update_f_select: bad size (ws=%d n=%lld ld=%lld repeat=%d)", ws_size, (long long) n_cols, (long long) ld, repeat);
+    TSVM_REQUIRE(row_type == TSVM_ROW_F64 || row_type == TSVM_ROW_F32, "tsvm_update_f_select: unknown row type %d", row_type);
+    TSVM_REQUIRE(y && alpha && out && workspace, "tsvm_update_f_select: null pointer");
+    TSVM_REQUIRE(n_select >= 1 && n_select <= MAX_WS, "tsvm_update_f_select: n_select %d outside [1, %d]", n_select, MAX_WS);
+    TSVM_REQUIRE(n_marked >= 0 && (n_marked == 0 || marked), "tsvm_update_f_select: bad marked list");
+    const int64_t n = n_cols * repeat;
+    TSVM_REQUIRE(n <= 0x7fffffffLL, "tsvm_update_f_select: %lld instances, at most 2^31 - 1", (long long) n);
+    SelFuse sf;
+    sf.w = sel_workspace(workspace, n);
+    sf.g = sel_geom(n, n_select, nu);
+    sf.y = y; sf.alpha = alpha; sf.Cp = Cp; sf.Cn = Cn; sf.marked = marked; sf.n_marked = n_marked;
+    hipStream_t s = tsvm_s(stream);
+    if (nu) dispatch_update_f<4>(f, alpha_diff, ws_size, k_rows, row_type, slots, ld, n_cols, repeat, sf, s);
+    else dispatch_update_f<2>(f, alpha_diff, ws_size, k_rows, row_type, slots, ld, n_cols, repeat, sf, s);
+    TSVM_LAUNCH_CHECK();
+    return select_working_set(f, y, alpha, n, Cp, Cn, marked, n_marked, out, n_select, nu, workspace, true,
+                              out_folded ? (int) n_cols : 0, out_folded, 1, stream);
 }
 
 size_t tsvm_select_workspace(int64_t n) {
@@ -720,13 +864,13 @@ size_t tsvm_select_workspace(int64_t n) {
 int tsvm_select_working_set(const double *f, const int *y, const double *alpha, int64_t n, double Cp, double Cn,
                             const int *marked, int n_marked, int *out, int n_select, int nu, void *workspace,
                             tsvm_stream stream) {
-    return select_working_set(f, y, alpha, n, Cp, Cn, marked, n_marked, out, n_select, nu, workspace, false, 0, nullptr, stream);
+    return select_working_set(f, y, alpha, n, Cp, Cn, marked, n_marked, out, n_select, nu, workspace, false, 0, nullptr, 0, stream);
 }
 
 int tsvm_select_working_set_again(const double *f, const int *y, const double *alpha, int64_t n, double Cp, double Cn,
                                   const int *marked, int n_marked, int *out, int n_select, int nu, void *workspace,
                                   tsvm_stream stream) {
-    return select_working_set(f, y, alpha, n, Cp, Cn, marked, n_marked, out, n_select, nu, workspace, true, 0, nullptr, stream);
+    return select_working_set(f, y, alpha, n, Cp, Cn, marked, n_marked, out, n_select, nu, workspace, true, 0, nullptr, 0, stream);
 }
 
 int tsvm_select_working_set_folded(const double *f, const int *y, const double *alpha, int64_t n, double Cp, double Cn,
@@ -734,7 +878,7 @@ int tsvm_select_working_set_folded(const double *f, const int *y, const double *
                                    int again, int fold_n, int *out_folded, tsvm_stream stream) {
     TSVM_REQUIRE(fold_n >= 1, "tsvm_select_working_set_folded: fold_n %d < 1", fold_n);
     return select_working_set(f, y, alpha, n, Cp, Cn, marked, n_marked, out, n_select, nu, workspace, again != 0, fold_n, out_folded,
-                              stream);
+                              0, stream);
 }
 
 }  // extern "C"

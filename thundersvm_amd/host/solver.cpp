@@ -397,6 +397,7 @@ struct SolveTask::Impl {
     float_type previous_local_diff = INFINITY, last_local_diff = INFINITY, second_last_local_diff = INFINITY;
     PhaseTimer timer;
     bool select_ahead = false, block_first = false, select_enqueued = false;
+    bool fuse_select = false;   // update_f also makes the first pass of the selection that follows
     int iter = 0;
 
     Impl(const CSMOSolver &solver, const KernelMatrix &k_mat, const std::vector<int> &y, std::vector<float_type> &alpha,
@@ -500,6 +501,9 @@ struct SolveTask::Impl {
         // straight from update_f into it; if the diff then says stop, that selection was simply not needed.
         // (Not when tracing, which reads the working set back after each iteration, nor when profiling.)
         select_ahead = !solver.trace && !solver.profile;
+        // With stacked copies (SVR) a thread of update_f has twice the instances to classify after its rows have
+        // streamed by, each behind memory reads that wait on a saturated HBM: measured slower than the separate pass.
+        fuse_select = rep == 1;
         // The solver reads the ws x ws block of the kernel matrix.  With few features the block is cheap to
         // compute on its own, without the stored rows, so it and the solver can be enqueued before the host
         // does the cache bookkeeping.  With many features that small launch (64 workgroups walking the whole
@@ -575,22 +579,25 @@ struct SolveTask::Impl {
 
     // Working-set selection of iteration `it`: the first one picks ws_size ids, later ones keep the last
     // half of the previous set and pick q new ids (csmosolver.cpp:63-77).
+    // Moves the window to where the selection of iteration `it` > 0 writes: q ids further, or back to the start of
+    // the buffer with the half that stays copied in front.
+    void advance_window() {
+        int next = sel_off + q;
+        if (next + ws_size > (int) d_ws.size()) {
+            TSVM_HIP_CHECK(hipMemcpyAsync(d_ws.data(), d_ws.data() + next, sizeof(int) * q, hipMemcpyDeviceToDevice, sa));
+            if (rep > 1)
+                TSVM_HIP_CHECK(hipMemcpyAsync(d_ws_folded.data(), d_ws_folded.data() + next, sizeof(int) * q,
+                                              hipMemcpyDeviceToDevice, sa));
+            next = 0;
+        }
+        sel_off = next;
+    }
+
     void launch_select(int it) {
         const int n_sel = it == 0 ? ws_size : q;
         hipStream_t sel = sa;
-        if (it == 0) {
-            sel_off = 0;
-        } else {
-            int next = sel_off + q;
-            if (next + ws_size > (int) d_ws.size()) {
-                TSVM_HIP_CHECK(hipMemcpyAsync(d_ws.data(), d_ws.data() + next, sizeof(int) * q, hipMemcpyDeviceToDevice, sel));
-                if (rep > 1)
-                    TSVM_HIP_CHECK(hipMemcpyAsync(d_ws_folded.data(), d_ws_folded.data() + next, sizeof(int) * q,
-                                                  hipMemcpyDeviceToDevice, sel));
-                next = 0;
-            }
-            sel_off = next;
-        }
+        if (it == 0) sel_off = 0;
+        else advance_window();
         const int *kept = it == 0 ? nullptr : d_ws.data() + sel_off;            // the half that stays: no candidates
         int *out = d_ws.data() + sel_off + (it == 0 ? 0 : q);
         if (rep > 1) {
@@ -787,6 +794,15 @@ struct SolveTask::Impl {
 
     void enqueue_update() {
         if (!on_one_stream) TSVM_HIP_CHECK(hipStreamWaitEvent(sa, solved, 0));   // alpha_diff, alpha and diff come from the solver
+        if (select_ahead && fuse_select) {
+            // the next selection's first pass over the instances rides on update_f's last one
+            advance_window();
+            abi_check(tsvm_update_f_select(d_f.data(), d_alpha_diff.data(), ws_size, k_rows, row_type, slots, ld, n_u, rep,
+                                           d_y.data(), d_alpha.data(), Cp, Cn, d_ws.data() + sel_off, q, d_ws.data() + sel_off + q, q,
+                                           nu, d_sel_ws.data(), rep > 1 ? d_ws_folded.data() + sel_off + q : nullptr, sa));
+            select_enqueued = true;
+            return;
+        }
         timer.begin();
         abi_check(tsvm_update_f(d_f.data(), d_alpha_diff.data(), ws_size, k_rows, row_type, slots, ld, n_u, rep, sa));
         timer.end(stats.ms_update_f);
