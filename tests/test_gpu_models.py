@@ -33,9 +33,10 @@ def _compare(train, test, prm, ws=0, trace=8):
     gd, gw = gm.trace()
     od, ow = om.trace()
     k = min(len(gd), len(od), trace)
-    assert np.array_equal(gw[:k], ow[:k]), "working sets diverge at outer iteration %d" % np.flatnonzero(
-        (gw[:k] != ow[:k]).any(axis=1))[0]
-    assert np.array_equal(gd[:k], od[:k])
+    if k:
+        assert np.array_equal(gw[:k], ow[:k]), "working sets diverge at outer iteration %d" % np.flatnonzero(
+            (gw[:k] != ow[:k]).any(axis=1))[0]
+        assert np.array_equal(gd[:k], od[:k])
     for b in range(gm.n_binary):
         st = gm.stats(b)
         assert st["n_iter"] == om.n_iter[b] and st["local_iter"] == om.local_iter[b]
@@ -141,6 +142,60 @@ def test_sparse_multiclass(kernel):
 def test_workload_c5_small():
     w = D.workload_c5(scale=0.01)
     _compare(w["train"], w["test"], make_param(**w["params"]), trace=64)
+
+
+@pytest.mark.parametrize("wl,scale", [("c1", 1.0), ("c2", 0.03), ("c3", 0.04), ("c4", 0.01), ("c5", 0.004)])
+def test_untraced_training_matches_the_oracle(wl, scale):
+    """Without a trace the production schedule runs: the next selection is enqueued ahead of the host's look at the
+    stopping rule, update_f makes that selection's first pass, class pairs run side by side.  Same iteration counts,
+    alpha, f, rho, coefficients and decision values as the oracle."""
+    w = getattr(D, "workload_" + wl)(scale) if wl != "c1" else D.workload_c1()
+    _compare(w["train"], w["test"], make_param(**w["params"]), trace=0)
+
+
+def _csr(rows, y):
+    ptr, col, val = [0], [], []
+    for r in rows:
+        for c, v in r:
+            col.append(c)
+            val.append(v)
+        ptr.append(len(col))
+    return D.CsrData(np.array(ptr, dtype=np.int64), np.array(col, dtype=np.int32),
+                     np.array(val, dtype=np.float32).astype(np.float64), np.array(y, dtype=np.float64))
+
+
+@pytest.mark.parametrize("case", ["two_points", "empty_rows", "duplicates_with_opposite_labels", "class_of_one",
+                                  "exactly_one_working_set", "one_more_than_a_working_set", "feature_zero_only"])
+@pytest.mark.parametrize("trace", [8, 0])
+def test_degenerate_inputs(case, trace):
+    """Inputs at the edges of what the reference accepts (dataset.cpp:190-234 groups whatever labels appear;
+    kernelmatrix.cpp:183-205 takes rows without any feature): the smallest two-class problem, instances with no
+    features, identical instances with opposite labels (alpha runs into C), a class with a single instance in a
+    three-class problem, exactly one working set of instances and one more, and a data set whose only feature is
+    feature 0.  All against the oracle, traced and with the production schedule."""
+    rng = np.random.default_rng(17)
+    prm = make_param(svm_type=0, kernel_type=2, gamma=0.5, C=10)
+    if case == "two_points":
+        d = _csr([[(1, 1.0)], [(1, -1.0), (2, 0.5)]], [1, -1])
+    elif case == "empty_rows":
+        rows = [[(c, float(v)) for c, v in zip(range(1, 6), rng.standard_normal(5))] for _ in range(60)]
+        for i in (0, 7, 8, 59):
+            rows[i] = []
+        d = _csr(rows, np.where(np.arange(60) % 3 == 0, 1, -1))
+    elif case == "duplicates_with_opposite_labels":
+        base = [[(c, float(v)) for c, v in zip(range(1, 4), rng.standard_normal(3))] for _ in range(20)]
+        d = _csr(base + base, [1] * 20 + [-1] * 20)
+    elif case == "class_of_one":
+        rows = [[(c, float(v)) for c, v in zip(range(1, 5), rng.standard_normal(4) + (i % 2))] for i in range(41)]
+        d = _csr(rows, [i % 2 for i in range(40)] + [7])
+    elif case in ("exactly_one_working_set", "one_more_than_a_working_set"):
+        n = 1024 if case == "exactly_one_working_set" else 1025
+        yy = np.where(rng.random(n) < 0.5, 1, -1)
+        rows = [[(c, float(v)) for c, v in zip(range(1, 9), rng.standard_normal(8) + 0.3 * yy[i])] for i in range(n)]
+        d = _csr(rows, yy)
+    else:
+        d = _csr([[(0, float(v))] for v in rng.standard_normal(50)], np.where(np.arange(50) % 2 == 0, 1, -1))
+    _compare(d, d, prm, trace=trace)
 
 
 def test_max_iter_cap():
