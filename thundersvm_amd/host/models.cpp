@@ -1,3 +1,4 @@
+#include <chrono>
 #include "models.h"
 #include <deque>
 
@@ -340,8 +341,7 @@ void SVC::train(const DataSet &dataset, SvmParam p) {   // svc.cpp:41-145
     std::vector<char> is_sv(n, 0);
     int k = 0;
     // pairs in flight: up to eight when every pair's solver gets a CU of its own and the pairs advance independently
-    // (at most three of them large pairs, train_pairs_in_lockstep), three when the pairs alternate between a solver
-    // phase and a chip-wide phase
+    // (train_pairs_in_lockstep), three when the pairs alternate between a solver phase and a chip-wide phase
     const int lanes = std::min(pair_lanes > 0 ? pair_lanes : SolveTask::cu_split_available() ? 8 : 3, n_binary_models);
     if (lanes > 1 && !profile && !trace_first) {
         train_pairs_in_lockstep(grouped, lanes, alpha);
@@ -357,14 +357,18 @@ void SVC::train(const DataSet &dataset, SvmParam p) {   // svc.cpp:41-145
                 finish_binary(p, alpha[k]);
             }
     }
-    k = 0;
+    // (the pairs' parts of what follows are independent of one another: one host thread per pair)
+    std::vector<std::pair<int, int>> pair_of;
     for (int i = 0; i < n_classes; ++i)
-        for (int j = i + 1; j < n_classes; ++j, ++k) {
-            const std::vector<int> ids = grouped.original_index(i, j);
-            for (size_t l = 0; l < ids.size(); ++l)
-                if (alpha[k][l] != 0) is_sv[ids[l]] = 1;
-            if (keep_binary) binary_alpha.push_back(alpha[k]);
-        }
+        for (int j = i + 1; j < n_classes; ++j) pair_of.push_back({i, j});
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int kk = 0; kk < n_binary_models; ++kk) {
+        const std::vector<int> ids = grouped.original_index(pair_of[kk].first, pair_of[kk].second);
+        for (size_t l = 0; l < ids.size(); ++l)
+            if (alpha[kk][l] != 0) __atomic_store_n(&is_sv[ids[l]], (char) 1, __ATOMIC_RELAXED);   // several pairs may mark one instance
+    }
+    if (keep_binary)
+        for (int kk = 0; kk < n_binary_models; ++kk) binary_alpha.push_back(alpha[kk]);
     // support vectors class by class, in grouped order
     for (int c = 0; c < n_classes; ++c)
         for (int id : grouped.original_index(c))
@@ -379,18 +383,18 @@ void SVC::train(const DataSet &dataset, SvmParam p) {   // svc.cpp:41-145
     coef.assign((size_t) (n_classes - 1) * n_total_sv, 0);
     std::vector<int> sv_start(n_classes, 0);
     for (int c = 1; c < n_classes; ++c) sv_start[c] = sv_start[c - 1] + n_sv[c - 1];
-    k = 0;
-    for (int i = 0; i < n_classes; ++i)
-        for (int j = i + 1; j < n_classes; ++j, ++k) {
-            const std::vector<int> ids = grouped.original_index(i, j);
-            const int ci = grouped.count()[i];
-            int at = sv_start[i];
-            for (int l = 0; l < ci; ++l)
-                if (is_sv[ids[l]]) coef[(size_t) (j - 1) * n_total_sv + at++] = alpha[k][l];
-            at = sv_start[j];
-            for (size_t l = ci; l < ids.size(); ++l)
-                if (is_sv[ids[l]]) coef[(size_t) i * n_total_sv + at++] = alpha[k][l];
-        }
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int kk = 0; kk < n_binary_models; ++kk) {   // (every pair writes two segments of coef that no other pair writes)
+        const int i = pair_of[kk].first, j = pair_of[kk].second;
+        const std::vector<int> ids = grouped.original_index(i, j);
+        const int ci = grouped.count()[i];
+        int at = sv_start[i];
+        for (int l = 0; l < ci; ++l)
+            if (is_sv[ids[l]]) coef[(size_t) (j - 1) * n_total_sv + at++] = alpha[kk][l];
+        at = sv_start[j];
+        for (size_t l = ci; l < ids.size(); ++l)
+            if (is_sv[ids[l]]) coef[(size_t) i * n_total_sv + at++] = alpha[kk][l];
+    }
     if (param.kernel_type == SvmParam::LINEAR) {   // explicit w per pair (svc.cpp:111-135)
         const size_t nf = grouped.n_features();
         linear_coef.assign((size_t) n_binary_models * (grouped.is_zero_based() ? nf + 1 : nf), 0);
