@@ -59,8 +59,14 @@ static int max2power(double n) { return (int) pow(2, floor(log2f(float(n)))); } 
 // trajectory -- is the reference's wherever its memory budget starts to bind (n + n_features above ~10^6 with the
 // default 8192 MiB).  Small model members (rho, n_sv, label) are left out.
 int SvmModel::get_working_set_size(const KernelMatrix &k_mat, size_t held_bytes) {
-    if (ws_override > 0) return ws_override;
     const size_t n_instances = k_mat.n_instances(), n_features = k_mat.n_features();
+    if (ws_override > 0) {
+        // (a working set larger than the problem cannot be filled: the selection would hand out instance ids of -1)
+        if ((size_t) ws_override > n_instances)
+            throw std::invalid_argument("working-set size " + std::to_string(ws_override) + " forced on a problem of " +
+                                        std::to_string(n_instances) + " instances");
+        return ws_override;
+    }
     const size_t used = k_mat.reference_syncmem_bytes() + n_instances * (sizeof(int) + 2 * sizeof(float_type)) + held_bytes;
     if (param.max_mem_size < used) throw std::bad_alloc();
     const size_t free_mem = param.max_mem_size - used;

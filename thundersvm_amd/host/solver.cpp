@@ -407,6 +407,9 @@ struct SolveTask::Impl {
           out_max_iter(out_max_iter), n((int) k_mat.n_instances()), n_u((int) k_mat.n_columns()), rep(k_mat.repeat()),
           row_type(k_mat.row_type()), row_esz(k_mat.row_elem_size()), q(ws_size / 2), ld(((int64_t) n_u + 7) / 8 * 8),
           nu(solver.is_nu()), ldk(tsvm_smo_solve_block_ld(ws_size)), timer(solver.profile) {
+        if (ws_size < 1 || ws_size > n || ws_size > 1024)
+            throw std::invalid_argument("SolveTask: working-set size " + std::to_string(ws_size) + " for " + std::to_string(n) +
+                                        " instances (1 .. min(instances, 1024))");
         wall0 = std::chrono::steady_clock::now();
         (void) process_epoch();
         stats.ws_size = ws_size;
@@ -503,7 +506,7 @@ struct SolveTask::Impl {
         select_ahead = !solver.trace && !solver.profile;
         // With stacked copies (SVR) a thread of update_f has twice the instances to classify after its rows have
         // streamed by, each behind memory reads that wait on a saturated HBM: measured slower than the separate pass.
-        fuse_select = rep == 1;
+        fuse_select = rep == 1 && q > 0;
         // The solver reads the ws x ws block of the kernel matrix.  With few features the block is cheap to
         // compute on its own, without the stored rows, so it and the solver can be enqueued before the host
         // does the cache bookkeeping.  With many features that small launch (64 workgroups walking the whole
