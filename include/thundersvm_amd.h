@@ -261,7 +261,9 @@ size_t tsvm_select_workspace(int64_t n);
 /* sort_f + select_working_set fused (smo_kernel.cpp:321-332; csmosolver.cpp:123-165;
  * nusmosolver.cpp:48-118): writes into out[0..n_select) the ids the reference's alternating scan
  * over the (f, index)-sorted order would pick, skipping the ids in marked[0..n_marked).
- * nu != 0 selects the four-pointer NuSMOSolver rule. */
+ * nu != 0 selects the four-pointer NuSMOSolver rule.  When the candidates run out before n_select ids are found
+ * (n_select larger than the number of unmarked instances) the remaining entries of out are -1: such a working set
+ * must not be handed to the solver entry points, which index with every id they are given. */
 int tsvm_select_working_set(const double *f, const int *y, const double *alpha, int64_t n, double Cp, double Cn,
                             const int *marked, int n_marked, int *out, int n_select, int nu, void *workspace,
                             tsvm_stream stream);
