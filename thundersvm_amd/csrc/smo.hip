@@ -438,11 +438,12 @@ __global__ __launch_bounds__(UF_T) void update_f_kernel(double *__restrict__ f, 
 // workgroup walks one contiguous chunk of the instances and keeps the chunk's marked instances (the half of the
 // previous working set that stays, csmosolver.cpp:65-71: never candidates) as a bit field in LDS.
 #define SEL_CHUNK_MAX 65536
+template <int NS>   // NS = g.n_sides: two sides need half the LDS of four, and a workgroup finds room on a busy CU sooner
 __global__ __launch_bounds__(SEL_T) void sel_pass_kernel(SelWorkspace w, const double *__restrict__ f,
                                                          const int *__restrict__ y, const double *__restrict__ alpha,
                                                          int64_t n, double Cp, double Cn, SelGeom g, int p,
                                                          const int *__restrict__ marked, int n_marked) {
-    __shared__ uint32_t lhist[SEL_MAX_SIDES][SEL_BINS];
+    __shared__ uint32_t lhist[NS][SEL_BINS];
     __shared__ SelState st[SEL_MAX_SIDES];
     __shared__ uint32_t scratch[SEL_T + 16];
     __shared__ uint32_t mark_bits[SEL_CHUNK_MAX / 32];
@@ -462,7 +463,7 @@ __global__ __launch_bounds__(SEL_T) void sel_pass_kernel(SelWorkspace w, const d
     bool any = false;
     for (int s = 0; s < g.n_sides; ++s) any |= !st[s].done;
     if (!any) return;
-    for (int e = tid; e < SEL_MAX_SIDES * SEL_BINS; e += SEL_T) (&lhist[0][0])[e] = 0;
+    for (int e = tid; e < NS * SEL_BINS; e += SEL_T) (&lhist[0][0])[e] = 0;
     bool is_key; int shift, width;
     sel_digit_geom(p, g.idx_bits, is_key, shift, width);
     const uint32_t dmask = (1u << width) - 1;
@@ -560,7 +561,7 @@ __device__ void sel_tail(const SelWorkspace &w, int64_t n, const SelGeom &g, int
     const int tid = threadIdx.x, nt = blockDim.x;
     for (int p = p_full; p < g.n_pass && sel_undecided(g, st); ++p) {
         if (tid < g.n_sides) w.state[p * SEL_MAX_SIDES + tid] = st[tid];
-        for (int e = tid; e < SEL_MAX_SIDES * SEL_BINS; e += nt) (&lhist[0][0])[e] = 0;
+        for (int e = tid; e < g.n_sides * SEL_BINS; e += nt) (&lhist[0][0])[e] = 0;
         __syncthreads();
         bool is_key; int shift, width;
         sel_digit_geom(p, g.idx_bits, is_key, shift, width);
@@ -586,11 +587,12 @@ __device__ __forceinline__ bool comp_less(uint64_t ka, uint32_t ia, uint64_t kb,
 
 // (fold_n > 0: the ids are also written modulo fold_n to out_folded, for problems whose instances are stacked
 // copies of fold_n stored rows)
+template <int NS>   // NS = g.n_sides (32 KB of LDS with two sides, 64 KB with four)
 __global__ __launch_bounds__(MAX_WS) void sel_final_kernel(SelWorkspace w, int64_t n, SelGeom g, int p_full,
                                                            int *__restrict__ out, int fold_n, int *__restrict__ out_folded) {
-    __shared__ uint64_t sk[SEL_MAX_SIDES][MAX_WS];
-    __shared__ uint32_t si[SEL_MAX_SIDES][MAX_WS];
-    __shared__ int pos_other[SEL_MAX_SIDES][MAX_WS];  // position of the same instance in the paired side's list, or -1
+    __shared__ uint64_t sk[NS][MAX_WS];
+    __shared__ uint32_t si[NS][MAX_WS];
+    __shared__ int pos_other[NS][MAX_WS];  // position of the same instance in the paired side's list, or -1
     __shared__ int cnt[SEL_MAX_SIDES];
     __shared__ int conflict;
     __shared__ SelState st[SEL_MAX_SIDES];
@@ -807,12 +809,14 @@ static int select_working_set(const double *f, const int *y, const double *alpha
         TSVM_LAUNCH_CHECK();
     }
     for (int p = first_pass; p < p_full; ++p) {
-        hipLaunchKernelGGL(sel_pass_kernel, dim3(grid), dim3(SEL_T), 0, s, w, f, y, alpha, n, Cp, Cn, g, p, marked, n_marked);
+        if (nu) hipLaunchKernelGGL(sel_pass_kernel<4>, dim3(grid), dim3(SEL_T), 0, s, w, f, y, alpha, n, Cp, Cn, g, p, marked, n_marked);
+        else hipLaunchKernelGGL(sel_pass_kernel<2>, dim3(grid), dim3(SEL_T), 0, s, w, f, y, alpha, n, Cp, Cn, g, p, marked, n_marked);
         TSVM_LAUNCH_CHECK();
     }
     hipLaunchKernelGGL(sel_compact_kernel, dim3(grid), dim3(SEL_T), 0, s, w, n, g, p_full);
     TSVM_LAUNCH_CHECK();
-    hipLaunchKernelGGL(sel_final_kernel, dim3(1), dim3(MAX_WS), 0, s, w, n, g, p_full, out, fold_n, out_folded);
+    if (nu) hipLaunchKernelGGL(sel_final_kernel<4>, dim3(1), dim3(MAX_WS), 0, s, w, n, g, p_full, out, fold_n, out_folded);
+    else hipLaunchKernelGGL(sel_final_kernel<2>, dim3(1), dim3(MAX_WS), 0, s, w, n, g, p_full, out, fold_n, out_folded);
     TSVM_LAUNCH_CHECK();
     return 0;
 }
