@@ -57,3 +57,43 @@ def _case(seed):
 def test_random_small_problem(seed):
     data, prm, ws, trace = _case(seed)
     T._compare(data, data, make_param(max_iter=30, **prm), ws=ws, trace=trace)
+
+
+def _sparse_case(seed):
+    """Few non-zeros among hundreds to thousands of features: the rows stay in CSR form on the device."""
+    rng = np.random.default_rng(seed)
+    svm_type = int(rng.choice([0, 0, 0, 1, 2, 3, 4]))
+    kt = int(rng.choice([0, 1, 2, 2, 3]))
+    n = int(rng.choice([5, 40, 300, 1100, 3000]))
+    d = int(rng.choice([600, 3000, 21000]))
+    avg = float(rng.choice([0.5, 3, 12]))
+    n_cls = int(rng.choice([2, 2, 3, 4])) if svm_type in (0, 1) else 1
+    cnt = rng.poisson(avg, size=n)
+    ptr = np.zeros(n + 1, dtype=np.int64)
+    np.cumsum(cnt, out=ptr[1:])
+    col = np.concatenate([np.sort(rng.choice(d, size=c, replace=False)) + 1 for c in cnt] + [np.zeros(0, dtype=np.int64)])
+    val = rng.standard_normal(len(col)).astype(np.float32).astype(np.float64)
+    if svm_type in (0, 1):
+        y = rng.integers(0, n_cls, size=n).astype(np.float64)
+        if len(np.unique(y)) < 2:
+            y[0], y[1] = 0, 1
+        smallest = int(np.sort(np.bincount(y.astype(int))[np.bincount(y.astype(int)) > 0])[:2].sum())
+    else:
+        y = rng.standard_normal(n)
+        smallest = n * (2 if svm_type in (3, 4) else 1)
+    prm = dict(svm_type=svm_type, kernel_type=kt, C=float(rng.choice([0.1, 1, 10])), gamma=float(rng.choice([0.01, 0.1, 0.5])),
+               coef0=float(rng.choice([0, 0.5])), degree=int(rng.choice([2, 3])), nu=float(rng.choice([0.1, 0.3, 0.5])),
+               p=float(rng.choice([0.01, 0.1])))
+    if kt == 3:
+        prm["gamma"] = 0.01
+    ws = int(rng.choice([0, 0, 64, 256]))
+    if ws > smallest:
+        ws = 0
+    trace = int(rng.choice([0, 0, 16]))
+    return D.CsrData(ptr, col.astype(np.int32), val, y), prm, ws, trace
+
+
+@pytest.mark.parametrize("seed", range(9000, 9040))
+def test_random_sparse_problem(seed):
+    data, prm, ws, trace = _sparse_case(seed)
+    T._compare(data, data, make_param(max_iter=30, **prm), ws=ws, trace=trace)
