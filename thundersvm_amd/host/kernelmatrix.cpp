@@ -1,3 +1,4 @@
+#include <memory>
 #include "kernelmatrix.h"
 #include <stdexcept>
 
@@ -95,8 +96,10 @@ std::shared_ptr<DeviceRows> DeviceRows::from_host(const DataSet::node2d &all, co
     for (size_t i = 0; i < n_rows; ++i) ptr[i + 1] += ptr[i];
     r.nnz = (size_t) ptr[n_rows];
     r.n_features = (size_t) max_index + 1;
-    std::vector<kernel_type> val(r.nnz);
-    std::vector<int> col(r.nnz);
+    // (not value-initialised: a std::vector would be zero-filled by one thread, 12 bytes per non-zero, before the
+    // threads below write every element anyway)
+    std::unique_ptr<kernel_type[]> val(new kernel_type[r.nnz]);
+    std::unique_ptr<int[]> col(new int[r.nnz]);
     int all_float = 1;
 #pragma omp parallel for schedule(static) reduction(min : all_float)
     for (size_t i = 0; i < n_rows; ++i) {
@@ -110,8 +113,10 @@ std::shared_ptr<DeviceRows> DeviceRows::from_host(const DataSet::node2d &all, co
         }
     }
     r.values_fit_float = all_float != 0;
-    r.val.upload(val);
-    r.col.upload(col);
+    r.val.resize(r.nnz);
+    r.val.upload(val.get(), r.nnz);
+    r.col.resize(r.nnz);
+    r.col.upload(col.get(), r.nnz);
     r.row_ptr.upload(ptr);
     r.self_dot.resize(r.n);
     abi_check(tsvm_csr_self_dot(r.val.data(), r.row_ptr.data(), (int64_t) r.n, r.self_dot.data(), nullptr));
