@@ -220,6 +220,31 @@ def test_forced_working_set_larger_than_the_problem_is_rejected():
     Model(0).train(tiny, make_param(svm_type=0, kernel_type=2, gamma=0.5, C=10), ws_override=32)
 
 
+def test_training_calls_from_two_threads_take_turns():
+    """The row arena and the pooled streams are shared by all calls of a process: calls made from several host threads
+    (ctypes releases the interpreter lock) are serialised by the library and give the models of sequential calls."""
+    import threading
+    w1, w2 = D.workload_c4(scale=0.004), D.workload_c5(scale=0.003)
+    jobs = [(w1["train"], make_param(**w1["params"])), (w2["train"], make_param(**w2["params"]))]
+    want = [Model(p.svm_type).train(d, p) for d, p in jobs]
+    got = [None, None]
+
+    def run(k):
+        d, p = jobs[k]
+        got[k] = Model(p.svm_type).train(d, p)
+
+    for _ in range(3):
+        threads = [threading.Thread(target=run, args=(k,)) for k in range(2)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        for k in range(2):
+            assert got[k] is not None
+            assert np.array_equal(got[k].coef, want[k].coef) and np.array_equal(got[k].rho, want[k].rho)
+            assert np.array_equal(got[k].sv_indices, want[k].sv_indices)
+
+
 def test_max_iter_cap():
     w = D.workload_c1(scale=0.5)
     prm = make_param(**w["params"])

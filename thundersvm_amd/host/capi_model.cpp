@@ -49,6 +49,7 @@ SvmParam to_param(const tsvm_param &p) {
 
 #define TSVM_GUARD(body)            \
     try {                           \
+        std::lock_guard<std::recursive_mutex> one_at_a_time(tsvm::device_work_mutex()); \
         body;                       \
         return 0;                   \
     } catch (const std::exception &e) { \

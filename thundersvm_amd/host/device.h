@@ -3,6 +3,7 @@
 // an explicit call (the reference's implicit host_data()/device_data() mirroring,
 // src/thundersvm/syncmem.cpp:58-108, is what forces a device-host round trip per solver iteration).
 #pragma once
+#include <mutex>
 #include <hip/hip_runtime.h>
 
 #include <new>
@@ -34,6 +35,12 @@ size_t &device_bytes_in_use();   // running total of DeviceBuffer allocations (t
 // rows plus the row cache).  Releasing a multi-gigabyte allocation costs up to seconds on this platform,
 // so the 21 one-vs-one solves of a 7-class problem must not each allocate and free their own pool.
 // Not counted in device_bytes_in_use().
+// One training or prediction call at a time per process: the row arena, the pooled CU-masked streams and the staging
+// buffers are shared by all of them (the reference is not re-entrant either: one cuSPARSE handle, one SyncMem
+// counter).  The model-level entry points hold this lock for their duration, so calls from several host threads
+// take turns instead of sharing those buffers.
+std::recursive_mutex &device_work_mutex();
+
 class RowArena {
 public:
     static RowArena &instance();

@@ -14,6 +14,11 @@ size_t &device_bytes_in_use() {
     return bytes;
 }
 
+std::recursive_mutex &device_work_mutex() {
+    static std::recursive_mutex m;
+    return m;
+}
+
 RowArena &RowArena::instance() {
     static RowArena arena;
     return arena;

@@ -20,6 +20,7 @@ SvmModel *as_model(void *m) { return static_cast<SvmModel *>(m); }
 template <typename F>
 bool guarded(const char *what, F &&f) {
     try {
+        std::lock_guard<std::recursive_mutex> one_at_a_time(tsvm::device_work_mutex());   // shared arena and streams
         f();
         return true;
     } catch (const std::exception &e) {
