@@ -337,6 +337,35 @@ def test_dense_rbf_many_columns_few_features(n, d, m):
     assert np.array_equal(got32[slots].astype(np.float64), want)
 
 
+@pytest.mark.parametrize("gamma", [0.5, 0.02, -0.5, -0.01])
+def test_rbf_arguments_on_both_sides_of_expf_s_range(gamma):
+    """Rows at very different scales: arguments of expf inside its range, in the subnormal results' stretch
+    (-104 .. -87.3), below it (the value is 0) and, with a negative gamma, above 88.7 (infinity), mixed within one
+    wavefront's stores and in whole tiles of their own; float and double rows, bit for bit."""
+    rng = np.random.default_rng(3)
+    n, d, m = 1500, 20, 200
+    x = rng.standard_normal((n, d)).astype(np.float32)
+    scale = np.ones(n, dtype=np.float32)
+    scale[rng.random(n) < 0.2] = 3.0
+    scale[rng.random(n) < 0.05] = 12.0
+    scale[600:900] = 2.5          # whole tiles of mid-range arguments
+    scale[900:1200] = 0.05        # and of arguments close to zero
+    x *= scale[:, None]
+    data = from_dense(x)
+    prm = dict(gamma=gamma)
+    okm = O.KernelMatrix(data.ptr, data.col, data.val, O.make_param(kernel_type=O.RBF, expf_mode=1, **prm))
+    x_d, nf, ld, sd, _ = _device_km(data, O.RBF, prm)
+    idx = rng.integers(0, n, size=m).astype(np.int32)
+    want = okm.get_rows(idx)
+    assert (want == 0).any() or gamma < 0
+    assert np.isinf(want).any() or gamma > 0
+    tiny = np.float32(1.2e-38)
+    assert ((want > 0) & (want < tiny)).any() or gamma < 0 or gamma < 0.1
+    for row_type in (capi.ROW_F32, capi.ROW_F64):
+        got = G.host(G.get_rows_dense(x_d, ld, n, nf, sd, x_d, ld, G.dev(idx), m, sd, O.RBF, row_type=row_type, **prm))
+        assert np.array_equal(got.astype(np.float64), want)
+
+
 @pytest.mark.parametrize("n,d,ws", [(300, 20, 64), (5000, 54, 1024), (2600, 200, 1024)])
 def test_row_store_managed_on_the_device(n, d, ws):
     """A row store with a slot for every instance, run the way the solver runs it: tsvm_row_slots_assign decides the

@@ -449,7 +449,7 @@ __global__ __launch_bounds__(256, 3) void get_rows_dense_stream_kernel(
         }
         // one value: the indicator columns' share, then the kernel function.  IND = 1..4: that many additions,
         // unrolled (the addend is 1.0 or 0.0: no branch); IND = 5: max_ones of them in a loop
-        auto finish = [&](double dot, double sdi, uint64_t mi, int tj) -> TO {
+        auto with_indicators = [&](double dot, uint64_t mi, int tj) -> double {
             if (IND) {
                 const int cnt = __popcll(mi & mj[tj]);
                 if (IND <= 4) {
@@ -459,7 +459,10 @@ __global__ __launch_bounds__(256, 3) void get_rows_dense_stream_kernel(
                     for (int t = 0; t < max_ones; ++t) dot += cnt > t ? 1.0 : 0.0;
                 }
             }
-            return tsvm_epilogue_as<TO>(dot, sdi, sdj[tj], kp, exp_tab);
+            return dot;
+        };
+        auto finish = [&](double dot, double sdi, uint64_t mi, int tj) -> TO {
+            return tsvm_epilogue_as<TO>(with_indicators(dot, mi, tj), sdi, sdj[tj], kp, exp_tab);
         };
         // interior tiles store without a test, four columns at a time; edge tiles (and outputs whose rows are not
         // 16-byte aligned) test and store every element
@@ -474,8 +477,25 @@ __global__ __launch_bounds__(256, 3) void get_rows_dense_stream_kernel(
                     const uint64_t mi = IND ? s_mi[r] : 0;
                     TO *orow = out + (int64_t) ((uint64_t) (uint32_t) s_slot[r] * (uint32_t) ldo) + jb;
                     vec4_t res;
+                    if constexpr (KT == TSVM_RBF && sizeof(TO) == 4) {
+                        // expf's two out-of-range cases cost four instructions per value; one look at the largest
+                        // magnitude among the wavefront's arguments (a NaN passes: it needs neither case) tells whether
+                        // any value of this store needs them.  Every instruction saved is an issue slot for the MFMAs.
+                        float xs[4];
 #pragma unroll
-                    for (int tj = 0; tj < 4; ++tj) res[tj] = finish(acc[ti][tj][v], sdi, mi, tj);
+                        for (int tj = 0; tj < 4; ++tj) xs[tj] = tsvm_rbf_arg(with_indicators(acc[ti][tj][v], mi, tj), sdi, sdj[tj], kp);
+                        const float mx = fmaxf(fmaxf(fabsf(xs[0]), fabsf(xs[1])), fmaxf(fabsf(xs[2]), fabsf(xs[3])));
+                        if (__builtin_amdgcn_ballot_w64(mx > 88.0f) == 0) {
+#pragma unroll
+                            for (int tj = 0; tj < 4; ++tj) res[tj] = tsvm_expf_in_range(xs[tj], exp_tab);
+                        } else {
+#pragma unroll
+                            for (int tj = 0; tj < 4; ++tj) res[tj] = tsvm_expf(xs[tj], exp_tab);
+                        }
+                    } else {
+#pragma unroll
+                        for (int tj = 0; tj < 4; ++tj) res[tj] = finish(acc[ti][tj][v], sdi, mi, tj);
+                    }
                     store_streaming((vec4_t *) orow, res);
                 }
             }

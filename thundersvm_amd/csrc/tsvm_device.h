@@ -30,14 +30,15 @@ __constant__ const uint64_t TSVM_EXP2F_TAB[32] = {
 // expf of a float argument, evaluated in double and rounded once to float: the table-driven
 // algorithm glibc (>= 2.27) uses for expf, in the form its FMA build takes (libm's bits on all 2^32 arguments).  `tab` points at the 32-entry table (LDS or constant).
 // The reference's kernels call libm expf on the host (kernelmatrix_kernel.cpp:71-72,87-89).
-__device__ __forceinline__ float tsvm_expf(float x, const uint64_t *tab) {
+// The routine without its two out-of-range cases: the right result for -0x1.9fe368p6 <= x <= 0x1.62e42ep6 and for NaN.
+__device__ __forceinline__ float tsvm_expf_in_range(float x, const uint64_t *tab) {
     const double InvLn2N = 0x1.71547652b82fep+0 * 32;
     const double SHIFT = 0x1.8p+52;
     const double C0 = 0x1.c6af84b912394p-5 / 32 / 32 / 32;
     const double C1 = 0x1.ebfce50fac4f3p-3 / 32 / 32;
     const double C2 = 0x1.62e42ff0c52d6p-1 / 32;
-    // The main path runs unconditionally and the out-of-range cases are selected afterwards (no
-    // branches in the epilogue); a NaN argument comes out as NaN through the arithmetic itself.
+    // (the out-of-range cases are selected afterwards, in tsvm_expf: no branches in the epilogue; a NaN argument
+    // comes out as NaN through the arithmetic itself)
     // (k and r both come straight from the exact product x * 32/ln2, as in the library's FMA build, where the
     // compiler fuses the product into the addition of SHIFT and into the subtraction of k: with a rounded product
     // two of the 2^32 arguments gave a neighbouring float)
@@ -55,7 +56,10 @@ __device__ __forceinline__ float tsvm_expf(float x, const uint64_t *tab) {
     double y = __builtin_fma(C2, r, 1.0);
     y = __builtin_fma(zz, r2, y);
     y = y * s;
-    float res = (float) y;
+    return (float) y;
+}
+__device__ __forceinline__ float tsvm_expf(float x, const uint64_t *tab) {
+    float res = tsvm_expf_in_range(x, tab);
     res = x > 0x1.62e42ep6f ? __builtin_inff() : res;   // > log(2^128)
     res = x < -0x1.9fe368p6f ? 0.0f : res;              // < log(2^-150)
     return res;
@@ -255,6 +259,12 @@ __device__ __noinline__ float tsvm_tanhf(float x) {
     return jx >= 0 ? z : -z;
 }
 
+// The argument of the RBF kernel's expf (kernelmatrix_kernel.cpp:87-89): -(sd0 + sd1 - 2*dot) * gamma, as a float;
+// 2*dot is exact, so the fma rounds exactly where the subtraction would.
+__device__ __forceinline__ float tsvm_rbf_arg(double dot, double sd0, double sd1, const KernelParam &p) {
+    return (float) (-__builtin_fma(-2.0, dot, sd0 + sd1) * p.gamma);
+}
+
 // Kernel epilogues (kernelmatrix_kernel.cpp:61-108).  sd0/sd1 are the two rows' self dot products.
 // The RBF / polynomial / sigmoid values are floats by definition (expf / powf / tanhf); this returns that
 // float, so that a caller storing float rows pays for no round trip through double.
@@ -269,11 +279,7 @@ __device__ __forceinline__ float tsvm_epilogue_f32(double dot, double sd0, doubl
             const float arg = (float) __builtin_fma(p.gamma, dot, p.coef0);
             return tsvm_tanhf(arg);
         }
-        default: {
-            // -(sd0 + sd1 - 2*dot) * gamma; 2*dot is exact, so the fma rounds exactly where the subtraction would
-            const double arg = -__builtin_fma(-2.0, dot, sd0 + sd1) * p.gamma;
-            return tsvm_expf((float) arg, tab);
-        }
+        default: return tsvm_expf(tsvm_rbf_arg(dot, sd0, sd1, p), tab);
     }
 }
 
