@@ -419,10 +419,27 @@ __global__ __launch_bounds__(256, 3) void get_rows_dense_stream_kernel(
                     acc[ti][tj] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[ti], bf[tj], acc[ti][tj], 0, 0, 0);
         };
         if (n_kt > 0) {
-            for (int kt = 0; kt + 1 < n_kt; ++kt) {
+            // K tiles whose successor is a whole tile: this thread's loads walk along its two rows with one running
+            // pointer each and constant offsets (an address computed per load costs the matrix cores an issue slot
+            // per instruction: 24 of them per 32 MFMAs before this loop was written this way)
+            const double *pa = a_ptr + a_k, *pb = x_ptr + b_k;
+            for (int kt = 0; kt + 2 < n_kt; ++kt) {
                 stage_tile(false);
                 __syncthreads();
-                load_tile(kt + 1, kt + 2 == n_kt);
+                pa += KTILE;
+                pb += KTILE;
+#pragma unroll
+                for (int q = 0; q < A_VEC; ++q) ra[q] = *(const v4d *) (pa + 4 * q);
+#pragma unroll
+                for (int q = 0; q < B_VEC; ++q) rb[q] = *(const v4d *) (pb + 4 * q);
+#pragma unroll
+                for (int ks = 0; ks < KTILE / 4; ++ks) mma_step(ks);
+                __syncthreads();
+            }
+            if (n_kt >= 2) {   // the tile before the last: its successor may reach past the row and is loaded with care
+                stage_tile(false);
+                __syncthreads();
+                load_tile(n_kt - 1, true);
 #pragma unroll
                 for (int ks = 0; ks < KTILE / 4; ++ks) mma_step(ks);
                 __syncthreads();
