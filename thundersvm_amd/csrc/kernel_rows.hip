@@ -401,62 +401,44 @@ __global__ __launch_bounds__(256, 3) void get_rows_dense_stream_kernel(
             s_mj[gen][tid] = pre_m;
         }
         v4d acc[TI][4];
-        // one group of four columns of the staged tile.  `fresh` (the same for the whole workgroup): the accumulators
-        // start from zero through the instruction's own third operand, instead of 32 moves per column tile, each of
-        // which would cost the matrix cores an issue slot.
-        auto mma_step = [&](int ks, bool fresh) {
+#pragma unroll
+        for (int ti = 0; ti < TI; ++ti)
+#pragma unroll
+            for (int tj = 0; tj < 4; ++tj) acc[ti][tj] = (v4d){0.0, 0.0, 0.0, 0.0};
+        auto mma_step = [&](int ks) {
             double af[TI], bf[4];
             const int kk = (ks * 4 + lk) * LS;
 #pragma unroll
             for (int t = 0; t < TI; ++t) af[t] = As[kk + wi * (16 * TI) + t * 16 + lrow];
 #pragma unroll
             for (int t = 0; t < 4; ++t) bf[t] = Bs[kk + wj * 64 + t * 16 + lrow];
-            if (fresh) {
-#pragma unroll
-                for (int ti = 0; ti < TI; ++ti)
-#pragma unroll
-                    for (int tj = 0; tj < 4; ++tj)
-                        acc[ti][tj] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[ti], bf[tj], (v4d){0.0, 0.0, 0.0, 0.0}, 0, 0, 0);
-            } else {
-#pragma unroll
-                for (int ti = 0; ti < TI; ++ti)
-#pragma unroll
-                    for (int tj = 0; tj < 4; ++tj)
-                        acc[ti][tj] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[ti], bf[tj], acc[ti][tj], 0, 0, 0);
-            }
-        };
-        if (n_kt == 0) {
 #pragma unroll
             for (int ti = 0; ti < TI; ++ti)
 #pragma unroll
-                for (int tj = 0; tj < 4; ++tj) acc[ti][tj] = (v4d){0.0, 0.0, 0.0, 0.0};
-        }
+                for (int tj = 0; tj < 4; ++tj)
+                    acc[ti][tj] = __builtin_amdgcn_mfma_f64_16x16x4f64(af[ti], bf[tj], acc[ti][tj], 0, 0, 0);
+        };
         if (n_kt > 0) {
-            // K tiles whose successor is a whole tile: this thread's loads walk along its two rows with one running
-            // pointer each and constant offsets (an address computed per load costs the matrix cores an issue slot
-            // per instruction: 24 of them per 32 MFMAs before this loop was written this way)
+            // While the successor of a K tile is a whole tile, this thread's loads walk along its two rows with one
+            // running pointer each and constant offsets: an address computed per load costs the matrix cores an issue
+            // slot per instruction (24 of them per 32 MFMAs before the loop was written this way).  The last tile may
+            // reach past the row and is loaded with care.
             const double *pa = a_ptr + a_k, *pb = x_ptr + b_k;
-            for (int kt = 0; kt + 2 < n_kt; ++kt) {
+            for (int kt = 0; kt + 1 < n_kt; ++kt) {
                 stage_tile(false);
                 __syncthreads();
-                pa += KTILE;
-                pb += KTILE;
+                if (kt + 2 < n_kt) {
+                    pa += KTILE;
+                    pb += KTILE;
 #pragma unroll
-                for (int q = 0; q < A_VEC; ++q) ra[q] = *(const v4d *) (pa + 4 * q);
+                    for (int q = 0; q < A_VEC; ++q) ra[q] = *(const v4d *) (pa + 4 * q);
 #pragma unroll
-                for (int q = 0; q < B_VEC; ++q) rb[q] = *(const v4d *) (pb + 4 * q);
-                mma_step(0, kt == 0);
+                    for (int q = 0; q < B_VEC; ++q) rb[q] = *(const v4d *) (pb + 4 * q);
+                } else {
+                    load_tile(n_kt - 1, true);
+                }
 #pragma unroll
-                for (int ks = 1; ks < KTILE / 4; ++ks) mma_step(ks, false);
-                __syncthreads();
-            }
-            if (n_kt >= 2) {   // the tile before the last: its successor may reach past the row and is loaded with care
-                stage_tile(false);
-                __syncthreads();
-                load_tile(n_kt - 1, true);
-                mma_step(0, n_kt == 2);
-#pragma unroll
-                for (int ks = 1; ks < KTILE / 4; ++ks) mma_step(ks, false);
+                for (int ks = 0; ks < KTILE / 4; ++ks) mma_step(ks);
                 __syncthreads();
             }
             stage_tile(true);
@@ -467,10 +449,9 @@ __global__ __launch_bounds__(256, 3) void get_rows_dense_stream_kernel(
             if (n_kt > 0) load_tile(0, n_kt == 1);
         }
         if (n_kt > 0) {
-            mma_step(0, n_kt == 1);
 #pragma unroll
-            for (int ks = 1; ks < KTILE / 4; ++ks)
-                if (ks < n_ks_last) mma_step(ks, false);
+            for (int ks = 0; ks < KTILE / 4; ++ks)
+                if (ks < n_ks_last) mma_step(ks);
             __syncthreads();   // every wavefront is done with the staged tile before the next one is written
         }
         double sdj[4];
