@@ -278,7 +278,10 @@ __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
 // is the serial chain over the indicator columns, bit for bit (a pre-summed count would round differently).
 // mask_x / mask_a hold one bit per indicator column and row; max_ones bounds the set bits of a row.
 // ------------------------------------------------------------------------------------------------
-template <int KT, typename TO, int IND>
+// LONG_K: the K loop for three and more K tiles keeps the tile before the last in a block of its own, so that the
+// tiles before it need no test of which kind of load comes next; shapes with fewer K tiles get the shorter code
+// (measured in training runs: the larger kernel costs a short K loop more than the test costs a long one).
+template <int KT, typename TO, int IND, bool LONG_K = false>
 __global__ __launch_bounds__(256, 3) void get_rows_dense_stream_kernel(
     const double *__restrict__ x, int64_t ldx, const int *__restrict__ x_idx, int64_t n, int d,
     const double *__restrict__ sd_x, const double *__restrict__ a, int64_t lda, const int *__restrict__ a_idx, int m,
@@ -424,22 +427,46 @@ __global__ __launch_bounds__(256, 3) void get_rows_dense_stream_kernel(
             // slot per instruction (24 of them per 32 MFMAs before the loop was written this way).  The last tile may
             // reach past the row and is loaded with care.
             const double *pa = a_ptr + a_k, *pb = x_ptr + b_k;
-            for (int kt = 0; kt + 1 < n_kt; ++kt) {
-                stage_tile(false);
-                __syncthreads();
-                if (kt + 2 < n_kt) {
+            if constexpr (LONG_K) {
+                for (int kt = 0; kt + 2 < n_kt; ++kt) {
+                    stage_tile(false);
+                    __syncthreads();
                     pa += KTILE;
                     pb += KTILE;
 #pragma unroll
                     for (int q = 0; q < A_VEC; ++q) ra[q] = *(const v4d *) (pa + 4 * q);
 #pragma unroll
                     for (int q = 0; q < B_VEC; ++q) rb[q] = *(const v4d *) (pb + 4 * q);
-                } else {
-                    load_tile(n_kt - 1, true);
-                }
 #pragma unroll
-                for (int ks = 0; ks < KTILE / 4; ++ks) mma_step(ks);
-                __syncthreads();
+                    for (int ks = 0; ks < KTILE / 4; ++ks) mma_step(ks);
+                    __syncthreads();
+                }
+                if (n_kt >= 2) {   // the tile before the last
+                    stage_tile(false);
+                    __syncthreads();
+                    load_tile(n_kt - 1, true);
+#pragma unroll
+                    for (int ks = 0; ks < KTILE / 4; ++ks) mma_step(ks);
+                    __syncthreads();
+                }
+            } else {
+                for (int kt = 0; kt + 1 < n_kt; ++kt) {
+                    stage_tile(false);
+                    __syncthreads();
+                    if (kt + 2 < n_kt) {
+                        pa += KTILE;
+                        pb += KTILE;
+#pragma unroll
+                        for (int q = 0; q < A_VEC; ++q) ra[q] = *(const v4d *) (pa + 4 * q);
+#pragma unroll
+                        for (int q = 0; q < B_VEC; ++q) rb[q] = *(const v4d *) (pb + 4 * q);
+                    } else {
+                        load_tile(n_kt - 1, true);
+                    }
+#pragma unroll
+                    for (int ks = 0; ks < KTILE / 4; ++ks) mma_step(ks);
+                    __syncthreads();
+                }
             }
             stage_tile(true);
         }
@@ -1011,7 +1038,13 @@ static int get_rows_dense(const double *x, int64_t ldx, const int *x_idx, int64_
     do {                                                                                                              \
         if (ti == 2) {                                                                                                \
             switch (ind_mode) {                                                                                       \
-                case 0: GR_STREAM(KTYPE, TO, 0); break;                                                               \
+                case 0:                                                                                               \
+                    if (d > 32)                                                                                       \
+                        hipLaunchKernelGGL((get_rows_dense_stream_kernel<KTYPE, TO, 0, true>), sgrid, block, 0, tsvm_s(stream), x, ldx, \
+                                           x_idx, n, d, sd_x, a, lda, a_idx, m, sd_a, kp, (TO *) out, out_slots, ldo, m_blocks, \
+                                           (unsigned) n_blocks, tpw, m_dev, mask_x, mask_a, max_ones, vec_ok);        \
+                    else GR_STREAM(KTYPE, TO, 0);                                                                     \
+                    break;                                                                                            \
                 case 1: GR_STREAM(KTYPE, TO, 1); break;                                                               \
                 case 2: GR_STREAM(KTYPE, TO, 2); break;                                                               \
                 case 3: GR_STREAM(KTYPE, TO, 3); break;                                                               \
