@@ -278,10 +278,10 @@ __global__ __launch_bounds__(256, (TI == 2 ? 3 : 2)) void get_rows_dense_kernel(
 // is the serial chain over the indicator columns, bit for bit (a pre-summed count would round differently).
 // mask_x / mask_a hold one bit per indicator column and row; max_ones bounds the set bits of a row.
 // ------------------------------------------------------------------------------------------------
-// LONG_K: the K loop for three and more K tiles keeps the tile before the last in a block of its own, so that the
+// K_TILES = 3: the K loop for three and more K tiles keeps the tile before the last in a block of its own, so that the
 // tiles before it need no test of which kind of load comes next; shapes with fewer K tiles get the shorter code
 // (measured in training runs: the larger kernel costs a short K loop more than the test costs a long one).
-template <int KT, typename TO, int IND, bool LONG_K = false>
+template <int KT, typename TO, int IND, int K_TILES = 2>   // K_TILES: 1 = a single K tile (d <= 16), 2 = any number, 3 = three and more (LONG_K)
 __global__ __launch_bounds__(256, 3) void get_rows_dense_stream_kernel(
     const double *__restrict__ x, int64_t ldx, const int *__restrict__ x_idx, int64_t n, int d,
     const double *__restrict__ sd_x, const double *__restrict__ a, int64_t lda, const int *__restrict__ a_idx, int m,
@@ -342,7 +342,7 @@ __global__ __launch_bounds__(256, 3) void get_rows_dense_stream_kernel(
     if (a_idx) a_r = a_idx[a_r];
     const double *a_ptr = a + (uint64_t) (uint32_t) a_r * (uint32_t) lda;
 
-    const int n_kt = (d + KTILE - 1) / KTILE;
+    const int n_kt = K_TILES == 1 ? (d > 0 ? 1 : 0) : (d + KTILE - 1) / KTILE;   // (K_TILES == 1: the host has checked d <= KTILE)
     const int n_ks_last = (d - (n_kt - 1) * KTILE + 3) / 4;   // groups of four columns in the last K tile, 1 .. KTILE / 4
     v4d ra[A_VEC], rb[B_VEC];
     double pre_sd = 0.0;      // the next tile's column data for column tid (threads below 128)
@@ -427,7 +427,9 @@ __global__ __launch_bounds__(256, 3) void get_rows_dense_stream_kernel(
             // slot per instruction (24 of them per 32 MFMAs before the loop was written this way).  The last tile may
             // reach past the row and is loaded with care.
             const double *pa = a_ptr + a_k, *pb = x_ptr + b_k;
-            if constexpr (LONG_K) {
+            if constexpr (K_TILES == 1) {
+                // (nothing in front of the only tile)
+            } else if constexpr (K_TILES == 3) {
                 for (int kt = 0; kt + 2 < n_kt; ++kt) {
                     stage_tile(false);
                     __syncthreads();
@@ -1030,17 +1032,22 @@ static int get_rows_dense(const double *x, int64_t ldx, const int *x_idx, int64_
     // four results per store need every group of four columns of every output row 16-byte aligned
     const int vec_ok = ((uintptr_t) out % 16 == 0) && (ldo % 4 == 0);
     const int ind_mode = !mask_x ? 0 : (max_ones >= 1 && max_ones <= 4) ? max_ones : 5;   // additions unrolled up to four
+#define GR_STREAM_K(KTYPE, TO, IND, KT_)                                                                               \
+    hipLaunchKernelGGL((get_rows_dense_stream_kernel<KTYPE, TO, IND, KT_>), sgrid, block, 0, tsvm_s(stream), x, ldx, x_idx, n, d, \
+                       sd_x, a, lda, a_idx, m, sd_a, kp, (TO *) out, out_slots, ldo, m_blocks, (unsigned) n_blocks, tpw, m_dev, \
+                       mask_x, mask_a, max_ones, vec_ok)
 #define GR_STREAM(KTYPE, TO, IND)                                                                                     \
-    hipLaunchKernelGGL((get_rows_dense_stream_kernel<KTYPE, TO, IND>), sgrid, block, 0, tsvm_s(stream), x, ldx, x_idx, n, d, sd_x, \
-                       a, lda, a_idx, m, sd_a, kp, (TO *) out, out_slots, ldo, m_blocks, (unsigned) n_blocks, tpw, m_dev, mask_x, \
-                       mask_a, max_ones, vec_ok)
+    do {                                                                                                              \
+        if (d <= 16) GR_STREAM_K(KTYPE, TO, IND, 1);                                                                  \
+        else GR_STREAM_K(KTYPE, TO, IND, 2);                                                                          \
+    } while (0)
 #define GR_LAUNCH_T(KTYPE, TO)                                                                                        \
     do {                                                                                                              \
         if (ti == 2) {                                                                                                \
             switch (ind_mode) {                                                                                       \
                 case 0:                                                                                               \
                     if (d > 32)                                                                                       \
-                        hipLaunchKernelGGL((get_rows_dense_stream_kernel<KTYPE, TO, 0, true>), sgrid, block, 0, tsvm_s(stream), x, ldx, \
+                        hipLaunchKernelGGL((get_rows_dense_stream_kernel<KTYPE, TO, 0, 3>), sgrid, block, 0, tsvm_s(stream), x, ldx, \
                                            x_idx, n, d, sd_x, a, lda, a_idx, m, sd_a, kp, (TO *) out, out_slots, ldo, m_blocks, \
                                            (unsigned) n_blocks, tpw, m_dev, mask_x, mask_a, max_ones, vec_ok);        \
                     else GR_STREAM(KTYPE, TO, 0);                                                                     \
@@ -1069,6 +1076,7 @@ static int get_rows_dense(const double *x, int64_t ldx, const int *x_idx, int64_
 #undef GR_LAUNCH
 #undef GR_LAUNCH_T
 #undef GR_STREAM
+#undef GR_STREAM_K
     TSVM_LAUNCH_CHECK();
     return 0;
 }
