@@ -313,7 +313,8 @@ def test_row_subsets_on_device():
     assert np.array_equal(G.host(oval), sub.val) and np.array_equal(G.host(ocol), sub.col)
 
 
-@pytest.mark.parametrize("n,d,m", [(131072 + 77, 7, 133), (140001, 54, 512), (131072, 90, 200), (135000, 200, 1024), (133333, 16, 65)])
+@pytest.mark.parametrize("n,d,m", [(131072 + 77, 7, 133), (140001, 54, 512), (131072, 90, 200), (135000, 200, 1024), (133333, 16, 65),
+                                   (131072 + 5, 24, 100), (131333, 33, 70)])   # one, two, three and more K tiles of 16 columns
 def test_dense_rbf_many_columns_few_features(n, d, m):
     """The shapes of the multi-class and regression workloads (hundreds of thousands of columns, tens of features):
     float and double rows, output slots, ragged last tiles in both directions."""
