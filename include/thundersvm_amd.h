@@ -308,6 +308,33 @@ int tsvm_sum_kernel_values(const double *coef, int total_sv, const int *sv_start
                            const double *rho, const void *k_mat, int row_type, int64_t ldk, double *dec_values,
                            int n_classes, int64_t n_instances, tsvm_stream stream);
 
+/* SvmModel::predict_dec_values in one pass (src/thundersvm/model/svmmodel.cpp:74-117: KernelMatrix::get_rows of the
+ * batch against the support vectors, then sum_kernel_values, kernelmatrix_kernel.cpp:110-147): the same decision
+ * values, with the kernel values reduced in registers instead of being written out as a batch x support-vector
+ * matrix.  Dense support vectors only.
+ *
+ * The caller lays the model out once: the support vectors of class s occupy the padded columns
+ * [128 * T_s, 128 * T_s + n_sv[s]) where T_s = sum over earlier classes of ceil(n_sv / 128), n_pad = 128 * T_k;
+ * col_map[p] = row of sv_x behind padded column p (padding: any valid row); coef_t[p * stride + c] = coefficient
+ * row c (0 .. k-2, the layout of include/thundersvm/model/svmmodel.h:154-164) of that support vector, zero for
+ * padding and for c >= k-1; stride = tsvm_predict_nc_stride(n_classes, d, masks given) (0: this shape is not taken,
+ * use tsvm_get_rows_* and tsvm_sum_kernel_values).  chunks[2q], chunks[2q+1] = first and one-past-last 128-column
+ * tile of chunk q; a chunk lies inside one class, chunks are ordered by class, class_chunk_start[s] = first chunk of
+ * class s (k + 1 entries).  Each workgroup takes one chunk and 64 (d <= 128 or masks) or 128 batch rows.
+ * a: the batch, dense [m][lda] in sv_x's column layout, with its rows' self dot products sd_a.  mask_sv / mask_a
+ * (both or neither) and max_ones as in tsvm_get_rows_dense_indicator, d then counting the columns before the
+ * indicator columns.  partial: workspace of max(n_chunks, 1) * m * (k-1) doubles.
+ * dec_values[r * P + p] as tsvm_sum_kernel_values defines it; sums run over the lanes of a wavefront and over the
+ * chunks in a fixed order (the reference adds the support vectors one after the other), so values agree with the
+ * two-call form to rounding, not bit for bit. */
+int tsvm_predict_nc_stride(int n_classes, int d, int has_masks);
+int tsvm_predict_dec_values_dense(const double *sv_x, int64_t ldx, int d, const double *sd_sv, const uint64_t *mask_sv,
+                                  const int *col_map, int64_t n_pad, const double *coef_t, const int *chunks,
+                                  int n_chunks, const int *class_chunk_start, const double *rho, int n_classes,
+                                  const double *a, int64_t lda, int64_t m, const double *sd_a, const uint64_t *mask_a,
+                                  int max_ones, int kernel_type, double gamma, double coef0, int degree, double *partial,
+                                  double *dec_values, tsvm_stream stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -60,6 +60,9 @@ SIGNATURES = {
     "tsvm_select_working_set_folded": (_int, [_p, _p, _p, _i64, _dbl, _dbl, _p, _int, _p, _int, _int, _p, _int, _int, _p, _p]),
     "tsvm_update_f_select": (_int, [_p, _p, _int, _p, _int, _p, _i64, _i64, _int, _p, _p, _dbl, _dbl, _p, _int, _p, _int, _int, _p, _p, _p]),
     "tsvm_sum_kernel_values": (_int, [_p, _int, _p, _p, _p, _p, _int, _i64, _p, _int, _i64, _p]),
+    "tsvm_predict_nc_stride": (_int, [_int, _int, _int]),
+    "tsvm_predict_dec_values_dense": (_int, [_p, _i64, _int, _p, _p, _p, _i64, _p, _p, _int, _p, _p, _int, _p, _i64, _i64, _p, _p,
+                                             _int, _int, _dbl, _dbl, _int, _p, _p, _p]),
 }
 
 _LIB = None

@@ -349,6 +349,15 @@ __device__ __forceinline__ double readlane_f64(double v, int lane) {
     return __hiloint2double(hi, lo);
 }
 
+// Sum over the sixteen lanes of a DPP row (lanes 16r .. 16r+15); every lane of the row returns it.
+__device__ __forceinline__ double dpp_row_sum_f64(double v) {
+    v += dpp_f64<TSVM_DPP_XOR1>(v);
+    v += dpp_f64<TSVM_DPP_XOR2>(v);
+    v += dpp_f64<TSVM_DPP_HALF_MIRROR>(v);
+    v += dpp_f64<TSVM_DPP_MIRROR>(v);
+    return v;
+}
+
 // Wavefront reductions used by the local solvers.  A (value, index) lexicographic minimum -- the
 // smallest value wins and, among equal values, the smallest index: the serial loops' "first strict
 // improvement" rule (smo_kernel.cpp:43-49,80-89) -- is taken in two branch-free passes: the minimum

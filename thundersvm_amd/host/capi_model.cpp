@@ -145,7 +145,7 @@ int tsvm_model_predict(void *model, void *dataset, int batch_size, double *dec_v
     TSVM_GUARD({
         SvmModel &m = *((Handle *) model)->model;
         const DataSet &ds = *(DataSet *) dataset;
-        std::vector<float_type> out = m.predict(ds.instances(), batch_size);
+        std::vector<float_type> out = m.predict(ds, batch_size);
         if (labels) memcpy(labels, out.data(), sizeof(double) * out.size());
         if (dec_values) memcpy(dec_values, m.get_dec_value().data(), sizeof(double) * m.get_dec_value().size());
     })

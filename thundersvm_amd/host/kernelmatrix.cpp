@@ -368,11 +368,12 @@ void KernelMatrix::get_rows(const DataSet::node2d &instances, void *d_out, int64
     get_rows(instances.data(), instances.size(), d_out, ld);
 }
 
-void KernelMatrix::get_rows(const std::vector<DataSet::node> *instances, size_t n_rows, void *d_out, int64_t ld) const {
+// The batch goes to the device as CSR (flattened by all cores into pinned memory, copied asynchronously) together
+// with its rows' self dot products; with dense stored rows it is also laid out as a dense matrix of the stored rows'
+// width (columns >= n_features are dropped from the products, kernelmatrix.cpp:392, but stay in the self dot).
+KernelMatrix::StagedBatch KernelMatrix::stage_batch(const std::vector<DataSet::node> *instances, size_t n_rows) const {
     const DeviceRows &R = *rows_;
     const int m = (int) n_rows;
-    if (m == 0) return;
-    // The batch goes to the device as CSR: flattened by all cores into pinned memory, copied asynchronously.
     TSVM_HIP_CHECK(hipStreamSynchronize(nullptr));   // a previous batch's copies have left the staging memory
     h_ptr_.reserve((size_t) m + 1);
     int64_t *ptr = h_ptr_.data();
@@ -383,10 +384,18 @@ void KernelMatrix::get_rows(const std::vector<DataSet::node> *instances, size_t 
     h_col_.reserve(total);
     kernel_type *val = h_val_.data();
     int *col = h_col_.data();
-#pragma omp parallel for schedule(static)
+    // (indicator columns of the stored rows: the batch can use them when its own values there are zeros and ones)
+    const int ind_lo = R.ind_first >= 0 ? R.ind_first : 0x7fffffff, ind_hi = (int) R.n_features;
+    int not_indicator = 0;
+#pragma omp parallel for schedule(static) reduction(max : not_indicator)
     for (int r = 0; r < m; ++r) {
         size_t e = (size_t) ptr[r];
-        for (const auto &nd : instances[r]) { val[e] = nd.value; col[e] = nd.index; ++e; }
+        for (const auto &nd : instances[r]) {
+            val[e] = nd.value;
+            col[e] = nd.index;
+            if (nd.index >= ind_lo && nd.index < ind_hi && nd.value != 0.0 && nd.value != 1.0) not_indicator = 1;
+            ++e;
+        }
     }
     if (b_val_.size() < total) { b_val_.resize(total); b_col_.resize(total); }
     if (b_ptr_.size() < (size_t) m + 1) b_ptr_.resize(m + 1);
@@ -397,20 +406,34 @@ void KernelMatrix::get_rows(const std::vector<DataSet::node> *instances, size_t 
     TSVM_HIP_CHECK(hipMemcpyAsync(b_ptr_.data(), ptr, ((size_t) m + 1) * sizeof(int64_t), hipMemcpyHostToDevice, nullptr));
     if (stage_sd_.size() < (size_t) m) stage_sd_.resize(m);
     abi_check(tsvm_csr_self_dot(b_val_.data(), b_ptr_.data(), m, stage_sd_.data(), nullptr));
-    const int n = (int) n_unique_;
+    StagedBatch out;
+    out.sd = stage_sd_.data();
+    out.indicator_values = R.ind_first >= 0 && !not_indicator;
     if (R.dense) {
         if (stage_.size() < (size_t) m * R.ld) stage_.resize((size_t) m * R.ld);
-        // columns >= R.n_features are dropped: the staging matrix is only R.n_features wide
         abi_check(tsvm_csr_to_dense(b_val_.data(), b_col_.data(), b_ptr_.data(), m, stage_.data(), R.ld, nullptr));
-        abi_check(tsvm_get_rows_dense(R.x.data(), R.ld, nullptr, n, (int) R.n_features, R.self_dot.data(), stage_.data(), R.ld, nullptr, m,
-                                      stage_sd_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
+        out.a = stage_.data();
+        out.lda = R.ld;
+    }
+    return out;
+}
+
+void KernelMatrix::get_rows(const std::vector<DataSet::node> *instances, size_t n_rows, void *d_out, int64_t ld) const {
+    const DeviceRows &R = *rows_;
+    const int m = (int) n_rows;
+    if (m == 0) return;
+    const StagedBatch b = stage_batch(instances, n_rows);
+    const int n = (int) n_unique_;
+    if (R.dense) {
+        abi_check(tsvm_get_rows_dense(R.x.data(), R.ld, nullptr, n, (int) R.n_features, R.self_dot.data(), b.a, b.lda, nullptr, m,
+                                      b.sd, (int) param.kernel_type, param.gamma, param.coef0, param.degree,
                                       d_out, row_type(), nullptr, ld, nullptr));
     } else {
         if (stage_.size() < (size_t) m * R.n_features) stage_.resize((size_t) m * R.n_features);
         abi_check(tsvm_csr_stage_rows(b_val_.data(), b_col_.data(), b_ptr_.data(), nullptr, m, (int) R.n_features,
                                       stage_.data(), nullptr));
         abi_check(tsvm_get_rows_csr(R.val.data(), R.col.data(), R.row_ptr.data(), nullptr, n, R.self_dot.data(), stage_.data(), m,
-                                    stage_sd_.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
+                                    b.sd, (int) param.kernel_type, param.gamma, param.coef0, param.degree,
                                     d_out, row_type(), nullptr, ld, nullptr));
     }
 }

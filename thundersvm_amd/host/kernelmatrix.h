@@ -75,6 +75,18 @@ public:
     void get_rows(const DataSet::node2d &instances, void *d_out, int64_t ld) const;
     void get_rows(const std::vector<DataSet::node> *instances, size_t m, void *d_out, int64_t ld) const;   // the same for a slice
 
+    // An external batch on the device: dense [m][lda] in the stored rows' column layout (dense stored rows only) and
+    // the rows' self dot products; valid until the next call that stages a batch.  indicator_values: the stored rows
+    // have indicator columns and the batch holds only zeros and ones there.
+    struct StagedBatch {
+        const kernel_type *a = nullptr;
+        int64_t lda = 0;
+        const kernel_type *sd = nullptr;
+        bool indicator_values = false;
+    };
+    StagedBatch stage_batch(const std::vector<DataSet::node> *instances, size_t m) const;
+    const DeviceRows &rows() const { return *rows_; }
+
     const kernel_type *diag() const { return diag_.data(); }          // device, n_instances() entries
     const kernel_type *self_dot() const { return rows_->self_dot.data(); }  // device, n_columns() entries
     size_t n_instances() const { return n_unique_ * repeat_; }        // rows of the matrix the solver sees

@@ -35,6 +35,7 @@ void SvmModel::model_setup(const DataSet &, SvmParam &p) {   // svmmodel.cpp:22-
     n_sv.assign(n_classes, 0);
     sv.clear();
     sv_k_mat.reset();
+    predict_plan_.reset();
     sv_indices.clear();
     coef.clear();
     linear_coef.clear();
@@ -95,55 +96,6 @@ void SvmModel::run_solver(CSMOSolver &solver, const KernelMatrix &k_mat, const s
     solver.solve(k_mat, y, alpha, rho_out, f_val, param.epsilon, Cp, Cn, ws, max_iter);
     solver_stats.push_back(solver.stats);
     if (keep_binary) binary_f.push_back(f_val);
-}
-
-// Decision values for a batch of rows (svmmodel.cpp:74-117): kernel values against all support
-// vectors, then the per-class-pair reduction, batch by batch, all on the device.
-void SvmModel::predict_dec_values(const DataSet::node2d &instances, std::vector<float_type> &dec, int batch_size) const {
-    dec.assign(instances.size() * (size_t) n_binary_models, 0);
-    if (instances.empty()) return;
-    std::vector<int> sv_start(n_classes, 0);
-    for (int c = 1; c < n_classes; ++c) sv_start[c] = sv_start[c - 1] + n_sv[c - 1];
-    const size_t T = sv.size();
-    if (T == 0) {
-        for (size_t r = 0; r < instances.size(); ++r)
-            for (int p = 0; p < n_binary_models; ++p) dec[r * n_binary_models + p] = -rho[p];
-        return;
-    }
-    // the support vectors' device copy is built by the first predict call and kept for the next ones (the
-    // reference rebuilds it per call, svmmodel.cpp:84)
-    if (!sv_k_mat) sv_k_mat.reset(new KernelMatrix(sv, param));
-    const KernelMatrix &k_mat = *sv_k_mat;
-    if (batch_size == -1) {
-        const size_t used = tsvm::device_bytes_in_use();
-        const size_t free_mem = param.max_mem_size > used ? param.max_mem_size - used : 0;
-        batch_size = (int) std::min(free_mem / sizeof(float_type) / (T + k_mat.n_features()), size_t(10000));
-        if (batch_size < 1) batch_size = 1;
-    }
-    DeviceBuffer<int> d_start, d_count;
-    DeviceBuffer<float_type> d_coef, d_rho;
-    d_start.upload(sv_start);
-    d_count.upload(n_sv);
-    d_coef.upload(coef);
-    d_rho.upload(rho);
-    const size_t bmax = std::min((size_t) batch_size, instances.size());
-    // kernel values of one batch: taken from the persistent row arena (no allocation per call)
-    // (rows padded to 16 elements: get_rows then writes whole aligned vectors)
-    const int64_t ldk = ((int64_t) T + 15) / 16 * 16;
-    void *d_k = tsvm::RowArena::instance().acquire(bmax * (size_t) ldk * k_mat.row_elem_size(), false);
-    DeviceBuffer<float_type> d_dec(bmax * n_binary_models);
-    for (size_t b0 = 0; b0 < instances.size(); b0 += batch_size) {
-        const size_t bm = std::min((size_t) batch_size, instances.size() - b0);
-        k_mat.get_rows(instances.data() + b0, bm, d_k, ldk);
-        abi_check(tsvm_sum_kernel_values(d_coef.data(), (int) T, d_start.data(), d_count.data(), d_rho.data(), d_k,
-                                         k_mat.row_type(), ldk, d_dec.data(), n_classes, (int64_t) bm, nullptr));
-        d_dec.download(dec.data() + b0 * n_binary_models, bm * n_binary_models);
-    }
-}
-
-std::vector<float_type> SvmModel::predict(const DataSet::node2d &instances, int batch_size) {   // svmmodel.cpp:157-171
-    predict_dec_values(instances, dec_values, batch_size);
-    return dec_values;
 }
 
 // Stratified folds in class order (svmmodel.cpp:31-71).
@@ -245,6 +197,7 @@ void SvmModel::load_from_file(std::string path) {
 // svmmodel.cpp:280-383
 void SvmModel::load_from_string(std::string data) {
     sv_k_mat.reset();
+    predict_plan_.reset();
     std::stringstream iss(data);
     std::string key;
     while (iss >> key) {
@@ -658,9 +611,8 @@ void SVC::train_pairs_in_lockstep(const DataSet &grouped, int lanes, std::vector
     }
 }
 
-std::vector<float_type> SVC::predict(const DataSet::node2d &instances, int batch_size) {   // svc.cpp:179-185
-    predict_dec_values(instances, dec_values, batch_size);
-    return predict_label(dec_values, (int) instances.size());
+std::vector<float_type> SVC::finish_predict(int n_instances) {   // svc.cpp:179-185
+    return predict_label(dec_values, n_instances);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1009,8 +961,8 @@ void OneClassSVC::train(const DataSet &dataset, SvmParam p) {
     if (param.kernel_type == SvmParam::LINEAR) compute_linear_coef_single_model(dataset.n_features(), dataset.is_zero_based());
 }
 
-std::vector<float_type> OneClassSVC::predict(const DataSet::node2d &instances, int batch_size) {   // oneclass_svc.cpp:59-66
-    std::vector<float_type> dec = SvmModel::predict(instances, batch_size);
+std::vector<float_type> OneClassSVC::finish_predict(int) {   // oneclass_svc.cpp:59-66
+    std::vector<float_type> dec = dec_values;
     for (auto &v : dec) v = v > 0 ? 1 : -1;
     return dec;
 }

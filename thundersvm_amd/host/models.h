@@ -14,8 +14,12 @@ class SvmModel {
 public:
     virtual ~SvmModel() = default;
     virtual void train(const DataSet &dataset, SvmParam param) = 0;
-    virtual std::vector<float_type> predict(const DataSet::node2d &instances, int batch_size = -1);
+    std::vector<float_type> predict(const DataSet::node2d &instances, int batch_size = -1);
     void predict_dec_values(const DataSet::node2d &instances, std::vector<float_type> &dec_values, int batch_size) const;
+    // The same for the instances of a DataSet; when the DataSet has a device-resident copy of its rows in the dense
+    // layout (DeviceRows::of), the kernels read the rows where they lie: nothing is assembled on the host or uploaded.
+    std::vector<float_type> predict(const DataSet &dataset, int batch_size = -1);
+    void predict_dec_values(const DataSet &dataset, std::vector<float_type> &dec_values, int batch_size) const;
     virtual std::vector<float_type> cross_validation(DataSet dataset, SvmParam param, int n_fold);
 
     virtual void save_to_file(std::string path);
@@ -56,6 +60,15 @@ public:
 
 protected:
     virtual void model_setup(const DataSet &dataset, SvmParam &param);
+    // what predict returns once dec_values holds the decision values of n_instances rows: the values themselves,
+    // class labels (SVC) or the side of the boundary (OneClassSVC)
+    virtual std::vector<float_type> finish_predict(int n_instances) { return dec_values; }
+    // the model as the prediction kernels read it (support vectors in HBM, coefficients by padded column)
+    struct PredictPlan;
+    const PredictPlan &predict_plan() const;
+    // one batch, rows already on the device as a dense matrix; false when the kernels do not take this model's shape
+    bool predict_batch_fused(const PredictPlan &plan, const kernel_type *a, int64_t lda, const kernel_type *sd_a, size_t m,
+                             bool indicator_values, float_type *dec_out) const;
     void copy_support_vectors(const DataSet::node2d &instances);
     void run_solver(CSMOSolver &solver, const KernelMatrix &k_mat, const std::vector<int> &y, std::vector<float_type> &alpha,
                     float_type &rho, std::vector<float_type> &f_val, float_type Cp, float_type Cn, size_t held_bytes = 0);
@@ -66,6 +79,7 @@ protected:
     std::vector<float_type> linear_coef;
     DataSet::node2d sv;
     mutable std::shared_ptr<KernelMatrix> sv_k_mat;   // device copy of sv, built by the first predict call
+    mutable std::shared_ptr<PredictPlan> predict_plan_;
     std::vector<int> sv_indices;
     std::vector<int> n_sv;           // per class
     int n_total_sv = 0;
@@ -83,10 +97,10 @@ protected:
 class SVC : public SvmModel {
 public:
     void train(const DataSet &dataset, SvmParam param) override;
-    std::vector<float_type> predict(const DataSet::node2d &instances, int batch_size) override;
 
 protected:
     void model_setup(const DataSet &dataset, SvmParam &param) override;
+    std::vector<float_type> finish_predict(int n_instances) override;
     // One class pair (i, j) of the one-vs-one decomposition: its rows, labels, starting point and solver.
     struct BinaryProblem {
         int i = 0, j = 0, k = 0;
@@ -136,10 +150,10 @@ protected:
 class OneClassSVC : public SvmModel {
 public:
     void train(const DataSet &dataset, SvmParam param) override;
-    std::vector<float_type> predict(const DataSet::node2d &instances, int batch_size) override;
 
 protected:
     void model_setup(const DataSet &dataset, SvmParam &param) override;
+    std::vector<float_type> finish_predict(int n_instances) override;
 };
 
 // Factory keyed on SvmParam::SVM_TYPE (thundersvm-train.cpp:41-60).
