@@ -3,19 +3,22 @@
 
 Headline workload (`--workload c4`, the default): the 500,000 x 54, 7-class one-vs-one RBF C-SVC (gamma=1, C=3,
 seed 20244), the configuration the path's speed-up target is quoted on.  A "step" is one full training pass,
-`SvmModel::train` on a DataSet that already exists: the reference's "all training time" window
-(src/thundersvm/thundersvm-train.cpp:89-94: KernelMatrix construction + every class pair's SMO solve +
-coefficient assembly, excluding file load and model save).  `value` is measured with the data rows already
-resident in HBM when the timed region starts; the same pass from a DataSet that lives in host memory only (rows
-assembled and uploaded inside train) is reported beside it as `train_seconds_with_upload`.
+`SvmModel::train` on a DataSet that exists in host memory: the reference's "all training time" window
+(src/thundersvm/thundersvm-train.cpp:89-94: row assembly and upload, KernelMatrix construction, every class pair's
+SMO solve, coefficient assembly; no file load, no model save).  `value` is that window in a warm process; the same
+pass with the rows already resident in HBM is reported beside it (`train_seconds_rows_resident`), and the first
+call of a fresh process -- the thundersvm-train executable on the workload's text file -- as `cli` (load / train /
+save) and `train_seconds_cold`.
 
 The printed JSON line also carries
-  * roofline: the dominant bounded kernel of the headline workload, timed live with device events on its
-    launch stream at the shape of the workload's largest problem, plus the fraction the same kernel reaches
-    inside training (from a phase-profiled pass);
-  * configs: the same figures for the other benchmark configurations (C2 dense MFMA get_rows, C3 CSR get_rows with
-    both kernels, C5 epsilon-SVR with its 200,000-row predict): train seconds, outer / inner iterations, get_rows
-    TFLOP/s or GB/s, update_f GB/s, predict rows/s;
+  * roofline: the roofed kernel with the most device time in a training trace of the workload -- get_rows -- timed
+    live with device events on its launch stream at the shape of the workload's largest problem, against the roof
+    that bounds it there (few features: the bytes of the rows it writes; many: the fp64 matrix cores), with the
+    fraction it reaches inside training (from a phase-profiled pass); `roofline_update_f`: the same for update_f;
+  * predict: rows per second from host rows and from device-resident rows, flops per row and the fraction of the
+    fp64 MFMA peak;
+  * configs: the same figures for the other benchmark configurations (C1; C2 dense MFMA get_rows; C3 CSR get_rows
+    with both kernels; C5 epsilon-SVR with its 200,000-row predict);
   * cpu_baseline: the CPU oracle (a port of the reference's USE_CUDA=OFF path, OpenMP) timed on this host on a
     bounded sample: a few outer SMO iterations of three class pairs of different sizes; per-iteration time is
     fitted linearly in the pair's row count and applied to every pair's outer-iteration count from the GPU run
@@ -26,7 +29,11 @@ import argparse
 import gc
 import json
 import os
+import re
+import shutil
+import subprocess
 import sys
+import tempfile
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
@@ -46,6 +53,8 @@ def parse():
     ap.add_argument("--scale", type=float, default=1.0, help="row-count scale of the workloads (1.0 = benchmark shape)")
     ap.add_argument("--cpu-seconds", type=float, default=40.0, help="CPU time budget of the baseline sample (0 = skip)")
     ap.add_argument("--others", type=int, default=1, help="also measure the other benchmark configurations (sub-blocks)")
+    ap.add_argument("--cli", type=int, default=1, help="also run the thundersvm-train executable on the workload's text file (fresh process)")
+    ap.add_argument("--loader-only", action="store_true", help="only write the workload's LibSVM text and time the loader (no GPU)")
     ap.add_argument("--kernels-only", action="store_true",
                     help="only launch get_rows / update_f at the workload's shape plus a 1 GiB device copy (for rocprofv3 counter runs)")
     return ap.parse_args()
@@ -83,7 +92,7 @@ def kernel_figures(train, params):
     import numpy as np
     import torch
     from thundersvm_amd import capi
-    from thundersvm_amd.host_rules import choose_dense, indicator_columns
+    from thundersvm_amd.model import choose_dense, indicator_run
     train = largest_problem(train, params)
     n, d = train.n, train.n_features
     nf = d + 1
@@ -107,14 +116,15 @@ def kernel_figures(train, params):
         capi.call("tsvm_csr_to_dense", val_d.data_ptr(), col_d.data_ptr(), ptr_d.data_ptr(), n, x.data_ptr(), ld, None)
         counts = torch.empty(2 * nf, dtype=torch.int32, device="cuda")
         capi.call("tsvm_column_stats_dense", x.data_ptr(), ld, n, nf, counts.data_ptr(), None)
-        first = indicator_columns(counts.cpu().numpy(), nf)
+        stats = counts.cpu().numpy()
+        first = indicator_run(stats, nf)
         masks, max_ones = None, 0
         if first < nf:
             masks = torch.empty(n, dtype=torch.int64, device="cuda")
             mo = torch.zeros(1, dtype=torch.int32, device="cuda")
             capi.call("tsvm_indicator_masks", x.data_ptr(), ld, n, first, nf - first, masks.data_ptr(), mo.data_ptr(), None)
             max_ones = int(mo.cpu()[0])
-            if (nf + 3) // 4 - (first + 3) // 4 < 2 + 3 * max_ones:     # the rule KernelMatrix applies
+            if not indicator_run(stats, nf, max_ones)[1]:     # the rule KernelMatrix applies
                 masks = None
         if masks is not None:
             run = lambda: capi.call("tsvm_get_rows_dense_indicator", x.data_ptr(), ld, None, n, first, sd.data_ptr(), masks.data_ptr(),
@@ -135,7 +145,8 @@ def kernel_figures(train, params):
                                executed_mfma_tflops=2.0 * m * n * ((mfma_cols + 3) // 4 * 4) / ms / 1e9,
                                useful_tflops=2.0 * m * train.nnz / ms / 1e9, row_bytes_per_value=esz,
                                min_bytes=min_bytes, gbs=min_bytes / ms / 1e6, frac_hbm_peak=min_bytes / ms / 1e6 / HBM_PEAK_GBS,
-                               flop_per_byte=flops / min_bytes)
+                               flop_per_byte=flops / min_bytes, mfma_columns=int(mfma_cols),
+                               executed_frac_mfma_peak=2.0 * m * n * ((mfma_cols + 3) // 4 * 4) / ms / 1e9 / FP64_MFMA_PEAK_TFLOPS)
         del x
     else:
         w = torch.zeros((nf, m), dtype=torch.float32, device="cuda")
@@ -184,6 +195,80 @@ def profiled_traffic(workload, kernel_prefix):
             if m:
                 return float(m.group(2)) * 1e9
     return None
+
+
+def profiled_mfma_util(workload, kernel_prefix):
+    """MfmaUtil (%) of a kernel from the committed rocprofv3 counter summary of this workload, None if there is none."""
+    path = os.path.join(ROOT, "profiles", "get_rows_update_f_%s_counters.md" % workload)
+    if not os.path.exists(path):
+        return None
+    for line in open(path):
+        cells = [c.strip() for c in line.split("|")]
+        if len(cells) >= 7 and cells[1].startswith("`" + kernel_prefix) and re.fullmatch(r"[0-9.]+", cells[5] or "x"):
+            return float(cells[5])
+    return None
+
+
+def cli_flags(params):
+    flags = ["-s", str(params["svm_type"]), "-t", str(params["kernel_type"]), "-c", repr(float(params["C"]))]
+    if "gamma" in params:
+        flags += ["-g", repr(float(params["gamma"]))]
+    if "p" in params:
+        flags += ["-p", repr(float(params["p"]))]
+    if "epsilon" in params:
+        flags += ["-e", repr(float(params["epsilon"]))]
+    return flags
+
+
+def cli_and_loader(w, run_cli=True, loader_threads=(1, 0)):
+    """Writes the workload's training rows as LibSVM text, times the loader on one thread and on all, and runs the
+    thundersvm-train executable on the file in a fresh process (first call: row arena, masked streams and code objects
+    are made inside its training window).  Must run before this process touches the GPU."""
+    from thundersvm_amd import data as D
+    from thundersvm_amd.model import Dataset
+    tmp = tempfile.mkdtemp(prefix="tsvm_bench_")
+    out = {}
+    try:
+        path = os.path.join(tmp, "train.txt")
+        t0 = time.time()
+        D.save_libsvm(path, w["train"])
+        size = os.path.getsize(path)
+        out["file"] = dict(bytes=size, rows=w["train"].n, write_seconds=time.time() - t0)
+        loader = {}
+        for t in loader_threads:
+            best = None
+            for _ in range(2):
+                t0 = time.time()
+                ds = Dataset(path=path, threads=t)
+                dt = time.time() - t0
+                assert ds.n == w["train"].n
+                del ds
+                best = dt if best is None else min(best, dt)
+            loader["threads_%s" % ("all" if t == 0 else t)] = dict(seconds=best, mb_per_s=size / 1e6 / best)
+        loader["cores"] = host_cores()
+        if "threads_1" in loader and "threads_all" in loader:
+            loader["speedup"] = loader["threads_1"]["seconds"] / loader["threads_all"]["seconds"]
+        out["loader"] = loader
+        if run_cli:
+            exe = os.path.join(ROOT, "thundersvm_amd", "bin", "thundersvm-train")
+            model = os.path.join(tmp, "train.model")
+            t0 = time.time()
+            res = subprocess.run([exe] + cli_flags(w["params"]) + [path, model], capture_output=True, text=True, timeout=600)
+            wall = time.time() - t0
+            log = res.stderr + res.stdout
+            if res.returncode != 0:
+                out["cli"] = dict(error=log[-400:])
+            else:
+                grab = lambda key: float(re.search(key + r" = ([0-9.eE+-]+)", log).group(1))
+                out["cli"] = dict(command="thundersvm-train " + " ".join(cli_flags(w["params"])) + " train.txt train.model",
+                                  load_seconds=grab("data loading time"), train_seconds=grab("all training time"),
+                                  save_seconds=grab("model saving time"), process_seconds=wall,
+                                  model_bytes=os.path.getsize(model),
+                                  note="fresh process: the training window holds the first allocation of the row arena, the "
+                                       "creation of the CU-masked streams and the loading of the kernels' code objects")
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+    return out
 
 
 def host_cores():
@@ -286,28 +371,29 @@ def measure_config(name, w, steps, warmup, with_kernels=True, predict=True):
 
     for _ in range(warmup):
         one(ds)
+    # the step: SvmModel::train on a DataSet that lives in host memory (rows are assembled and uploaded inside train)
     model, secs = None, []
     for _ in range(steps):
         model = None
-        torch.cuda.synchronize()
-        t0 = time.time()
-        model = one(ds)
-        torch.cuda.synchronize()
-        secs.append(time.time() - t0)
-    # the same pass when the DataSet only exists in host memory: rows are assembled and uploaded inside train()
-    up = []
-    for _ in range(2):
         fresh = Dataset(train)
         torch.cuda.synchronize()
         t0 = time.time()
-        one(fresh)
+        model = one(fresh)
         torch.cuda.synchronize()
-        up.append(time.time() - t0)
+        secs.append(time.time() - t0)
         del fresh
+    # the same pass when the rows are already resident in HBM
+    res = []
+    for _ in range(min(steps, 3)):
+        torch.cuda.synchronize()
+        t0 = time.time()
+        one(ds)
+        torch.cuda.synchronize()
+        res.append(time.time() - t0)
     nb = model.n_binary
     st = [model.stats(b) for b in range(nb)]
     block = {"workload": "%s: %d x %d, %s" % (w["name"], train.n, train.n_features, json.dumps(params)),
-             "train_seconds": sum(secs) / len(secs), "train_seconds_steps": secs, "train_seconds_with_upload": min(up),
+             "train_seconds": sum(secs) / len(secs), "train_seconds_steps": secs, "train_seconds_rows_resident": min(res),
              "outer_iterations": int(sum(s["n_iter"] for s in st)), "inner_iterations": int(sum(s["local_iter"] for s in st)),
              "binary_problems": nb, "total_sv": int(model.total_sv),
              "rows_computed": int(sum(s["rows_computed"] for s in st)),
@@ -320,7 +406,7 @@ def measure_config(name, w, steps, warmup, with_kernels=True, predict=True):
     sizes = _problem_sizes(train, params, model)
     esz = 8 if params["kernel_type"] == 0 else 4
     d = train.n_features
-    from thundersvm_amd.host_rules import choose_dense
+    from thundersvm_amd.model import choose_dense
     if choose_dense(train.n, d + 1, train.nnz):
         rows_flops = sum(2.0 * s["rows_computed"] * n_cols * d for s, n_cols in zip(ps, sizes))
     else:
@@ -339,8 +425,32 @@ def measure_config(name, w, steps, warmup, with_kernels=True, predict=True):
         t0 = time.time()
         model.predict(ds_test)
         pt = time.time() - t0
-        block["predict"] = dict(rows=test.n, seconds=pt, rows_per_s=test.n / pt, n_sv=int(model.total_sv),
-                                note="test rows start in host memory")
+        dd_test = Dataset(test).to_device()
+        model.predict(dd_test)
+        ptd = []
+        for _ in range(3):
+            t0 = time.time()
+            model.predict(dd_test)
+            ptd.append(time.time() - t0)
+        ptd = min(ptd)
+        k = model.n_classes
+        n_sv = int(model.total_sv)
+        flops_row = 2.0 * n_sv * d + 2.0 * (k - 1) * n_sv
+        # what has to move: the batch, the support vectors, the coefficients, the decision values (no kernel values)
+        by = 8.0 * (test.n * d + n_sv * d + (k - 1) * n_sv + test.n * nb)
+        block["predict"] = dict(rows=test.n, n_sv=n_sv, classes=k, seconds=pt, rows_per_s=test.n / pt,
+                                note="rows_per_s: test rows start in host memory; *_device_rows: rows resident in HBM "
+                                     "(Dataset.to_device), decision values copied back",
+                                seconds_device_rows=ptd, rows_per_s_device_rows=test.n / ptd,
+                                flops_per_row=flops_row, tflops=flops_row * test.n / pt / 1e12,
+                                frac_mfma_peak=flops_row * test.n / pt / 1e12 / FP64_MFMA_PEAK_TFLOPS,
+                                tflops_device_rows=flops_row * test.n / ptd / 1e12,
+                                frac_mfma_peak_device_rows=flops_row * test.n / ptd / 1e12 / FP64_MFMA_PEAK_TFLOPS,
+                                bytes=by, frac_hbm_peak=by / ptd / 1e9 / HBM_PEAK_GBS,
+                                kernel="tsvm_predict_dec_values_dense (kernel values reduced in registers)"
+                                       if choose_dense(n_sv, d + 1, model._sv_nnz) else
+                                       "tsvm_get_rows_csr + tsvm_sum_kernel_values")
+        del dd_test, ds_test
     if with_kernels:
         block["kernels"] = kernel_figures(train, params)
     return block, model
@@ -362,15 +472,22 @@ def main():
         print("bench.py: this build runs on exactly one GPU (no collectives, no sharding); re-run with --gpus 1",
               file=sys.stderr)
         sys.exit(2)
-    import torch
     from thundersvm_amd import data as D
-
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible", file=sys.stderr)
-        sys.exit(1)
     gen = {"c1": lambda s: D.workload_c1(s), "c2": lambda s: D.workload_c2(s), "c3": lambda s: D.workload_c3(s),
            "c4": lambda s: D.workload_c4(s, n_test=int(50000 * s)), "c5": lambda s: D.workload_c5(s)}
     w = gen[args.workload](args.scale)
+
+    if args.loader_only:
+        print(json.dumps(cli_and_loader(w, run_cli=False, loader_threads=(1, 2, 4, 8, 0))))
+        return
+
+    # the executable in a fresh process, and the loader: before this process has touched the GPU
+    fresh = cli_and_loader(w, run_cli=True) if args.cli and not args.kernels_only else {}
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
 
     if args.kernels_only:
         src = torch.empty(1 << 27, dtype=torch.float64, device="cuda").normal_()
@@ -392,29 +509,46 @@ def main():
     kern = head["kernels"]
     uf, gr = kern["update_f"], kern["get_rows"]
     it = head["in_training"]
+    traffic_unit = "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled; from profiles/)"
+    phases = head["phase_ms"]
+    share = lambda key: phases[key] / max(sum(phases.values()), 1e-9)
     if "tflops" not in gr:
         roofline = dict(kernel=gr["kernel"], bound="hbm", achieved=gr["gbs"], peak=HBM_PEAK_GBS, unit="GB/s", frac=gr["frac_hbm_peak"],
-                        traffic=profiled_traffic(args.workload, "get_rows_csr"),
-                        traffic_unit="bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled; from profiles/)", launch_ms=gr["ms"],
+                        traffic=profiled_traffic(args.workload, "get_rows_csr"), traffic_unit=traffic_unit, launch_ms=gr["ms"],
                         algorithmic="12*nnz + 4*(n+1) + 4*m*d + %d*m*n bytes per launch, m=%d n=%d nnz=%d" % (
                             gr["row_bytes_per_value"], gr["m"], gr["n"], gr["nnz"]))
-    elif gr["d"] < 64:
-        # few features: get_rows is bound by writing the rows, and update_f (reading them back) is the kernel with the
-        # most device time among the bounded ones; both are HBM kernels
-        roofline = dict(kernel="update_f_kernel (ws 1024 x n %d, %d-byte kernel values)" % (uf["n"], uf["row_bytes_per_value"]),
-                        bound="hbm", achieved=uf["gbs"], peak=HBM_PEAK_GBS, unit="GB/s", frac=uf["frac_hbm_peak"],
-                        traffic=profiled_traffic(args.workload, "update_f"),
-                        traffic_unit="bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled; from profiles/)",
-                        launch_ms=uf["ms"], algorithmic="e*ws*n + 16*n + 8*ws bytes per launch, e=%d ws=1024 n=%d" % (uf["row_bytes_per_value"], uf["n"]),
-                        frac_in_training=it["update_f_gbs"] / HBM_PEAK_GBS,
-                        in_training="bytes of the rows with non-zero alpha_diff actually read, summed over a phase-profiled pass, over its update_f time")
+    elif 2.0 * gr["d"] / 8.0 < 2 * 9.8:
+        # few features (2d/8 flop per byte of a double-precision row is not far above the chip's 9.8 flop per byte):
+        # the roof of get_rows is the memory traffic of the rows it writes
+        roofline = dict(kernel=gr["kernel"], bound="hbm", achieved=gr["gbs"], peak=HBM_PEAK_GBS, unit="GB/s", frac=gr["frac_hbm_peak"],
+                        traffic=profiled_traffic(args.workload, "get_rows_dense"), traffic_unit=traffic_unit, launch_ms=gr["ms"],
+                        algorithmic="8*(m*d + n*d) + %d*m*n bytes per launch, m=%d n=%d d=%d" % (
+                            gr["row_bytes_per_value"], gr["m"], gr["n"], gr["d"]),
+                        mfma_util_percent=profiled_mfma_util(args.workload, "get_rows_dense"),
+                        executed_mfma_tflops=gr["executed_mfma_tflops"], executed_frac_mfma_peak=gr["executed_frac_mfma_peak"],
+                        algorithmic_tflops=gr["tflops"], algorithmic_frac_mfma_peak=gr["frac_mfma_peak"],
+                        in_training_algorithmic_tflops=it["get_rows_tflops"],
+                        note="the matrix cores execute %d of the %d columns; the others are indicator columns added in the epilogue" % (
+                            gr["mfma_columns"], gr["d"]) if gr["mfma_columns"] < gr["d"] else None)
     else:
         roofline = dict(kernel=gr["kernel"], bound="mfma", achieved=gr["tflops"], peak=FP64_MFMA_PEAK_TFLOPS,
                         unit="TFLOP/s", frac=gr["frac_mfma_peak"], traffic=profiled_traffic(args.workload, "get_rows_dense"),
-                        traffic_unit="bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled; from profiles/)",
-                        launch_ms=gr["ms"], algorithmic="2*m*n*d flops per launch, m=%d n=%d d=%d" % (gr["m"], gr["n"], gr["d"]),
+                        traffic_unit=traffic_unit, launch_ms=gr["ms"],
+                        algorithmic="2*m*n*d flops per launch, m=%d n=%d d=%d" % (gr["m"], gr["n"], gr["d"]),
+                        mfma_util_percent=profiled_mfma_util(args.workload, "get_rows_dense"),
                         frac_in_training=it["get_rows_tflops"] / FP64_MFMA_PEAK_TFLOPS,
                         in_training="2*rows*n*d over the get_rows time of a phase-profiled pass")
+    roofline["share_of_phase_time"] = share("ms_get_rows")
+    roofline_uf = dict(kernel="update_f_kernel (ws 1024 x n %d, %d-byte kernel values)" % (uf["n"], uf["row_bytes_per_value"]),
+                       bound="hbm", achieved=uf["gbs"], peak=HBM_PEAK_GBS, unit="GB/s", frac=uf["frac_hbm_peak"],
+                       traffic=profiled_traffic(args.workload, "update_f"), traffic_unit=traffic_unit, launch_ms=uf["ms"],
+                       algorithmic="e*ws*n + 16*n + 8*ws bytes per launch, e=%d ws=1024 n=%d" % (uf["row_bytes_per_value"], uf["n"]),
+                       frac_in_training=it["update_f_gbs"] / HBM_PEAK_GBS,
+                       in_training="bytes of the rows with non-zero alpha_diff actually read, summed over a phase-profiled pass, over its update_f time",
+                       share_of_phase_time=share("ms_update_f"))
+    unroofed = dict(local_solver_share_of_phase_time=share("ms_local"), selection_share_of_phase_time=share("ms_select"),
+                    note="shares of the summed phase times of one phase-profiled pass (one problem at a time); the local solver "
+                         "is one workgroup bound by latency and has no roof")
 
     cpu = None
     if args.cpu_seconds > 0:
@@ -443,19 +577,24 @@ def main():
                 del m
         gc.enable()
 
+    cli = fresh.get("cli")
     line = {
         "metric": "smo_train_wall_clock", "value": dt, "unit": "s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": dt * 1e3, "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f64",
         "data": "synthetic (seeded generator, float32-exact values)",
         "config": {"workload": head["workload"], "scale": args.scale, "working_set": 1024,
-                   "window": "SvmModel::train, data rows resident in HBM (thundersvm-train.cpp:89-94 without the upload; "
-                             "train_seconds_with_upload has it)"},
+                   "window": "SvmModel::train on a DataSet in host memory (thundersvm-train.cpp:89-94: rows assembled and "
+                             "uploaded inside), warm process; train_seconds_rows_resident: rows already in HBM; "
+                             "train_seconds_cold: the same window in the first call of a fresh process"},
         "step_seconds": head["train_seconds_steps"],
-        "train_seconds_with_upload": head["train_seconds_with_upload"],
+        "train_seconds_rows_resident": head["train_seconds_rows_resident"],
+        "train_seconds_cold": cli.get("train_seconds") if cli else None,
+        "cli": cli, "loader": fresh.get("loader"), "text_file": fresh.get("file"),
         "solver": {"outer_iterations": head["outer_iterations"], "inner_iterations": head["inner_iterations"],
                    "binary_problems": head["binary_problems"], "total_sv": head["total_sv"], "phase_ms": head["phase_ms"],
                    "cache_hit_rate": head["cache_hit_rate"], "in_training": head["in_training"]},
-        "roofline": roofline, "cpu_baseline": cpu, "kernels": kern, "predict": head.get("predict"), "configs": configs,
+        "roofline": roofline, "roofline_update_f": roofline_uf, "unroofed": unroofed, "cpu_baseline": cpu, "kernels": kern,
+        "predict": head.get("predict"), "configs": configs,
     }
     print(json.dumps(line))
 

@@ -60,8 +60,25 @@ int tsvm_model_train_csr(void *model, int64_t n, const int64_t *row_ptr, const i
  * not the conversion.  y may be NULL for prediction-only data. */
 void *tsvm_dataset_new_csr(int64_t n, const int64_t *row_ptr, const int *col, const double *val, const double *y);
 void *tsvm_dataset_load(const char *libsvm_file);
+/* DataSet::load_from_file (src/thundersvm/dataset.cpp:20-100) with the number of reading and parsing threads given
+ * (0: what OpenMP would start, as tsvm_dataset_load and the reference do). */
+void *tsvm_dataset_load_threads(const char *libsvm_file, int n_threads);
+/* What a DataSet holds (for checking a loader): returns the number of stored entries; then the rows as CSR
+ * (row_ptr: rows + 1 entries) with the file's feature ids, and the labels.  Any pointer may be NULL. */
+int64_t tsvm_dataset_info(void *dataset, int64_t *n_features, int *zero_based, int *has_labels);
+void tsvm_dataset_get_csr(void *dataset, int64_t *row_ptr, int *col, double *val, double *y);
 void tsvm_dataset_free(void *dataset);
 int64_t tsvm_dataset_rows(void *dataset);
+/* Layout rules of the host layer, for callers that drive the kernel-level C ABI themselves and want the kernels a
+ * training run would use.  choose_dense: dense row-major storage (1) or CSR (0) for n rows of n_features columns
+ * with nnz stored entries (the reference decides per column, CSR_DenseCSR, src/thundersvm/kernelmatrix.cpp:16-74;
+ * here one layout serves all columns).  indicator_run_start: first column of the trailing run of columns that
+ * hold only zeros and ones, from the 2 * n_features counts of tsvm_column_stats_dense (n_features: none);
+ * indicator_run_pays: whether get_rows leaves that run to its epilogue, given the largest number of ones a row
+ * has there (tsvm_indicator_masks). */
+int tsvm_rule_choose_dense(int64_t n, int64_t n_features, int64_t nnz);
+int tsvm_rule_indicator_run_start(const int *column_stats, int n_features);
+int tsvm_rule_indicator_run_pays(int n_features, int first, int max_ones);
 /* Uploads the DataSet's rows to HBM now (dense or CSR layout, with their self dot products) instead of at the
  * first training call that uses it; the copy stays with the DataSet, and every later training call, including
  * each class pair of a one-vs-one run, takes its rows from it on the device. */

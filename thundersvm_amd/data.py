@@ -79,13 +79,17 @@ def load_libsvm(path):
     return CsrData(ptr, col, val32.astype(np.float64), ys)
 
 
-def save_libsvm(path, data):
+def save_libsvm(path, data, rows_per_write=100000):
+    """LibSVM text with nine significant digits (float32-exact values survive the round trip)."""
+    n = data.n
+    ptr = data.ptr.tolist()
+    y = data.y.tolist() if data.y is not None else [0.0] * n
     with open(path, "w") as fh:
-        for i in range(data.n):
-            s, e = data.ptr[i], data.ptr[i + 1]
-            y = data.y[i] if data.y is not None else 0
-            feats = " ".join("%d:%.9g" % (c, v) for c, v in zip(data.col[s:e], data.val[s:e]))
-            fh.write(("%.9g " % y) + feats + "\n")
+        for r0 in range(0, n, rows_per_write):
+            r1 = min(n, r0 + rows_per_write)
+            e0, e1 = ptr[r0], ptr[r1]
+            toks = ["%d:%.9g" % cv for cv in zip(data.col[e0:e1].tolist(), data.val[e0:e1].tolist())]
+            fh.write("".join("%.9g %s\n" % (y[i], " ".join(toks[ptr[i] - e0:ptr[i + 1] - e0])) for i in range(r0, r1)))
 
 
 # ----------------------------------------------------------------------------------------------

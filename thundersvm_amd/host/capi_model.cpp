@@ -120,6 +120,52 @@ void *tsvm_dataset_load(const char *libsvm_file) {
     }
 }
 
+void *tsvm_dataset_load_threads(const char *libsvm_file, int n_threads) {
+    try {
+        DataSet *ds = new DataSet();
+        ds->load_from_file(libsvm_file, n_threads);
+        return ds;
+    } catch (const std::exception &e) {
+        fail(e);
+        return nullptr;
+    }
+}
+
+int64_t tsvm_dataset_info(void *dataset, int64_t *n_features, int *zero_based, int *has_labels) {
+    const DataSet &ds = *(DataSet *) dataset;
+    if (n_features) *n_features = (int64_t) ds.n_features();
+    if (zero_based) *zero_based = ds.is_zero_based();
+    if (has_labels) *has_labels = ds.y().size() == ds.n_instances();
+    int64_t nnz = 0;
+    for (const auto &row : ds.instances()) nnz += (int64_t) row.size();
+    return nnz;
+}
+
+void tsvm_dataset_get_csr(void *dataset, int64_t *row_ptr, int *col, double *val, double *y) {
+    const DataSet &ds = *(DataSet *) dataset;
+    int64_t e = 0;
+    for (size_t r = 0; r < ds.n_instances(); ++r) {
+        if (row_ptr) row_ptr[r] = e;
+        for (const auto &nd : ds.instances()[r]) {
+            if (col) col[e] = nd.index;
+            if (val) val[e] = nd.value;
+            ++e;
+        }
+        if (y && r < ds.y().size()) y[r] = ds.y()[r];
+    }
+    if (row_ptr) row_ptr[ds.n_instances()] = e;
+}
+
+int tsvm_rule_choose_dense(int64_t n, int64_t n_features, int64_t nnz) {
+    return KernelMatrix::choose_dense((size_t) n, (size_t) n_features, (size_t) nnz);
+}
+int tsvm_rule_indicator_run_start(const int *column_stats, int n_features) {
+    return DeviceRows::indicator_run_start(column_stats, n_features);
+}
+int tsvm_rule_indicator_run_pays(int n_features, int first, int max_ones) {
+    return DeviceRows::indicator_run_pays(n_features, first, max_ones);
+}
+
 int tsvm_dataset_to_device(void *dataset) {
     try {
         (void) DeviceRows::of(*(DataSet *) dataset);

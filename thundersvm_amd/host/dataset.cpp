@@ -1,52 +1,215 @@
 #include "dataset.h"
 
+#include <fcntl.h>
+#include <omp.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <algorithm>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <fstream>
+#include <memory>
 #include <stdexcept>
 
 DataSet::DataSet(const node2d &instances, int n_features, const std::vector<float_type> &y)
     : y_(y), instances_(instances), n_features_(n_features) {}
 
-// One pass over the file text.  Each token "i:v" is parsed the way the reference's sscanf("%d:%f")
-// does: v goes through float (src/thundersvm/dataset.cpp:72-80).  Row order is file order.
-void DataSet::load_from_file(std::string file_name) {
+// ------------------------------------------------------------------------------------------------
+// LibSVM text loader.  The reference reads 16 MB at a time and lets every OpenMP thread parse a run of whole lines
+// of the buffer (src/thundersvm/dataset.cpp:20-100); here the file is read once (every thread its share), cut into
+// runs of whole lines, four per thread, parsed side by side and joined in file order.  Each token "i:v" gives what
+// the reference's sscanf("%d:%f") gives: v is the correctly rounded float of the decimal text.
+// Unlike the reference, a last line without a newline is kept (the reference's buffer walk stops at the last newline
+// it has seen and loses that line) and blank lines are skipped (the reference turns one into an instance without
+// features and with label 0).
+// ------------------------------------------------------------------------------------------------
+namespace {
+
+const double kPow10[23] = {1e0,  1e1,  1e2,  1e3,  1e4,  1e5,  1e6,  1e7,  1e8,  1e9,  1e10, 1e11,
+                           1e12, 1e13, 1e14, 1e15, 1e16, 1e17, 1e18, 1e19, 1e20, 1e21, 1e22};
+
+inline bool is_blank(char c) { return c == ' ' || c == '\t' || c == '\r'; }
+
+// A decimal number without the library call where that is provably the same.  Up to 19 significant digits fit a
+// 64-bit integer w; when w < 2^53 and the decimal exponent is within +-22, w and 10^|e| are exact doubles and their
+// product or quotient is the correctly rounded double of the text (one rounding).  Returns false when the text is
+// anything else (more digits, a large exponent, "inf", "nan", a hexadecimal float): the caller asks strtod / strtof.
+inline bool fast_decimal(const char *p, const char *lim, const char **end, double *out) {
+    const char *s = p;
+    bool neg = false;
+    if (s < lim && (*s == '-' || *s == '+')) neg = *s++ == '-';
+    uint64_t w = 0;
+    int sig = 0, e10 = 0;
+    bool any = false;
+    for (; s < lim && *s >= '0' && *s <= '9'; ++s) {
+        any = true;
+        if (sig >= 19) return false;
+        w = w * 10 + (uint64_t) (*s - '0');
+        if (w) ++sig;
+    }
+    if (s < lim && *s == '.') {
+        for (++s; s < lim && *s >= '0' && *s <= '9'; ++s) {
+            any = true;
+            if (sig >= 19) return false;
+            w = w * 10 + (uint64_t) (*s - '0');
+            if (w) ++sig;
+            --e10;
+        }
+    }
+    if (!any) return false;
+    if (s < lim && (*s == 'e' || *s == 'E')) {
+        const char *t = s + 1;
+        bool eneg = false;
+        if (t < lim && (*t == '-' || *t == '+')) eneg = *t++ == '-';
+        if (t < lim && *t >= '0' && *t <= '9') {
+            int ex = 0;
+            for (; t < lim && *t >= '0' && *t <= '9'; ++t)
+                if (ex < 10000) ex = ex * 10 + (*t - '0');
+            e10 += eneg ? -ex : ex;
+            s = t;
+        }
+    }
+    if (s < lim && !is_blank(*s) && *s != '\n' && *s != ':') return false;   // something the simple grammar does not cover
+    if (w >> 53 || e10 < -22 || e10 > 22) return false;
+    double d = (double) w;
+    d = e10 < 0 ? d / kPow10[-e10] : d * kPow10[e10];
+    *out = neg ? -d : d;
+    *end = s;
+    return true;
+}
+
+// the float of sscanf("%f"): the decimal text rounded once, to float
+inline float parse_float(const char *p, const char *lim, const char **end) {
+    double d;
+    if (fast_decimal(p, lim, end, &d)) {
+        // Rounding the correctly rounded double to float gives the correctly rounded float unless the double lies
+        // exactly half way between two floats (rounding is monotonic, so the double can only be on the wrong side of
+        // that point by being that point).  Zero and float-normal magnitudes only.
+        uint64_t bits;
+        memcpy(&bits, &d, sizeof bits);
+        const double ad = d < 0 ? -d : d;
+        if (ad == 0.0 || (ad >= 0x1p-126 && ad < 0x1p127 && (bits & 0x1fffffffull) != 0x10000000ull)) return (float) d;
+    }
+    char *q;
+    const float v = strtof(p, &q);   // (the text is NUL-terminated)
+    *end = q;
+    return v;
+}
+
+inline double parse_double(const char *p, const char *lim, const char **end) {
+    double d;
+    if (fast_decimal(p, lim, end, &d)) return d;
+    char *q;
+    d = strtod(p, &q);
+    *end = q;
+    return d;
+}
+
+struct LoadedRun {
+    std::vector<float_type> y;
+    DataSet::node2d rows;
+    size_t max_index = 0;
+    bool zero_based = false;
+    bool bad = false;
+};
+
+void parse_run(const char *p, const char *end, LoadedRun &out) {
+    std::vector<DataSet::node> row;   // assembled here, copied out at its final size: one allocation per instance
+    while (p < end) {
+        const char *eol = (const char *) memchr(p, '\n', end - p);
+        if (!eol) eol = end;
+        while (p < eol && is_blank(*p)) ++p;
+        if (p < eol) {
+            const char *q;
+            out.y.push_back(parse_double(p, eol, &q));
+            if (q == p) { out.bad = true; return; }
+            p = q;
+            row.clear();
+            while (p < eol) {
+                while (p < eol && is_blank(*p)) ++p;
+                if (p >= eol) break;
+                long idx = 0;
+                bool neg = false;
+                const char *s = p;
+                if (*s == '-' || *s == '+') neg = *s++ == '-';
+                const char *digits = s;
+                for (; s < eol && *s >= '0' && *s <= '9'; ++s) idx = idx * 10 + (*s - '0');
+                if (s == digits || s >= eol || *s != ':') { out.bad = true; return; }
+                if (neg) idx = -idx;
+                p = s + 1;
+                const float v = parse_float(p, eol, &q);
+                if (q == p) { out.bad = true; return; }
+                p = q;
+                row.emplace_back((int) idx, (kernel_type) v);
+                if (idx == 0) out.zero_based = true;
+                if (idx > 0 && (size_t) idx > out.max_index) out.max_index = (size_t) idx;
+            }
+            out.rows.emplace_back(row.begin(), row.end());
+        }
+        p = eol + 1;
+    }
+}
+
+}  // namespace
+
+void DataSet::load_from_file(std::string file_name, int n_threads) {
     device_slot_ = std::make_shared<std::shared_ptr<void>>();   // new instances: any device copy is stale
     y_.clear();
     instances_.clear();
     n_features_ = 0;
     zero_based_ = false;
-    std::ifstream in(file_name, std::ios::binary);
-    if (!in.is_open()) throw std::runtime_error("file " + file_name + " not found");
-    std::string text((std::istreambuf_iterator<char>(in)), std::istreambuf_iterator<char>());
-    const char *p = text.c_str();
-    const char *end = p + text.size();
-    while (p < end) {
-        const char *eol = (const char *) memchr(p, '\n', end - p);
-        if (!eol) eol = end;
-        while (p < eol && (*p == ' ' || *p == '\t' || *p == '\r')) ++p;
-        if (p < eol) {
-            char *q;
-            y_.push_back(strtod(p, &q));
-            instances_.emplace_back();
-            auto &row = instances_.back();
-            p = q;
-            while (p < eol) {
-                while (p < eol && (*p == ' ' || *p == '\t' || *p == '\r')) ++p;
-                if (p >= eol) break;
-                long idx = strtol(p, &q, 10);
-                if (q == p || *q != ':') throw std::runtime_error("read error, using [index]:[value] format");
-                p = q + 1;
-                float v = strtof(p, &q);
-                if (q == p) throw std::runtime_error("read error, using [index]:[value] format");
-                p = q;
-                row.emplace_back((int) idx, (kernel_type) v);
-                if (idx == 0) zero_based_ = true;
-                if ((size_t) idx > n_features_) n_features_ = idx;
+    if (n_threads <= 0) n_threads = omp_get_max_threads();
+    const int fd = open(file_name.c_str(), O_RDONLY);
+    if (fd < 0) throw std::runtime_error("file " + file_name + " not found");
+    struct stat st;
+    if (fstat(fd, &st) != 0) { close(fd); throw std::runtime_error("file " + file_name + " cannot be read"); }
+    const size_t size = (size_t) st.st_size;
+    std::unique_ptr<char[]> text(new char[size + 1]);
+    text[size] = 0;
+    bool read_ok = true;
+    const size_t piece = (size + n_threads - 1) / std::max(n_threads, 1);
+#pragma omp parallel for num_threads(n_threads) schedule(static, 1)
+    for (int t = 0; t < n_threads; ++t) {
+        size_t off = std::min(size, (size_t) t * piece);
+        const size_t stop = std::min(size, off + piece);
+        while (off < stop) {
+            const ssize_t got = pread(fd, text.get() + off, stop - off, (off_t) off);
+            if (got <= 0) {
+#pragma omp atomic write
+                read_ok = false;
+                break;
             }
+            off += (size_t) got;
         }
-        p = eol + 1;
+    }
+    close(fd);
+    if (!read_ok) throw std::runtime_error("file " + file_name + " cannot be read");
+    // runs of whole lines: run r starts behind the first newline at or after byte r * size / n_runs
+    const int n_runs = n_threads == 1 ? 1 : n_threads * 4;
+    std::vector<size_t> cut(n_runs + 1, size);
+    cut[0] = 0;
+    for (int r = 1; r < n_runs; ++r) {
+        const size_t from = std::max(cut[r - 1], size / n_runs * r);
+        const char *nl = from < size ? (const char *) memchr(text.get() + from, '\n', size - from) : nullptr;
+        cut[r] = nl ? (size_t) (nl - text.get()) + 1 : size;
+    }
+    std::vector<LoadedRun> runs(n_runs);
+#pragma omp parallel for num_threads(n_threads) schedule(dynamic, 1)
+    for (int r = 0; r < n_runs; ++r) parse_run(text.get() + cut[r], text.get() + cut[r + 1], runs[r]);
+    size_t total = 0;
+    for (const LoadedRun &r : runs) {
+        if (r.bad) throw std::runtime_error("read error, using [index]:[value] format");
+        total += r.rows.size();
+        if (r.max_index > n_features_) n_features_ = r.max_index;
+        zero_based_ = zero_based_ || r.zero_based;
+    }
+    y_.reserve(total);
+    instances_.reserve(total);
+    for (LoadedRun &r : runs) {
+        y_.insert(y_.end(), r.y.begin(), r.y.end());
+        for (auto &row : r.rows) instances_.push_back(std::move(row));
     }
     TSVM_LOG << "#instances = " << n_instances() << ", #features = " << n_features();
 }

@@ -18,7 +18,9 @@ public:
     DataSet() = default;
     DataSet(const node2d &instances, int n_features, const std::vector<float_type> &y);
 
-    void load_from_file(std::string file_name);
+    // n_threads: threads that read and parse (0: as many as OpenMP would start, which the `-o` option sets, as in
+    // the reference)
+    void load_from_file(std::string file_name, int n_threads = 0);
     void load_from_python(float *y, char **x, int len);
     void load_from_sparse(int row_size, float *val, int *row_ptr, int *col_ptr, float *label);
     void load_from_dense(int row_size, int features, float *data, float *label);

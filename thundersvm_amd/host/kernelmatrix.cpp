@@ -189,22 +189,32 @@ const std::vector<int> &DeviceRows::column_stats() const {
     return column_stats_;
 }
 
-// The trailing run of columns whose values are all 0 or 1, if leaving it out of the matrix product saves more than
-// the additions it costs in the epilogue: one 4-column step of the matrix cores per value is worth about one
-// epilogue instruction, an indicator column that may match costs about three.
+// The trailing run of columns whose values are all 0 or 1 (at most 64 of them): its first column, n_features when
+// the last column is not such a column.  stats: the 2 * n_features counts of column_stats().
+int DeviceRows::indicator_run_start(const int *stats, int n_features) {
+    int first = n_features;
+    while (first > 0 && n_features - first < 64 && stats[n_features + first - 1] == 0) --first;
+    return first;
+}
+
+// Leaving the run to the kernel's epilogue pays when it saves more than the additions cost there: one 4-column step
+// of the matrix cores per value is worth about one epilogue instruction, an indicator column that may match about three.
+bool DeviceRows::indicator_run_pays(int n_features, int first, int max_ones) {
+    const int steps_saved = (n_features + 3) / 4 - (first + 3) / 4;
+    return steps_saved >= 2 + 3 * max_ones;
+}
+
 void DeviceRows::find_indicator_columns() {
     ind_first = -1;
     if (!dense || n == 0 || n_features == 0 || getenv("TSVM_NO_INDICATOR")) return;
     const std::vector<int> &stats = column_stats();
-    int first = (int) n_features;
-    while (first > 0 && (int) n_features - first < 64 && stats[n_features + first - 1] == 0) --first;
+    const int first = indicator_run_start(stats.data(), (int) n_features);
     if (first == (int) n_features) return;
     tsvm::DeviceBuffer<uint64_t> masks(n);
     tsvm::DeviceBuffer<int> d_max(1);
     abi_check(tsvm_indicator_masks(x.data(), ld, (int64_t) n, first, (int) n_features - first, masks.data(), d_max.data(), nullptr));
     const int max_ones = d_max.to_host()[0];
-    const int steps_saved = (int) ((n_features + 3) / 4) - (first + 3) / 4;
-    if (steps_saved < 2 + 3 * max_ones) return;
+    if (!indicator_run_pays((int) n_features, first, max_ones)) return;
     ind_first = first;
     ind_max_ones = max_ones;
     ind_mask = std::move(masks);

@@ -43,6 +43,8 @@ struct DeviceRows {
     int ind_first = -1, ind_max_ones = 0;
     tsvm::DeviceBuffer<uint64_t> ind_mask;       // [n]
     void find_indicator_columns();
+    static int indicator_run_start(const int *stats, int n_features);
+    static bool indicator_run_pays(int n_features, int first, int max_ones);
 
     // rows[0..n_rows) of `all` (rows == nullptr: the first n_rows), assembled on the host and uploaded
     static std::shared_ptr<DeviceRows> from_host(const DataSet::node2d &all, const int *rows, size_t n_rows);

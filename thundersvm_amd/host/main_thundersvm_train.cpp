@@ -19,7 +19,9 @@ int main(int argc, char **argv) {
     try {
         tsvm::Log::enabled() = !parser.quiet;
         DataSet train;
+        auto t_load = std::chrono::high_resolution_clock::now();
         train.load_from_file(parser.svmtrain_input_file_name);
+        TSVM_LOG << "data loading time = " << std::chrono::duration<float>(std::chrono::high_resolution_clock::now() - t_load).count();
         std::unique_ptr<SvmModel> model = make_model(parser.param_cmd.svm_type);
         if (parser.param_cmd.svm_type == SvmParam::NU_SVC) {   // feasibility of nu (thundersvm-train.cpp:57-70)
             train.group_classes();
@@ -49,7 +51,9 @@ int main(int argc, char **argv) {
             model->train(train, parser.param_cmd);
             std::chrono::duration<float> dt = std::chrono::high_resolution_clock::now() - start;
             TSVM_LOG << "all training time = " << dt.count();
+            auto t_save = std::chrono::high_resolution_clock::now();
             model->save_to_file(parser.model_file_name);
+            TSVM_LOG << "model saving time = " << std::chrono::duration<float>(std::chrono::high_resolution_clock::now() - t_save).count();
         }
     } catch (std::bad_alloc &) {
         fprintf(stderr, "out of memory, you may try \"-m memory size\" to constrain memory usage\n");

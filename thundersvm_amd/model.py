@@ -60,6 +60,15 @@ def host_lib():
         L.tsvm_dataset_new_csr.argtypes = [C.c_int64, _i64p, _ip, _dp, _dp]
         L.tsvm_dataset_load.restype = C.c_void_p
         L.tsvm_dataset_load.argtypes = [C.c_char_p]
+        L.tsvm_dataset_load_threads.restype = C.c_void_p
+        L.tsvm_dataset_load_threads.argtypes = [C.c_char_p, C.c_int]
+        L.tsvm_dataset_info.restype = C.c_int64
+        L.tsvm_dataset_info.argtypes = [C.c_void_p, _i64p, _ip, _ip]
+        L.tsvm_dataset_get_csr.restype = None
+        L.tsvm_dataset_get_csr.argtypes = [C.c_void_p, _i64p, _ip, _dp, _dp]
+        L.tsvm_rule_choose_dense.argtypes = [C.c_int64, C.c_int64, C.c_int64]
+        L.tsvm_rule_indicator_run_start.argtypes = [_ip, C.c_int]
+        L.tsvm_rule_indicator_run_pays.argtypes = [C.c_int, C.c_int, C.c_int]
         L.tsvm_dataset_free.argtypes = [C.c_void_p]
         L.tsvm_dataset_rows.restype = C.c_int64
         L.tsvm_dataset_rows.argtypes = [C.c_void_p]
@@ -81,6 +90,21 @@ def host_lib():
     return _HOST
 
 
+def choose_dense(n, n_features, nnz):
+    """KernelMatrix::choose_dense of the host layer: dense row-major rows (True) or CSR."""
+    return bool(host_lib().tsvm_rule_choose_dense(n, n_features, nnz))
+
+
+def indicator_run(column_stats, n_features, max_ones=None):
+    """First column of the trailing run of 0/1 columns (the host layer's rule, from tsvm_column_stats_dense's counts);
+    with max_ones also whether get_rows leaves the run to its epilogue."""
+    counts = np.ascontiguousarray(column_stats, dtype=np.int32)
+    first = host_lib().tsvm_rule_indicator_run_start(_p(counts, _ip), n_features)
+    if max_ones is None:
+        return first
+    return first, bool(host_lib().tsvm_rule_indicator_run_pays(n_features, first, max_ones))
+
+
 def _check(rc):
     if rc != 0:
         msg = host_lib().tsvm_model_last_error().decode()
@@ -96,10 +120,10 @@ def _p(a, t):
 class Dataset:
     """Rows held by the host layer's DataSet (converted once, reusable across train / predict calls)."""
 
-    def __init__(self, data=None, path=None):
+    def __init__(self, data=None, path=None, threads=0):
         L = host_lib()
         if path is not None:
-            self.h = C.c_void_p(L.tsvm_dataset_load(path.encode()))
+            self.h = C.c_void_p(L.tsvm_dataset_load_threads(path.encode(), threads))
         else:
             y = None if data.y is None else np.ascontiguousarray(data.y, dtype=np.float64)
             self.h = C.c_void_p(L.tsvm_dataset_new_csr(data.n, _p(data.ptr, _i64p), _p(data.col, _ip), _p(data.val, _dp),
@@ -107,6 +131,19 @@ class Dataset:
         if not self.h:
             raise capi.TsvmError(L.tsvm_model_last_error().decode())
         self.n = L.tsvm_dataset_rows(self.h)
+
+    def csr(self):
+        """The rows as the DataSet holds them: CsrData with the stored feature ids, plus (n_features, zero_based)."""
+        from .data import CsrData
+        L = host_lib()
+        nf, zb, hl = C.c_int64(), C.c_int(), C.c_int()
+        nnz = L.tsvm_dataset_info(self.h, C.byref(nf), C.byref(zb), C.byref(hl))
+        ptr = np.zeros(self.n + 1, dtype=np.int64)
+        col = np.zeros(nnz, dtype=np.int32)
+        val = np.zeros(nnz)
+        y = np.zeros(self.n)
+        L.tsvm_dataset_get_csr(self.h, _p(ptr, _i64p), _p(col, _ip), _p(val, _dp), _p(y, _dp))
+        return CsrData(ptr, col, val, y if hl.value else None), nf.value, bool(zb.value)
 
     def to_device(self):
         """Uploads the rows to HBM now; training calls on this Dataset then start from device-resident data."""
