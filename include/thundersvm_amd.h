@@ -198,20 +198,22 @@ int tsvm_c_smo_solve_static(const int *y, const double *f_val, double *alpha, do
                             int ws_size, double Cp, double Cn, const void *k_rows, int row_type, const int *slots,
                             int64_t ld, const double *k_diag, double eps, double *diff, int max_iter, tsvm_stream stream);
 
-/* Row stride (in doubles) of the ws x ws block the solver kernels read: ws rounded up to 256, 512 or 1024. */
+/* Row stride (in elements) of the ws x ws block the solver kernels read: ws rounded up to 256, 512 or 1024.
+ * block_type below: element type of the block, TSVM_ROW_F64 or, when the kernel rows are float (their values are
+ * floats to begin with), TSVM_ROW_F32: the same numbers in half the bytes, widened when the solver loads them. */
 int tsvm_smo_solve_block_ld(int ws_size);
 
 /* The block from stored kernel rows: kws[r*ldk + t] = element cols[t] of the row in slot slots[r] (slots == NULL:
  * slot r), r, t < ws_size, ldk = tsvm_smo_solve_block_ld(ws_size), columns t >= ws_size zero-filled; the gather that
  * replaces the strided reads k_mat_rows[row_len*i + working_set[t]] of smo_kernel.cpp:50-52,107-110. */
 int tsvm_smo_gather_block(const void *k_rows, int row_type, const int *slots, int64_t ld, const int *cols, int ws_size,
-                          double *kws, tsvm_stream stream);
+                          void *kws, int block_type, tsvm_stream stream);
 
 /* The block when slot_of_id[i] names the slot that holds instance i's row (a row cache that holds every row):
  * kws[r*ldk + t] = element ids[t] of the row in slot slot_of_id[ids[r]]; slots_out[r] receives that slot (the
  * table tsvm_update_f takes).  Nothing has to come from the host between the selection and this call. */
 int tsvm_smo_gather_block_by_id(const void *k_rows, int row_type, const int *slot_of_id, int64_t ld, const int *ids,
-                                int ws_size, double *kws, int *slots_out, tsvm_stream stream);
+                                int ws_size, void *kws, int block_type, int *slots_out, tsvm_stream stream);
 
 /* Slots for the new rows of a working set, decided on the device, for a row store with a slot for every
  * instance (the reference recomputes the rows of every working set, csmosolver.cpp:65-77; rows kept here are the
@@ -228,10 +230,10 @@ int tsvm_row_slots_assign(const int *ids_new, int n_new, int *slot_of_id, int *s
  * else of the kernel matrix, so it can run while the full rows are still being computed on another
  * stream.  C is passed as Cp for the nu variant (Cn unused). */
 int tsvm_c_smo_solve_block(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
-                           int ws_size, double Cp, double Cn, const double *kws, const double *k_diag, double eps,
+                           int ws_size, double Cp, double Cn, const void *kws, int block_type, const double *k_diag, double eps,
                            double *diff, int max_iter, tsvm_stream stream);
 int tsvm_nu_smo_solve_block(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
-                            int ws_size, double C, const double *kws, const double *k_diag, double eps, double *diff,
+                            int ws_size, double C, const void *kws, int block_type, const double *k_diag, double eps, double *diff,
                             int max_iter, tsvm_stream stream);
 
 /* No counterpart in the reference: the two block solvers above, made to run on a chosen accelerator die (XCD, 0..7).
@@ -242,11 +244,11 @@ int tsvm_nu_smo_solve_block(const int *y, const double *f_val, double *alpha, do
  * stream only; epoch: 1 for the first launch on a gate, then one more per launch; gate[2] receives the XCD the
  * solver ran on. */
 int tsvm_c_smo_solve_block_on_xcd(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
-                                  int ws_size, double Cp, double Cn, const double *kws, const double *k_diag, double eps,
+                                  int ws_size, double Cp, double Cn, const void *kws, int block_type, const double *k_diag, double eps,
                                   double *diff, int max_iter, int *gate, int epoch, int xcd, tsvm_stream stream);
 int tsvm_nu_smo_solve_block_on_xcd(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
-                                   int ws_size, double C, const double *kws, const double *k_diag, double eps, double *diff,
-                                   int max_iter, int *gate, int epoch, int xcd, tsvm_stream stream);
+                                   int ws_size, double C, const void *kws, int block_type, const double *k_diag, double eps,
+                                   double *diff, int max_iter, int *gate, int epoch, int xcd, tsvm_stream stream);
 
 /* nu_smo_solve (smo_kernel.cpp:127-298), same conventions; diff[1] is left untouched as in the
  * reference's CPU code. */

@@ -413,11 +413,13 @@ def test_row_store_managed_on_the_device(n, d, ws):
         assert G.host(miss_ids)[:len(want_miss)].tolist() == want_miss
         assert np.array_equal(G.host(slot_of), h_slot_of)
         assert np.array_equal(G.host(slots_ws), h_slot_of[ws_ids])
-        kws = torch.full((ws, ldk), 3.0, dtype=torch.float64, device="cuda")
+        # the block as doubles and as floats (float rows: the same numbers), turn by turn
+        bt, bdt = (capi.ROW_F64, torch.float64) if it % 2 else (capi.ROW_F32, torch.float32)
+        kws = torch.full((ws, ldk), 3.0, dtype=bdt, device="cuda")
         out_slots = torch.zeros(ws, dtype=torch.int32, device="cuda")
         capi.call("tsvm_smo_gather_block_by_id", G.ptr(store), capi.ROW_F32, G.ptr(slot_of), ldo, G.ptr(ids_d), ws, G.ptr(kws),
-                  G.ptr(out_slots), G.stream())
-        got = G.host(kws)
+                  bt, G.ptr(out_slots), G.stream())
+        got = G.host(kws).astype(np.float64)
         assert np.array_equal(got[:, :ws], all_rows[np.ix_(ws_ids, ws_ids)].astype(np.float64)) and (got[:, ws:] == 0).all()
         assert np.array_equal(G.host(out_slots), h_slot_of[ws_ids])
     assert used == n                                       # every instance has been seen: the store is complete
@@ -446,6 +448,13 @@ def test_working_set_block(name, kt, prm, n, d, ws):
     assert np.array_equal(got[:, :ws], rows[:, ids])
     assert np.array_equal(got[:, :ws], got[:, :ws].T)
     assert (got[:, ws:] == 9.0).all()
+    if kt != O.LINEAR:      # kernel values that are floats by definition: the block as float elements holds the same numbers
+        blk32 = torch.full((ws, ldk), 9.0, dtype=torch.float32, device="cuda")
+        capi.call("tsvm_get_rows_dense", G.ptr(x_d), ld, G.ptr(ids_d), ws, nf, G.ptr(sd), G.ptr(x_d), ld, G.ptr(ids_d), ws, G.ptr(sd),
+                  kt, prm.get("gamma", 0.0), prm.get("coef0", 0.0), prm.get("degree", 3), G.ptr(blk32), capi.ROW_F32, None, ldk,
+                  G.stream())
+        got32 = G.host(blk32).astype(np.float64)
+        assert np.array_equal(got32[:, :ws], got[:, :ws]) and (got32[:, ws:] == 9.0).all()
 
 
 def _mixed_rows(rng, n, n_cont, groups):

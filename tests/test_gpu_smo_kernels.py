@@ -130,6 +130,13 @@ def test_nu_smo_solve(n, ws):
     assert G.host(diff_d)[0] == diff_want[0]
     assert np.array_equal(G.host(a_d), a_want)
     assert np.array_equal(G.host(ad_d), ad_want)
+    # the same rows held as float: a float block inside, identical result
+    a_d, k32_d = G.dev(alpha), G.dev(k_rows.astype(np.float32))
+    capi.call("tsvm_nu_smo_solve", G.ptr(y_d), G.ptr(f_d), G.ptr(a_d), G.ptr(ad_d), G.ptr(ws_d), ws, Cc, G.ptr(k32_d),
+              capi.ROW_F32, None, n, G.ptr(dg_d), eps, G.ptr(diff_d), 100000, G.ptr(wsp), G.stream())
+    assert G.host(diff_d)[0] == diff_want[0]
+    assert np.array_equal(G.host(a_d), a_want)
+    assert np.array_equal(G.host(ad_d), ad_want)
 
 
 @pytest.mark.parametrize("nu", [False, True])
@@ -150,18 +157,21 @@ def test_smo_solve_block_on_a_chosen_xcd(n, ws, nu):
     block = np.zeros((ws, ldk))
     block[:, :ws] = k_rows[:, ws_ids]
     y_d, f_d, ws_d, b_d, dg_d = G.dev(y), G.dev(f), G.dev(ws_ids), G.dev(block), G.dev(diag)
+    assert np.array_equal(block.astype(np.float32).astype(np.float64), block)     # RBF values: a float block holds the same numbers
+    b32_d = G.dev(block.astype(np.float32))
     gate = torch.zeros(4, dtype=torch.int32, device="cuda")
     seen = set()
     for epoch, xcd in enumerate([0, 3, 7, 5, 1, 2, 6, 4, 0, 0], start=1):
         a_d = G.dev(alpha)
         ad_d = torch.zeros(ws, dtype=torch.float64, device="cuda")
         diff_d = torch.zeros(2, dtype=torch.float64, device="cuda")
+        blk, bt = (b_d, capi.ROW_F64) if epoch % 2 else (b32_d, capi.ROW_F32)
         if nu:
             capi.call("tsvm_nu_smo_solve_block_on_xcd", G.ptr(y_d), G.ptr(f_d), G.ptr(a_d), G.ptr(ad_d), G.ptr(ws_d), ws, Cc,
-                      G.ptr(b_d), G.ptr(dg_d), eps, G.ptr(diff_d), 100000, G.ptr(gate), epoch, xcd, G.stream())
+                      G.ptr(blk), bt, G.ptr(dg_d), eps, G.ptr(diff_d), 100000, G.ptr(gate), epoch, xcd, G.stream())
         else:
             capi.call("tsvm_c_smo_solve_block_on_xcd", G.ptr(y_d), G.ptr(f_d), G.ptr(a_d), G.ptr(ad_d), G.ptr(ws_d), ws, Cc, Cc,
-                      G.ptr(b_d), G.ptr(dg_d), eps, G.ptr(diff_d), 100000, G.ptr(gate), epoch, xcd, G.stream())
+                      G.ptr(blk), bt, G.ptr(dg_d), eps, G.ptr(diff_d), 100000, G.ptr(gate), epoch, xcd, G.stream())
         g = G.host(gate)
         assert g[0] == epoch and g[1] == 8 * epoch and 0 <= g[2] < 8
         seen.add(int(g[2]))
@@ -171,9 +181,11 @@ def test_smo_solve_block_on_a_chosen_xcd(n, ws, nu):
     # bad arguments are refused
     lib = capi.kernel_lib()
     assert lib.tsvm_c_smo_solve_block_on_xcd(G.ptr(y_d), G.ptr(f_d), G.ptr(a_d), G.ptr(ad_d), G.ptr(ws_d), ws, Cc, Cc, G.ptr(b_d),
-                                             G.ptr(dg_d), eps, G.ptr(diff_d), 10, G.ptr(gate), 0, 0, G.stream()) != 0
+                                             capi.ROW_F64, G.ptr(dg_d), eps, G.ptr(diff_d), 10, G.ptr(gate), 0, 0, G.stream()) != 0
     assert lib.tsvm_c_smo_solve_block_on_xcd(G.ptr(y_d), G.ptr(f_d), G.ptr(a_d), G.ptr(ad_d), G.ptr(ws_d), ws, Cc, Cc, G.ptr(b_d),
-                                             G.ptr(dg_d), eps, G.ptr(diff_d), 10, G.ptr(gate), 1, 8, G.stream()) != 0
+                                             capi.ROW_F64, G.ptr(dg_d), eps, G.ptr(diff_d), 10, G.ptr(gate), 1, 8, G.stream()) != 0
+    assert lib.tsvm_c_smo_solve_block_on_xcd(G.ptr(y_d), G.ptr(f_d), G.ptr(a_d), G.ptr(ad_d), G.ptr(ws_d), ws, Cc, Cc, G.ptr(b_d),
+                                             7, G.ptr(dg_d), eps, G.ptr(diff_d), 10, G.ptr(gate), 1, 0, G.stream()) != 0
 
 
 def _select_case(n, n_select, n_marked, seed, tie_mode, nu):

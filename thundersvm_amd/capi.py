@@ -47,13 +47,13 @@ SIGNATURES = {
     "tsvm_c_smo_solve_static": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _dbl, _p, _int, _p, _i64, _p, _dbl, _p, _int, _p]),
     "tsvm_nu_smo_solve": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _p, _int, _p, _i64, _p, _dbl, _p, _int, _p, _p]),
     "tsvm_smo_solve_block_ld": (_int, [_int]),
-    "tsvm_smo_gather_block": (_int, [_p, _int, _p, _i64, _p, _int, _p, _p]),
+    "tsvm_smo_gather_block": (_int, [_p, _int, _p, _i64, _p, _int, _p, _int, _p]),
     "tsvm_row_slots_assign": (_int, [_p, _int, _p, _p, _p, _p, _p, _int, _p, _p, _p]),
-    "tsvm_smo_gather_block_by_id": (_int, [_p, _int, _p, _i64, _p, _int, _p, _p, _p]),
-    "tsvm_c_smo_solve_block": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _dbl, _p, _p, _dbl, _p, _int, _p]),
-    "tsvm_nu_smo_solve_block": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _p, _p, _dbl, _p, _int, _p]),
-    "tsvm_c_smo_solve_block_on_xcd": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _dbl, _p, _p, _dbl, _p, _int, _p, _int, _int, _p]),
-    "tsvm_nu_smo_solve_block_on_xcd": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _p, _p, _dbl, _p, _int, _p, _int, _int, _p]),
+    "tsvm_smo_gather_block_by_id": (_int, [_p, _int, _p, _i64, _p, _int, _p, _int, _p, _p]),
+    "tsvm_c_smo_solve_block": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _dbl, _p, _int, _p, _dbl, _p, _int, _p]),
+    "tsvm_nu_smo_solve_block": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _p, _int, _p, _dbl, _p, _int, _p]),
+    "tsvm_c_smo_solve_block_on_xcd": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _dbl, _p, _int, _p, _dbl, _p, _int, _p, _int, _int, _p]),
+    "tsvm_nu_smo_solve_block_on_xcd": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _p, _int, _p, _dbl, _p, _int, _p, _int, _int, _p]),
     "tsvm_select_workspace": (C.c_size_t, [_i64]),
     "tsvm_select_working_set": (_int, [_p, _p, _p, _i64, _dbl, _dbl, _p, _int, _p, _int, _int, _p, _p]),
     "tsvm_select_working_set_again": (_int, [_p, _p, _p, _i64, _dbl, _dbl, _p, _int, _p, _int, _int, _p, _p]),

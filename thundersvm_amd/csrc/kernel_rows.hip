@@ -354,10 +354,10 @@ __global__ void indicator_masks_kernel(const double *__restrict__ x, int64_t ld,
 // diagonal are filled by the mirror writes of the others and get no workgroup.  Column tile j (128 wide) needs the
 // 64-row tiles 0 .. 2j+1, so workgroup c works on column tile j = the largest j with j(j+1) <= c, row tile
 // c - j(j+1); dealt out in this order, every XCD gets the same share of the work.
-template <int KT>
+template <int KT, typename TO>
 __global__ __launch_bounds__(256, 3) void get_rows_dense_sym_kernel(
     const double *__restrict__ x, int64_t ldx, const int *__restrict__ idx, int m, int d, const double *__restrict__ sd_x,
-    KernelParam kp, double *__restrict__ out, int64_t ldo, unsigned m_blocks) {
+    KernelParam kp, TO *__restrict__ out, int64_t ldo, unsigned m_blocks) {
     __shared__ double As[GrShape<2>::LDS_DOUBLES];
     __shared__ double Bs[GrShape<2>::LDS_DOUBLES];
     __shared__ uint64_t exp_tab[32];
@@ -370,7 +370,7 @@ __global__ __launch_bounds__(256, 3) void get_rows_dense_sym_kernel(
     if (i0 >= m) return;               // (the last column tile has fewer row tiles when m is not a multiple of 128)
     if (threadIdx.x < 32) exp_tab[threadIdx.x] = TSVM_EXP2F_TAB[threadIdx.x];
     __syncthreads();
-    get_rows_tile<KT, 2, double, true>(x, ldx, idx, m, d, sd_x, x, ldx, idx, m, sd_x, kp, out, nullptr, ldo, i0, j0, As, Bs, exp_tab);
+    get_rows_tile<KT, 2, TO, true>(x, ldx, idx, m, d, sd_x, x, ldx, idx, m, sd_x, kp, out, nullptr, ldo, i0, j0, As, Bs, exp_tab);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -771,27 +771,27 @@ static int get_rows_dense(const double *x, int64_t ldx, const int *x_idx, int64_
     dim3 grid((unsigned) (n_blocks * m_blocks)), block(256);
     // the solver's ws x ws block: symmetric, computed from the tiles on and above the diagonal
     const bool sym = x == a && ldx == lda && x_idx && x_idx == a_idx && n == m && sd_x == sd_a && !out_slots && !m_dev &&
-                     row_type == TSVM_ROW_F64 && ti == 2 && ldo >= n;
+                     ti == 2 && ldo >= n;
     if (sym) {
         grid = dim3((unsigned) (n_blocks * (n_blocks + 1)));   // column tile j: row tiles 0 .. 2j+1
-        switch (kernel_type) {
-            case TSVM_LINEAR:
-                hipLaunchKernelGGL(get_rows_dense_sym_kernel<TSVM_LINEAR>, grid, block, 0, tsvm_s(stream), x, ldx, x_idx, m, d, sd_x,
-                                   kp, (double *) out, ldo, m_blocks);
-                break;
-            case TSVM_POLY:
-                hipLaunchKernelGGL(get_rows_dense_sym_kernel<TSVM_POLY>, grid, block, 0, tsvm_s(stream), x, ldx, x_idx, m, d, sd_x, kp,
-                                   (double *) out, ldo, m_blocks);
-                break;
-            case TSVM_SIGMOID:
-                hipLaunchKernelGGL(get_rows_dense_sym_kernel<TSVM_SIGMOID>, grid, block, 0, tsvm_s(stream), x, ldx, x_idx, m, d, sd_x,
-                                   kp, (double *) out, ldo, m_blocks);
-                break;
-            default:
-                hipLaunchKernelGGL(get_rows_dense_sym_kernel<TSVM_RBF>, grid, block, 0, tsvm_s(stream), x, ldx, x_idx, m, d, sd_x, kp,
-                                   (double *) out, ldo, m_blocks);
-                break;
+#define GR_SYM(KTYPE, TO)                                                                                                      \
+    hipLaunchKernelGGL((get_rows_dense_sym_kernel<KTYPE, TO>), grid, block, 0, tsvm_s(stream), x, ldx, x_idx, m, d, sd_x, kp, (TO *) out, \
+                       ldo, m_blocks)
+        if (row_type == TSVM_ROW_F32) {
+            switch (kernel_type) {
+                case TSVM_POLY: GR_SYM(TSVM_POLY, float); break;
+                case TSVM_SIGMOID: GR_SYM(TSVM_SIGMOID, float); break;
+                default: GR_SYM(TSVM_RBF, float); break;
+            }
+        } else {
+            switch (kernel_type) {
+                case TSVM_LINEAR: GR_SYM(TSVM_LINEAR, double); break;
+                case TSVM_POLY: GR_SYM(TSVM_POLY, double); break;
+                case TSVM_SIGMOID: GR_SYM(TSVM_SIGMOID, double); break;
+                default: GR_SYM(TSVM_RBF, double); break;
+            }
         }
+#undef GR_SYM
         TSVM_LAUNCH_CHECK();
         return 0;
     }

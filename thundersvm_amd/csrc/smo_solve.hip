@@ -2,8 +2,8 @@
 // USE_CUDA=OFF semantics) as one LDS-resident workgroup on gfx950.
 //
 // Shape of the kernel.  One workgroup of 256 threads (one wavefront per SIMD of the CU) holds the
-// whole working set: element t = e*256 + tid lives in register slot e of thread tid (E = ws/256
-// slots, up to 4) with its f and diagonal; alpha lives in LDS (only two entries change per
+// whole working set: element t = tid*E + e lives in register slot e of thread tid (E = ws/256
+// slots, up to 4: a thread's elements are neighbours, so its share of a block row is one load) with its f and diagonal; alpha lives in LDS (only two entries change per
 // iteration) and the I_up / I_low membership of a thread's elements is a bit field in one register.
 // One inner iteration is
 //   1. (i, up) = first argmin of f over I_up and low = max of f over I_low: a per-thread scan of
@@ -37,25 +37,27 @@
 // reads, gathered once per call so that the two row reads per inner iteration
 // (smo_kernel.cpp:50-52,107-110) are contiguous; rows are padded to the solver's thread x slot grid
 // so every thread can load without a bounds test.
-template <typename TK>
+// TB: element type of the block.  Float kernel rows give a float block: the same values in half the bytes, widened
+// again when the solver loads them.
+template <typename TK, typename TB>
 __global__ void gather_ws_block_kernel(const TK *__restrict__ k_rows, const int *__restrict__ slots, int64_t ld,
-                                       const int *__restrict__ working_set, int ws, int ldk, double *__restrict__ kws) {
+                                       const int *__restrict__ working_set, int ws, int ldk, TB *__restrict__ kws) {
     const int r = blockIdx.x;
     const TK *row = k_rows + (int64_t) (slots ? slots[r] : r) * ld;
-    for (int t = threadIdx.x; t < ldk; t += blockDim.x) kws[(int64_t) r * ldk + t] = t < ws ? (double) row[working_set[t]] : 0.0;
+    for (int t = threadIdx.x; t < ldk; t += blockDim.x) kws[(int64_t) r * ldk + t] = t < ws ? (TB) row[working_set[t]] : (TB) 0;
 }
 
 // The same block when a table names the slot of every instance's row (a row cache that holds them all): row r
 // is the one of instance ids[r]; its slot is also written to slots_out[r], for update_f.
-template <typename TK>
+template <typename TK, typename TB>
 __global__ void gather_ws_block_by_id_kernel(const TK *__restrict__ k_rows, const int *__restrict__ slot_of_id, int64_t ld,
-                                             const int *__restrict__ ids, int ws, int ldk, double *__restrict__ kws,
+                                             const int *__restrict__ ids, int ws, int ldk, TB *__restrict__ kws,
                                              int *__restrict__ slots_out) {
     const int r = blockIdx.x;
     const int slot = slot_of_id[ids[r]];
     if (threadIdx.x == 0) slots_out[r] = slot;
     const TK *row = k_rows + (int64_t) slot * ld;
-    for (int t = threadIdx.x; t < ldk; t += blockDim.x) kws[(int64_t) r * ldk + t] = t < ws ? (double) row[ids[t]] : 0.0;
+    for (int t = threadIdx.x; t < ldk; t += blockDim.x) kws[(int64_t) r * ldk + t] = t < ws ? (TB) row[ids[t]] : (TB) 0;
 }
 
 // Slots for a working set's new rows when the row store has a slot for every instance (nothing is ever
@@ -132,25 +134,40 @@ __device__ __forceinline__ void wave_first_argmin(const double (&x)[E], int tid,
     m = wave_min_f64(m);
     int r = MAX_WS;
 #pragma unroll
-    for (int e = E - 1; e >= 0; --e) r = x[e] == m ? e * SV_T + tid : r;
+    for (int e = E - 1; e >= 0; --e) r = x[e] == m ? tid * E + e : r;
     idx = wave_min_i32(r);
     v = m;
 }
 
 // Replaces the `width` membership bits of element t in the bit field of the thread that owns it.
+template <int E>
 __device__ __forceinline__ unsigned set_member_bits(unsigned m, int tid, int t, unsigned bits, int width) {
-    const int sh = (t / SV_T) * width;
+    const int sh = (t % E) * width;
     const unsigned field = ((1u << width) - 1u) << sh;
-    return tid == (t & (SV_T - 1)) ? ((m & ~field) | (bits << sh)) : m;
+    return tid == t / E ? ((m & ~field) | (bits << sh)) : m;
+}
+
+// A thread's E consecutive elements of a block row: one 4E- or 8E-byte load, widened to double.
+template <int E, typename TB>
+__device__ __forceinline__ void load_row_elems(const TB *__restrict__ row, int tid, double (&out)[E]) {
+    if constexpr (E == 1) {
+        out[0] = (double) row[tid];
+    } else {
+        typedef TB vec_t __attribute__((ext_vector_type(E)));
+        const vec_t v = *(const vec_t *) (row + tid * E);
+#pragma unroll
+        for (int e = 0; e < E; ++e) out[e] = (double) v[e];
+    }
 }
 
 // Each wavefront knows its own best candidate a barrier and an LDS round trip before the workgroup
 // knows the winner, and the winner is always one of the four.  One load per lane, 128 bytes apart,
-// touches every cache line of a candidate's 8 KB row, so the row the workgroup then reads is already
-// on its way into the CU's L1 / the XCD's L2.  A wavefront without a candidate reports an index
+// touches every cache line of a candidate's row, so the row the workgroup then reads is already
+// on its way into the CU's L1 / the XCD's L2 (the four candidates' rows of a float block, 4 KB each, fit the L1 together).
+// A wavefront without a candidate reports an index
 // that may lie beyond the block's ws rows (an inactive element or MAX_WS): it touches row 0 instead.
 #define TSVM_TOUCH_ROW(kws, t, ws, ldk, lane) \
-    (((const unsigned *) ((kws) + (int64_t) ((t) < (ws) ? (t) : 0) * (ldk)))[(lane) * 32 < (ldk) * 2 ? (lane) * 32 : 0])
+    (((const unsigned *) ((kws) + (int64_t) ((t) < (ws) ? (t) : 0) * (ldk)))[(lane) * 32 < (int) ((ldk) * sizeof(*(kws)) / 4) ? (lane) * 32 : 0])
 
 // One solver on a chosen XCD.  A kernel of one workgroup runs on whichever XCD its stream's hardware queue starts
 // dealing at; launched as eight workgroups under a CU mask with one CU per XCD, one workgroup lands on every XCD, and
@@ -180,11 +197,11 @@ __device__ __forceinline__ bool solver_elected(int *gate, int epoch, int target_
 }
 
 // Elements beyond ws are given y = 0, which puts them in neither I_up nor I_low.
-template <int E>
+template <int E, typename TB>
 __global__ __launch_bounds__(SV_T) void c_smo_solve_kernel(
     const int *__restrict__ label, const double *__restrict__ f_val, double *__restrict__ alpha,
     double *__restrict__ alpha_diff, const int *__restrict__ working_set, int ws, double Cp, double Cn,
-    const double *__restrict__ kws, const double *__restrict__ k_diag, double eps, double *__restrict__ diff,
+    const TB *__restrict__ kws, const double *__restrict__ k_diag, double eps, double *__restrict__ diff,
     int max_iter, int *__restrict__ gate, int epoch, int target_xcd) {
     if (gate && !solver_elected(gate, epoch, target_xcd)) return;
     constexpr int LDK = E * SV_T;
@@ -204,7 +221,7 @@ __global__ __launch_bounds__(SV_T) void c_smo_solve_kernel(
     unsigned member = 0;   // bit 2e: element e is in I_up; bit 2e+1: in I_low
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-        const int t = e * SV_T + tid;
+        const int t = tid * E + e;
         const bool active = t < ws;
         const int w = active ? working_set[t] : 0;
         f[e] = active ? f_val[w] : 0.0;
@@ -254,7 +271,7 @@ __global__ __launch_bounds__(SV_T) void c_smo_solve_kernel(
         double fu[E];
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            s_f[par][e * SV_T + tid] = f[e];
+            s_f[par][tid * E + e] = f[e];
             fu[e] = (member >> (2 * e)) & 1u ? f[e] : TSVM_INF;
         }
         double v;
@@ -271,10 +288,9 @@ __global__ __launch_bounds__(SV_T) void c_smo_solve_kernel(
         int i;
         block_argmin(sA_v, sA_i, up_value, i, MAX_WS);
         i = up_value < TSVM_INF ? i : 0;
-        const double *row_i = kws + (int64_t) i * LDK;
+        const TB *row_i = kws + (int64_t) i * LDK;
         double kI[E];
-#pragma unroll
-        for (int e = 0; e < E; ++e) kI[e] = row_i[e * SV_T + tid];
+        load_row_elems<E, TB>(row_i, tid, kI);
         const double kd_i = s_kd[i];
         // j2 = first argmin of -b^2/a over I_low with f > up (smo_kernel.cpp:77-90)
         double qs[E];
@@ -303,11 +319,10 @@ __global__ __launch_bounds__(SV_T) void c_smo_solve_kernel(
         int j2;
         block_argmin(sB_v, sB_i, min_t, j2, MAX_WS);
         j2 = min_t < TSVM_INF ? j2 : 0;
-        const double *row_j = kws + (int64_t) j2 * LDK;
+        const TB *row_j = kws + (int64_t) j2 * LDK;
         double kJ[E];
-#pragma unroll
-        for (int e = 0; e < E; ++e) kJ[e] = row_j[e * SV_T + tid];
-        const double kIj = row_i[j2];
+        load_row_elems<E, TB>(row_j, tid, kJ);
+        const double kIj = (double) row_i[j2];
         // two-variable step (smo_kernel.cpp:92-103)
         const double a_i = s_a[i], y_i = (double) s_y[i];
         const double a_j0 = s_a[j2], y_j = (double) s_y[j2];
@@ -318,8 +333,8 @@ __global__ __launch_bounds__(SV_T) void c_smo_solve_kernel(
         const double l = alpha_i_diff < alpha_j_diff ? alpha_i_diff : alpha_j_diff;
         const double na_i = a_i + l * y_i;
         const double na_j = (j2 == i ? na_i : a_j0) - l * y_j;
-        member = set_member_bits(member, tid, i, (is_I_up(na_i, y_i, Cp, Cn) ? 1u : 0u) | (is_I_low(na_i, y_i, Cp, Cn) ? 2u : 0u), 2);
-        member = set_member_bits(member, tid, j2, (is_I_up(na_j, y_j, Cp, Cn) ? 1u : 0u) | (is_I_low(na_j, y_j, Cp, Cn) ? 2u : 0u), 2);
+        member = set_member_bits<E>(member, tid, i, (is_I_up(na_i, y_i, Cp, Cn) ? 1u : 0u) | (is_I_low(na_i, y_i, Cp, Cn) ? 2u : 0u), 2);
+        member = set_member_bits<E>(member, tid, j2, (is_I_up(na_j, y_j, Cp, Cn) ? 1u : 0u) | (is_I_low(na_j, y_j, Cp, Cn) ? 2u : 0u), 2);
         pend_i = i;
         pend_j = j2;
         pend_ai = na_i;
@@ -332,7 +347,7 @@ __global__ __launch_bounds__(SV_T) void c_smo_solve_kernel(
     __syncthreads();   // the pending alpha writes of the last step were made before the loop's exit test
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-        const int t = e * SV_T + tid;
+        const int t = tid * E + e;
         if (t < ws) {
             const double a = s_a[t];
             alpha_diff[t] = -(a - a_old[e]) * (double) s_y[t];
@@ -356,11 +371,11 @@ __device__ __forceinline__ unsigned nu_member_bits(double a, double y, double C)
     return (y > 0 && a < C ? 1u : 0u) | (y < 0 && a > 0 ? 2u : 0u) | (y > 0 && a > 0 ? 4u : 0u) | (y < 0 && a < C ? 8u : 0u);
 }
 
-template <int E>
+template <int E, typename TB>
 __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
     const int *__restrict__ label, const double *__restrict__ f_val, double *__restrict__ alpha,
     double *__restrict__ alpha_diff, const int *__restrict__ working_set, int ws, double C,
-    const double *__restrict__ kws, const double *__restrict__ k_diag, double eps, double *__restrict__ diff,
+    const TB *__restrict__ kws, const double *__restrict__ k_diag, double eps, double *__restrict__ diff,
     int max_iter, int *__restrict__ gate, int epoch, int target_xcd) {
     if (gate && !solver_elected(gate, epoch, target_xcd)) return;
     constexpr int LDK = E * SV_T;
@@ -378,7 +393,7 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
     unsigned member = 0;
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-        const int t = e * SV_T + tid;
+        const int t = tid * E + e;
         const bool active = t < ws;
         const int w = active ? working_set[t] : 0;
         f[e] = active ? f_val[w] : 0.0;
@@ -428,7 +443,7 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
         double fup[E], fun[E];
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            s_f[par][e * SV_T + tid] = f[e];
+            s_f[par][tid * E + e] = f[e];
             const unsigned b = member >> (4 * e);
             fup[e] = b & 1u ? f[e] : TSVM_INF;
             fun[e] = b & 2u ? f[e] : TSVM_INF;
@@ -450,14 +465,11 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
         block_argmin(sA_vn, sA_in, up_value_n, in, MAX_WS);
         ip = up_value_p < TSVM_INF ? ip : 0;
         in = up_value_n < TSVM_INF ? in : 0;
-        const double *row_p = kws + (int64_t) ip * LDK;
-        const double *row_n = kws + (int64_t) in * LDK;
+        const TB *row_p = kws + (int64_t) ip * LDK;
+        const TB *row_n = kws + (int64_t) in * LDK;
         double kIp[E], kIn[E];
-#pragma unroll
-        for (int e = 0; e < E; ++e) {
-            kIp[e] = row_p[e * SV_T + tid];
-            kIn[e] = row_n[e * SV_T + tid];
-        }
+        load_row_elems<E, TB>(row_p, tid, kIp);
+        load_row_elems<E, TB>(row_n, tid, kIn);
         const double kd_ip = s_kd[ip];
         double qp[E], qn[E];
         bool go = false;   // max(low_p - up_p, low_n - up_n) >= local_eps (smo_kernel.cpp:185)
@@ -492,12 +504,11 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
         const int i = take_p ? ip : in;
         const int j2 = take_p ? j2p : j2n;
         const double up_value = take_p ? up_value_p : up_value_n;
-        const double *row_i = take_p ? row_p : row_n;
-        const double *row_j = kws + (int64_t) j2 * LDK;
+        const TB *row_i = take_p ? row_p : row_n;
+        const TB *row_j = kws + (int64_t) j2 * LDK;
         double kJ[E];
-#pragma unroll
-        for (int e = 0; e < E; ++e) kJ[e] = row_j[e * SV_T + tid];
-        const double kIj = row_i[j2];
+        load_row_elems<E, TB>(row_j, tid, kJ);
+        const double kIj = (double) row_i[j2];
         const double a_i = s_a[i], y_i = (double) s_y[i];
         const double a_j0 = s_a[j2], y_j = (double) s_y[j2];
         const double alpha_i_diff = y_i > 0 ? C - a_i : a_i;
@@ -507,8 +518,8 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
         const double l = alpha_i_diff < alpha_j_diff ? alpha_i_diff : alpha_j_diff;
         const double na_i = a_i + l * y_i;
         const double na_j = (j2 == i ? na_i : a_j0) - l * y_j;
-        member = set_member_bits(member, tid, i, nu_member_bits(na_i, y_i, C), 4);
-        member = set_member_bits(member, tid, j2, nu_member_bits(na_j, y_j, C), 4);
+        member = set_member_bits<E>(member, tid, i, nu_member_bits(na_i, y_i, C), 4);
+        member = set_member_bits<E>(member, tid, j2, nu_member_bits(na_j, y_j, C), 4);
         pend_i = i;
         pend_j = j2;
         pend_ai = na_i;
@@ -521,7 +532,7 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
     __syncthreads();
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-        const int t = e * SV_T + tid;
+        const int t = tid * E + e;
         if (t < ws) {
             const double a = s_a[t];
             alpha_diff[t] = -(a - a_old[e]) * (double) s_y[t];
@@ -556,21 +567,30 @@ size_t tsvm_smo_solve_workspace(int ws_size) {
     return sizeof(double) * (size_t) ws_size * (size_t) solver_ldk(ws_size) + 256;
 }
 
+// A float block needs float rows (a double row's values would be rounded).
+static bool block_type_ok(int block_type, int row_type) {
+    return block_type == TSVM_ROW_F64 || (block_type == TSVM_ROW_F32 && row_type == TSVM_ROW_F32);
+}
+
 static int launch_gather(const void *k_rows, int row_type, const int *slots, int64_t ld, const int *working_set, int ws,
-                         void *workspace, hipStream_t s) {
+                         void *workspace, int block_type, hipStream_t s) {
     TSVM_REQUIRE(row_type == TSVM_ROW_F64 || row_type == TSVM_ROW_F32, "smo_solve: unknown row type %d", row_type);
-    if (row_type == TSVM_ROW_F32)
-        hipLaunchKernelGGL(gather_ws_block_kernel<float>, dim3(ws), dim3(256), 0, s, (const float *) k_rows, slots, ld,
+    TSVM_REQUIRE(block_type_ok(block_type, row_type), "smo_solve: block type %d not valid for row type %d", block_type, row_type);
+    if (row_type == TSVM_ROW_F32 && block_type == TSVM_ROW_F32)
+        hipLaunchKernelGGL((gather_ws_block_kernel<float, float>), dim3(ws), dim3(256), 0, s, (const float *) k_rows, slots, ld,
+                           working_set, ws, solver_ldk(ws), (float *) workspace);
+    else if (row_type == TSVM_ROW_F32)
+        hipLaunchKernelGGL((gather_ws_block_kernel<float, double>), dim3(ws), dim3(256), 0, s, (const float *) k_rows, slots, ld,
                            working_set, ws, solver_ldk(ws), (double *) workspace);
     else
-        hipLaunchKernelGGL(gather_ws_block_kernel<double>, dim3(ws), dim3(256), 0, s, (const double *) k_rows, slots, ld,
+        hipLaunchKernelGGL((gather_ws_block_kernel<double, double>), dim3(ws), dim3(256), 0, s, (const double *) k_rows, slots, ld,
                            working_set, ws, solver_ldk(ws), (double *) workspace);
     TSVM_LAUNCH_CHECK();
     return 0;
 }
 
 // The attribute query and the dynamic-LDS opt-in are made once per kernel and device, not per launch.
-#define TSVM_LAUNCH_SOLVER(KERNEL, EVAL, ...)                                                       \
+#define TSVM_LAUNCH_SOLVER(KERNEL, EVAL, TB, ...)                                                   \
     do {                                                                                            \
         static thread_local int dev_done_ = -1;                                                     \
         static thread_local size_t dyn_ = 0;                                                        \
@@ -578,19 +598,32 @@ static int launch_gather(const void *k_rows, int row_type, const int *slots, int
         TSVM_HIP(hipGetDevice(&dev_));                                                              \
         if (dev_done_ != dev_) {                                                                    \
             hipFuncAttributes fa_;                                                                  \
-            TSVM_HIP(hipFuncGetAttributes(&fa_, reinterpret_cast<const void *>(KERNEL<EVAL>)));     \
-            TSVM_HIP(reserve_cu(KERNEL<EVAL>, fa_.sharedSizeBytes, &dyn_));                          \
+            TSVM_HIP(hipFuncGetAttributes(&fa_, reinterpret_cast<const void *>(KERNEL<EVAL, TB>))); \
+            TSVM_HIP(reserve_cu(KERNEL<EVAL, TB>, fa_.sharedSizeBytes, &dyn_));                      \
             dev_done_ = dev_;                                                                       \
         }                                                                                           \
-        hipLaunchKernelGGL(KERNEL<EVAL>, dim3(solver_grid_), dim3(SV_T), solver_grid_ == 1 ? dyn_ : 0, s, __VA_ARGS__); \
+        hipLaunchKernelGGL((KERNEL<EVAL, TB>), dim3(solver_grid_), dim3(SV_T), solver_grid_ == 1 ? dyn_ : 0, s, __VA_ARGS__); \
     } while (0)
 
-#define TSVM_DISPATCH_E(KERNEL, ...)                                                            \
+#define TSVM_DISPATCH_E_T(KERNEL, TB, ...)                                                      \
     do {                                                                                        \
-        if (ws_size <= SV_T) TSVM_LAUNCH_SOLVER(KERNEL, 1, __VA_ARGS__);                        \
-        else if (ws_size <= 2 * SV_T) TSVM_LAUNCH_SOLVER(KERNEL, 2, __VA_ARGS__);               \
-        else TSVM_LAUNCH_SOLVER(KERNEL, 4, __VA_ARGS__);                                        \
+        if (ws_size <= SV_T) TSVM_LAUNCH_SOLVER(KERNEL, 1, TB, __VA_ARGS__);                    \
+        else if (ws_size <= 2 * SV_T) TSVM_LAUNCH_SOLVER(KERNEL, 2, TB, __VA_ARGS__);           \
+        else TSVM_LAUNCH_SOLVER(KERNEL, 4, TB, __VA_ARGS__);                                    \
     } while (0)
+
+// (kws_: the block; block_type_: its element type)
+#define TSVM_DISPATCH_E(KERNEL, PRE, POST)                                                                           \
+    do {                                                                                                             \
+        if (block_type_ == TSVM_ROW_F32) {                                                                           \
+            const float *kws = (const float *) kws_;                                                                 \
+            TSVM_DISPATCH_E_T(KERNEL, float, TSVM_UNPACK PRE, kws, TSVM_UNPACK POST);                                \
+        } else {                                                                                                     \
+            const double *kws = (const double *) kws_;                                                               \
+            TSVM_DISPATCH_E_T(KERNEL, double, TSVM_UNPACK PRE, kws, TSVM_UNPACK POST);                               \
+        }                                                                                                            \
+    } while (0)
+#define TSVM_UNPACK(...) __VA_ARGS__
 
 int tsvm_c_smo_solve(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
                      int ws_size, double Cp, double Cn, const void *k_rows, int row_type, const int *slots, int64_t ld,
@@ -602,11 +635,12 @@ int tsvm_c_smo_solve(const int *y, const double *f_val, double *alpha, double *a
     hipStream_t s = tsvm_s(stream);
     int *gate_ = nullptr;
     const int epoch_ = 0, target_xcd_ = 0, solver_grid_ = 1;
-    int rc = launch_gather(k_rows, row_type, slots, ld, working_set, ws_size, workspace, s);
+    const int block_type_ = row_type;   // the block keeps the rows' element type
+    int rc = launch_gather(k_rows, row_type, slots, ld, working_set, ws_size, workspace, block_type_, s);
     if (rc) return rc;
-    const double *kws = (const double *) workspace;
-    TSVM_DISPATCH_E(c_smo_solve_kernel, y, f_val, alpha, alpha_diff, working_set, ws_size, Cp, Cn, kws, k_diag, eps, diff,
-                    max_iter, gate_, epoch_, target_xcd_);
+    const void *kws_ = workspace;
+    TSVM_DISPATCH_E(c_smo_solve_kernel, (y, f_val, alpha, alpha_diff, working_set, ws_size, Cp, Cn),
+                    (k_diag, eps, diff, max_iter, gate_, epoch_, target_xcd_));
     TSVM_LAUNCH_CHECK();
     return 0;
 }
@@ -650,11 +684,12 @@ int tsvm_c_smo_solve_static(const int *y, const double *f_val, double *alpha, do
     const int epoch_ = 0, target_xcd_ = 0, solver_grid_ = 1;
     // the gather writes every element of the ws x ldk block the solver reads (columns beyond ws as zeros), so
     // nothing of the previous call's content is read
-    rc = launch_gather(k_rows, row_type, slots, ld, working_set, ws_size, block, s);
+    const int block_type_ = row_type;
+    rc = launch_gather(k_rows, row_type, slots, ld, working_set, ws_size, block, block_type_, s);
     if (rc) return rc;
-    const double *kws = block;
-    TSVM_DISPATCH_E(c_smo_solve_kernel, y, f_val, alpha, alpha_diff, working_set, ws_size, Cp, Cn, kws, k_diag, eps, diff,
-                    max_iter, gate_, epoch_, target_xcd_);
+    const void *kws_ = block;
+    TSVM_DISPATCH_E(c_smo_solve_kernel, (y, f_val, alpha, alpha_diff, working_set, ws_size, Cp, Cn),
+                    (k_diag, eps, diff, max_iter, gate_, epoch_, target_xcd_));
     TSVM_LAUNCH_CHECK();
     return 0;
 }
@@ -662,23 +697,28 @@ int tsvm_c_smo_solve_static(const int *y, const double *f_val, double *alpha, do
 int tsvm_smo_solve_block_ld(int ws_size) { return ws_size < 1 ? 0 : solver_ldk(ws_size); }
 
 int tsvm_smo_gather_block(const void *k_rows, int row_type, const int *slots, int64_t ld, const int *cols, int ws_size,
-                          double *kws, tsvm_stream stream) {
+                          void *kws, int block_type, tsvm_stream stream) {
     TSVM_REQUIRE(k_rows && cols && kws, "tsvm_smo_gather_block: null pointer");
     TSVM_REQUIRE(ws_size >= 1 && ws_size <= MAX_WS, "tsvm_smo_gather_block: ws_size %d outside [1, %d]", ws_size, MAX_WS);
-    return launch_gather(k_rows, row_type, slots, ld, cols, ws_size, kws, tsvm_s(stream));
+    return launch_gather(k_rows, row_type, slots, ld, cols, ws_size, kws, block_type, tsvm_s(stream));
 }
 
 int tsvm_smo_gather_block_by_id(const void *k_rows, int row_type, const int *slot_of_id, int64_t ld, const int *ids,
-                                int ws_size, double *kws, int *slots_out, tsvm_stream stream) {
+                                int ws_size, void *kws, int block_type, int *slots_out, tsvm_stream stream) {
     TSVM_REQUIRE(k_rows && slot_of_id && ids && kws && slots_out, "tsvm_smo_gather_block_by_id: null pointer");
     TSVM_REQUIRE(ws_size >= 1 && ws_size <= MAX_WS, "tsvm_smo_gather_block_by_id: ws_size %d outside [1, %d]", ws_size, MAX_WS);
     TSVM_REQUIRE(row_type == TSVM_ROW_F64 || row_type == TSVM_ROW_F32, "tsvm_smo_gather_block_by_id: unknown row type %d", row_type);
-    if (row_type == TSVM_ROW_F32)
-        hipLaunchKernelGGL(gather_ws_block_by_id_kernel<float>, dim3(ws_size), dim3(256), 0, tsvm_s(stream), (const float *) k_rows,
-                           slot_of_id, ld, ids, ws_size, solver_ldk(ws_size), kws, slots_out);
+    TSVM_REQUIRE(block_type_ok(block_type, row_type), "tsvm_smo_gather_block_by_id: block type %d not valid for row type %d", block_type,
+                 row_type);
+    if (row_type == TSVM_ROW_F32 && block_type == TSVM_ROW_F32)
+        hipLaunchKernelGGL((gather_ws_block_by_id_kernel<float, float>), dim3(ws_size), dim3(256), 0, tsvm_s(stream),
+                           (const float *) k_rows, slot_of_id, ld, ids, ws_size, solver_ldk(ws_size), (float *) kws, slots_out);
+    else if (row_type == TSVM_ROW_F32)
+        hipLaunchKernelGGL((gather_ws_block_by_id_kernel<float, double>), dim3(ws_size), dim3(256), 0, tsvm_s(stream),
+                           (const float *) k_rows, slot_of_id, ld, ids, ws_size, solver_ldk(ws_size), (double *) kws, slots_out);
     else
-        hipLaunchKernelGGL(gather_ws_block_by_id_kernel<double>, dim3(ws_size), dim3(256), 0, tsvm_s(stream), (const double *) k_rows,
-                           slot_of_id, ld, ids, ws_size, solver_ldk(ws_size), kws, slots_out);
+        hipLaunchKernelGGL((gather_ws_block_by_id_kernel<double, double>), dim3(ws_size), dim3(256), 0, tsvm_s(stream),
+                           (const double *) k_rows, slot_of_id, ld, ids, ws_size, solver_ldk(ws_size), (double *) kws, slots_out);
     TSVM_LAUNCH_CHECK();
     return 0;
 }
@@ -696,55 +736,61 @@ int tsvm_row_slots_assign(const int *ids_new, int n_new, int *slot_of_id, int *s
 }
 
 static int c_block(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set, int ws_size,
-                   double Cp, double Cn, const double *kws, const double *k_diag, double eps, double *diff, int max_iter,
-                   int *gate_, int epoch_, int target_xcd_, tsvm_stream stream) {
-    TSVM_REQUIRE(y && f_val && alpha && alpha_diff && working_set && kws && k_diag && diff, "tsvm_c_smo_solve_block: null pointer");
+                   double Cp, double Cn, const void *kws_, int block_type_, const double *k_diag, double eps, double *diff,
+                   int max_iter, int *gate_, int epoch_, int target_xcd_, tsvm_stream stream) {
+    TSVM_REQUIRE(y && f_val && alpha && alpha_diff && working_set && kws_ && k_diag && diff, "tsvm_c_smo_solve_block: null pointer");
     TSVM_REQUIRE(ws_size >= 1 && ws_size <= MAX_WS, "tsvm_c_smo_solve_block: ws_size %d outside [1, %d]", ws_size, MAX_WS);
+    TSVM_REQUIRE(block_type_ == TSVM_ROW_F64 || block_type_ == TSVM_ROW_F32, "tsvm_c_smo_solve_block: unknown block type %d", block_type_);
     hipStream_t s = tsvm_s(stream);
     const int solver_grid_ = gate_ ? TSVM_SOLVER_GRID_ON_XCD : 1;
-    TSVM_DISPATCH_E(c_smo_solve_kernel, y, f_val, alpha, alpha_diff, working_set, ws_size, Cp, Cn, kws, k_diag, eps, diff,
-                    max_iter, gate_, epoch_, target_xcd_);
+    TSVM_DISPATCH_E(c_smo_solve_kernel, (y, f_val, alpha, alpha_diff, working_set, ws_size, Cp, Cn),
+                    (k_diag, eps, diff, max_iter, gate_, epoch_, target_xcd_));
     TSVM_LAUNCH_CHECK();
     return 0;
 }
 
 static int nu_block(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set, int ws_size,
-                    double C, const double *kws, const double *k_diag, double eps, double *diff, int max_iter, int *gate_,
-                    int epoch_, int target_xcd_, tsvm_stream stream) {
-    TSVM_REQUIRE(y && f_val && alpha && alpha_diff && working_set && kws && k_diag && diff, "tsvm_nu_smo_solve_block: null pointer");
+                    double C, const void *kws_, int block_type_, const double *k_diag, double eps, double *diff, int max_iter,
+                    int *gate_, int epoch_, int target_xcd_, tsvm_stream stream) {
+    TSVM_REQUIRE(y && f_val && alpha && alpha_diff && working_set && kws_ && k_diag && diff, "tsvm_nu_smo_solve_block: null pointer");
     TSVM_REQUIRE(ws_size >= 1 && ws_size <= MAX_WS, "tsvm_nu_smo_solve_block: ws_size %d outside [1, %d]", ws_size, MAX_WS);
+    TSVM_REQUIRE(block_type_ == TSVM_ROW_F64 || block_type_ == TSVM_ROW_F32, "tsvm_nu_smo_solve_block: unknown block type %d", block_type_);
     hipStream_t s = tsvm_s(stream);
     const int solver_grid_ = gate_ ? TSVM_SOLVER_GRID_ON_XCD : 1;
-    TSVM_DISPATCH_E(nu_smo_solve_kernel, y, f_val, alpha, alpha_diff, working_set, ws_size, C, kws, k_diag, eps, diff,
-                    max_iter, gate_, epoch_, target_xcd_);
+    TSVM_DISPATCH_E(nu_smo_solve_kernel, (y, f_val, alpha, alpha_diff, working_set, ws_size, C),
+                    (k_diag, eps, diff, max_iter, gate_, epoch_, target_xcd_));
     TSVM_LAUNCH_CHECK();
     return 0;
 }
 
 int tsvm_c_smo_solve_block(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
-                           int ws_size, double Cp, double Cn, const double *kws, const double *k_diag, double eps,
+                           int ws_size, double Cp, double Cn, const void *kws, int block_type, const double *k_diag, double eps,
                            double *diff, int max_iter, tsvm_stream stream) {
-    return c_block(y, f_val, alpha, alpha_diff, working_set, ws_size, Cp, Cn, kws, k_diag, eps, diff, max_iter, nullptr, 0, 0, stream);
+    return c_block(y, f_val, alpha, alpha_diff, working_set, ws_size, Cp, Cn, kws, block_type, k_diag, eps, diff, max_iter, nullptr, 0,
+                   0, stream);
 }
 
 int tsvm_nu_smo_solve_block(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
-                            int ws_size, double C, const double *kws, const double *k_diag, double eps, double *diff,
+                            int ws_size, double C, const void *kws, int block_type, const double *k_diag, double eps, double *diff,
                             int max_iter, tsvm_stream stream) {
-    return nu_block(y, f_val, alpha, alpha_diff, working_set, ws_size, C, kws, k_diag, eps, diff, max_iter, nullptr, 0, 0, stream);
+    return nu_block(y, f_val, alpha, alpha_diff, working_set, ws_size, C, kws, block_type, k_diag, eps, diff, max_iter, nullptr, 0, 0,
+                    stream);
 }
 
 int tsvm_c_smo_solve_block_on_xcd(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
-                                  int ws_size, double Cp, double Cn, const double *kws, const double *k_diag, double eps,
+                                  int ws_size, double Cp, double Cn, const void *kws, int block_type, const double *k_diag, double eps,
                                   double *diff, int max_iter, int *gate, int epoch, int xcd, tsvm_stream stream) {
     TSVM_REQUIRE(gate && epoch >= 1 && xcd >= 0 && xcd < TSVM_SOLVER_GRID_ON_XCD, "tsvm_c_smo_solve_block_on_xcd: bad gate, epoch or xcd");
-    return c_block(y, f_val, alpha, alpha_diff, working_set, ws_size, Cp, Cn, kws, k_diag, eps, diff, max_iter, gate, epoch, xcd, stream);
+    return c_block(y, f_val, alpha, alpha_diff, working_set, ws_size, Cp, Cn, kws, block_type, k_diag, eps, diff, max_iter, gate, epoch,
+                   xcd, stream);
 }
 
 int tsvm_nu_smo_solve_block_on_xcd(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
-                                   int ws_size, double C, const double *kws, const double *k_diag, double eps, double *diff,
-                                   int max_iter, int *gate, int epoch, int xcd, tsvm_stream stream) {
+                                   int ws_size, double C, const void *kws, int block_type, const double *k_diag, double eps,
+                                   double *diff, int max_iter, int *gate, int epoch, int xcd, tsvm_stream stream) {
     TSVM_REQUIRE(gate && epoch >= 1 && xcd >= 0 && xcd < TSVM_SOLVER_GRID_ON_XCD, "tsvm_nu_smo_solve_block_on_xcd: bad gate, epoch or xcd");
-    return nu_block(y, f_val, alpha, alpha_diff, working_set, ws_size, C, kws, k_diag, eps, diff, max_iter, gate, epoch, xcd, stream);
+    return nu_block(y, f_val, alpha, alpha_diff, working_set, ws_size, C, kws, block_type, k_diag, eps, diff, max_iter, gate, epoch, xcd,
+                    stream);
 }
 
 int tsvm_nu_smo_solve(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
@@ -757,11 +803,12 @@ int tsvm_nu_smo_solve(const int *y, const double *f_val, double *alpha, double *
     hipStream_t s = tsvm_s(stream);
     int *gate_ = nullptr;
     const int epoch_ = 0, target_xcd_ = 0, solver_grid_ = 1;
-    int rc = launch_gather(k_rows, row_type, slots, ld, working_set, ws_size, workspace, s);
+    const int block_type_ = row_type;
+    int rc = launch_gather(k_rows, row_type, slots, ld, working_set, ws_size, workspace, block_type_, s);
     if (rc) return rc;
-    const double *kws = (const double *) workspace;
-    TSVM_DISPATCH_E(nu_smo_solve_kernel, y, f_val, alpha, alpha_diff, working_set, ws_size, C, kws, k_diag, eps, diff,
-                    max_iter, gate_, epoch_, target_xcd_);
+    const void *kws_ = workspace;
+    TSVM_DISPATCH_E(nu_smo_solve_kernel, (y, f_val, alpha, alpha_diff, working_set, ws_size, C),
+                    (k_diag, eps, diff, max_iter, gate_, epoch_, target_xcd_));
     TSVM_LAUNCH_CHECK();
     return 0;
 }

@@ -349,13 +349,13 @@ void KernelMatrix::get_rows_counted(const int *d_idx, int m_max, const int *d_m,
 }
 
 // K(x_idx[r], x_idx[t]) for r, t < m: the same kernels with the column set restricted to the m rows,
-// so every value is bit-identical to the corresponding entry of a full kernel row.
-void KernelMatrix::get_block(const int *d_idx, int m, kernel_type *d_out, int64_t ld, hipStream_t stream) const {
+// so every value is bit-identical to the corresponding entry of a full kernel row.  Elements are row_type() wide.
+void KernelMatrix::get_block(const int *d_idx, int m, void *d_out, int64_t ld, hipStream_t stream) const {
     const DeviceRows &R = *rows_;
     if (R.dense) {
         abi_check(tsvm_get_rows_dense(R.x.data(), R.ld, d_idx, m, (int) R.n_features, R.self_dot.data(), R.x.data(), R.ld, d_idx, m,
                                       R.self_dot.data(), (int) param.kernel_type, param.gamma, param.coef0, param.degree,
-                                      d_out, TSVM_ROW_F64, nullptr, ld, stream));
+                                      d_out, row_type(), nullptr, ld, stream));
         return;
     }
     const int wt = R.values_fit_float ? TSVM_ROW_F32 : TSVM_ROW_F64;
@@ -367,7 +367,7 @@ void KernelMatrix::get_block(const int *d_idx, int m, kernel_type *d_out, int64_
     abi_check(tsvm_gather_f64(R.self_dot.data(), d_idx, m, stage_blk_sd_.data(), stream));
     abi_check(tsvm_get_rows_csr_staged(R.val.data(), R.col.data(), R.row_ptr.data(), d_idx, m, R.self_dot.data(),
                                        stage_blk_.data(), wt, m, stage_blk_sd_.data(), (int) param.kernel_type, param.gamma,
-                                       param.coef0, param.degree, d_out, TSVM_ROW_F64, nullptr, ld, stream));
+                                       param.coef0, param.degree, d_out, row_type(), nullptr, ld, stream));
     abi_check(tsvm_csr_scatter_rows(R.val.data(), R.col.data(), R.row_ptr.data(), d_idx, m, (int) R.n_features,
                                     stage_blk_.data(), wt, 1, stream));
 }

@@ -71,8 +71,8 @@ public:
     // the same when only the device knows how many rows there are (*d_m of at most m_max; dense layout only)
     void get_rows_counted(const int *d_idx, int m_max, const int *d_m, void *d_out, int64_t ld, const int *d_out_slots,
                           hipStream_t stream) const;
-    // the m x m block K(x_idx[r], x_idx[t]) -> d_out[r*ld + t] (what the local solver reads; always double)
-    void get_block(const int *d_idx, int m, kernel_type *d_out, int64_t ld, hipStream_t stream = nullptr) const;
+    // the m x m block K(x_idx[r], x_idx[t]) -> d_out[r*ld + t] (what the local solver reads; row_type() elements)
+    void get_block(const int *d_idx, int m, void *d_out, int64_t ld, hipStream_t stream = nullptr) const;
     // kernel rows of an external batch -> element i*ld + j of d_out (row_type() elements)
     void get_rows(const DataSet::node2d &instances, void *d_out, int64_t ld) const;
     void get_rows(const std::vector<DataSet::node> *instances, size_t m, void *d_out, int64_t ld) const;   // the same for a slice

@@ -747,7 +747,7 @@ struct SolveTask::Impl {
             block_on_solver_cus = t_block + 0.4e-3 <= t_rows;
         }
         if (caching && all_cached) {
-            abi_check(tsvm_smo_gather_block_by_id(k_rows, row_type, d_slot_of.data(), ld, ws_u(), ws_size, d_kws.data(),
+            abi_check(tsvm_smo_gather_block_by_id(k_rows, row_type, d_slot_of.data(), ld, ws_u(), ws_size, d_kws.data(), row_type,
                                                   d_slots_a.data(), sa));
             slots = d_slots_a.data();
         } else if (block_on_solver_cus) {
@@ -757,7 +757,7 @@ struct SolveTask::Impl {
         } else if (block_first) {
             k_mat.get_block(ws_u(), ws_size, d_kws.data(), ldk, sa);
         } else {
-            abi_check(tsvm_smo_gather_block(k_rows, row_type, slots, ld, ws_u(), ws_size, d_kws.data(), sa));
+            abi_check(tsvm_smo_gather_block(k_rows, row_type, slots, ld, ws_u(), ws_size, d_kws.data(), row_type, sa));
         }
         timer.end(stats.ms_local);
         if (!on_one_stream && !block_on_solver_cus) TSVM_HIP_CHECK(hipEventRecord(block_done, sa));
@@ -778,18 +778,18 @@ struct SolveTask::Impl {
             ++solver_epoch;
             if (nu)
                 abi_check(tsvm_nu_smo_solve_block_on_xcd(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), ws_ids(), ws_size, Cp,
-                                                         d_kws.data(), k_mat.diag(), eps, d_diff, max_iter, d_gate.data(), solver_epoch,
-                                                         solver_xcd, st));
+                                                         d_kws.data(), row_type, k_mat.diag(), eps, d_diff, max_iter, d_gate.data(),
+                                                         solver_epoch, solver_xcd, st));
             else
                 abi_check(tsvm_c_smo_solve_block_on_xcd(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), ws_ids(), ws_size, Cp,
-                                                        Cn, d_kws.data(), k_mat.diag(), eps, d_diff, max_iter, d_gate.data(), solver_epoch,
-                                                        solver_xcd, st));
+                                                        Cn, d_kws.data(), row_type, k_mat.diag(), eps, d_diff, max_iter, d_gate.data(),
+                                                        solver_epoch, solver_xcd, st));
         } else if (nu) {
             abi_check(tsvm_nu_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), ws_ids(), ws_size,
-                                              Cp, d_kws.data(), k_mat.diag(), eps, d_diff, max_iter, st));
+                                              Cp, d_kws.data(), row_type, k_mat.diag(), eps, d_diff, max_iter, st));
         } else {
             abi_check(tsvm_c_smo_solve_block(d_y.data(), d_f.data(), d_alpha.data(), d_alpha_diff.data(), ws_ids(), ws_size,
-                                             Cp, Cn, d_kws.data(), k_mat.diag(), eps, d_diff, max_iter, st));
+                                             Cp, Cn, d_kws.data(), row_type, k_mat.diag(), eps, d_diff, max_iter, st));
         }
         timer.end(stats.ms_local);
         if (!on_one_stream) TSVM_HIP_CHECK(hipEventRecord(solved, ss));
