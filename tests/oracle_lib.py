@@ -21,13 +21,19 @@ class OrcParam(C.Structure):
 
 
 def make_param(svm_type=C_SVC, kernel_type=RBF, degree=3, gamma=0.0, coef0=0.0, C_=1.0, nu=0.5, p=0.1,
-               epsilon=0.001, max_mem_size=8192 << 20, max_iter=-1, expf_mode=1):
-    """Defaults follow include/thundersvm/svmparam.h:14-29 (p and epsilon are float literals there)."""
+               epsilon=0.001, max_mem_size=8192 << 20, max_iter=-1, expf_mode=1, weights=None):
+    """Defaults follow include/thundersvm/svmparam.h:14-29 (p and epsilon are float literals there).
+    weights: {class label: factor on C}."""
     prm = OrcParam()
     prm.svm_type, prm.kernel_type, prm.degree, prm.expf_mode = svm_type, kernel_type, degree, expf_mode
     prm.gamma, prm.coef0, prm.C, prm.nu = gamma, coef0, C_, nu
     prm.p, prm.epsilon = p, epsilon
     prm.max_mem_size, prm.max_iter, prm.nr_weight = max_mem_size, max_iter, 0
+    if weights:
+        prm._keep = (np.array(list(weights.keys()), dtype=np.int32), np.array(list(weights.values()), dtype=np.float64))
+        prm.nr_weight = len(weights)
+        prm.weight_label = prm._keep[0].ctypes.data_as(C.POINTER(C.c_int))
+        prm.weight = prm._keep[1].ctypes.data_as(C.POINTER(C.c_double))
     return prm
 
 

@@ -171,6 +171,29 @@ def test_failures_are_reported_through_succeed():
     lib.model_free(C.c_void_p(m))
 
 
+def test_probability_estimates_with_class_weights():
+    """The five fold models of a probability run train with the class weights of the run (svc.cpp:428-462 hands them
+    the same parameters): probabilities against the oracle's, which differ visibly from the unweighted ones."""
+    lib = _lib()
+    d = D.load_libsvm(FIXTURE)
+    weights = {int(d.y[0]): 6.0, int(d.y[-1]): 0.25}
+    m, _, n_classes, ok = _fit(lib, d, 0, 2, True, gamma=0.5, cost=0.5, probability=1, weights=weights)
+    assert ok == 1 and n_classes == 3
+    lab, dec = _predict(lib, m, d, True, 3)
+    prob = np.zeros(d.n * 3, dtype=np.float32)
+    lib.get_pro(C.c_void_p(m), _fp(prob))
+    prob = prob.reshape(d.n, 3)
+    want = {}
+    for name, w in (("weighted", weights), ("plain", None)):
+        op = O.make_param(svm_type=0, kernel_type=2, gamma=0.5, C_=0.5, epsilon=float(np.float32(0.001)), expf_mode=1, weights=w)
+        pa, pb = O.probability_train(d.ptr, d.col, d.val, d.y, op)
+        om = O.Model(d.ptr, d.col, d.val, d.y, op)
+        want[name] = O.predict_probability(om.predict_dec_values(d.ptr, d.col, d.val), pa, pb, 3)
+    assert np.abs(prob - want["weighted"]).max() < 1e-6
+    assert np.abs(want["weighted"] - want["plain"]).max() > 1e-3      # the weights matter on this problem
+    lib.model_free(C.c_void_p(m))
+
+
 @pytest.mark.parametrize("sparse", [True, False])
 def test_probability_estimates(sparse):
     """probability = 1 (svc.cpp:137-143, 289-314, 432-491): probA / probB from the 5-fold decision values, coupled

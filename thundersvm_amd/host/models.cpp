@@ -43,11 +43,14 @@ void SvmModel::model_setup(const DataSet &, SvmParam &p) {   // svmmodel.cpp:22-
     binary_alpha.clear();
     binary_f.clear();
     param = p;
-    // The class weights are the caller's arrays and need not outlive this call: SVC::model_setup folds them into
-    // c_weight while they are alive, and the model's own copy of the parameters drops the pointers.
-    param.nr_weight = 0;
-    param.weight_label = nullptr;
-    param.weight = nullptr;
+    // The class weights are the caller's arrays and need not outlive this call, while the model's own copy of the
+    // parameters lives as long as the model (probability_train hands it to the fold models, svc.cpp:428-462): the
+    // model keeps its own copy of the two arrays and points its parameters at them.
+    own_weight_label.assign(p.weight_label, p.weight_label + (p.weight_label ? p.nr_weight : 0));
+    own_weight.assign(p.weight, p.weight + (p.weight ? p.nr_weight : 0));
+    param.nr_weight = (int) std::min(own_weight_label.size(), own_weight.size());
+    param.weight_label = param.nr_weight ? own_weight_label.data() : nullptr;
+    param.weight = param.nr_weight ? own_weight.data() : nullptr;
 }
 
 static int max2power(double n) { return (int) pow(2, floor(log2f(float(n)))); }   // util/common.h:20-23

@@ -75,6 +75,8 @@ protected:
     void compute_linear_coef_single_model(size_t n_feature, bool zero_based);
 
     SvmParam param;
+    std::vector<int> own_weight_label;        // what param.weight_label / param.weight point at
+    std::vector<float_type> own_weight;
     std::vector<float_type> coef;
     std::vector<float_type> linear_coef;
     DataSet::node2d sv;
