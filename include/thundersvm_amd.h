@@ -193,7 +193,11 @@ int tsvm_c_smo_solve(const int *y, const double *f_val, double *alpha, double *a
  * The ws x ws block goes into a static device array of 1024 x 1024 doubles (8 MiB per device, held until the
  * process ends); ws_size > 1024 is rejected with TSVM_EINVAL.  The call allocates and frees nothing.  Every call on
  * a device shares that device's array: calls that overlap on one device (different streams or threads) race, the
- * caller has to order them.  Results are those of tsvm_c_smo_solve. */
+ * caller has to order them.  Results are those of tsvm_c_smo_solve.
+ * The first call on a device looks up the array's address and the kernels' attributes (and the runtime may load the
+ * library's code object then): make that call, or tsvm_c_smo_solve_static_init(), once per device outside any graph
+ * capture; calls after it only launch kernels. */
+int tsvm_c_smo_solve_static_init(void);
 int tsvm_c_smo_solve_static(const int *y, const double *f_val, double *alpha, double *alpha_diff, const int *working_set,
                             int ws_size, double Cp, double Cn, const void *k_rows, int row_type, const int *slots,
                             int64_t ld, const double *k_diag, double eps, double *diff, int max_iter, tsvm_stream stream);

@@ -131,23 +131,6 @@ int tsvm_cmdparser_train(int argc, char **argv, tsvm_param *param, int *gamma_se
  * process ends, because releasing it costs up to seconds). */
 int tsvm_release_device_cache(void);
 
-/* Self-test of the host's bounded wait for the local solver's report (no device needed): waits on a word that
- * nobody writes, with a stream that reports "still running", and returns 0 when the wait gave up with its
- * time-out error after timeout_ms (within a second of it), -1 otherwise.  never_written != 0 makes the stream
- * report "drained" instead: the wait must then fail with its "finished without reporting" error at once. */
-int tsvm_selftest_solver_wait(int timeout_ms, int never_written);
-
-/* Self-test of the device buffer type that stands in for the reference's SyncArray (needs a device): byte
- * accounting on allocation, resize, move and destruction, and an upload / download round trip; the cases of
- * src/test/test_syncmem.cpp and test_syncarray.cpp that apply.  0 on success, -1 with a message otherwise. */
-int tsvm_selftest_device_buffer(void);
-
-/* Test hook (no GPU needed): drives the kernel-row cache's bookkeeping as a solve does, with a first working set of ws
- * ids and ws/2 new ids per iteration, on the cyclic sequence 0, 1, ..., n_ids-1, 0, ..., and checks after every
- * iteration that each working-set row has a slot of its own, is pinned and off the eviction list.  Returns the
- * number of hits, or -1 (tsvm_model_last_error says what broke). */
-long long tsvm_selftest_row_cache(int n_ids, int slots, int ws, int iterations);
-
 int tsvm_model_save(void *model, const char *path);
 int tsvm_model_load(void *model, const char *path);
 

@@ -78,11 +78,12 @@ def test_no_cpu_fallback():
 def test_bounded_wait_for_the_local_solver():
     """The host's wait for the solver's report gives up with an error instead of spinning for ever (host only:
     the word is never written, no kernel is involved)."""
-    lib = model.host_lib()
-    assert lib.tsvm_selftest_solver_wait(300, 0) == 0, lib.tsvm_model_last_error()
-    assert b"TSVM_SOLVER_TIMEOUT_MS" in lib.tsvm_model_last_error()
-    assert lib.tsvm_selftest_solver_wait(60000, 1) == 0, lib.tsvm_model_last_error()
-    assert b"without reporting" in lib.tsvm_model_last_error()
+    import selftest_lib
+    lib = selftest_lib.lib()
+    assert lib.tsvm_selftest_solver_wait(300, 0) == 0, lib.tsvm_selftest_last_error()
+    assert b"TSVM_SOLVER_TIMEOUT_MS" in lib.tsvm_selftest_last_error()
+    assert lib.tsvm_selftest_solver_wait(60000, 1) == 0, lib.tsvm_selftest_last_error()
+    assert b"without reporting" in lib.tsvm_selftest_last_error()
 
 
 def test_row_cache_bookkeeping():
@@ -91,20 +92,19 @@ def test_row_cache_bookkeeping():
     (every row is evicted just before its turn comes again); rows that were computed leave at the tail instead, so a
     resident set survives and hits once per cycle.  After every iteration the hook checks that the working set's rows
     are pinned, own their slots and are off the eviction list."""
-    import ctypes
-    lib = model.host_lib()
-    lib.tsvm_selftest_row_cache.restype = ctypes.c_longlong
+    import selftest_lib
+    lib = selftest_lib.lib()
     ws, q = 64, 32
     # every id has a slot: each id misses exactly once
     n_ids, iters = 1000, 200
     lookups = ws + q * (iters - 1)
-    assert lib.tsvm_selftest_row_cache(n_ids, 1000, ws, iters) == lookups - n_ids, lib.tsvm_model_last_error()
+    assert lib.tsvm_selftest_row_cache(n_ids, 1000, ws, iters) == lookups - n_ids, lib.tsvm_selftest_last_error()
     # 1000 ids, 400 slots: a resident set of about 400 - ws rows hits in every later cycle
     hits = lib.tsvm_selftest_row_cache(n_ids, 400, ws, iters)
-    assert hits >= 0, lib.tsvm_model_last_error()
+    assert hits >= 0, lib.tsvm_selftest_last_error()
     cycles = lookups // n_ids
     assert hits >= (cycles - 1) * 250, hits          # least-recently-used order: 0
     assert hits <= lookups - n_ids
     # the smallest cache the solver uses (four working sets) and a cycle barely longer than it
-    assert lib.tsvm_selftest_row_cache(4 * ws + 8, 4 * ws, ws, 300) >= 0, lib.tsvm_model_last_error()
-    assert lib.tsvm_selftest_row_cache(10, 400, ws, 10) == -1 and b"bad arguments" in lib.tsvm_model_last_error()
+    assert lib.tsvm_selftest_row_cache(4 * ws + 8, 4 * ws, ws, 300) >= 0, lib.tsvm_selftest_last_error()
+    assert lib.tsvm_selftest_row_cache(10, 400, ws, 10) == -1 and b"bad arguments" in lib.tsvm_selftest_last_error()

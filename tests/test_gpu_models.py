@@ -472,7 +472,7 @@ def test_device_buffer_accounting_and_round_trip():
     """DeviceBuffer<T>, the device-only stand-in for SyncArray<T>: the checks of the reference's
     src/test/test_syncmem.cpp:7-50 and test_syncarray.cpp:7-60 that apply to a buffer without a host mirror
     (allocation counted once, released on destruction and on resize, moves transfer ownership without
-    counting twice, upload -> download round trip), run inside the host library."""
-    from thundersvm_amd.model import host_lib
-    lib = host_lib()
-    assert lib.tsvm_selftest_device_buffer() == 0, lib.tsvm_model_last_error()
+    counting twice, upload -> download round trip), run by the test-only native library."""
+    import selftest_lib
+    lib = selftest_lib.lib()
+    assert lib.tsvm_selftest_device_buffer() == 0, lib.tsvm_selftest_last_error()

@@ -33,7 +33,7 @@ def _both(n, ws, row_type, seed_off, check_device_free=True):
                       G.ptr(k_d), row_type, G.ptr(s_d), n, G.ptr(dg_d), eps, G.ptr(diff_d), max_iter, G.stream())
             torch.cuda.synchronize()
             assert torch.cuda.memory_allocated() == before
-            # (the first call on a device may make the runtime load the library's code object, static array included)
+            # (after tsvm_c_smo_solve_static_init nothing is left to look up or load)
             assert not check_device_free or torch.cuda.mem_get_info()[0] == free_before
         else:
             wsp = torch.empty(capi.kernel_lib().tsvm_smo_solve_workspace(ws), dtype=torch.uint8, device="cuda")
@@ -46,7 +46,9 @@ def _both(n, ws, row_type, seed_off, check_device_free=True):
 
 
 def test_static_solver_matches_workspace_solver_twice():
-    _both(2000, 1024, capi.ROW_F64, 0, check_device_free=False)    # fills the whole static block
+    # once per device, outside any capture: the array's address, the kernels' attributes, the code object
+    assert capi.kernel_lib().tsvm_c_smo_solve_static_init() == 0, capi.kernel_lib().tsvm_last_error()
+    _both(2000, 1024, capi.ROW_F64, 0)    # fills the whole static block
     _both(700, 100, capi.ROW_F32, 1)      # smaller: reads nothing the first call left behind
     _both(900, 300, capi.ROW_F64, 2)
 

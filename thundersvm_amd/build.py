@@ -53,9 +53,21 @@ def build_host(extra=()):
     return HOST_LIB
 
 
+def build_selftests():
+    """The test-only library (tests/native): self-tests of host-layer pieces, linked against the host library."""
+    src = os.path.join(os.path.dirname(HERE), "tests", "native", "selftest.cpp")
+    if not os.path.exists(src):
+        return None
+    out = os.path.join(os.path.dirname(src), "libtsvm_selftest.so")
+    _run(["g++", "-O2", "-fPIC", "-std=c++17", "-fopenmp", "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include", src, "-shared", "-o", out,
+          "-L", HERE, "-lthundersvm", "-ltsvm_hip", "-Wl,-rpath,$ORIGIN/../../thundersvm_amd", "-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,/opt/rocm/lib"])
+    return out
+
+
 def build_all():
     build_kernels()
     build_host()
+    build_selftests()
 
 
 if __name__ == "__main__":

@@ -44,6 +44,7 @@ SIGNATURES = {
     "tsvm_update_f": (_int, [_p, _p, _int, _p, _int, _p, _i64, _i64, _int, _p]),
     "tsvm_smo_solve_workspace": (C.c_size_t, [_int]),
     "tsvm_c_smo_solve": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _dbl, _p, _int, _p, _i64, _p, _dbl, _p, _int, _p, _p]),
+    "tsvm_c_smo_solve_static_init": (_int, []),
     "tsvm_c_smo_solve_static": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _dbl, _p, _int, _p, _i64, _p, _dbl, _p, _int, _p]),
     "tsvm_nu_smo_solve": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _p, _int, _p, _i64, _p, _dbl, _p, _int, _p, _p]),
     "tsvm_smo_solve_block_ld": (_int, [_int]),

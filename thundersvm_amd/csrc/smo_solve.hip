@@ -26,7 +26,9 @@
 #include "tsvm_device.h"
 #include "tsvm_internal.h"
 
+#include <map>
 #include <mutex>
+#include <utility>
 
 #define TSVM_INF __builtin_inf()
 #define MAX_WS 1024
@@ -551,11 +553,30 @@ __global__ __launch_bounds__(SV_T) void nu_smo_solve_kernel(
 // The solver workgroup asks for the rest of the CU's 160 KB of LDS as (unused) dynamic shared memory:
 // no other workgroup can then be placed on its CU, so a kernel running concurrently on another
 // stream cannot take issue slots, LDS bandwidth or L1 space away from the latency-bound solver.
-template <typename K>
-static hipError_t reserve_cu(K kernel, size_t static_lds, size_t *dyn) {
+static hipError_t reserve_cu(const void *kernel, size_t static_lds, size_t *dyn) {
     const size_t cu_lds = 160 * 1024;
     *dyn = cu_lds > static_lds + 1024 ? cu_lds - static_lds - 1024 : 0;
-    return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int) *dyn);
+    return hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int) *dyn);
+}
+
+// The dynamic LDS a solver kernel is launched with on the current device.  The attribute query and the opt-in are made
+// once per kernel and device (whichever host thread comes first), not per launch.
+static int solver_dyn_lds(const void *kernel, size_t *dyn) {
+    static std::mutex mu;
+    static std::map<std::pair<const void *, int>, size_t> table;
+    int dev = 0;
+    TSVM_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lock(mu);
+    auto it = table.find(std::make_pair(kernel, dev));
+    if (it == table.end()) {
+        hipFuncAttributes fa;
+        TSVM_HIP(hipFuncGetAttributes(&fa, kernel));
+        size_t d = 0;
+        TSVM_HIP(reserve_cu(kernel, fa.sharedSizeBytes, &d));
+        it = table.emplace(std::make_pair(kernel, dev), d).first;
+    }
+    *dyn = it->second;
+    return 0;
 }
 
 extern "C" {
@@ -589,20 +610,14 @@ static int launch_gather(const void *k_rows, int row_type, const int *slots, int
     return 0;
 }
 
-// The attribute query and the dynamic-LDS opt-in are made once per kernel and device, not per launch.
 #define TSVM_LAUNCH_SOLVER(KERNEL, EVAL, TB, ...)                                                   \
     do {                                                                                            \
-        static thread_local int dev_done_ = -1;                                                     \
-        static thread_local size_t dyn_ = 0;                                                        \
-        int dev_ = 0;                                                                               \
-        TSVM_HIP(hipGetDevice(&dev_));                                                              \
-        if (dev_done_ != dev_) {                                                                    \
-            hipFuncAttributes fa_;                                                                  \
-            TSVM_HIP(hipFuncGetAttributes(&fa_, reinterpret_cast<const void *>(KERNEL<EVAL, TB>))); \
-            TSVM_HIP(reserve_cu(KERNEL<EVAL, TB>, fa_.sharedSizeBytes, &dyn_));                      \
-            dev_done_ = dev_;                                                                       \
+        size_t dyn_ = 0;                                                                            \
+        if (solver_grid_ == 1) {                                                                    \
+            const int rc_ = solver_dyn_lds(reinterpret_cast<const void *>(KERNEL<EVAL, TB>), &dyn_); \
+            if (rc_) return rc_;                                                                    \
         }                                                                                           \
-        hipLaunchKernelGGL((KERNEL<EVAL, TB>), dim3(solver_grid_), dim3(SV_T), solver_grid_ == 1 ? dyn_ : 0, s, __VA_ARGS__); \
+        hipLaunchKernelGGL((KERNEL<EVAL, TB>), dim3(solver_grid_), dim3(SV_T), dyn_, s, __VA_ARGS__); \
     } while (0)
 
 #define TSVM_DISPATCH_E_T(KERNEL, TB, ...)                                                      \
@@ -666,6 +681,21 @@ static int solver_block_address(double **out) {
         g_solver_block_ptr[dev] = p;
     }
     *out = g_solver_block_ptr[dev];
+    return 0;
+}
+
+int tsvm_c_smo_solve_static_init(void) {
+    double *block = nullptr;
+    int rc = solver_block_address(&block);
+    if (rc) return rc;
+    size_t dyn = 0;
+    const void *kernels[] = {reinterpret_cast<const void *>(c_smo_solve_kernel<1, float>), reinterpret_cast<const void *>(c_smo_solve_kernel<2, float>),
+                             reinterpret_cast<const void *>(c_smo_solve_kernel<4, float>), reinterpret_cast<const void *>(c_smo_solve_kernel<1, double>),
+                             reinterpret_cast<const void *>(c_smo_solve_kernel<2, double>), reinterpret_cast<const void *>(c_smo_solve_kernel<4, double>)};
+    for (const void *k : kernels) {
+        rc = solver_dyn_lds(k, &dyn);
+        if (rc) return rc;
+    }
     return 0;
 }
 

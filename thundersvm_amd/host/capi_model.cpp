@@ -344,72 +344,6 @@ int tsvm_release_device_cache(void) {
     TSVM_GUARD({ tsvm::RowArena::instance().release(); })
 }
 
-int tsvm_selftest_device_buffer(void) {
-    TSVM_GUARD({
-        using tsvm::DeviceBuffer;
-        auto expect = [](bool ok, const char *what) { if (!ok) throw std::runtime_error(std::string("DeviceBuffer: ") + what); };
-        const size_t base = tsvm::device_bytes_in_use();
-        {
-            DeviceBuffer<char> a(100);
-            expect(a.data() != nullptr && a.size() == 100, "allocation");
-            expect(tsvm::device_bytes_in_use() == base + 100, "one allocation counted");
-            DeviceBuffer<char> b;                       // nothing allocated, nothing counted
-            expect(b.data() == nullptr && tsvm::device_bytes_in_use() == base + 100, "empty buffer");
-            b.resize(100);
-            expect(tsvm::device_bytes_in_use() == base + 200, "second allocation counted");
-            {
-                DeviceBuffer<char> t(100);
-                expect(tsvm::device_bytes_in_use() == base + 300, "third allocation counted");
-                DeviceBuffer<char> moved(std::move(t));   // ownership moves, the bytes are counted once
-                expect(t.data() == nullptr && t.size() == 0 && moved.size() == 100, "move");
-                expect(tsvm::device_bytes_in_use() == base + 300, "move does not count twice");
-            }
-            expect(tsvm::device_bytes_in_use() == base + 200, "destruction releases");
-            DeviceBuffer<int> d(100);
-            expect(d.size() == 100 && tsvm::device_bytes_in_use() == base + 200 + 100 * sizeof(int), "typed size");
-            d.resize(20);                               // a resize starts over, as SyncArray::resize does
-            expect(d.size() == 20 && tsvm::device_bytes_in_use() == base + 200 + 20 * sizeof(int), "resize");
-            std::vector<int> host(10);
-            for (int i = 0; i < 10; ++i) host[i] = i;
-            d.upload(host.data(), 10, 5);               // interior offsets are accepted
-            for (int i = 0; i < 10; ++i) host[i] = -1;
-            d.download(host.data(), 10, 5);
-            for (int i = 0; i < 10; ++i) expect(host[i] == i, "round trip");
-            d.zero();
-            const std::vector<int> z = d.to_host();
-            for (int v : z) expect(v == 0, "zero fill");
-        }
-        expect(tsvm::device_bytes_in_use() == base, "everything released");
-    })
-}
-
-long long tsvm_selftest_row_cache(int n_ids, int slots, int ws, int iterations) {
-    std::string what;
-    const long long hits = tsvm::row_cache_selftest(n_ids, slots, ws, iterations, what);
-    if (hits < 0) g_error = "row cache: " + what;
-    return hits;
-}
-
-int tsvm_selftest_solver_wait(int timeout_ms, int never_written) {
-    static volatile uint64_t word;
-    word = 0x7ff8dead00000001ull;
-    const auto t0 = std::chrono::steady_clock::now();
-    try {
-        if (never_written)
-            tsvm::wait_while_pending(&word, word, timeout_ms, [](void *) { return hipSuccess; }, nullptr);
-        else
-            tsvm::wait_while_pending(&word, word, timeout_ms, [](void *) { return hipErrorNotReady; }, nullptr);
-    } catch (const std::runtime_error &e) {
-        const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
-        g_error = e.what();
-        const bool timed_out = g_error.find("TSVM_SOLVER_TIMEOUT_MS") != std::string::npos;
-        if (never_written) return !timed_out && ms < 1000.0 ? 0 : -1;
-        return timed_out && ms >= timeout_ms && ms < timeout_ms + 1000.0 ? 0 : -1;
-    }
-    g_error = "the wait returned although the word never changed";
-    return -1;
-}
-
 int tsvm_model_save(void *model, const char *path) {
     TSVM_GUARD({ ((Handle *) model)->model->save_to_file(path); })
 }

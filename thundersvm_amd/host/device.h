@@ -90,6 +90,8 @@ public:
     T *data() { return ptr_; }
     const T *data() const { return ptr_; }
     size_t size() const { return count_; }
+    // Gives the memory up without freeing it: for a device that has stopped answering, where hipFree would not return.
+    void abandon() { ptr_ = nullptr; count_ = 0; }
 
     void upload(const T *host, size_t count, size_t offset = 0) {
         if (count) TSVM_HIP_CHECK(hipMemcpy(ptr_ + offset, host, count * sizeof(T), hipMemcpyHostToDevice));

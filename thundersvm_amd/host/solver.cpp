@@ -1,4 +1,5 @@
 #include "solver.h"
+#include "row_cache.h"
 
 #include <chrono>
 #include <map>
@@ -9,87 +10,13 @@
 
 using tsvm::abi_check;
 using tsvm::DeviceBuffer;
+using tsvm::RowCache;
 
 namespace {
 
 inline bool up_set(float_type a, float_type y, float_type Cp, float_type Cn) { return (y > 0 && a < Cp) || (y < 0 && a > 0); }
 inline bool low_set(float_type a, float_type y, float_type Cp, float_type Cn) { return (y > 0 && a > 0) || (y < 0 && a < Cn); }
 inline bool free_sv(float_type a, float_type y, float_type Cp, float_type Cn) { return a > 0 && (y > 0 ? a < Cp : a < Cn); }
-
-// Kernel-row cache bookkeeping (host side).  Rows of the kernel matrix live in slots of one HBM pool;
-// slot_of maps an instance id to its slot, an intrusive doubly linked list keeps the slots that may be evicted in
-// eviction order (tail first).  The device only ever sees slot numbers.  The reference keeps no rows
-// beyond the previous working set's second half (csmosolver.cpp:33-42,65-77); cached rows are the
-// rows get_rows would recompute, so the cache cannot change a result.
-//
-// Which row goes.  A row is pinned (out of the list) while it is in the working set, two outer iterations as a rule.
-// When it leaves, a row that was found in the cache when it entered goes to the front of the list; a row that had to
-// be computed goes to the tail, where the next misses take its slot first (all but every 64th such row, which goes
-// to the front, so that the cache's content can drift).  Plain least-recently-used order loses against SMO's access
-// pattern whenever the rows that keep coming back outnumber the slots: the selection works through them in turn,
-// and every row is evicted shortly before it is wanted again (a 426,315-instance class pair with 35,000 slots: 1 %
-// hits; with this order 26 %, and the best any order could do, knowing the future, is 39 %).
-struct RowCache {
-    int cap = 0, used = 0, head = -1, tail = -1;
-    long long released_misses = 0;
-    std::vector<int> slot_of, id_of, prev, next, pins;
-    std::vector<char> was_hit;
-    void init(int n, int capacity) {
-        cap = capacity;
-        slot_of.assign(n, -1);
-        id_of.assign(cap, -1);
-        prev.assign(cap, -1);
-        next.assign(cap, -1);
-        pins.assign(cap, 0);
-        was_hit.assign(cap, 0);
-    }
-    void unlink(int s) {
-        if (prev[s] >= 0) next[prev[s]] = next[s]; else head = next[s];
-        if (next[s] >= 0) prev[next[s]] = prev[s]; else tail = prev[s];
-    }
-    void push_front(int s) {
-        prev[s] = -1;
-        next[s] = head;
-        if (head >= 0) prev[head] = s;
-        head = s;
-        if (tail < 0) tail = s;
-    }
-    void push_back(int s) {
-        next[s] = -1;
-        prev[s] = tail;
-        if (tail >= 0) next[tail] = s;
-        tail = s;
-        if (head < 0) head = s;
-    }
-    int lookup(int id) {                 // slot of a cached row, pinned from now on, or -1
-        const int s = slot_of[id];
-        if (s >= 0) {
-            if (pins[s]++ == 0) { unlink(s); was_hit[s] = 1; }
-        }
-        return s;
-    }
-    int insert(int id) {                 // slot for a new row, pinned: a free one, else the list's tail (-1: every slot is pinned)
-        int s;
-        if (used < cap) {
-            s = used++;
-        } else {
-            s = tail;
-            if (s < 0) return -1;
-            unlink(s);
-            slot_of[id_of[s]] = -1;
-        }
-        id_of[s] = id;
-        slot_of[id] = s;
-        pins[s] = 1;
-        was_hit[s] = 0;
-        return s;
-    }
-    void release(int s) {                // the row has left the working set
-        if (--pins[s] > 0) return;
-        if (was_hit[s] || (++released_misses & 63) == 0) push_front(s);
-        else push_back(s);
-    }
-};
 
 struct PhaseTimer {
     bool on;
@@ -177,55 +104,6 @@ bool make_lane_group(int n_lanes, LaneGroup &g) {
 }  // namespace
 
 namespace tsvm {
-
-// Drives RowCache the way a solve does (first working set of ws rows, then q = ws / 2 new rows per iteration while the
-// previous new half stays pinned) on a cyclic sequence of n_ids ids, and checks after every step that each row of the
-// working set has a slot of its own and that the tables agree.  Returns the number of hits, or -1 with `what` set.
-long long row_cache_selftest(int n_ids, int slots, int ws, int iterations, std::string &what) {
-    if (n_ids < ws || slots < 2 * ws || ws < 2 || ws % 2) { what = "bad arguments"; return -1; }
-    RowCache c;
-    c.init(n_ids, slots);
-    const int q = ws / 2;
-    std::vector<int> ids(ws), slot(ws);
-    long long hits = 0;
-    int next_id = 0;
-    for (int it = 0; it < iterations; ++it) {
-        const int n_new = it == 0 ? ws : q, first_new = it == 0 ? 0 : q;
-        if (it > 0) {
-            for (int t = 0; t < q; ++t) c.release(slot[t]);
-            for (int t = 0; t < q; ++t) { ids[t] = ids[t + q]; slot[t] = slot[t + q]; }
-        }
-        for (int t = 0; t < n_new; ++t) {
-            const int id = next_id;
-            next_id = (next_id + 1) % n_ids;
-            int s = c.lookup(id);
-            if (s >= 0) ++hits;
-            else s = c.insert(id);
-            if (s < 0) { what = "no slot left for a working-set row"; return -1; }
-            ids[first_new + t] = id;
-            slot[first_new + t] = s;
-        }
-        std::vector<char> taken(slots, 0);
-        for (int t = 0; t < ws; ++t) {
-            if (slot[t] < 0 || slot[t] >= slots || c.slot_of[ids[t]] != slot[t] || c.id_of[slot[t]] != ids[t]) {
-                what = "a working-set row lost its slot";
-                return -1;
-            }
-            if (taken[slot[t]] && n_ids >= 2 * ws) { what = "two working-set rows share a slot"; return -1; }
-            taken[slot[t]] = 1;
-            if (c.pins[slot[t]] < 1) { what = "a working-set row is not pinned"; return -1; }
-        }
-        int listed = 0;
-        for (int s2 = c.head; s2 >= 0; s2 = c.next[s2]) {
-            if (c.pins[s2] != 0) { what = "a pinned row is on the eviction list"; return -1; }
-            if (++listed > slots) { what = "the eviction list has a cycle"; return -1; }
-        }
-        int pinned = 0;
-        for (int s2 = 0; s2 < c.used; ++s2) pinned += c.pins[s2] > 0;
-        if (listed + pinned != c.used) { what = "rows neither pinned nor listed"; return -1; }
-    }
-    return hits;
-}
 
 long long solver_timeout_ms() {
     const char *e = getenv("TSVM_SOLVER_TIMEOUT_MS");
@@ -348,9 +226,18 @@ struct SolveTask::Impl {
     bool wait_by_event = false;
     hipStream_t solver_stream = nullptr;
     volatile uint64_t *diff_word() const { return reinterpret_cast<volatile uint64_t *>(h_diff + (nu ? 0 : 1)); }
+    // Set when a wait for the solver gave up: the device is taken to be hung, and the destructor then touches neither
+    // the streams nor the device memory (synchronising, destroying or freeing would block for good); the task's streams
+    // stay marked as in use, its memory stays allocated, and the error reaches the caller.
+    bool abandoned = false;
     void wait_for_diff() {
-        tsvm::wait_while_pending(diff_word(), DIFF_PENDING, tsvm::solver_timeout_ms(),
-                                 [](void *st) { return hipStreamQuery((hipStream_t) st); }, solver_stream);
+        try {
+            tsvm::wait_while_pending(diff_word(), DIFF_PENDING, tsvm::solver_timeout_ms(),
+                                     [](void *st) { return hipStreamQuery((hipStream_t) st); }, solver_stream);
+        } catch (...) {
+            abandoned = true;
+            throw;
+        }
     }
     // the same wait as a poll (one look per call; the stream is asked, and the time-out checked, every 200 ms)
     std::chrono::steady_clock::time_point solver_enqueued, next_stream_check;
@@ -370,12 +257,18 @@ struct SolveTask::Impl {
         next_stream_check = now + std::chrono::milliseconds(200);
         const hipError_t e = hipStreamQuery(solver_stream);
         if (e == hipSuccess) {
-            if (*diff_word() == DIFF_PENDING) throw std::runtime_error("SolveTask: the local solver finished without reporting");
+            if (*diff_word() == DIFF_PENDING) {
+                abandoned = true;
+                throw std::runtime_error("SolveTask: the local solver finished without reporting");
+            }
         } else if (e != hipErrorNotReady) {
+            abandoned = true;
             TSVM_HIP_CHECK(e);
         }
-        if (now - solver_enqueued > std::chrono::milliseconds(tsvm::solver_timeout_ms()))
+        if (now - solver_enqueued > std::chrono::milliseconds(tsvm::solver_timeout_ms())) {
+            abandoned = true;
             throw std::runtime_error("SolveTask: no word from the local solver (TSVM_SOLVER_TIMEOUT_MS); the device may be hung");
+        }
         return false;
     }
     bool ids_arrived() const {
@@ -518,6 +411,12 @@ struct SolveTask::Impl {
     }
 
     ~Impl() {
+        if (abandoned) {   // nothing that could wait for the device
+            for (DeviceBuffer<int> *b : {&d_y, &d_ws, &d_slots_a, &d_slots_b, &d_ws_folded, &d_gate, &d_slot_of, &d_cache_state}) b->abandon();
+            for (DeviceBuffer<float_type> *b : {&d_alpha, &d_f, &d_alpha_diff, &d_kws}) b->abandon();
+            d_sel_ws.abandon();
+            return;
+        }
         if (sa) (void) hipStreamSynchronize(sa);   // a selection enqueued ahead may still be running
         if (ss && ss != sa) (void) hipStreamSynchronize(ss);
         if (ids && ids != sa) { (void) hipStreamSynchronize(ids); (void) hipStreamDestroy(ids); }

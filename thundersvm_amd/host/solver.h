@@ -33,8 +33,6 @@ struct SolverStats {
 class SolveTask;
 
 namespace tsvm {
-// checks the kernel-row cache's bookkeeping on a scripted sequence (see solver.cpp); hits or -1
-long long row_cache_selftest(int n_ids, int slots, int ws, int iterations, std::string &what);
 // Spins until *word no longer holds `pending`.  Every 200 ms `stream_state()` is asked for the state of the stream
 // that is to write the word (hipSuccess: everything enqueued has run; hipErrorNotReady: still running; anything else
 // is thrown as that error).  Throws std::runtime_error when the stream has drained without the word changing, or
