@@ -145,6 +145,31 @@ int tsvm_get_rows_csr(const double *val, const int *col, const int64_t *row_ptr,
                       const double *w, int m, const double *sd_w, int kernel_type, double gamma, double coef0,
                       int degree, void *out, int row_type, const int *out_slots, int64_t ldo, tsvm_stream stream);
 
+/* The CSR product on a sliced copy of the stored rows (the role of dns_csr_mul, kernelmatrix_kernel.cpp:149-160, with
+ * the operands' roles exchanged: the stored rows are streamed, the working rows wait in LDS).
+ * Sliced layout (sliced ELL, slices of 64 rows): entry k of row 64 s + l lies at slice_ptr[s] + 64 k + l; slice s is
+ * as wide as its longest row (tsvm_csr_slice_widths gives the widths, the caller turns them into slice_ptr[s + 1] =
+ * slice_ptr[s] + 64 * width[s], ceil(n / 64) + 1 entries); tsvm_csr_to_sliced fills it from the CSR arrays, padding
+ * with column pad_col (= n_features) and value 0; values are stored as val_type (TSVM_ROW_F32 only when every value
+ * is exactly a float).
+ * tsvm_get_rows_csr_sliced: out[slot(i) * ldo + j] = kappa(row a_idx[i] of the CSR matrix (a_val, a_col, a_ptr), stored
+ * row j) for i < m, j < n; sd_a is indexed by the CSR row (a_idx == NULL: rows 0 .. m-1).  Sums run over a stored row's
+ * entries in stored order; entries whose feature does not occur in a block of sixteen working rows add exact zeros
+ * and are skipped.  max_row_nnz: an upper bound on the entries of any working row; the working rows' block is held in
+ * tsvm_get_rows_csr_sliced_lds(n_features, max_row_nnz, val_type) bytes of LDS (a table of n_features 16-bit entries
+ * and a tile with a row of sixteen doubles for every feature that occurs in the block; a block with more such features
+ * than the tile has rows is done in two halves): when that returns 0 the shape does not fit (eight of the longest
+ * rows must) and the call is rejected (use tsvm_get_rows_csr_staged). */
+int tsvm_csr_slice_widths(const int64_t *row_ptr, int64_t n, int *widths, tsvm_stream stream);
+int tsvm_csr_to_sliced(const double *val, const int *col, const int64_t *row_ptr, int64_t n, const int64_t *slice_ptr, int pad_col,
+                       int *ell_col, void *ell_val, int val_type, tsvm_stream stream);
+size_t tsvm_get_rows_csr_sliced_lds(int n_features, int max_row_nnz, int val_type);
+int tsvm_get_rows_csr_sliced(const int *ell_col, const void *ell_val, int val_type, const int64_t *slice_ptr, int64_t n,
+                             const double *sd_x, const double *a_val, const int *a_col, const int64_t *a_ptr, const int *a_idx,
+                             int m, const double *sd_a, int n_features, int max_row_nnz, int kernel_type, double gamma,
+                             double coef0, int degree, void *out, int row_type, const int *out_slots, int64_t ldo,
+                             tsvm_stream stream);
+
 /* Device-side row subsets, so that a sub-problem (one class pair of a one-vs-one run, svc.cpp:147-150) takes its
  * rows from a data set already resident in HBM instead of a host copy:
  * dense: out row r = x row idx[r] (rows of ld doubles, ld % 4 == 0);

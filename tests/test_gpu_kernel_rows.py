@@ -158,6 +158,82 @@ def test_float_rows_rejected_for_linear_kernel():
                   G.ptr(out), capi.ROW_F32, None, 8, G.stream())
 
 
+def _sliced_copy(data, n, nf, val_type):
+    """The stored rows in slices of 64 (tsvm_csr_slice_widths, tsvm_csr_to_sliced), checked against a numpy layout."""
+    val_d, col_d, ptr_d = G.dev(data.val), G.dev(data.col), G.dev(data.ptr)
+    n_slices = (n + 63) // 64
+    widths = torch.zeros(n_slices, dtype=torch.int32, device="cuda")
+    capi.call("tsvm_csr_slice_widths", G.ptr(ptr_d), n, G.ptr(widths), G.stream())
+    lens = np.diff(data.ptr)
+    want_w = np.array([lens[s * 64:(s + 1) * 64].max(initial=0) for s in range(n_slices)])
+    assert np.array_equal(G.host(widths), want_w)
+    sp = np.concatenate([[0], np.cumsum(64 * want_w)]).astype(np.int64)
+    sp_d = G.dev(sp)
+    ell_col = torch.full((int(sp[-1]),), -5, dtype=torch.int32, device="cuda")
+    ell_val = torch.full((int(sp[-1]),), 7.0, dtype=torch.float32 if val_type == capi.ROW_F32 else torch.float64, device="cuda")
+    capi.call("tsvm_csr_to_sliced", G.ptr(val_d), G.ptr(col_d), G.ptr(ptr_d), n, G.ptr(sp_d), nf, G.ptr(ell_col), G.ptr(ell_val),
+              val_type, G.stream())
+    ec, ev = G.host(ell_col), G.host(ell_val).astype(np.float64)
+    for j in (0, 1, 63, 64, n // 2, n - 1):
+        s, l = j // 64, j % 64
+        ent = sp[s] + 64 * np.arange(want_w[s]) + l
+        k = lens[j]
+        assert np.array_equal(ec[ent[:k]], data.col[data.ptr[j]:data.ptr[j + 1]]) and (ec[ent[k:]] == nf).all()
+        assert np.array_equal(ev[ent[:k]], data.val[data.ptr[j]:data.ptr[j + 1]]) and (ev[ent[k:]] == 0).all()
+    return (val_d, col_d, ptr_d), sp_d, ell_col, ell_val
+
+
+@pytest.mark.parametrize("n,d,m,max_k", [(700, 3000, 70, 40), (5000, 3000, 512, 40), (3000, 20958, 130, 90), (1000, 50, 16, 50),
+                                         (333, 9000, 1, 30)])
+@pytest.mark.parametrize("name,kt,prm", KERNELS)
+def test_csr_sliced_path(name, kt, prm, n, d, m, max_k):
+    """tsvm_get_rows_csr_sliced (stored rows streamed from their sliced copy, working rows as a tile in LDS) against the
+    oracle's rows, bit for bit: skewed feature frequencies (a few features in almost every row, a long tail), empty rows,
+    a working set that is not a multiple of sixteen, duplicates in the working set, output slots, both value types."""
+    rng = np.random.default_rng(n + m)
+    p_col = 1.0 / np.arange(1, d + 1) ** 1.1
+    p_col /= p_col.sum()
+    ptr, col, val = [0], [], []
+    for i in range(n):
+        k = int(rng.integers(0, max_k + 1)) if i % 7 else 0
+        c = np.sort(rng.choice(d, size=min(k, d), replace=False, p=p_col)) + 1
+        col.extend(c)
+        val.extend(rng.standard_normal(len(c)).astype(np.float32))
+        ptr.append(len(col))
+    data = CsrData(ptr, col, np.asarray(val, dtype=np.float64))
+    p = O.make_param(kernel_type=kt, expf_mode=1, **prm)
+    okm = O.KernelMatrix(data.ptr, data.col, data.val, p)
+    nf = okm.n_features
+    max_nnz = int(np.diff(data.ptr).max())
+    idx = rng.integers(0, n, size=m).astype(np.int32)
+    if m > 3: idx[3] = idx[1]
+    idx_d = G.dev(idx)
+    want = okm.get_rows(idx)
+    slots = rng.permutation(m + 5)[:m].astype(np.int32)
+    slots_d = G.dev(slots)
+    for val_type in (capi.ROW_F32, capi.ROW_F64):
+        lds = capi.kernel_lib().tsvm_get_rows_csr_sliced_lds(nf, max_nnz, val_type)
+        assert 0 < lds <= 160 * 1024, lds
+        (val_d, col_d, ptr_d), sp_d, ell_col, ell_val = _sliced_copy(data, n, nf, val_type)
+        sd = torch.empty(n, dtype=torch.float64, device="cuda")
+        capi.call("tsvm_csr_self_dot", G.ptr(val_d), G.ptr(ptr_d), n, G.ptr(sd), G.stream())
+        row_types = [capi.ROW_F64] if kt == O.LINEAR else [capi.ROW_F64, capi.ROW_F32]
+        for rt in row_types:
+            ldo = n + 3
+            out = torch.full((m + 5, ldo), -3.0, dtype=torch.float32 if rt == capi.ROW_F32 else torch.float64, device="cuda")
+            capi.call("tsvm_get_rows_csr_sliced", G.ptr(ell_col), G.ptr(ell_val), val_type, G.ptr(sp_d), n, G.ptr(sd), G.ptr(val_d),
+                      G.ptr(col_d), G.ptr(ptr_d), G.ptr(idx_d), m, G.ptr(sd), nf, max_nnz, kt, prm.get("gamma", 0.0),
+                      prm.get("coef0", 0.0), prm.get("degree", 3), G.ptr(out), rt, G.ptr(slots_d), ldo, G.stream())
+            got = G.host(out).astype(np.float64)
+            _check(name, got[slots][:, :n], want)
+            untouched = np.setdiff1d(np.arange(m + 5), slots)
+            assert (got[untouched] == -3.0).all() and (got[:, n:] == -3.0).all()
+    # shapes the kernel does not take are refused: rows so long that eight of them overflow the tile, feature tables
+    # larger than the LDS
+    assert capi.kernel_lib().tsvm_get_rows_csr_sliced_lds(20000, 5000, capi.ROW_F32) == 0
+    assert capi.kernel_lib().tsvm_get_rows_csr_sliced_lds(200000, 10, capi.ROW_F32) == 0
+
+
 @pytest.mark.parametrize("n", [700, 5000])   # four / sixteen stored rows per workgroup
 @pytest.mark.parametrize("name,kt,prm", KERNELS)
 def test_csr_path(name, kt, prm, n):

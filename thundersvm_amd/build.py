@@ -23,15 +23,14 @@ def build_kernels(extra=(), only=None):
     """One object per source file, compiled side by side, then one link.  `only`: recompile just these sources and
     reuse the other objects of an earlier call (development)."""
     import concurrent.futures
-    import tempfile
     srcs = sorted(f for f in os.listdir(CSRC) if f.endswith(".hip"))
-    objdir = os.environ.get("TSVM_OBJ_DIR") or tempfile.mkdtemp(prefix="tsvm_obj_")
+    objdir = os.environ.get("TSVM_OBJ_DIR") or os.path.join(HERE, "build", "obj")   # (kept: `only` reuses the other objects)
     os.makedirs(objdir, exist_ok=True)
     objs = [os.path.join(objdir, f[:-4] + ".o") for f in srcs]
     todo = [(f, o) for f, o in zip(srcs, objs) if only is None or f in only or not os.path.exists(o)]
     with concurrent.futures.ThreadPoolExecutor(max_workers=min(6, max(1, len(todo)))) as pool:
         list(pool.map(lambda fo: _run(["hipcc", *HIP_FLAGS, *extra, "-c", "-o", fo[1], os.path.join(CSRC, fo[0])]), todo))
-    _run(["hipcc", "--offload-arch=gfx950", "-fPIC", "-shared", "-o", KERNEL_LIB, *objs])
+    _run(["hipcc", *HIP_FLAGS, *extra, "-shared", "-o", KERNEL_LIB, *objs])
     return KERNEL_LIB
 
 

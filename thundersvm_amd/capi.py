@@ -37,6 +37,11 @@ SIGNATURES = {
     "tsvm_csr_scatter_rows": (_int, [_p, _p, _p, _p, _int, _int, _p, _int, _int, _p]),
     "tsvm_get_rows_csr": (_int, [_p, _p, _p, _p, _i64, _p, _p, _int, _p, _int, _dbl, _dbl, _int, _p, _int, _p, _i64, _p]),
     "tsvm_get_rows_csr_staged": (_int, [_p, _p, _p, _p, _i64, _p, _p, _int, _int, _p, _int, _dbl, _dbl, _int, _p, _int, _p, _i64, _p]),
+    "tsvm_csr_slice_widths": (_int, [_p, _i64, _p, _p]),
+    "tsvm_csr_to_sliced": (_int, [_p, _p, _p, _i64, _p, _int, _p, _p, _int, _p]),
+    "tsvm_get_rows_csr_sliced_lds": (C.c_size_t, [_int, _int, _int]),
+    "tsvm_get_rows_csr_sliced": (_int, [_p, _p, _int, _p, _i64, _p, _p, _p, _p, _p, _int, _p, _int, _int, _int, _dbl, _dbl, _int,
+                                        _p, _int, _p, _i64, _p]),
     "tsvm_fold_ids": (_int, [_p, _int, _int, _p, _p]),
     "tsvm_gather_rows_f64": (_int, [_p, _i64, _p, _i64, _p, _p]),
     "tsvm_csr_gather_rows": (_int, [_p, _p, _p, _p, _i64, _p, _p, _p, _p]),

@@ -455,6 +455,219 @@ __global__ __launch_bounds__(256) void get_rows_csr_kernel(
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// CSR get_rows on a sliced copy of the stored rows.
+//
+// The kernel above reads the staged working rows once per stored non-zero: m values for every entry of the matrix,
+// gigabytes through the L2 per call.  Here the roles are turned round.  The stored rows are kept a second time in
+// slices of 64 rows (sliced ELL): entry k of row 64 s + l lies at slice_ptr[s] + 64 k + l, rows shorter than their
+// slice's longest are padded with the column n_features and the value 0, so a wavefront reads 64 rows' k-th entries
+// as one contiguous run.  One thread owns one stored row j and sixteen accumulators, one per working row of the
+// workgroup's block of sixteen; the block's working rows live in LDS as a dense tile over the features that occur
+// in them (a 16-bit table maps a feature to its tile row, or to "absent").  Every stored entry is read once per
+// block of sixteen working rows (from the L2: all blocks walk the same rows at the same time), looked up in LDS, and
+// if present multiplied into the sixteen sums.  Products with absent features are zero and are left out; the others
+// are added in stored order, so every sum is the serial chain of the reference, bit for bit.
+// ------------------------------------------------------------------------------------------------
+#define SL_T 1024   // threads = stored rows per step of a workgroup (sixteen slices)
+#define SL_IB 16    // working rows per workgroup
+
+template <typename TV>
+__global__ void csr_slice_fill_kernel(const double *__restrict__ val, const int *__restrict__ col,
+                                      const int64_t *__restrict__ row_ptr, int64_t n, const int64_t *__restrict__ slice_ptr,
+                                      int pad_col, int *__restrict__ ell_col, TV *__restrict__ ell_val) {
+    const int64_t s = blockIdx.x;
+    const int lane = threadIdx.x & 63;
+    const int64_t base = slice_ptr[s];
+    const int width = (int) ((slice_ptr[s + 1] - base) >> 6);
+    const int64_t j = s * 64 + lane;
+    const int64_t e0 = j < n ? row_ptr[j] : 0, len = j < n ? row_ptr[j + 1] - e0 : 0;
+    for (int k = threadIdx.x >> 6; k < width; k += blockDim.x >> 6) {
+        const bool live = k < len;
+        ell_col[base + (int64_t) k * 64 + lane] = live ? col[e0 + k] : pad_col;
+        ell_val[base + (int64_t) k * 64 + lane] = live ? (TV) val[e0 + k] : (TV) 0;
+    }
+}
+
+__global__ void csr_slice_widths_kernel(const int64_t *__restrict__ row_ptr, int64_t n, int *__restrict__ widths) {
+    const int64_t j = (int64_t) blockIdx.x * 64 + (threadIdx.x & 63);
+    int len = j < n ? (int) (row_ptr[j + 1] - row_ptr[j]) : 0;
+#pragma unroll
+    for (int msk = 32; msk >= 1; msk >>= 1) len = max(len, __shfl_xor(len, msk, 64));
+    if ((threadIdx.x & 63) == 0) widths[blockIdx.x] = len;
+}
+
+// LDS layout of the kernel below: tile double[4][slot_cap][4] | remap u16[d + 2] | bits u32[words] | base u32[words].
+// The tile takes what the other tables leave of SL_LDS_BUDGET.
+#define SL_LDS_BUDGET (156 * 1024)
+struct SlicedLds {
+    size_t remap, bits, base, total;
+    int slot_cap;
+};
+static SlicedLds sliced_lds(int d) {
+    SlicedLds l;
+    const size_t words = ((size_t) d + 1 + 31) / 32;
+    const size_t tables = (((size_t) d + 2) * 2 + 15) / 16 * 16 + 2 * words * 4 + 16;
+    const size_t room = SL_LDS_BUDGET > tables ? SL_LDS_BUDGET - tables : 0;
+    l.slot_cap = (int) std::min<size_t>(room / (SL_IB * sizeof(double)), 0xfffe);
+    l.remap = (size_t) l.slot_cap * SL_IB * sizeof(double);
+    l.bits = l.remap + (((size_t) d + 2) * 2 + 15) / 16 * 16;
+    l.base = l.bits + words * 4;
+    l.total = l.base + words * 4 + 16;
+    return l;
+}
+
+// The working rows' tile holds doubles: a float there would have to be widened once per use, and on this part the
+// conversion instruction runs at a quarter of the rate of a double-precision multiply-add (with a float tile the
+// kernel took 0.36 ms at 512 x 72,000 rows of ~50 entries, the conversions two thirds of it).
+// A block of sixteen working rows whose features outnumber the tile's rows is done in two halves (the host has
+// checked that eight of the longest rows fit).
+template <int KT, typename TO, typename TV>
+__global__ __launch_bounds__(SL_T) void get_rows_csr_sliced_kernel(
+    const int *__restrict__ ell_col, const TV *__restrict__ ell_val, const int64_t *__restrict__ slice_ptr, int64_t n,
+    const double *__restrict__ sd_x, const double *__restrict__ a_val, const int *__restrict__ a_col,
+    const int64_t *__restrict__ a_ptr, const int *__restrict__ a_idx, int m, const double *__restrict__ sd_a, int d,
+    int slot_cap, KernelParam kp_in, TO *__restrict__ out, const int *__restrict__ out_slots, int64_t ldo, unsigned n_ib,
+    int steps, size_t off_remap, size_t off_bits, size_t off_base) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    __shared__ uint64_t exp_tab[32];
+    __shared__ double s_sdi[SL_IB];
+    KernelParam kp = kp_in;
+    kp.kernel_type = KT;
+    __shared__ int64_t s_orow[SL_IB];
+    __shared__ int64_t s_arow[SL_IB];
+    __shared__ unsigned s_wave_total[SL_T / 64];
+    double *tile = (double *) lds;
+    uint16_t *remap = (uint16_t *) (lds + off_remap);
+    unsigned *bits = (unsigned *) (lds + off_bits);
+    unsigned *wbase = (unsigned *) (lds + off_base);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const unsigned logical = xcd_remap(blockIdx.x, gridDim.x);
+    const int i0 = (int) (logical % n_ib) * SL_IB;
+    const int64_t chunk = logical / n_ib;
+    const int n_words = (d + 1 + 31) / 32;
+    const int wpt = (n_words + SL_T - 1) / SL_T;
+    const int64_t n_slices = (n + 63) / 64;
+    typedef double tile4 __attribute__((ext_vector_type(4)));
+    if (tid < 32) exp_tab[tid] = TSVM_EXP2F_TAB[tid];
+    if (tid < SL_IB) {
+        const int i = i0 + tid < m ? i0 + tid : m - 1;
+        const int64_t row = a_idx ? (int64_t) a_idx[i] : (int64_t) i;
+        s_arow[tid] = row;
+        s_sdi[tid] = sd_a ? sd_a[row] : 0.0;
+        s_orow[tid] = (int64_t) (out_slots ? out_slots[i] : i) * ldo;
+    }
+    __syncthreads();
+    int r0 = 0, nr = SL_IB;   // the working rows of this pass: r0 .. r0 + nr - 1 of the block, at tile positions 0 .. nr - 1
+    while (r0 < SL_IB) {
+        // which features occur in the pass's rows (wavefront p walks row r0 + p)
+        const bool row_live = wave < nr && i0 + r0 + wave < m;
+        const int64_t ae0 = row_live ? a_ptr[s_arow[r0 + wave]] : 0, ae1 = row_live ? a_ptr[s_arow[r0 + wave] + 1] : 0;
+        for (int w = tid; w < n_words; w += SL_T) bits[w] = 0;
+        __syncthreads();
+        for (int64_t e = ae0 + lane; e < ae1; e += 64) {
+            const int c = a_col[e];
+            if (c >= 0 && c < d) atomicOr(&bits[c >> 5], 1u << (c & 31));
+        }
+        __syncthreads();
+        // tile rows in feature order: exclusive prefix sums of the words' bit counts
+        unsigned mine = 0;
+        for (int q = 0; q < wpt; ++q) {
+            const int w = tid * wpt + q;
+            mine += w < n_words ? __popc(bits[w]) : 0;
+        }
+        unsigned incl = mine;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const unsigned t = __shfl_up(incl, off, 64);
+            if (lane >= off) incl += t;
+        }
+        if (lane == 63) s_wave_total[wave] = incl;
+        __syncthreads();
+        unsigned before = 0, n_slots = 0;
+        for (int w = 0; w < SL_T / 64; ++w) {
+            before += w < wave ? s_wave_total[w] : 0;
+            n_slots += s_wave_total[w];
+        }
+        if (n_slots > (unsigned) slot_cap && nr > SL_IB / 2) {   // (uniform) too many features: this half first, then the other
+            nr = SL_IB / 2;
+            __syncthreads();
+            continue;
+        }
+        unsigned run = before + incl - mine;
+        for (int q = 0; q < wpt; ++q) {
+            const int w = tid * wpt + q;
+            if (w < n_words) {
+                wbase[w] = run;
+                run += __popc(bits[w]);
+            }
+        }
+        __syncthreads();
+        for (int c = tid; c <= d; c += SL_T) {
+            const unsigned word = bits[c >> 5], bit = 1u << (c & 31);
+            remap[c] = (word & bit) ? (uint16_t) (wbase[c >> 5] + __popc(word & (bit - 1u))) : (uint16_t) 0xffff;
+        }
+        // The tile in four parts, one per group of four working rows: part g holds 4 values per tile row, [slot_cap][4],
+        // so that the 64 lanes of a read, each at another tile row, spread over the LDS banks.
+        for (unsigned e = tid; e < (unsigned) slot_cap * SL_IB; e += SL_T) tile[e] = 0.0;
+        __syncthreads();
+        for (int64_t e = ae0 + lane; e < ae1; e += 64) {
+            const int c = a_col[e];
+            if (c >= 0 && c < d) {
+                const unsigned slot = remap[c];
+                if (slot < (unsigned) slot_cap) tile[((unsigned) (wave >> 2) * slot_cap + slot) * 4 + (wave & 3)] = a_val[e];
+            }
+        }
+        __syncthreads();
+
+        for (int step = 0; step < steps; ++step) {
+            const int64_t slice = (chunk * steps + step) * (SL_T / 64) + wave;
+            if (slice >= n_slices) break;   // (wavefront-uniform; no barrier inside this loop)
+            const int64_t base = slice_ptr[slice];
+            const int width = (int) ((slice_ptr[slice + 1] - base) >> 6);
+            const int64_t j = slice * 64 + lane;
+            double acc[SL_IB];
+#pragma unroll
+            for (int r = 0; r < SL_IB; ++r) acc[r] = 0.0;
+            const int *pc = ell_col + base + lane;
+            const TV *pv = ell_val + base + lane;
+            auto take = [&](int c, double v) {
+                const unsigned slot = remap[c];
+                if (slot != 0xffffu) {
+                    const tile4 *t = (const tile4 *) tile + slot;
+#pragma unroll
+                    for (int g = 0; g < SL_IB / 4; ++g) {
+                        const tile4 a4 = t[(size_t) g * slot_cap];
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) acc[g * 4 + u] = __builtin_fma(v, a4[u], acc[g * 4 + u]);
+                    }
+                }
+            };
+            int k = 0;
+            for (; k + 4 <= width; k += 4) {   // four entries' loads go out together; the products keep stored order
+                int c[4];
+                TV v[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    c[u] = pc[(int64_t) (k + u) * 64];
+                    v[u] = pv[(int64_t) (k + u) * 64];
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) take(c[u], (double) v[u]);
+            }
+            for (; k < width; ++k) take(pc[(int64_t) k * 64], (double) pv[(int64_t) k * 64]);
+            if (j < n) {
+                const double sdj = sd_x ? sd_x[j] : 0.0;
+#pragma unroll
+                for (int p = 0; p < SL_IB; ++p)
+                    if (p < nr && i0 + r0 + p < m) out[s_orow[r0 + p] + j] = tsvm_epilogue_as<TO>(acc[p], s_sdi[r0 + p], sdj, kp, exp_tab);
+            }
+        }
+        r0 += nr;
+        __syncthreads();   // every wavefront is done with the tile before the next pass rebuilds it
+    }
+}
+
 // out row r = x row idx[r]; rows are ld doubles long, ld a multiple of 4, moved as 32-byte vectors
 __global__ void gather_rows_f64_kernel(const v4d *__restrict__ x, int64_t ld4, const int *__restrict__ idx, int64_t m,
                                        v4d *__restrict__ out) {
@@ -974,6 +1187,98 @@ int tsvm_get_rows_csr_staged(const double *val, const int *col, const int64_t *r
                              tsvm_stream stream) {
     return get_rows_csr(val, col, row_ptr, x_idx, n, sd_x, w, w_type, m, sd_w, kernel_type, gamma, coef0, degree, out, row_type,
                         out_slots, ldo, stream);
+}
+
+int tsvm_csr_slice_widths(const int64_t *row_ptr, int64_t n, int *widths, tsvm_stream stream) {
+    TSVM_REQUIRE(row_ptr && widths && n >= 0, "tsvm_csr_slice_widths: bad argument");
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(csr_slice_widths_kernel, dim3(grid_for(n, 64)), dim3(64), 0, tsvm_s(stream), row_ptr, n, widths);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+int tsvm_csr_to_sliced(const double *val, const int *col, const int64_t *row_ptr, int64_t n, const int64_t *slice_ptr, int pad_col,
+                       int *ell_col, void *ell_val, int val_type, tsvm_stream stream) {
+    TSVM_REQUIRE(row_ptr && slice_ptr && ell_col && ell_val && n >= 0, "tsvm_csr_to_sliced: bad argument");
+    TSVM_REQUIRE(val_type == TSVM_ROW_F64 || val_type == TSVM_ROW_F32, "tsvm_csr_to_sliced: unknown value type %d", val_type);
+    if (n == 0) return 0;
+    const dim3 grid(grid_for(n, 64)), block(256);
+    if (val_type == TSVM_ROW_F32)
+        hipLaunchKernelGGL(csr_slice_fill_kernel<float>, grid, block, 0, tsvm_s(stream), val, col, row_ptr, n, slice_ptr, pad_col, ell_col,
+                           (float *) ell_val);
+    else
+        hipLaunchKernelGGL(csr_slice_fill_kernel<double>, grid, block, 0, tsvm_s(stream), val, col, row_ptr, n, slice_ptr, pad_col, ell_col,
+                           (double *) ell_val);
+    TSVM_LAUNCH_CHECK();
+    return 0;
+}
+
+size_t tsvm_get_rows_csr_sliced_lds(int n_features, int max_row_nnz, int val_type) {
+    (void) val_type;
+    if (n_features < 1 || max_row_nnz < 0) return 0;
+    const SlicedLds l = sliced_lds(n_features);
+    // half a block of the longest rows has to fit the tile (whole blocks that do not are done in two halves)
+    if ((int64_t) l.slot_cap < std::min<int64_t>((int64_t) (SL_IB / 2) * std::max(max_row_nnz, 1), (int64_t) n_features)) return 0;
+    return l.total;
+}
+
+int tsvm_get_rows_csr_sliced(const int *ell_col, const void *ell_val, int val_type, const int64_t *slice_ptr, int64_t n,
+                             const double *sd_x, const double *a_val, const int *a_col, const int64_t *a_ptr, const int *a_idx,
+                             int m, const double *sd_a, int n_features, int max_row_nnz, int kernel_type, double gamma,
+                             double coef0, int degree, void *out, int row_type, const int *out_slots, int64_t ldo,
+                             tsvm_stream stream) {
+    TSVM_REQUIRE(ell_col && ell_val && slice_ptr && a_col && a_val && a_ptr && out, "tsvm_get_rows_csr_sliced: null pointer");
+    TSVM_REQUIRE(val_type == TSVM_ROW_F64 || val_type == TSVM_ROW_F32, "tsvm_get_rows_csr_sliced: unknown value type %d", val_type);
+    TSVM_REQUIRE(n >= 0 && m >= 0 && ldo >= n && n_features >= 1, "tsvm_get_rows_csr_sliced: bad size");
+    TSVM_REQUIRE(kernel_type >= 0 && kernel_type <= 4, "tsvm_get_rows_csr_sliced: unknown kernel type %d", kernel_type);
+    TSVM_REQUIRE(row_type_ok(row_type, kernel_type), "tsvm_get_rows_csr_sliced: row type %d not valid for kernel type %d", row_type,
+                 kernel_type);
+    TSVM_REQUIRE((kernel_type != TSVM_RBF && kernel_type != TSVM_PRECOMPUTED) || (sd_x && sd_a),
+                 "tsvm_get_rows_csr_sliced: RBF needs self dot products");
+    const size_t lds_bytes = tsvm_get_rows_csr_sliced_lds(n_features, max_row_nnz, val_type);
+    TSVM_REQUIRE(lds_bytes > 0, "tsvm_get_rows_csr_sliced: %d features with rows of up to %d entries do not fit the LDS", n_features,
+                 max_row_nnz);
+    if (n == 0 || m == 0) return 0;
+    KernelParam kp{kernel_type, degree, gamma, coef0};
+    const SlicedLds l = sliced_lds(n_features);
+    const unsigned n_ib = (unsigned) ((m + SL_IB - 1) / SL_IB);
+    // a workgroup takes `steps` runs of 1024 stored rows: enough workgroups for three rounds of the chip, few enough
+    // that building the tile (once per workgroup) stays a small part
+    const int64_t runs = (n + SL_T - 1) / SL_T;
+    const int steps = (int) std::max<int64_t>(1, std::min<int64_t>(8, runs * n_ib / 768));
+    const int64_t chunks = (runs + steps - 1) / steps;
+    TSVM_REQUIRE(chunks * n_ib < (int64_t) 0x7fffffff, "tsvm_get_rows_csr_sliced: grid too large");
+    const dim3 grid((unsigned) (chunks * n_ib)), block(SL_T);
+#define SL_LAUNCH_K(KTYPE, TO, TV)                                                                                           \
+    do {                                                                                                                     \
+        static bool opted_ = false;                                                                                          \
+        if (!opted_) {                                                                                                       \
+            TSVM_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(get_rows_csr_sliced_kernel<KTYPE, TO, TV>),          \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, SL_LDS_BUDGET));                        \
+            opted_ = true;                                                                                                   \
+        }                                                                                                                    \
+        hipLaunchKernelGGL((get_rows_csr_sliced_kernel<KTYPE, TO, TV>), grid, block, l.total, tsvm_s(stream), ell_col,       \
+                           (const TV *) ell_val, slice_ptr, n, sd_x, a_val, a_col, a_ptr, a_idx, m, sd_a, n_features, l.slot_cap, kp, \
+                           (TO *) out, out_slots, ldo, n_ib, steps, l.remap, l.bits, l.base);                                \
+    } while (0)
+#define SL_LAUNCH(TO, TV)                                              \
+    do {                                                               \
+        switch (kernel_type) {                                         \
+            case TSVM_LINEAR: SL_LAUNCH_K(TSVM_LINEAR, double, TV); break; \
+            case TSVM_POLY: SL_LAUNCH_K(TSVM_POLY, TO, TV); break;     \
+            case TSVM_SIGMOID: SL_LAUNCH_K(TSVM_SIGMOID, TO, TV); break; \
+            default: SL_LAUNCH_K(TSVM_RBF, TO, TV); break;             \
+        }                                                              \
+    } while (0)
+    if (row_type == TSVM_ROW_F32) {
+        if (val_type == TSVM_ROW_F32) SL_LAUNCH(float, float); else SL_LAUNCH(float, double);
+    } else {
+        if (val_type == TSVM_ROW_F32) SL_LAUNCH(double, float); else SL_LAUNCH(double, double);
+    }
+#undef SL_LAUNCH_K
+#undef SL_LAUNCH
+    TSVM_LAUNCH_CHECK();
+    return 0;
 }
 
 int tsvm_gather_rows_f64(const double *x, int64_t ld, const int *idx, int64_t m, double *out, tsvm_stream stream) {

@@ -137,8 +137,36 @@ std::shared_ptr<DeviceRows> DeviceRows::from_host(const DataSet::node2d &all, co
         r.find_indicator_columns();
     } else {
         r.host_row_ptr = std::move(ptr);
+        r.build_sliced();
     }
     return out;
+}
+
+// The sliced copy of CSR rows (row offsets are known on the host).
+void DeviceRows::build_sliced() {
+    sliced_lds = 0;
+    max_row_nnz = 0;
+    if (dense || n == 0 || getenv("TSVM_NO_SLICED")) return;
+    for (size_t i = 0; i < n; ++i) max_row_nnz = std::max(max_row_nnz, (int) (host_row_ptr[i + 1] - host_row_ptr[i]));
+    const int vt = values_fit_float ? TSVM_ROW_F32 : TSVM_ROW_F64;
+    const size_t need = tsvm_get_rows_csr_sliced_lds((int) n_features, max_row_nnz, vt);
+    if (need == 0) return;
+    const size_t n_slices = (n + 63) / 64;
+    std::vector<int64_t> sp(n_slices + 1, 0);
+    for (size_t s = 0; s < n_slices; ++s) {
+        int64_t w = 0;
+        for (size_t i = s * 64; i < std::min(n, s * 64 + 64); ++i) w = std::max(w, host_row_ptr[i + 1] - host_row_ptr[i]);
+        sp[s + 1] = sp[s] + 64 * w;
+    }
+    // (a few very long rows would blow the padded copy up: then the plain CSR kernel stays in charge)
+    if ((size_t) sp[n_slices] > 4 * nnz + 64 * n_slices) return;
+    slice_ptr.upload(sp);
+    ell_col.resize((size_t) sp[n_slices]);
+    ell_val.resize((size_t) sp[n_slices] * (values_fit_float ? sizeof(float) : sizeof(double)));
+    abi_check(tsvm_csr_to_sliced(val.data(), col.data(), row_ptr.data(), (int64_t) n, slice_ptr.data(), (int) n_features, ell_col.data(),
+                                 ell_val.data(), vt, nullptr));
+    TSVM_HIP_CHECK(hipDeviceSynchronize());
+    sliced_lds = need;
 }
 
 std::shared_ptr<DeviceRows> DeviceRows::subset(const DeviceRows &base, const int *rows, size_t n_rows) {
@@ -174,6 +202,7 @@ std::shared_ptr<DeviceRows> DeviceRows::subset(const DeviceRows &base, const int
         r.col.resize(r.nnz);
         abi_check(tsvm_csr_gather_rows(base.val.data(), base.col.data(), base.row_ptr.data(), d_rows.data(), (int64_t) n_rows,
                                        r.row_ptr.data(), r.val.data(), r.col.data(), nullptr));
+        r.build_sliced();
     }
     TSVM_HIP_CHECK(hipDeviceSynchronize());   // d_rows is released on return
     return out;
@@ -317,9 +346,16 @@ void KernelMatrix::get_rows(const int *d_idx, int m, void *d_out, int64_t ld, co
                                       d_out, row_type(), d_out_slots, ld, stream));
         return;
     }
+    const int wt = R.values_fit_float ? TSVM_ROW_F32 : TSVM_ROW_F64;
+    if (R.sliced_lds) {   // the stored rows streamed once per sixteen working rows, the working rows in LDS
+        abi_check(tsvm_get_rows_csr_sliced(R.ell_col.data(), R.ell_val.data(), wt, R.slice_ptr.data(), n, R.self_dot.data(),
+                                           R.val.data(), R.col.data(), R.row_ptr.data(), d_idx, m, R.self_dot.data(),
+                                           (int) R.n_features, R.max_row_nnz, (int) param.kernel_type, param.gamma, param.coef0,
+                                           param.degree, d_out, row_type(), d_out_slots, ld, stream));
+        return;
+    }
     // The staging matrix [n_features][m] is kept all-zero between uses: the working rows' non-zeros are written
     // into it and taken out again afterwards (nnz entries each way instead of a fill of n_features x m).
-    const int wt = R.values_fit_float ? TSVM_ROW_F32 : TSVM_ROW_F64;
     grow_zeroed(stage_w_, (size_t) m * R.n_features * (R.values_fit_float ? sizeof(float) : sizeof(double)), stream);
     if (stage_sd_.size() < (size_t) m) stage_sd_.resize(m);
     abi_check(tsvm_csr_scatter_rows(R.val.data(), R.col.data(), R.row_ptr.data(), d_idx, m, (int) R.n_features,

@@ -32,6 +32,14 @@ struct DeviceRows {
     tsvm::DeviceBuffer<int> col;
     tsvm::DeviceBuffer<int64_t> row_ptr;
     std::vector<int64_t> host_row_ptr;           // CSR layout only: needed to lay out a subset
+    // CSR layout: the rows a second time in slices of 64 (sliced ELL, see tsvm_get_rows_csr_sliced), which get_rows
+    // streams; values as float when values_fit_float.  sliced_lds == 0: the shape does not fit that kernel.
+    tsvm::DeviceBuffer<int> ell_col;
+    tsvm::DeviceBuffer<unsigned char> ell_val;
+    tsvm::DeviceBuffer<int64_t> slice_ptr;
+    int max_row_nnz = 0;
+    size_t sliced_lds = 0;
+    void build_sliced();
     tsvm::DeviceBuffer<kernel_type> self_dot;    // [n]
     // per column c < n_features: [c] = entries (dense: non-zero values; CSR: stored entries), [n_features + c] = values
     // that are neither 0 nor 1; counted on the device on first use
