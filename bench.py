@@ -57,6 +57,8 @@ def parse():
     ap.add_argument("--loader-only", action="store_true", help="only write the workload's LibSVM text and time the loader (no GPU)")
     ap.add_argument("--kernels-only", action="store_true",
                     help="only launch get_rows / update_f at the workload's shape plus a 1 GiB device copy (for rocprofv3 counter runs)")
+    ap.add_argument("--predict-only", action="store_true",
+                    help="only train once and predict the workload's test rows, plus a 1 GiB device copy (for rocprofv3 runs)")
     return ap.parse_args()
 
 
@@ -377,6 +379,42 @@ def cpu_baseline(train, params, model, budget_s):
                 estimate=True)
 
 
+def measure_predict(model, test, d, nb):
+    """Predicts `test` once from host memory and three times from rows resident in HBM (best of three)."""
+    import numpy as np
+    from thundersvm_amd.model import Dataset, choose_dense
+    ds_test = Dataset(test)
+    model.predict(test.rows(np.arange(min(test.n, 256))))
+    t0 = time.time()
+    model.predict(ds_test)
+    pt = time.time() - t0
+    dd_test = Dataset(test).to_device()
+    model.predict(dd_test)
+    ptd = []
+    for _ in range(3):
+        t0 = time.time()
+        model.predict(dd_test)
+        ptd.append(time.time() - t0)
+    ptd = min(ptd)
+    k = model.n_classes
+    n_sv = int(model.total_sv)
+    flops_row = 2.0 * n_sv * d + 2.0 * (k - 1) * n_sv
+    # what has to move: the batch, the support vectors, the coefficients, the decision values (no kernel values)
+    by = 8.0 * (test.n * d + n_sv * d + (k - 1) * n_sv + test.n * nb)
+    return dict(rows=test.n, n_sv=n_sv, classes=k, seconds=pt, rows_per_s=test.n / pt,
+                note="rows_per_s: test rows start in host memory; *_device_rows: rows resident in HBM "
+                     "(Dataset.to_device), decision values copied back",
+                seconds_device_rows=ptd, rows_per_s_device_rows=test.n / ptd,
+                flops_per_row=flops_row, tflops=flops_row * test.n / pt / 1e12,
+                frac_mfma_peak=flops_row * test.n / pt / 1e12 / FP64_MFMA_PEAK_TFLOPS,
+                tflops_device_rows=flops_row * test.n / ptd / 1e12,
+                frac_mfma_peak_device_rows=flops_row * test.n / ptd / 1e12 / FP64_MFMA_PEAK_TFLOPS,
+                bytes=by, frac_hbm_peak=by / ptd / 1e9 / HBM_PEAK_GBS,
+                kernel="tsvm_predict_dec_values_dense (kernel values reduced in registers)"
+                       if choose_dense(n_sv, d + 1, model._sv_nnz) else
+                       "tsvm_get_rows_csr + tsvm_sum_kernel_values")
+
+
 def measure_config(name, w, steps, warmup, with_kernels=True, predict=True):
     """Trains `steps` times (after `warmup`) on device-resident rows, once more from host rows, once phase-profiled;
     predicts the test rows; times the kernels at the workload's shape."""
@@ -443,37 +481,7 @@ def measure_config(name, w, steps, warmup, with_kernels=True, predict=True):
         "note": "from one phase-profiled pass (one problem at a time, every phase timed with device events); ms_local includes the ws x ws block"}
     del pm
     if predict and test is not None:
-        ds_test = Dataset(test)
-        model.predict(test.rows(np.arange(min(test.n, 256))))
-        t0 = time.time()
-        model.predict(ds_test)
-        pt = time.time() - t0
-        dd_test = Dataset(test).to_device()
-        model.predict(dd_test)
-        ptd = []
-        for _ in range(3):
-            t0 = time.time()
-            model.predict(dd_test)
-            ptd.append(time.time() - t0)
-        ptd = min(ptd)
-        k = model.n_classes
-        n_sv = int(model.total_sv)
-        flops_row = 2.0 * n_sv * d + 2.0 * (k - 1) * n_sv
-        # what has to move: the batch, the support vectors, the coefficients, the decision values (no kernel values)
-        by = 8.0 * (test.n * d + n_sv * d + (k - 1) * n_sv + test.n * nb)
-        block["predict"] = dict(rows=test.n, n_sv=n_sv, classes=k, seconds=pt, rows_per_s=test.n / pt,
-                                note="rows_per_s: test rows start in host memory; *_device_rows: rows resident in HBM "
-                                     "(Dataset.to_device), decision values copied back",
-                                seconds_device_rows=ptd, rows_per_s_device_rows=test.n / ptd,
-                                flops_per_row=flops_row, tflops=flops_row * test.n / pt / 1e12,
-                                frac_mfma_peak=flops_row * test.n / pt / 1e12 / FP64_MFMA_PEAK_TFLOPS,
-                                tflops_device_rows=flops_row * test.n / ptd / 1e12,
-                                frac_mfma_peak_device_rows=flops_row * test.n / ptd / 1e12 / FP64_MFMA_PEAK_TFLOPS,
-                                bytes=by, frac_hbm_peak=by / ptd / 1e9 / HBM_PEAK_GBS,
-                                kernel="tsvm_predict_dec_values_dense (kernel values reduced in registers)"
-                                       if choose_dense(n_sv, d + 1, model._sv_nnz) else
-                                       "tsvm_get_rows_csr + tsvm_sum_kernel_values")
-        del dd_test, ds_test
+        block["predict"] = measure_predict(model, test, d, nb)
     if with_kernels:
         block["kernels"] = kernel_figures(train, params)
     return block, model
@@ -505,19 +513,25 @@ def main():
         return
 
     # the executable in a fresh process, and the loader: before this process has touched the GPU
-    fresh = cli_and_loader(w, run_cli=True) if args.cli and not args.kernels_only else {}
+    fresh = cli_and_loader(w, run_cli=True) if args.cli and not (args.kernels_only or args.predict_only) else {}
 
     import torch
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
 
-    if args.kernels_only:
+    if args.kernels_only or args.predict_only:
         src = torch.empty(1 << 27, dtype=torch.float64, device="cuda").normal_()
         dst = torch.empty_like(src)
         dst.copy_(src)                      # plain copy of known size: 1 GiB read + 1 GiB written
         torch.cuda.synchronize()
         del src, dst
+        if args.predict_only:
+            from thundersvm_amd.model import Dataset, Model, make_param
+            prm = make_param(**w["params"])
+            model = Model(prm.svm_type).train(Dataset(w["train"]).to_device(), prm)
+            print(json.dumps(measure_predict(model, w["test"], w["train"].n_features, model.n_binary)))
+            return
         print(json.dumps(kernel_figures(w["train"], w["params"])))
         return
 

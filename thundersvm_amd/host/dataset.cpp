@@ -198,18 +198,21 @@ void DataSet::load_from_file(std::string file_name, int n_threads) {
     std::vector<LoadedRun> runs(n_runs);
 #pragma omp parallel for num_threads(n_threads) schedule(dynamic, 1)
     for (int r = 0; r < n_runs; ++r) parse_run(text.get() + cut[r], text.get() + cut[r + 1], runs[r]);
-    size_t total = 0;
-    for (const LoadedRun &r : runs) {
-        if (r.bad) throw std::runtime_error("read error, using [index]:[value] format");
-        total += r.rows.size();
-        if (r.max_index > n_features_) n_features_ = r.max_index;
-        zero_based_ = zero_based_ || r.zero_based;
+    std::vector<size_t> first(n_runs + 1, 0);
+    for (int r = 0; r < n_runs; ++r) {
+        if (runs[r].bad) throw std::runtime_error("read error, using [index]:[value] format");
+        first[r + 1] = first[r] + runs[r].rows.size();
+        if (runs[r].max_index > n_features_) n_features_ = runs[r].max_index;
+        zero_based_ = zero_based_ || runs[r].zero_based;
     }
-    y_.reserve(total);
-    instances_.reserve(total);
-    for (LoadedRun &r : runs) {
-        y_.insert(y_.end(), r.y.begin(), r.y.end());
-        for (auto &row : r.rows) instances_.push_back(std::move(row));
+    y_.resize(first[n_runs]);
+    instances_.resize(first[n_runs]);
+#pragma omp parallel for num_threads(n_threads) schedule(dynamic, 1)
+    for (int r = 0; r < n_runs; ++r) {
+        LoadedRun &run = runs[r];
+        std::copy(run.y.begin(), run.y.end(), y_.begin() + first[r]);
+        std::move(run.rows.begin(), run.rows.end(), instances_.begin() + first[r]);
+        run = LoadedRun();      // the run's own arrays are released by the thread that moved it
     }
     TSVM_LOG << "#instances = " << n_instances() << ", #features = " << n_features();
 }
