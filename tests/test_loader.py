@@ -105,6 +105,31 @@ def test_number_forms_and_layout(tmp_path):
         _same(one, Dataset(path=path, threads=t).csr())
 
 
+def test_file_that_ends_on_a_page_boundary(tmp_path):
+    """The file is parsed from a mapping of its pages: a file whose size is a whole number of pages has nothing behind
+    its last byte, so a last line without a newline must not be handed to a library call that reads on (its last token
+    here is one the short decimal parser leaves to strtof: 25 digits)."""
+    page = os.sysconf("SC_PAGE_SIZE")
+    last = "-1 1:0.5 3:1.000000059604644775390625"
+    for final_newline in (False, True):
+        body = "".join("1 1:%d.25 2:%d\n" % (i, i % 7) for i in range(3000))
+        end = last + ("\n" if final_newline else "")
+        pad = (-(len(body) + len(end))) % page
+        assert pad == 0 or pad >= 8
+        if pad:
+            body += "2 5:" + "0" * (pad - 6) + "1\n"        # a line of exactly `pad` bytes
+        text = body + end
+        assert len(text) % page == 0
+        path = str(tmp_path / ("page_%d.txt" % final_newline))
+        open(path, "w").write(text)
+        one = Dataset(path=path, threads=1).csr()
+        _against_python(path, one)
+        assert one[0].n == 3000 + (1 if pad else 0) + 1 and one[0].y[-1] == -1.0
+        assert one[0].val[-1] == 1.0      # 1 + 2^-24, the midpoint between two floats, rounds to the even one
+        for t in (3, 16):
+            _same(one, Dataset(path=path, threads=t).csr())
+
+
 def test_bad_input(tmp_path):
     from thundersvm_amd import capi
     path = str(tmp_path / "bad.txt")

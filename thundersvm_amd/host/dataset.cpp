@@ -2,6 +2,7 @@
 
 #include <fcntl.h>
 #include <omp.h>
+#include <sys/mman.h>
 #include <sys/stat.h>
 #include <unistd.h>
 
@@ -18,7 +19,7 @@ DataSet::DataSet(const node2d &instances, int n_features, const std::vector<floa
 
 // ------------------------------------------------------------------------------------------------
 // LibSVM text loader.  The reference reads 16 MB at a time and lets every OpenMP thread parse a run of whole lines
-// of the buffer (src/thundersvm/dataset.cpp:20-100); here the file is read once (every thread its share), cut into
+// of the buffer (src/thundersvm/dataset.cpp:20-100); here the whole file is mapped, cut into
 // runs of whole lines, four per thread, parsed side by side and joined in file order.  Each token "i:v" gives what
 // the reference's sscanf("%d:%f") gives: v is the correctly rounded float of the decimal text.
 // Unlike the reference, a last line without a newline is kept (the reference's buffer walk stops at the last newline
@@ -160,44 +161,74 @@ void DataSet::load_from_file(std::string file_name, int n_threads) {
     instances_.clear();
     n_features_ = 0;
     zero_based_ = false;
-    if (n_threads <= 0) n_threads = omp_get_max_threads();
     const int fd = open(file_name.c_str(), O_RDONLY);
     if (fd < 0) throw std::runtime_error("file " + file_name + " not found");
     struct stat st;
     if (fstat(fd, &st) != 0) { close(fd); throw std::runtime_error("file " + file_name + " cannot be read"); }
     const size_t size = (size_t) st.st_size;
-    std::unique_ptr<char[]> text(new char[size + 1]);
-    text[size] = 0;
-    bool read_ok = true;
-    const size_t piece = (size + n_threads - 1) / std::max(n_threads, 1);
+    if (n_threads <= 0) n_threads = omp_get_max_threads();
+    // The file's pages are parsed where the page cache holds them (a private read-only mapping: no copy, every thread
+    // faults in the part it parses).  The library calls behind parse_float / parse_double need text that ends in a
+    // character no number contains: inside the mapping that is the line's newline, so the mapping is parsed up to
+    // the last newline, and a last line without one is parsed from a NUL-terminated copy.
+    struct Mapping {
+        void *p = MAP_FAILED;
+        size_t n = 0;
+        ~Mapping() { if (p != MAP_FAILED) munmap(p, n); }
+    } map;
+    std::unique_ptr<char[]> copy;
+    const char *text = nullptr;
+    if (size > 0) {
+        map.p = mmap(nullptr, size, PROT_READ, MAP_PRIVATE, fd, 0);
+        map.n = size;
+    }
+    if (map.p != MAP_FAILED) {
+        text = (const char *) map.p;
+    } else if (size > 0) {   // a file that cannot be mapped (a pipe, a special file system): read it, every thread its share
+        copy.reset(new char[size + 1]);
+        copy[size] = 0;
+        bool read_ok = true;
+        const size_t piece = (size + n_threads - 1) / std::max(n_threads, 1);
 #pragma omp parallel for num_threads(n_threads) schedule(static, 1)
-    for (int t = 0; t < n_threads; ++t) {
-        size_t off = std::min(size, (size_t) t * piece);
-        const size_t stop = std::min(size, off + piece);
-        while (off < stop) {
-            const ssize_t got = pread(fd, text.get() + off, stop - off, (off_t) off);
-            if (got <= 0) {
+        for (int t = 0; t < n_threads; ++t) {
+            size_t off = std::min(size, (size_t) t * piece);
+            const size_t stop = std::min(size, off + piece);
+            while (off < stop) {
+                const ssize_t got = pread(fd, copy.get() + off, stop - off, (off_t) off);
+                if (got <= 0) {
 #pragma omp atomic write
-                read_ok = false;
-                break;
+                    read_ok = false;
+                    break;
+                }
+                off += (size_t) got;
             }
-            off += (size_t) got;
         }
+        if (!read_ok) { close(fd); throw std::runtime_error("file " + file_name + " cannot be read"); }
+        text = copy.get();
     }
     close(fd);
-    if (!read_ok) throw std::runtime_error("file " + file_name + " cannot be read");
-    // runs of whole lines: run r starts behind the first newline at or after byte r * size / n_runs
-    const int n_runs = n_threads == 1 ? 1 : n_threads * 4;
-    std::vector<size_t> cut(n_runs + 1, size);
+    size_t body = size;   // the part that ends in a newline
+    if (map.p != MAP_FAILED) {
+        const void *last_nl = memrchr(text, '\n', size);
+        body = last_nl ? (size_t) ((const char *) last_nl - text) + 1 : 0;
+    }
+    const std::string tail = body < size ? std::string(text + body, size - body) : std::string();
+    // runs of whole lines: run r starts behind the first newline at or after byte r * body / n_runs
+    const int n_body_runs = n_threads == 1 ? 1 : n_threads * 4;
+    const int n_runs = n_body_runs + 1;                     // the last run is the line without a newline, if any
+    std::vector<size_t> cut(n_body_runs + 1, body);
     cut[0] = 0;
-    for (int r = 1; r < n_runs; ++r) {
-        const size_t from = std::max(cut[r - 1], size / n_runs * r);
-        const char *nl = from < size ? (const char *) memchr(text.get() + from, '\n', size - from) : nullptr;
-        cut[r] = nl ? (size_t) (nl - text.get()) + 1 : size;
+    for (int r = 1; r < n_body_runs; ++r) {
+        const size_t from = std::max(cut[r - 1], body / n_body_runs * r);
+        const char *nl = from < body ? (const char *) memchr(text + from, '\n', body - from) : nullptr;
+        cut[r] = nl ? (size_t) (nl - text) + 1 : body;
     }
     std::vector<LoadedRun> runs(n_runs);
 #pragma omp parallel for num_threads(n_threads) schedule(dynamic, 1)
-    for (int r = 0; r < n_runs; ++r) parse_run(text.get() + cut[r], text.get() + cut[r + 1], runs[r]);
+    for (int r = 0; r < n_runs; ++r) {
+        if (r < n_body_runs) parse_run(text + cut[r], text + cut[r + 1], runs[r]);
+        else parse_run(tail.c_str(), tail.c_str() + tail.size(), runs[r]);
+    }
     std::vector<size_t> first(n_runs + 1, 0);
     for (int r = 0; r < n_runs; ++r) {
         if (runs[r].bad) throw std::runtime_error("read error, using [index]:[value] format");
