@@ -291,6 +291,23 @@ def cli_and_loader(w, run_cli=True, loader_threads=(1, 0)):
                                   model_bytes=os.path.getsize(model),
                                   note="fresh process: the training window holds the first allocation of the row arena, the "
                                        "creation of the CU-masked streams and the loading of the kernels' code objects")
+                if w.get("test") is not None:
+                    # thundersvm-predict on the model just written and the workload's test rows as text
+                    test_path, pred_path = os.path.join(tmp, "test.txt"), os.path.join(tmp, "test.predict")
+                    D.save_libsvm(test_path, w["test"])
+                    t0 = time.time()
+                    res = subprocess.run([os.path.join(ROOT, "thundersvm_amd", "bin", "thundersvm-predict"), test_path, model, pred_path],
+                                         capture_output=True, text=True, timeout=600)
+                    wall = time.time() - t0
+                    log = res.stderr + res.stdout
+                    if res.returncode != 0:
+                        out["cli_predict"] = dict(error=log[-400:])
+                    else:
+                        out["cli_predict"] = dict(command="thundersvm-predict test.txt train.model test.predict", rows=w["test"].n,
+                                                  model_load_seconds=grab("model loading time"), data_load_seconds=grab("data loading time"),
+                                                  predict_seconds=grab("prediction time"), process_seconds=wall,
+                                                  note="fresh process: prediction time holds the upload of the support vectors, "
+                                                       "the first allocation of the row arena and the loading of the code objects")
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
     return out
@@ -626,7 +643,7 @@ def main():
         "step_seconds": head["train_seconds_steps"],
         "train_seconds_rows_resident": head["train_seconds_rows_resident"],
         "train_seconds_cold": cli.get("train_seconds") if cli else None,
-        "cli": cli, "loader": fresh.get("loader"), "text_file": fresh.get("file"),
+        "cli": cli, "cli_predict": fresh.get("cli_predict"), "loader": fresh.get("loader"), "text_file": fresh.get("file"),
         "solver": {"outer_iterations": head["outer_iterations"], "inner_iterations": head["inner_iterations"],
                    "binary_problems": head["binary_problems"], "total_sv": head["total_sv"], "phase_ms": head["phase_ms"],
                    "cache_hit_rate": head["cache_hit_rate"], "in_training": head["in_training"]},

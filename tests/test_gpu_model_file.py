@@ -92,3 +92,35 @@ def test_libsvm_style_model_with_double_values(tmp_path):
     lab, dec = m.predict(D.from_dense(x, np.zeros(3), keep_zeros=False))
     assert np.abs(dec[:, 0] - np.array(want)).max() < 1e-6
     assert lab.tolist() == [1.0 if v > 0 else -1.0 for v in want]
+
+
+def test_support_vector_lines_of_a_large_model(tmp_path):
+    """The support-vector lines are written by several threads, runs of lines each; joined they are the lines a single
+    writer makes: every coefficient with 16 significant digits, every value with 8, in the model's own order."""
+    rng = np.random.default_rng(12)
+    k, per, d = 4, 900, 6
+    centres = rng.standard_normal((k, d))
+    cls = rng.permutation(np.repeat(np.arange(k), per))
+    x = (centres[cls] + 1.2 * rng.standard_normal((k * per, d))).astype(np.float32)
+    x[rng.random(x.shape) < 0.3] = 0.0                      # rows of different lengths
+    tr = D.from_dense(x, (cls + 1).astype(np.float64))
+    m = Model(0).train(tr, make_param(svm_type=0, kernel_type=2, gamma=0.4, C=2.0))
+    assert m.total_sv > 2000                                # many runs of 256 lines and more
+    out = str(tmp_path / "big.model")
+    m.save(out)
+    lines = open(out).read().split("\n")
+    start = lines.index("SV ") + 1
+    body = lines[start:]
+    assert body[-1] == "" and len(body) == m.total_sv + 1
+    coef = m.coef.reshape(k - 1, m.total_sv)
+    for i in range(m.total_sv):
+        lo, hi = m.sv_ptr[i], m.sv_ptr[i + 1]
+        want = "".join("%.16g " % coef[j, i] for j in range(k - 1))
+        want += "".join("%d:%.8g " % (c, v) for c, v in zip(m.sv_col[lo:hi], m.sv_val[lo:hi]))
+        assert body[i] == want, i
+    # and the text loads back to the same model text
+    m2 = Model(0)
+    m2.load(out)
+    out2 = str(tmp_path / "big2.model")
+    m2.save(out2)
+    assert open(out2).read() == open(out).read()

@@ -1,6 +1,7 @@
 // thundersvm-predict: src/thundersvm/thundersvm-predict.cpp:18-106.
 #include <hip/hip_runtime.h>
 
+#include <chrono>
 #include <cstdio>
 #include <fstream>
 
@@ -31,12 +32,20 @@ int main(int argc, char **argv) {
         std::unique_ptr<SvmModel> model = make_model((SvmParam::SVM_TYPE) type);
         TSVM_HIP_CHECK(hipSetDevice(parser.gpu_id));
         model->set_max_memory_size_Byte(parser.param_cmd.max_mem_size);
+        auto now = [] { return std::chrono::high_resolution_clock::now(); };
+        auto since = [&](std::chrono::high_resolution_clock::time_point t) { return std::chrono::duration<float>(now() - t).count(); };
+        auto t0 = now();
         model->load_from_file(parser.svmpredict_model_file_name);
+        TSVM_LOG << "model loading time = " << since(t0);
         DataSet test;
+        t0 = now();
         test.load_from_file(parser.svmpredict_input_file);
+        TSVM_LOG << "data loading time = " << since(t0);
+        t0 = now();
         std::vector<float_type> predict_y = model->predict(test.instances(), -1);
+        TSVM_LOG << "prediction time = " << since(t0);
         std::ofstream out(parser.svmpredict_output_file);
-        for (float_type v : predict_y) out << v << std::endl;
+        for (float_type v : predict_y) out << v << '\n';   // (the reference ends each line with std::endl: the same bytes)
         if (type == SvmParam::C_SVC || type == SvmParam::NU_SVC)
             TSVM_LOG << "Accuracy = " << accuracy_score(predict_y, test.y());
         else if (type == SvmParam::EPSILON_SVR || type == SvmParam::NU_SVR)

@@ -1,6 +1,9 @@
 #include <chrono>
 #include "models.h"
+#include "text_parse.h"
 #include <deque>
+
+#include <omp.h>
 
 #include <algorithm>
 #include <cmath>
@@ -174,13 +177,29 @@ std::string SvmModel::save_to_string() {
         s << std::endl;
     }
     s << "SV " << std::endl;
+    // The support-vector lines are most of a large model's text (C4: 167,298 lines, 43 MB): runs of lines are written
+    // side by side into strings of their own and joined in order.  "%.16g" / "%.8g" are what the stream writes for
+    // setprecision(16) / setprecision(8) (its num_put goes through the same printf conversion in the C locale).
     const int rows = (param.svm_type == SvmParam::NU_SVC || param.svm_type == SvmParam::C_SVC) ? n_classes - 1 : 1;
-    for (size_t i = 0; i < sv.size(); ++i) {
-        for (int j = 0; j < rows; ++j) s << std::setprecision(16) << coef[j * sv.size() + i] << " ";
-        for (const auto &nd : sv[i]) s << nd.index << ":" << std::setprecision(8) << nd.value << " ";
-        s << std::endl;
+    const size_t n = sv.size();
+    const int n_runs = (int) std::max<size_t>(1, std::min<size_t>((size_t) omp_get_max_threads() * 4, n / 256));
+    std::vector<std::string> run_text(n_runs);
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int r = 0; r < n_runs; ++r) {
+        std::string &o = run_text[r];
+        char buf[64];
+        for (size_t i = n * r / n_runs; i < n * (r + 1) / n_runs; ++i) {
+            for (int j = 0; j < rows; ++j) o.append(buf, snprintf(buf, sizeof buf, "%.16g ", (double) coef[j * n + i]));
+            for (const auto &nd : sv[i]) o.append(buf, snprintf(buf, sizeof buf, "%d:%.8g ", nd.index, (double) nd.value));
+            o.push_back('\n');
+        }
     }
-    return s.str();
+    std::string text = s.str();
+    size_t total = text.size();
+    for (const std::string &o : run_text) total += o.size();
+    text.reserve(total);
+    for (const std::string &o : run_text) text += o;
+    return text;
 }
 
 void SvmModel::save_to_file(std::string path) {
@@ -248,26 +267,81 @@ void SvmModel::load_from_string(std::string data) {
             float_type v;
             while (ls >> v) linear_coef.push_back(v);
         } else if (key == "SV") {
+            // One line per support vector: `rows` coefficients, then index:value tokens (svmmodel.cpp:356-381).  The
+            // lines are most of a large model's text: they are cut into runs of whole lines and parsed side by side,
+            // each number the correctly rounded double of its text, as the stream extraction and sscanf("%lf") of the
+            // reference give.  Exactly total_sv lines are read; missing ones leave empty vectors with zero coefficients.
             const bool cls = param.svm_type == SvmParam::C_SVC || param.svm_type == SvmParam::NU_SVC;
             const int rows = cls ? n_classes - 1 : 1;
-            sv.clear();
+            sv.assign(n_total_sv, {});
             coef.assign((size_t) rows * n_total_sv, 0);
-            std::string line;
-            std::getline(iss, line);
-            for (int i = 0; i < n_total_sv; ++i) {
-                std::getline(iss, line);
-                std::stringstream ls(line);
-                for (int j = 0; j < rows; ++j) ls >> coef[(size_t) j * n_total_sv + i];
-                sv.emplace_back();
-                std::string tuple;
-                while (ls >> tuple) {
-                    int idx;
-                    double v;
-                    if (sscanf(tuple.c_str(), "%d:%lf", &idx, &v) != 2) throw std::runtime_error("error when loading model file");
-                    sv.back().emplace_back(idx, v);
-                    sv_max_index = std::max(sv_max_index, idx);
+            const char *text = data.c_str();
+            const size_t size = data.size();
+            size_t pos = (size_t) iss.tellg();
+            const char *nl0 = pos < size ? (const char *) memchr(text + pos, '\n', size - pos) : nullptr;
+            pos = nl0 ? (size_t) (nl0 - text) + 1 : size;                 // behind the rest of the "SV" line
+            const int n_runs = (int) std::max<size_t>(1, std::min<size_t>((size_t) omp_get_max_threads() * 4, (size - pos) >> 16));
+            std::vector<size_t> cut(n_runs + 1, size);
+            cut[0] = pos;
+            for (int r = 1; r < n_runs; ++r) {
+                const size_t from = std::max(cut[r - 1], pos + (size - pos) / n_runs * r);
+                const char *nl = from < size ? (const char *) memchr(text + from, '\n', size - from) : nullptr;
+                cut[r] = nl ? (size_t) (nl - text) + 1 : size;
+            }
+            std::vector<size_t> first_line(n_runs + 1, 0);                // lines (newlines) before each run
+#pragma omp parallel for schedule(static, 1)
+            for (int r = 0; r < n_runs; ++r) {
+                size_t c = 0;
+                for (const char *q = text + cut[r], *e = text + cut[r + 1]; q < e; ++c) {
+                    const char *nl = (const char *) memchr(q, '\n', e - q);
+                    if (!nl) break;
+                    q = nl + 1;
+                }
+                first_line[r + 1] = c;
+            }
+            for (int r = 0; r < n_runs; ++r) first_line[r + 1] += first_line[r];
+            std::vector<int> run_max(n_runs, 0);
+            std::vector<char> run_bad(n_runs, 0);
+#pragma omp parallel for schedule(dynamic, 1)
+            for (int r = 0; r < n_runs; ++r) {
+                const char *q = text + cut[r], *e = text + cut[r + 1];
+                std::vector<DataSet::node> row;
+                for (size_t i = first_line[r]; q < e && i < (size_t) n_total_sv; ++i) {
+                    const char *eol = (const char *) memchr(q, '\n', e - q);
+                    if (!eol) eol = e;
+                    const char *t;
+                    for (int j = 0; j < rows; ++j) {
+                        while (q < eol && tsvm::is_blank(*q)) ++q;
+                        if (q >= eol) break;                              // a short line: the other coefficients stay 0
+                        coef[(size_t) j * n_total_sv + i] = tsvm::parse_double(q, eol, &t);
+                        if (t == q) { run_bad[r] = 1; break; }
+                        q = t;
+                    }
+                    row.clear();
+                    while (!run_bad[r]) {
+                        while (q < eol && tsvm::is_blank(*q)) ++q;
+                        if (q >= eol) break;
+                        char *after;
+                        const long idx = strtol(q, &after, 10);
+                        if (after == q || after >= eol || *after != ':') { run_bad[r] = 1; break; }
+                        q = after + 1;
+                        if (q >= eol || tsvm::is_blank(*q)) { run_bad[r] = 1; break; }   // "index:" without a value
+                        const double v = tsvm::parse_double(q, eol, &t);
+                        if (t == q) { run_bad[r] = 1; break; }
+                        q = t;
+                        row.emplace_back((int) idx, v);
+                        run_max[r] = std::max(run_max[r], (int) idx);
+                    }
+                    if (run_bad[r]) break;
+                    sv[i].assign(row.begin(), row.end());
+                    q = eol + 1;
                 }
             }
+            for (int r = 0; r < n_runs; ++r) {
+                if (run_bad[r]) throw std::runtime_error("error when loading model file");
+                sv_max_index = std::max(sv_max_index, run_max[r]);
+            }
+            break;                                                        // nothing follows the support vectors
         }
     }
     if (param.svm_type != SvmParam::C_SVC && param.svm_type != SvmParam::NU_SVC) {
