@@ -36,7 +36,7 @@ typedef struct tsvm_param {
     int verbose;
     const int *weight_label;
     const double *weight;
-    int64_t cache_bytes;    /* HBM kernel-row cache budget: -1 = three quarters of the free device memory, 0 = off */
+    int64_t cache_bytes;    /* HBM kernel-row cache budget: -1 = nine tenths of the free device memory, 0 = off */
     int pair_lanes;         /* class pairs of a one-vs-one run in flight at a time: 0 = automatic (8 when each pair's local
                              * solver gets a compute unit of its own, else 3 pairs advanced in lockstep), 1 = one at a time */
 } tsvm_param;

@@ -44,7 +44,7 @@ std::recursive_mutex &device_work_mutex();
 class RowArena {
 public:
     static RowArena &instance();
-    // bytes a solve may use when the caller gave no explicit budget: three quarters of what is free or already held
+    // bytes a solve may use when the caller gave no explicit budget: nine tenths of what is free or already held
     size_t auto_budget();
     void *acquire(size_t bytes, bool auto_sized);
     void release();

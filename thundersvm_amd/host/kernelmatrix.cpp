@@ -28,13 +28,15 @@ size_t RowArena::auto_budget() {
     if (full_budget_) return cap_;   // the arena already is the budget: never chase small changes in free memory
     size_t free_b = 0, total_b = 0;
     TSVM_HIP_CHECK(hipMemGetInfo(&free_b, &total_b));
-    // Three quarters of what is free or already held, unless TSVM_ARENA_PERCENT (10..90) says otherwise: kernel rows
-    // are what the memory is for (hits grow in proportion to the slots, the set-up of a class pair or a prediction
-    // takes a few GB at most).  Half gave 1.80 s / 1.77 s on the seven-class and the regression benchmark, three
-    // quarters 1.71 / 1.63, 85 % 1.68 / 1.59; allocating the arena costs about 5 ms per GB, once per process.
+    // Nine tenths of what is free or already held, unless TSVM_ARENA_PERCENT (10..95) says otherwise: kernel rows
+    // are what the memory is for (hits grow in proportion to the slots; the set-up of a class pair or a prediction
+    // takes a few GB at most, and partial sums of predictions come out of the arena itself).  On the seven-class and
+    // the regression benchmark: half 1.80 s / 1.77 s, three quarters 1.71 / 1.63, 85 % 1.68 / 1.59 with the kernels
+    // of that time; with the present ones three quarters 1.576 / 1.586 (hits 46.8 % / 37.7 %), nine tenths
+    // 1.530 / 1.550 (50.9 % / 43.7 %).
     const char *e = getenv("TSVM_ARENA_PERCENT");
-    const int asked = e ? atoi(e) : 75;
-    const size_t pct = (size_t) (asked < 10 ? 10 : asked > 90 ? 90 : asked);
+    const int asked = e ? atoi(e) : 90;
+    const size_t pct = (size_t) (asked < 10 ? 10 : asked > 95 ? 95 : asked);
     return (free_b + cap_) / 100 * pct;
 }
 

@@ -53,7 +53,7 @@ public:
     mutable SolverStats stats;
     SolverTrace *trace = nullptr;
     bool profile = false;
-    // Budget of the HBM kernel-row cache in bytes: -1 = three quarters of the free device memory, 0 = no cache.
+    // Budget of the HBM kernel-row cache in bytes: -1 = nine tenths of the free device memory, 0 = no cache.
     long long cache_bytes = -1;
 
 protected:
