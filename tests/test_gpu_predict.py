@@ -141,3 +141,29 @@ def test_long_chunks_and_many_support_vectors(monkeypatch):
     gm, _ = _check(D.from_dense(x, y), D.from_dense(xt, np.zeros(len(xt))), make_param(svm_type=0, kernel_type=2, gamma=0.5, C=1.0),
                    monkeypatch)
     assert gm.total_sv > 8000
+
+
+def test_sparse_class_pair_whose_rows_are_all_empty():
+    """A wide, sparse three-class problem in which two classes' rows hold no feature at all: their class pair is a CSR
+    sub-problem without a single stored entry (every kernel value is kappa(0, 0)), so there is nothing to slice for the
+    CSR kernels; training and prediction still agree with the oracle."""
+    rng = np.random.default_rng(3)
+    ptr, col, val, y = [0], [], [], []
+    for i in range(12):
+        cls = i % 3 + 1
+        if cls == 3:
+            c = np.sort(rng.choice(np.arange(1, 400), 3, replace=False))
+            col += list(c)
+            val += list(rng.standard_normal(3).astype(np.float32))
+        ptr.append(len(col))
+        y.append(float(cls))
+    tr = D.CsrData(ptr, col, val, y)
+    xt = rng.standard_normal((4, 399)).astype(np.float32) * (rng.random((4, 399)) < 0.01)
+    te = D.from_dense(xt, np.zeros(4))
+    prm = make_param(svm_type=0, kernel_type=2, gamma=0.01, C=1.0)
+    gm = Model(0).train(tr, prm)
+    om = O.Model(tr.ptr, tr.col, tr.val, tr.y, _oparam(prm))
+    assert gm.total_sv == om.total_sv and np.array_equal(gm.coef, om.coef) and np.array_equal(gm.rho, om.rho)
+    _, gdec = gm.predict(te)
+    _, odec = om.predict(te.ptr, te.col, te.val, 100)
+    assert np.abs(gdec - odec).max() < 1e-6

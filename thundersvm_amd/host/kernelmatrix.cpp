@@ -162,6 +162,7 @@ void DeviceRows::build_sliced() {
     }
     // (a few very long rows would blow the padded copy up: then the plain CSR kernel stays in charge)
     if ((size_t) sp[n_slices] > 4 * nnz + 64 * n_slices) return;
+    if (sp[n_slices] == 0) return;   // every row is empty: nothing to slice, the plain kernel writes kappa(0, 0)
     slice_ptr.upload(sp);
     ell_col.resize((size_t) sp[n_slices]);
     ell_val.resize((size_t) sp[n_slices] * (values_fit_float ? sizeof(float) : sizeof(double)));
