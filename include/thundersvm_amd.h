@@ -286,6 +286,14 @@ int tsvm_nu_smo_solve(const int *y, const double *f_val, double *alpha, double *
                       const double *k_diag, double eps, double *diff, int max_iter, void *workspace,
                       tsvm_stream stream);
 
+/* Sends ids[0 .. n_ids) (device memory, e.g. what a selection has just written) to host memory the device can write
+ * (pinned and mapped: hipHostMalloc with hipHostMallocMapped, device pointer from hipHostGetDevicePointer), taken
+ * modulo fold_n when fold_n > 0, and then, behind a system-wide fence, writes `word` to host_ids[word_at]
+ * (word_at >= n_ids): a host thread that polls that word sees the ids once it sees the word.  It has no counterpart in
+ * the reference, whose select_working_set runs on the host (csmosolver.cpp:123-165); it replaces a device-to-host copy
+ * and the event behind it for callers that keep a host-side table of which kernel row lives where. */
+int tsvm_report_ids(const int *ids, int n_ids, int fold_n, int *host_ids, int word_at, int word, tsvm_stream stream);
+
 /* Bytes of device workspace tsvm_select_working_set needs for n instances. */
 size_t tsvm_select_workspace(int64_t n);
 

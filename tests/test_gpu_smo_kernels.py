@@ -377,3 +377,23 @@ def test_empty_inputs_are_no_ops():
     zeros = torch.zeros(4, dtype=torch.float64, device="cuda")
     capi.call("tsvm_update_f", G.ptr(f), G.ptr(zeros), 4, G.ptr(out), capi.ROW_F64, None, 8, 5, 1, G.stream())
     assert (G.host(f) == 3.0).all()
+
+
+def test_report_ids_to_host_memory():
+    """tsvm_report_ids: the ids land in host memory the device can write, folded when asked, and the word the host polls
+    is there once the stream has run (a host-side row store reads its new ids this way instead of through a copy)."""
+    rng = np.random.default_rng(4)
+    ids = rng.integers(0, 50000, size=512).astype(np.int32)
+    ids[7] = -1                                             # a side that ran dry leaves -1
+    ids_d = G.dev(ids)
+    host = torch.full((1024 + 16,), -7, dtype=torch.int32).pin_memory()
+    for n_ids, fold, word in [(512, 0, 1), (512, 20000, 2), (100, 0, 3), (0, 0, 4)]:
+        capi.call("tsvm_report_ids", G.ptr(ids_d), n_ids, fold, host.data_ptr(), 1024, word, G.stream())
+        torch.cuda.synchronize()
+        got = host.numpy()
+        want = ids[:n_ids].copy()
+        if fold:
+            want[want >= 0] %= fold
+        assert np.array_equal(got[:n_ids], want) and got[1024] == word
+    with pytest.raises(capi.TsvmError):
+        capi.call("tsvm_report_ids", G.ptr(ids_d), 600, 0, host.data_ptr(), 512, 1, G.stream())      # the word would lie inside the ids

@@ -61,6 +61,7 @@ SIGNATURES = {
     "tsvm_c_smo_solve_block_on_xcd": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _dbl, _p, _int, _p, _dbl, _p, _int, _p, _int, _int, _p]),
     "tsvm_nu_smo_solve_block_on_xcd": (_int, [_p, _p, _p, _p, _p, _int, _dbl, _p, _int, _p, _dbl, _p, _int, _p, _int, _int, _p]),
     "tsvm_select_workspace": (C.c_size_t, [_i64]),
+    "tsvm_report_ids": (_int, [_p, _int, _int, _p, _int, _int, _p]),
     "tsvm_select_working_set": (_int, [_p, _p, _p, _i64, _dbl, _dbl, _p, _int, _p, _int, _int, _p, _p]),
     "tsvm_select_working_set_again": (_int, [_p, _p, _p, _i64, _dbl, _dbl, _p, _int, _p, _int, _int, _p, _p]),
     "tsvm_select_working_set_folded": (_int, [_p, _p, _p, _i64, _dbl, _dbl, _p, _int, _p, _int, _int, _p, _int, _int, _p, _p]),

@@ -727,6 +727,23 @@ __global__ __launch_bounds__(MAX_WS) void sel_final_kernel(SelWorkspace w, int64
     }
 }
 
+// The ids a selection has just written, sent to the host by the device itself: host_ids is host memory the device
+// can write (pinned, mapped); the ids go there (modulo fold_n when fold_n > 0) and then, behind a system-wide fence,
+// `word` goes to host_ids[word_at], which the host polls.  One small kernel in stream order behind the selection,
+// in place of a copy, an event and the wake-up of a thread that sleeps on it.
+__global__ __launch_bounds__(256) void report_ids_kernel(const int *__restrict__ ids, int n_ids, int fold_n,
+                                                         int *__restrict__ host_ids, int word_at, int word) {
+    for (int t = threadIdx.x; t < n_ids; t += 256) {
+        const int id = ids[t];
+        host_ids[t] = fold_n > 0 && id >= 0 ? id % fold_n : id;
+    }
+    __threadfence_system();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        __hip_atomic_store(&host_ids[word_at], word, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // C ABI
 // ------------------------------------------------------------------------------------------------
@@ -858,6 +875,15 @@ int tsvm_update_f_select(double *f, const double *alpha_diff, int ws_size, const
     TSVM_LAUNCH_CHECK();
     return select_working_set(f, y, alpha, n, Cp, Cn, marked, n_marked, out, n_select, nu, workspace, true,
                               out_folded ? (int) n_cols : 0, out_folded, 1, stream);
+}
+
+int tsvm_report_ids(const int *ids, int n_ids, int fold_n, int *host_ids, int word_at, int word, tsvm_stream stream) {
+    TSVM_REQUIRE(ids && host_ids, "tsvm_report_ids: null pointer");
+    TSVM_REQUIRE(n_ids >= 0 && n_ids <= MAX_WS && word_at >= n_ids && fold_n >= 0, "tsvm_report_ids: bad size (n_ids=%d word_at=%d fold_n=%d)",
+                 n_ids, word_at, fold_n);
+    hipLaunchKernelGGL(report_ids_kernel, dim3(1), dim3(256), 0, tsvm_s(stream), ids, n_ids, fold_n, host_ids, word_at, word);
+    TSVM_LAUNCH_CHECK();
+    return 0;
 }
 
 size_t tsvm_select_workspace(int64_t n) {

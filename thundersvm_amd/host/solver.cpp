@@ -177,7 +177,7 @@ struct SolveTask::Impl {
     // The chip-wide work of a task is enqueued on stream `sa` (`ids` is the stream the newly selected ids are read
     // back on for the host-side cache bookkeeping: the same one).
     hipStream_t sa = nullptr, ids = nullptr;
-    hipEvent_t selected = nullptr, ids_ready = nullptr, diff_ready = nullptr;
+    hipEvent_t selected = nullptr, diff_ready = nullptr;
     // A task that runs alone splits the chip: the local solver (one workgroup, a chain of dependent steps) gets a
     // stream `ss` restricted to one CU of every XCD, everything else runs on `sa`, restricted to the other CUs.
     // The solver then runs next to this iteration's get_rows at nearly its stand-alone speed; sharing CUs with a
@@ -214,6 +214,7 @@ struct SolveTask::Impl {
     DeviceBuffer<int> d_cache_state;                  // slots in use, rows to compute
     int *h_cache_info = nullptr, *d_cache_info = nullptr;   // the same two numbers in pinned host memory
     int *h_ids = nullptr, *h_slots = nullptr;
+    int *d_ids_host = nullptr;   // h_ids as the device addresses it
     // diff (the solver's 16 bytes for the host, smo_kernel.cpp:87,120) lives in pinned host memory that the device
     // writes directly: no copy in the stream between update_f and the next selection
     double *h_diff = nullptr, *d_diff = nullptr;
@@ -271,12 +272,39 @@ struct SolveTask::Impl {
         }
         return false;
     }
+    // The new ids come to the host from the device itself (tsvm_report_ids, in stream order behind the selection):
+    // h_ids[ws_size] takes the number of the report once its ids are in h_ids.
+    int ids_seq = 0;
     bool ids_arrived() const {
         if (!(caching && !all_cached && !device_cache)) return true;
-        const hipError_t e = hipEventQuery(ids_ready);
-        if (e == hipSuccess) return true;
-        if (e != hipErrorNotReady) TSVM_HIP_CHECK(e);
-        return false;
+        if (*(volatile int *) (h_ids + ws_size) != ids_seq) return false;
+        __atomic_thread_fence(__ATOMIC_ACQUIRE);
+        return true;
+    }
+    void wait_for_ids() {
+        using clock = std::chrono::steady_clock;
+        const auto start = clock::now();
+        auto next_check = start + std::chrono::milliseconds(200);
+        for (unsigned long long spins = 1; !ids_arrived(); ++spins) {
+            if (spins % 4096 != 0) continue;
+            const auto now = clock::now();
+            if (now < next_check) continue;
+            next_check = now + std::chrono::milliseconds(200);
+            const hipError_t e = hipStreamQuery(ids);
+            if (e == hipSuccess) {
+                if (!ids_arrived()) {
+                    abandoned = true;
+                    throw std::runtime_error("SolveTask: the selection finished without reporting its ids");
+                }
+            } else if (e != hipErrorNotReady) {
+                abandoned = true;
+                TSVM_HIP_CHECK(e);
+            }
+            if (now - start > std::chrono::milliseconds(tsvm::solver_timeout_ms())) {
+                abandoned = true;
+                throw std::runtime_error("SolveTask: no ids from the selection (TSVM_SOLVER_TIMEOUT_MS); the device may be hung");
+            }
+        }
     }
     int rotation_base = 0;   // iteration at which d_slots_a was valid
     long long window_lookups = 0, window_hits = 0, window_first = 0, first_touches = 0;
@@ -331,7 +359,6 @@ struct SolveTask::Impl {
         // anything else of the iteration, so it waits for nothing but the selection.
         ids = sa;
         TSVM_HIP_CHECK(hipEventCreateWithFlags(&selected, hipEventDisableTiming));
-        TSVM_HIP_CHECK(hipEventCreateWithFlags(&ids_ready, hipEventDisableTiming));
         TSVM_HIP_CHECK(hipEventCreateWithFlags(&diff_ready, hipEventDisableTiming));
         TSVM_HIP_CHECK(hipEventCreateWithFlags(&block_done, hipEventDisableTiming));
         TSVM_HIP_CHECK(hipEventCreateWithFlags(&solved, hipEventDisableTiming));
@@ -375,7 +402,9 @@ struct SolveTask::Impl {
         cur_ids.resize(ws_size);
         TSVM_HIP_CHECK(hipHostMalloc((void **) &h_diff, 2 * sizeof(double), hipHostMallocMapped | hipHostMallocCoherent));
         TSVM_HIP_CHECK(hipHostGetDevicePointer((void **) &d_diff, h_diff, 0));
-        TSVM_HIP_CHECK(hipHostMalloc((void **) &h_ids, ws_size * sizeof(int)));
+        TSVM_HIP_CHECK(hipHostMalloc((void **) &h_ids, (ws_size + 16) * sizeof(int), hipHostMallocMapped | hipHostMallocCoherent));
+        TSVM_HIP_CHECK(hipHostGetDevicePointer((void **) &d_ids_host, h_ids, 0));
+        h_ids[ws_size] = 0;
         TSVM_HIP_CHECK(hipHostMalloc((void **) &h_slots, 3 * ws_size * sizeof(int)));
         h_diff[0] = h_diff[1] = 0;
         if (!caching) {
@@ -425,7 +454,6 @@ struct SolveTask::Impl {
         if (block_done) (void) hipEventDestroy(block_done);
         if (solved) (void) hipEventDestroy(solved);
         if (selected) (void) hipEventDestroy(selected);
-        if (ids_ready) (void) hipEventDestroy(ids_ready);
         if (diff_ready) (void) hipEventDestroy(diff_ready);
         if (h_diff) (void) hipHostFree(h_diff);
         if (h_cache_info) (void) hipHostFree(h_cache_info);
@@ -524,10 +552,8 @@ struct SolveTask::Impl {
         ws_off = sel_off;
         timer.end(stats.ms_select);
         if (caching && !all_cached && !device_cache) {
-            // the new ids travel to the host, on their own stream if there is one
-            if (ids != sa) TSVM_HIP_CHECK(hipStreamWaitEvent(ids, selected, 0));
-            TSVM_HIP_CHECK(hipMemcpyAsync(h_ids, ws_ids() + first_new, sizeof(int) * n_new, hipMemcpyDeviceToHost, ids));
-            TSVM_HIP_CHECK(hipEventRecord(ids_ready, ids));
+            // the new ids travel to the host: written there by a small kernel behind the selection
+            abi_check(tsvm_report_ids(ws_ids() + first_new, n_new, 0, d_ids_host, ws_size, ++ids_seq, ids));
         }
     }
 
@@ -549,7 +575,7 @@ struct SolveTask::Impl {
             slots = d_slots_a.data();
         } else if (caching) {
             // look the new ids up and compute only the rows that are not cached
-            TSVM_HIP_CHECK(hipEventSynchronize(ids_ready));
+            wait_for_ids();
             if (iter > 0) {
                 // the first half of the previous working set leaves; the second half moves up and stays pinned
                 for (int t = 0; t < q; ++t) cache.release(cur_slots[t]);
