@@ -575,9 +575,9 @@ struct SolveTask::Impl {
             slots = d_slots_a.data();
         } else if (caching) {
             // look the new ids up and compute only the rows that are not cached
-            wait_for_ids();
             if (iter > 0) {
                 // the first half of the previous working set leaves; the second half moves up and stays pinned
+                // (known without the new ids: done while they are still on their way)
                 for (int t = 0; t < q; ++t) cache.release(cur_slots[t]);
                 for (int t = 0; t < q; ++t) {
                     cur_ids[t] = cur_ids[t + q];
@@ -586,6 +586,7 @@ struct SolveTask::Impl {
             }
             miss_ids.clear();
             miss_slots.clear();
+            wait_for_ids();
             for (int t = 0; t < n_new; ++t) {
                 const int id = h_ids[t] % n_u;   // a second member with the same folded id hits the slot just assigned
                 int s = cache.lookup(id);
