@@ -292,7 +292,9 @@ def cli_and_loader(w, run_cli=True, loader_threads=(1, 0)):
                                   note="fresh process: the training window holds the first allocation of the row arena, the "
                                        "creation of the CU-masked streams and the loading of the kernels' code objects; the "
                                        "executable takes half of the free device memory for kernel rows (a process that trains "
-                                       "once pays the arena's allocation and release once), the library nine tenths")
+                                       "once pays the arena's allocation and release once), the library nine tenths; on a device "
+                                       "whose memory another process has just given back (a test run right before, say) the "
+                                       "arena's allocation waits for the driver to clear it: 2.5 to 4 s more")
                 if w.get("test") is not None:
                     # thundersvm-predict on the model just written and the workload's test rows as text
                     test_path, pred_path = os.path.join(tmp, "test.txt"), os.path.join(tmp, "test.predict")
