@@ -291,7 +291,7 @@ def cli_and_loader(w, run_cli=True, loader_threads=(1, 0)):
                                   model_bytes=os.path.getsize(model),
                                   note="fresh process: the training window holds the first allocation of the row arena, the "
                                        "creation of the CU-masked streams and the loading of the kernels' code objects; the "
-                                       "executable takes half of the free device memory for kernel rows (a process that trains "
+                                       "executable takes 45 % of the free device memory for kernel rows (a process that trains "
                                        "once pays the arena's allocation and release once), the library nine tenths; on a device "
                                        "whose memory another process has just given back (a test run right before, say) the "
                                        "arena's allocation waits for the driver to clear it: 2.5 to 4 s more")

@@ -17,11 +17,14 @@ int main(int argc, char **argv) {
         fprintf(stderr, "%s\n%s", e.what(), CMDParser::train_usage());
         return 1;
     }
-    // A process that trains once and exits pays for the row arena's allocation and release once per training: about
-    // 5 ms per GB up to three quarters of the device's memory and 30 ms per GB beyond (216 GB: 0.5 s at exit, 258 GB:
-    // 1.8 s).  The library's default (nine tenths of the free memory) suits processes that train again and again; here
-    // half is taken unless the environment says otherwise.
-    setenv("TSVM_ARENA_PERCENT", "50", 0);
+    // A process that trains once and exits pays for the row arena's allocation and release once per training: the
+    // release alone takes 0.5 s for three quarters of the device's memory and 1.8 s for nine tenths, and the driver clears
+    // released memory in the background (about 40 GB/s) before it hands it out again, so a process that asks for more
+    // than the untouched rest right after another has exited waits for that (two such runs with half of the memory
+    // each: the second trains in 5.8 s instead of 1.75 s).  The library's default (nine tenths of the free memory) suits
+    // processes that train again and again; here less than half is taken unless the environment says otherwise, so that
+    // one run after another finds an untouched half.
+    setenv("TSVM_ARENA_PERCENT", "45", 0);
     try {
         tsvm::Log::enabled() = !parser.quiet;
         DataSet train;
